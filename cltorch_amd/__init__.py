@@ -1,0 +1,13 @@
+"""MI355X-native backend behind cltorch's ``torch.ClTensor`` operator API.
+
+``libthcl_hip.so`` (built by ``python -m cltorch_amd.build``) is the product: a
+C-ABI library exporting the reference's ``THClTensor_*`` entry points for the
+pointwise / copy / reduce / addmm path.  ``ClTensor`` mirrors the Lua methods
+on top of it.  Importing this package does not touch a GPU; the first tensor
+does, and raises if no device or no built library is present.
+"""
+from .tensor import (ClError, ClTensor, finish, getDeviceCount, mm, setAddFinish, state,  # noqa: F401
+                     synchronize)
+from . import _lib  # noqa: F401
+
+__all__ = ["ClTensor", "ClError", "mm", "synchronize", "finish", "getDeviceCount", "setAddFinish", "state"]

@@ -1,0 +1,328 @@
+// Pointwise apply engine, host side + the ahead-of-time kernels.
+//
+// Mirrors THClTensor_pointwiseApply (reference: src/lib/THClApply.cpp:145-240):
+// element counts must agree, at most 25 dims, a written operand that overlaps
+// itself is staged through a dense temporary.  What differs is the planning:
+// instead of one kernel shape specialised per (dims...) tuple, a call is
+// classified into one of five kernel families (dense 128-bit, dense scalar,
+// joint-strided 128-bit, joint-strided scalar, per-operand generic).
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "apply_device.h"
+#include "internal.h"
+
+namespace {
+
+enum PlanKind { K_CONTIG_V4 = 0, K_CONTIG_S, K_JOINT_V4, K_JOINT_S, K_GENERIC, K_NONE };
+const char *const kKindSuffix[] = {"_contig_v4", "_contig_s", "_joint_v4", "_joint_s", "_generic"};
+
+struct ApplyPlan {
+  PlanKind kind = K_NONE;
+  unsigned grid = 0;
+  thcl_rt *rt = nullptr;
+  ThclContigParams c;
+  ThclJointParams j;
+  ThclGenericParams g;
+};
+
+constexpr unsigned kMaxGrid = 1u << 22;
+constexpr long kUnitsPerTile = THCL_APPLY_THREADS * THCL_APPLY_UNROLL;
+
+
+bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+
+// Fills `plan`; returns false when there is nothing to launch.
+bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan) {
+  const int n = call.n;
+  THClTensor *const *t = call.t;
+  const long total = THClTensor_nElement(state, t[0]);
+  for (int i = 1; i < n; i++)
+    THCL_CHECK(THClTensor_nElement(state, t[i]) == total, "element size mismatch between tensors 1 and %d", i + 1);
+  for (int i = 0; i < n; i++)
+    THCL_CHECK(t[i]->nDimension <= THCL_MAX_DIMS, "Apply: too many dimensions in tensor %d", i + 1);
+  if (total == 0) return false;
+  for (int i = 0; i < n; i++)
+    THCL_CHECK(t[i]->storage && t[i]->storage->wrapper, "tensor %d has no device storage", i + 1);
+  thcl_check_same_device(state, 3, t[0], n > 1 ? t[1] : nullptr, n > 2 ? t[2] : nullptr);
+  plan.rt = thcl_ctx(state, t[0]->storage->device);
+
+  float *p[3] = {nullptr, nullptr, nullptr};
+  for (int i = 0; i < n; i++) p[i] = thcl_dptr(t[i]);
+
+  bool all_contig = true;
+  for (int i = 0; i < n; i++) all_contig = all_contig && THClTensor_isContiguous(state, t[i]);
+
+  JointLayout J;
+  if (!all_contig) {
+    J = thcl_joint_collapse(n, t);
+    if (J.valid && J.dims == 1) {
+      bool unit = true;
+      for (int i = 0; i < n; i++) unit = unit && J.strides[i][0] == 1;
+      if (unit) all_contig = true;  // e.g. identically transposed views of dense tensors
+    }
+  }
+
+  if (all_contig) {
+    bool al = true;
+    for (int i = 0; i < n; i++) al = al && aligned16(p[i]);
+    plan.kind = al ? K_CONTIG_V4 : K_CONTIG_S;
+    ThclContigParams &c = plan.c;
+    memset(&c, 0, sizeof(c));
+    for (int i = 0; i < 3; i++) c.p[i] = p[i];
+    c.pt[0] = call.pt[0];
+    c.pt[1] = call.pt[1];
+    c.val[0] = call.val[0];
+    c.val[1] = call.val[1];
+    c.n = (thcl_u64)total;
+    const long units = al ? (total >> 2) : total;
+    const long tiles = (units + kUnitsPerTile - 1) / kUnitsPerTile;
+    c.ntiles = (thcl_u64)tiles;
+    plan.grid = (unsigned)(tiles < 1 ? 1 : (tiles > kMaxGrid ? kMaxGrid : tiles));
+    return true;
+  }
+
+  // strided paths index with 32 bits
+  THCL_CHECK(total < (1l << 31), THCL_DIM_WARNING);
+
+  bool joint_ok = J.valid && J.dims <= THCL_JOINT_MAX_DIMS;
+  if (joint_ok)
+    for (int i = 0; i < n && joint_ok; i++)
+      for (int d = 0; d < J.dims; d++)
+        if (J.strides[i][d] < 0 || J.strides[i][d] >= (1l << 32)) joint_ok = false;
+
+  if (joint_ok) {
+    const int last = J.dims - 1;
+    bool vec = (J.sizes[last] % 4 == 0);
+    for (int i = 0; i < n && vec; i++) {
+      vec = vec && J.strides[i][last] == 1 && aligned16(p[i]);
+      for (int d = 0; d < last; d++) vec = vec && (J.strides[i][d] % 4 == 0);
+    }
+    plan.kind = vec ? K_JOINT_V4 : K_JOINT_S;
+    ThclJointParams &j = plan.j;
+    memset(&j, 0, sizeof(j));
+    for (int i = 0; i < 3; i++) j.p[i] = p[i];
+    j.pt[0] = call.pt[0];
+    j.pt[1] = call.pt[1];
+    j.val[0] = call.val[0];
+    j.val[1] = call.val[1];
+    j.dims = J.dims;
+    const long units = vec ? total / 4 : total;
+    j.nunits = (thcl_u32)units;
+    for (int d = 0; d < J.dims; d++) {
+      long s = J.sizes[d];
+      if (vec && d == last) s /= 4;
+      j.size[d] = thcl_make_divisor(s);
+      for (int i = 0; i < n; i++) j.stride[i][d] = (thcl_u32)J.strides[i][d];
+    }
+    const long tiles = (units + kUnitsPerTile - 1) / kUnitsPerTile;
+    j.ntiles = (thcl_u32)tiles;
+    plan.grid = (unsigned)(tiles > kMaxGrid ? kMaxGrid : tiles);
+    return true;
+  }
+
+  plan.kind = K_GENERIC;
+  ThclGenericParams &g = plan.g;
+  memset(&g, 0, sizeof(g));
+  for (int i = 0; i < 3; i++) g.p[i] = p[i];
+  g.pt[0] = call.pt[0];
+  g.pt[1] = call.pt[1];
+  g.val[0] = call.val[0];
+  g.val[1] = call.val[1];
+  g.n = (thcl_u32)total;
+  for (int i = 0; i < n; i++) {
+    Layout L = thcl_collapse(t[i]);
+    g.op[i].dims = L.dims;
+    for (int d = 0; d < L.dims; d++) {
+      THCL_CHECK(L.strides[d] >= 0 && L.strides[d] < (1l << 32), THCL_DIM_WARNING);
+      g.op[i].size[d] = thcl_make_divisor(L.sizes[d]);
+      g.op[i].stride[d] = (thcl_u32)L.strides[d];
+    }
+  }
+  const long tiles = (total + kUnitsPerTile - 1) / kUnitsPerTile;
+  g.ntiles = (thcl_u32)tiles;
+  plan.grid = (unsigned)(tiles > kMaxGrid ? kMaxGrid : tiles);
+  return true;
+}
+
+// ---------------------------------------------------------- fixed kernels ---
+#define X(name, nt, stmt)                                                                             \
+  struct Op_##name {                                                                                  \
+    static constexpr int NT = nt;                                                                     \
+    static __device__ __forceinline__ void run(float &o, float a, float b, float v1, float v2, float p1, \
+                                               float p2) {                                            \
+      (void)a; (void)b; (void)v1; (void)v2; (void)p1; (void)p2;                                        \
+      stmt;                                                                                           \
+    }                                                                                                 \
+  };
+THCL_FIXED_OPS(X)
+#undef X
+}  // namespace
+
+#define X(name, nt, stmt) THCL_DEFINE_APPLY_KERNELS(thcl_k_##name, Op_##name, nt)
+THCL_FIXED_OPS(X)
+#undef X
+
+namespace {
+struct KernelSet {
+  int nt;
+  void (*contig_v4)(ThclContigParams);
+  void (*contig_s)(ThclContigParams);
+  void (*joint_v4)(ThclJointParams);
+  void (*joint_s)(ThclJointParams);
+  void (*generic)(ThclGenericParams);
+};
+const KernelSet kFixed[OP_COUNT] = {
+#define X(name, nt, stmt) \
+  {nt, thcl_k_##name##_contig_v4, thcl_k_##name##_contig_s, thcl_k_##name##_joint_v4, thcl_k_##name##_joint_s, thcl_k_##name##_generic},
+    THCL_FIXED_OPS(X)
+#undef X
+};
+
+void launch_fixed(const KernelSet &ks, ApplyPlan &plan) {
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(plan.rt);
+  dim3 grid(plan.grid), block(THCL_APPLY_THREADS);
+  switch (plan.kind) {
+    case K_CONTIG_V4: hipLaunchKernelGGL(ks.contig_v4, grid, block, 0, stream, plan.c); break;
+    case K_CONTIG_S: hipLaunchKernelGGL(ks.contig_s, grid, block, 0, stream, plan.c); break;
+    case K_JOINT_V4: hipLaunchKernelGGL(ks.joint_v4, grid, block, 0, stream, plan.j); break;
+    case K_JOINT_S: hipLaunchKernelGGL(ks.joint_s, grid, block, 0, stream, plan.j); break;
+    case K_GENERIC: hipLaunchKernelGGL(ks.generic, grid, block, 0, stream, plan.g); break;
+    default: return;
+  }
+  hipError_t e = hipGetLastError();
+  THCL_CHECK(e == hipSuccess, "apply kernel launch failed: %s", hipGetErrorString(e));
+}
+
+void launch_expr(THClState *state, const std::string &expr, int nt, ApplyPlan &plan) {
+  std::string key = std::to_string(nt) + "|" + expr;
+  std::string entry = std::string("thcl_user") + kKindSuffix[plan.kind];
+  std::string source;
+  if (!thcl_rt_kernel_cached(plan.rt, key.c_str())) source = thcl_expr_source(expr, nt);
+  thcl_rt_kernel *k = thcl_rt_kernel_get(plan.rt, key.c_str(), source.c_str(), entry.c_str());
+  THCL_CHECK(k != nullptr, "%s", thcl_rt_error());
+  void *params = nullptr;
+  size_t bytes = 0;
+  switch (plan.kind) {
+    case K_CONTIG_V4:
+    case K_CONTIG_S: params = &plan.c; bytes = sizeof(plan.c); break;
+    case K_JOINT_V4:
+    case K_JOINT_S: params = &plan.j; bytes = sizeof(plan.j); break;
+    default: params = &plan.g; bytes = sizeof(plan.g); break;
+  }
+  THCL_CHECK(thcl_rt_launch(plan.rt, k, plan.grid, 1, 1, THCL_APPLY_THREADS, 1, 1, 0, params, bytes) == 0, "%s",
+             thcl_rt_error());
+  (void)state;
+}
+
+// Runs `body(call)` with operand 0 replaced by a dense temporary when it
+// aliases itself, then scatters the temporary back (any writer may win), as
+// the reference does (src/lib/THClApply.cpp:183-190,231-237).
+template <class F>
+void with_overlap_fixup(THClState *state, ApplyCall &call, F body) {
+  THClTensor *orig = nullptr;
+  if (!call.ignore_overlap && call.t[0]->nDimension > 0 && thcl_overlapping(call.t[0])) {
+    orig = call.t[0];
+    call.t[0] = THClTensor_newContiguous(state, orig);
+  }
+  try {
+    body(call);
+  } catch (...) {
+    if (orig) {
+      THClTensor_free(state, call.t[0]);
+      call.t[0] = orig;
+    }
+    throw;
+  }
+  if (orig) {
+    ApplyCall back;
+    back.n = 2;
+    back.t[0] = orig;
+    back.t[1] = call.t[0];
+    back.ignore_overlap = true;
+    thcl_apply_fixed(state, OP_COPY, back);
+    THClTensor_free(state, call.t[0]);
+    call.t[0] = orig;
+  }
+}
+}  // namespace
+
+void thcl_apply_fixed(THClState *state, ThclOp op, ApplyCall &call) {
+  THCL_CHECK(op >= 0 && op < OP_COUNT, "unknown operator %d", (int)op);
+  const KernelSet &ks = kFixed[op];
+  THCL_CHECK(ks.nt == call.n, "operator %d takes %d tensors, got %d", (int)op, ks.nt, call.n);
+  with_overlap_fixup(state, call, [&](ApplyCall &c) {
+    ApplyPlan plan;
+    if (!make_plan(state, c, plan)) return;
+    launch_fixed(ks, plan);
+    thcl_after_launch(state, plan.rt);
+  });
+}
+
+void thcl_apply_expr(THClState *state, const std::string &expr, ApplyCall &call) {
+  with_overlap_fixup(state, call, [&](ApplyCall &c) {
+    ApplyPlan plan;
+    if (!make_plan(state, c, plan)) return;
+    launch_expr(state, expr, c.n, plan);
+    thcl_after_launch(state, plan.rt);
+  });
+}
+
+void thcl_fill_contig(thcl_rt *rt, float *dst, float value, long n) {
+  if (n <= 0) return;
+  ApplyPlan plan;
+  plan.rt = rt;
+  ThclContigParams &c = plan.c;
+  memset(&c, 0, sizeof(c));
+  c.p[0] = dst;
+  c.val[0] = value;
+  c.n = (thcl_u64)n;
+  const bool al = aligned16(dst);
+  plan.kind = al ? K_CONTIG_V4 : K_CONTIG_S;
+  const long units = al ? (n >> 2) : n;
+  const long tiles = (units + kUnitsPerTile - 1) / kUnitsPerTile;
+  c.ntiles = (thcl_u64)tiles;
+  plan.grid = (unsigned)(tiles < 1 ? 1 : (tiles > kMaxGrid ? kMaxGrid : tiles));
+  launch_fixed(kFixed[OP_FILL], plan);
+}
+
+// ------------------------------------------------------------ test hooks ---
+// Host-only helpers so the layout logic can be checked without a device.
+extern "C" {
+unsigned thcl_dbg_divide(unsigned n, long d) {
+  ThclDivisor dv = thcl_make_divisor(d);
+  return (unsigned)((((unsigned long long)n * dv.magic) >> 32) + n) >> dv.shift;
+}
+
+// kind of kernel a call with these layouts would use; -1 when invalid.
+// ptr_align[i]: byte misalignment to assume for operand i's first element.
+int thcl_dbg_plan_kind(int n, const int *ndims, const long *sizes, const long *strides, const long *offsets,
+                       int *out_dims, long *out_sizes, long *out_strides) {
+  THClTensor hdr[3];
+  THClTensor *tp[3];
+  THClStorage st[3];
+  long sz[3][THCL_MAX_DIMS], sd[3][THCL_MAX_DIMS];
+  for (int i = 0; i < n; i++) {
+    memset(&hdr[i], 0, sizeof(THClTensor));
+    memset(&st[i], 0, sizeof(THClStorage));
+    for (int d = 0; d < ndims[i]; d++) {
+      sz[i][d] = sizes[i * THCL_MAX_DIMS + d];
+      sd[i][d] = strides[i * THCL_MAX_DIMS + d];
+    }
+    hdr[i].size = sz[i];
+    hdr[i].stride = sd[i];
+    hdr[i].nDimension = ndims[i];
+    hdr[i].storageOffset = offsets[i];
+    tp[i] = &hdr[i];
+  }
+  JointLayout J = thcl_joint_collapse(n, tp);
+  if (!J.valid) return -1;
+  *out_dims = J.dims;
+  for (int d = 0; d < J.dims; d++) {
+    out_sizes[d] = J.sizes[d];
+    for (int i = 0; i < n; i++) out_strides[i * THCL_MAX_DIMS + d] = J.strides[i][d];
+  }
+  return J.dims;
+}
+}

@@ -1,0 +1,320 @@
+// Device side of the pointwise apply engine.  This text is compiled twice: by
+// hipcc for the fixed operators, and at run time by hipRTC with a user
+// expression wrapped into an operator struct.  It therefore includes nothing
+// and uses only built-in types.
+//
+// What it replaces: the templated OpenCL kernel THClTensor_pointwiseApplyD
+// (reference: src/lib/THClApply.cl:47-102), one work-item per element with a
+// `%`,`/` chain per operand and per dimension.  Here:
+//   * contiguous operands move as 128-bit vectors, several in flight per lane;
+//   * same-shaped strided operands share one index decomposition (joint
+//     layout), done per 4-element unit when the innermost run allows it, with
+//     multiply-shift division;
+//   * operands of different shapes fall back to one decomposition per operand.
+//
+// An operator is a struct with
+//   static constexpr int NT;   // tensors it touches (1..3), operand 0 is written
+//   static __device__ void run(float &o, float a, float b, float v1, float v2, float p1, float p2);
+// `o` holds operand 0's old value on entry; loads whose value the operator
+// never reads are removed by the compiler, so write-only operators (fill,
+// copy) cost no read of operand 0.
+#ifndef THCL_APPLY_DEVICE_H
+#define THCL_APPLY_DEVICE_H
+
+#define THCL_APPLY_THREADS 256
+#define THCL_APPLY_UNROLL 4
+#define THCL_JOINT_MAX_DIMS 8
+#define THCL_GENERIC_MAX_DIMS 25
+
+typedef float thcl_f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int thcl_u32;
+typedef unsigned long long thcl_u64;
+
+// n / d for n < 2^31 by multiply-high and shift (d >= 1).
+struct ThclDivisor {
+  thcl_u32 d, magic, shift, pad;
+};
+__device__ __forceinline__ thcl_u32 thcl_div(thcl_u32 n, const ThclDivisor &dv) {
+  return (__umulhi(n, dv.magic) + n) >> dv.shift;
+}
+#ifndef __HIPCC_RTC__
+// host side: magic = floor(2^32 * (2^shift - d) / d) + 1 with 2^shift >= d
+inline ThclDivisor thcl_make_divisor(long d) {
+  ThclDivisor r;
+  r.d = (thcl_u32)d;
+  unsigned shift = 0;
+  while (shift < 32 && (1ull << shift) < (unsigned long long)d) shift++;
+  const unsigned long long magic =
+      ((1ull << 32) * ((1ull << shift) - (unsigned long long)d)) / (unsigned long long)d + 1;
+  r.magic = (thcl_u32)magic;
+  r.shift = shift;
+  r.pad = 0;
+  return r;
+}
+#endif
+
+struct ThclContigParams {
+  float *p[3];
+  const float *pt[2];
+  float val[2];
+  thcl_u64 n;       // elements
+  thcl_u64 ntiles;  // tiles of THREADS*UNROLL units
+};
+
+struct ThclJointParams {
+  float *p[3];
+  const float *pt[2];
+  float val[2];
+  thcl_u32 nunits;  // units = n / VEC
+  thcl_u32 ntiles;
+  int dims;
+  ThclDivisor size[THCL_JOINT_MAX_DIMS];       // in units along the innermost dim
+  thcl_u32 stride[3][THCL_JOINT_MAX_DIMS];     // in elements
+};
+
+struct ThclGenericOperand {
+  int dims;
+  int pad;
+  ThclDivisor size[THCL_GENERIC_MAX_DIMS];
+  thcl_u32 stride[THCL_GENERIC_MAX_DIMS];
+  thcl_u32 pad2;
+};
+struct ThclGenericParams {
+  float *p[3];
+  const float *pt[2];
+  float val[2];
+  thcl_u32 n;
+  thcl_u32 ntiles;
+  ThclGenericOperand op[3];
+};
+
+template <class Op>
+__device__ __forceinline__ void thcl_apply_one(float &o, float a, float b, float v1, float v2, float p1, float p2) {
+  Op::run(o, a, b, v1, v2, p1, p2);
+}
+
+// ------------------------------------------------------------ contiguous ---
+// All operands dense and 16-byte aligned.  A tile is THREADS*UNROLL float4
+// units; lane l of a block touches units l, l+THREADS, ... so every wave reads
+// whole 1 KiB lines.  Loads of a tile are issued before any arithmetic.
+template <class Op, int NT>
+__device__ __forceinline__ void thcl_apply_contig_v4(const ThclContigParams &P) {
+  const float p1 = P.pt[0] ? *P.pt[0] : 0.f;
+  const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
+  const float v1 = P.val[0], v2 = P.val[1];
+  const thcl_u64 n4 = P.n >> 2;
+  thcl_f4 *o4 = (thcl_f4 *)P.p[0];
+  const thcl_f4 *a4 = (const thcl_f4 *)P.p[1];
+  const thcl_f4 *b4 = (const thcl_f4 *)P.p[2];
+  for (thcl_u64 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
+    const thcl_u64 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
+    thcl_f4 o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
+    if (base + (THCL_APPLY_UNROLL - 1) * THCL_APPLY_THREADS < n4) {
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+        const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
+        o[k] = __builtin_nontemporal_load(o4 + i);
+        if (NT > 1) a[k] = __builtin_nontemporal_load(a4 + i);
+        if (NT > 2) b[k] = __builtin_nontemporal_load(b4 + i);
+      }
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          float oo = o[k][c];
+          thcl_apply_one<Op>(oo, NT > 1 ? a[k][c] : 0.f, NT > 2 ? b[k][c] : 0.f, v1, v2, p1, p2);
+          o[k][c] = oo;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++)
+        __builtin_nontemporal_store(o[k], o4 + base + (thcl_u64)k * THCL_APPLY_THREADS);
+    } else {
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+        const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
+        if (i < n4) {
+          thcl_f4 ov = o4[i], av, bv;
+          if (NT > 1) av = a4[i];
+          if (NT > 2) bv = b4[i];
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            float oo = ov[c];
+            thcl_apply_one<Op>(oo, NT > 1 ? av[c] : 0.f, NT > 2 ? bv[c] : 0.f, v1, v2, p1, p2);
+            ov[c] = oo;
+          }
+          o4[i] = ov;
+        }
+      }
+    }
+  }
+  // the last n % 4 elements
+  const thcl_u64 rem = P.n & 3;
+  if (blockIdx.x == 0 && threadIdx.x < rem) {
+    const thcl_u64 i = (n4 << 2) + threadIdx.x;
+    float oo = P.p[0][i];
+    thcl_apply_one<Op>(oo, NT > 1 ? P.p[1][i] : 0.f, NT > 2 ? P.p[2][i] : 0.f, v1, v2, p1, p2);
+    P.p[0][i] = oo;
+  }
+}
+
+// Dense operands whose addresses are not all 16-byte aligned: one dword per
+// lane, still whole lines per wave.
+template <class Op, int NT>
+__device__ __forceinline__ void thcl_apply_contig_s(const ThclContigParams &P) {
+  const float p1 = P.pt[0] ? *P.pt[0] : 0.f;
+  const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
+  const float v1 = P.val[0], v2 = P.val[1];
+  for (thcl_u64 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
+    const thcl_u64 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
+    float o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
+#pragma unroll
+    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
+      if (i < P.n) {
+        o[k] = P.p[0][i];
+        if (NT > 1) a[k] = P.p[1][i];
+        if (NT > 2) b[k] = P.p[2][i];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
+      if (i < P.n) {
+        float oo = o[k];
+        thcl_apply_one<Op>(oo, NT > 1 ? a[k] : 0.f, NT > 2 ? b[k] : 0.f, v1, v2, p1, p2);
+        P.p[0][i] = oo;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------- joint strided ---
+// Operands share sizes; dims were ordered by the written operand's stride and
+// merged on the host.  A unit is VEC consecutive elements of the innermost
+// dim (VEC = 4 needs unit stride there plus 16-byte aligned rows).
+template <class Op, int NT, int VEC>
+__device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
+  const float p1 = P.pt[0] ? *P.pt[0] : 0.f;
+  const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
+  const float v1 = P.val[0], v2 = P.val[1];
+  for (thcl_u32 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
+    const thcl_u32 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
+    thcl_u64 off[THCL_APPLY_UNROLL][3];
+#pragma unroll
+    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      thcl_u32 u = base + k * THCL_APPLY_THREADS;
+      thcl_u64 o0 = 0, o1 = 0, o2 = 0;
+      for (int d = P.dims - 1; d > 0; d--) {
+        const thcl_u32 q = thcl_div(u, P.size[d]);
+        const thcl_u32 r = u - q * P.size[d].d;
+        const thcl_u32 rr = (d == P.dims - 1) ? r * VEC : r;
+        o0 += (thcl_u64)rr * P.stride[0][d];
+        if (NT > 1) o1 += (thcl_u64)rr * P.stride[1][d];
+        if (NT > 2) o2 += (thcl_u64)rr * P.stride[2][d];
+        u = q;
+      }
+      const thcl_u32 r0 = (P.dims == 1) ? u * VEC : u;
+      off[k][0] = o0 + (thcl_u64)r0 * P.stride[0][0];
+      off[k][1] = o1 + (thcl_u64)r0 * P.stride[1][0];
+      off[k][2] = o2 + (thcl_u64)r0 * P.stride[2][0];
+    }
+    if (VEC == 4) {
+      thcl_f4 o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+        if (base + k * THCL_APPLY_THREADS < P.nunits) {
+          o[k] = *(const thcl_f4 *)(P.p[0] + off[k][0]);
+          if (NT > 1) a[k] = *(const thcl_f4 *)(P.p[1] + off[k][1]);
+          if (NT > 2) b[k] = *(const thcl_f4 *)(P.p[2] + off[k][2]);
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+        if (base + k * THCL_APPLY_THREADS < P.nunits) {
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            float oo = o[k][c];
+            thcl_apply_one<Op>(oo, NT > 1 ? a[k][c] : 0.f, NT > 2 ? b[k][c] : 0.f, v1, v2, p1, p2);
+            o[k][c] = oo;
+          }
+          *(thcl_f4 *)(P.p[0] + off[k][0]) = o[k];
+        }
+      }
+    } else {
+      float o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+        if (base + k * THCL_APPLY_THREADS < P.nunits) {
+          o[k] = P.p[0][off[k][0]];
+          if (NT > 1) a[k] = P.p[1][off[k][1]];
+          if (NT > 2) b[k] = P.p[2][off[k][2]];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+        if (base + k * THCL_APPLY_THREADS < P.nunits) {
+          float oo = o[k];
+          thcl_apply_one<Op>(oo, NT > 1 ? a[k] : 0.f, NT > 2 ? b[k] : 0.f, v1, v2, p1, p2);
+          P.p[0][off[k][0]] = oo;
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------- generic ---
+// Operands agree only in element count: each decomposes the linear index over
+// its own collapsed dims (the reference's scheme, with cheaper division).
+__device__ __forceinline__ thcl_u64 thcl_generic_offset(thcl_u32 i, const ThclGenericOperand &L) {
+  thcl_u64 off = 0;
+  for (int d = L.dims - 1; d > 0; d--) {
+    const thcl_u32 q = thcl_div(i, L.size[d]);
+    off += (thcl_u64)(i - q * L.size[d].d) * L.stride[d];
+    i = q;
+  }
+  return off + (thcl_u64)i * L.stride[0];
+}
+
+template <class Op, int NT>
+__device__ __forceinline__ void thcl_apply_generic(const ThclGenericParams &P) {
+  const float p1 = P.pt[0] ? *P.pt[0] : 0.f;
+  const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
+  const float v1 = P.val[0], v2 = P.val[1];
+  for (thcl_u32 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
+    const thcl_u32 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      const thcl_u32 i = base + k * THCL_APPLY_THREADS;
+      if (i < P.n) {
+        const thcl_u64 o0 = thcl_generic_offset(i, P.op[0]);
+        float oo = P.p[0][o0];
+        float a = 0.f, b = 0.f;
+        if (NT > 1) a = P.p[1][thcl_generic_offset(i, P.op[1])];
+        if (NT > 2) b = P.p[2][thcl_generic_offset(i, P.op[2])];
+        thcl_apply_one<Op>(oo, a, b, v1, v2, p1, p2);
+        P.p[0][o0] = oo;
+      }
+    }
+  }
+}
+
+// Entry points for one operator; K is a name prefix.
+#define THCL_DEFINE_APPLY_KERNELS(K, Op, NT)                                                             \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_contig_v4(ThclContigParams P) {  \
+    thcl_apply_contig_v4<Op, NT>(P);                                                                     \
+  }                                                                                                      \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_contig_s(ThclContigParams P) {   \
+    thcl_apply_contig_s<Op, NT>(P);                                                                      \
+  }                                                                                                      \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_v4(ThclJointParams P) {    \
+    thcl_apply_joint<Op, NT, 4>(P);                                                                      \
+  }                                                                                                      \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_s(ThclJointParams P) {     \
+    thcl_apply_joint<Op, NT, 1>(P);                                                                      \
+  }                                                                                                      \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_generic(ThclGenericParams P) {   \
+    thcl_apply_generic<Op, NT>(P);                                                                       \
+  }
+
+#endif  // THCL_APPLY_DEVICE_H

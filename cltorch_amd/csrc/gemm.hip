@@ -1,0 +1,287 @@
+// fp32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32), column-major BLAS
+// semantics: C[m x n] = alpha * op(A) * op(B) + beta * C.
+//
+// What it replaces: the clblasSgemm call of THClBlas_gemm (reference:
+// src/lib/THClBlas.cpp:381-449), whose arithmetic lives in clBLAS.
+//
+// Shape of the kernel: 256 threads = 4 waves in a 2x2 arrangement over a
+// BM x BN block tile; K advances in slabs of 16 staged through double-buffered
+// LDS (one barrier per slab), the next slab's global loads are issued before
+// the current slab's MFMAs.  Operands that are contiguous along m/n in memory
+// sit in LDS as [k][mn] and are read one dword per MFMA; operands contiguous
+// along k sit as [mn][k+4] and are read 128 bits per four MFMAs.  Within a
+// group of 8 k-values, MFMA step s consumes k = s (lanes 0-31) and k = 4+s
+// (lanes 32-63) for both operands, which is what makes the 128-bit read usable.
+// Blocks are renumbered so the blocks an XCD receives form a compact patch of
+// the tile grid and share its L2.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "internal.h"
+
+namespace {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 16;
+constexpr int KPITCH = BK + 4;  // [mn][k] rows: odd number of 16-byte chunks -> conflict-free 128-bit reads
+
+struct GemmParams {
+  const float *a, *b;
+  float *c;
+  int m, n, k;
+  int lda, ldb, ldc;
+  float alpha, beta;
+  int tiles_m, tiles_n;
+  int group_m;  // tiles along m per scheduling group
+};
+
+// One operand tile in LDS.  KC: contiguous along k in global memory.
+template <int BMN, bool KC>
+struct TileLds {
+  static constexpr int FLOATS = KC ? BMN * KPITCH : BK * BMN;
+};
+
+// global -> registers: each thread carries BMN*BK/256/4 float4
+template <int BMN, bool KC, bool EDGE>
+struct TileLoader {
+  static constexpr int NV = BMN * BK / 256 / 4;
+  f4 r[NV];
+
+  // g: operand base; ld: leading dim; mn0: first row/col of the tile; k0: first k; lim_mn/lim_k: extents
+  __device__ __forceinline__ void load(const float *g, int ld, int mn0, int k0, int lim_mn, int lim_k) {
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      const int f = threadIdx.x + 256 * p;
+      if (KC) {
+        const int mn = f / (BK / 4), kq = f % (BK / 4);
+        const float *src = g + (size_t)(mn0 + mn) * ld + k0 + kq * 4;
+        if (!EDGE) {
+          r[p] = *(const f4 *)src;
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; c++)
+            r[p][c] = (mn0 + mn < lim_mn && k0 + kq * 4 + c < lim_k) ? src[c] : 0.f;
+        }
+      } else {
+        const int kk = f / (BMN / 4), q = f % (BMN / 4);
+        const float *src = g + (size_t)(k0 + kk) * ld + mn0 + q * 4;
+        if (!EDGE) {
+          r[p] = *(const f4 *)src;
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; c++)
+            r[p][c] = (k0 + kk < lim_k && mn0 + q * 4 + c < lim_mn) ? src[c] : 0.f;
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void store(float *lds) const {
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      const int f = threadIdx.x + 256 * p;
+      if (KC) {
+        const int mn = f / (BK / 4), kq = f % (BK / 4);
+        *(f4 *)(lds + mn * KPITCH + kq * 4) = r[p];
+      } else {
+        const int kk = f / (BMN / 4), q = f % (BMN / 4);
+        *(f4 *)(lds + kk * BMN + q * 4) = r[p];
+      }
+    }
+  }
+};
+
+// fragments of one 8-k group for the wave's sub-tiles: frag[t][s], t = 32-wide sub-tile, s = MFMA step
+template <int BMN, bool KC, int NT>
+__device__ __forceinline__ void read_frags(const float *lds, int mn_wave0, int kgroup, float (&frag)[NT][4]) {
+  const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    const int mn = mn_wave0 + t * 32 + l32;
+    if (KC) {
+      const f4 v = *(const f4 *)(lds + mn * KPITCH + kgroup * 8 + 4 * h);
+#pragma unroll
+      for (int s = 0; s < 4; s++) frag[t][s] = v[s];
+    } else {
+#pragma unroll
+      for (int s = 0; s < 4; s++) frag[t][s] = lds[(kgroup * 8 + 4 * h + s) * BMN + mn];
+    }
+  }
+}
+
+// TA: op(A) = A^T (A stored k-contiguous); TB: op(B) = B^T (B stored n-contiguous)
+template <int BM, int BN, bool TA, bool TB, bool EDGE>
+__global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
+  constexpr bool AKC = TA;    // 'n': a[i + l*lda] (m-contiguous); 't': a[l + i*lda] (k-contiguous)
+  constexpr bool BKC = !TB;   // 'n': b[l + j*ldb] (k-contiguous); 't': b[j + l*ldb] (n-contiguous)
+  constexpr int WM = BM / 2, WN = BN / 2;   // wave tile
+  constexpr int MT = WM / 32, NT = WN / 32; // 32x32 MFMA tiles per wave
+  constexpr int AF = TileLds<BM, AKC>::FLOATS, BF = TileLds<BN, BKC>::FLOATS;
+  __shared__ __attribute__((aligned(16))) float lds[2 * (AF + BF)];
+
+  // XCD-aware renumbering: consecutive hardware block ids go to different
+  // XCDs, so give XCD x the x-th contiguous chunk of logical ids.
+  const int nblocks = P.tiles_m * P.tiles_n;
+  int bid = blockIdx.x;
+  {
+    const int per = nblocks / 8;
+    if (per > 0 && bid < per * 8) bid = (bid % 8) * per + bid / 8;
+  }
+  // grouped order: walk group_m tiles down m, then step along n
+  int tm, tn;
+  {
+    const int gsz = P.group_m * P.tiles_n;
+    const int g = bid / gsz, r = bid % gsz;
+    const int m_first = g * P.group_m;
+    const int m_count = (P.tiles_m - m_first < P.group_m) ? (P.tiles_m - m_first) : P.group_m;
+    tm = m_first + r % m_count;
+    tn = r / m_count;
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int wave = threadIdx.x >> 6;
+  const int wm0 = (wave & 1) * WM, wn0 = (wave >> 1) * WN;
+
+  f16v acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  TileLoader<BM, AKC, EDGE> la;
+  TileLoader<BN, BKC, EDGE> lb;
+  const int KT = (P.k + BK - 1) / BK;
+
+  la.load(P.a, P.lda, m0, 0, P.m, P.k);
+  lb.load(P.b, P.ldb, n0, 0, P.n, P.k);
+  la.store(lds);
+  lb.store(lds + AF);
+  __syncthreads();
+
+  for (int kt = 0; kt < KT; kt++) {
+    const int cur = kt & 1;
+    float *As = lds + cur * (AF + BF);
+    float *Bs = As + AF;
+    if (kt + 1 < KT) {
+      la.load(P.a, P.lda, m0, (kt + 1) * BK, P.m, P.k);
+      lb.load(P.b, P.ldb, n0, (kt + 1) * BK, P.n, P.k);
+    }
+#pragma unroll
+    for (int kg = 0; kg < BK / 8; kg++) {
+      float fa[MT][4], fb[NT][4];
+      read_frags<BM, AKC, MT>(As, wm0, kg, fa);
+      read_frags<BN, BKC, NT>(Bs, wn0, kg, fb);
+#pragma unroll
+      for (int s = 0; s < 4; s++)
+#pragma unroll
+        for (int i = 0; i < MT; i++)
+#pragma unroll
+          for (int j = 0; j < NT; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) {
+      float *An = lds + (cur ^ 1) * (AF + BF);
+      la.store(An);
+      lb.store(An + AF);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane holds rows 8*(r/4) + 4*(lane/32) + (r%4) of column lane%32
+  const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+      const int col = n0 + wn0 + j * 32 + l32;
+#pragma unroll
+      for (int rq = 0; rq < 4; rq++) {
+        const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
+        float *cp = P.c + (size_t)col * P.ldc + row;
+        if (!EDGE) {
+          f4 v;
+#pragma unroll
+          for (int c = 0; c < 4; c++) v[c] = P.alpha * acc[i][j][rq * 4 + c];
+          if (P.beta != 0.f) {
+            const f4 old = *(const f4 *)cp;
+#pragma unroll
+            for (int c = 0; c < 4; c++) v[c] += P.beta * old[c];
+          }
+          *(f4 *)cp = v;
+        } else {
+          if (col < P.n) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+              if (row + c < P.m) {
+                float v = P.alpha * acc[i][j][rq * 4 + c];
+                if (P.beta != 0.f) v += P.beta * cp[c];
+                cp[c] = v;
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, bool EDGE>
+void launch_tt(bool ta, bool tb, dim3 grid, hipStream_t s, const GemmParams &P) {
+  dim3 block(256);
+  if (!ta && !tb) hipLaunchKernelGGL((sgemm_mfma<BM, BN, false, false, EDGE>), grid, block, 0, s, P);
+  else if (ta && !tb) hipLaunchKernelGGL((sgemm_mfma<BM, BN, true, false, EDGE>), grid, block, 0, s, P);
+  else if (!ta && tb) hipLaunchKernelGGL((sgemm_mfma<BM, BN, false, true, EDGE>), grid, block, 0, s, P);
+  else hipLaunchKernelGGL((sgemm_mfma<BM, BN, true, true, EDGE>), grid, block, 0, s, P);
+}
+
+bool al16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+}  // namespace
+
+void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m, long n, long k, float alpha,
+                const float *a, long lda, const float *b, long ldb, float beta, float *c, long ldc) {
+  const bool ta = (transa == 't' || transa == 'T'), tb = (transb == 't' || transb == 'T');
+  THCL_CHECK(ta || transa == 'n' || transa == 'N', "gemm: transa must be 'n' or 't'");
+  THCL_CHECK(tb || transb == 'n' || transb == 'N', "gemm: transb must be 'n' or 't'");
+  THCL_CHECK(m <= INT32_MAX && n <= INT32_MAX && k <= INT32_MAX && lda <= INT32_MAX && ldb <= INT32_MAX &&
+                 ldc <= INT32_MAX,
+             "gemm only supports m, n, k, lda, ldb, ldc with the bound [val] <= %d", INT32_MAX);
+  if (m <= 0 || n <= 0) return;
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  GemmParams P;
+  memset(&P, 0, sizeof(P));
+  P.a = a;
+  P.b = b;
+  P.c = c;
+  P.m = (int)m;
+  P.n = (int)n;
+  P.k = (int)(k > 0 ? k : 0);
+  P.lda = (int)lda;
+  P.ldb = (int)ldb;
+  P.ldc = (int)ldc;
+  P.alpha = alpha;
+  P.beta = beta;
+  // tile choice: 128x128 by default; 64-wide tiles when a dimension is small
+  const int bm = (m >= 128 && (m % 128 == 0 || m >= 1024)) ? 128 : 64;
+  const int bn = (n >= 128 && (n % 128 == 0 || n >= 1024)) ? 128 : 64;
+  const bool fast = (m % bm == 0) && (n % bn == 0) && (k % BK == 0) && k > 0 && (lda % 4 == 0) && (ldb % 4 == 0) &&
+                    (ldc % 4 == 0) && al16(a) && al16(b) && al16(c);
+  P.tiles_m = (int)((m + bm - 1) / bm);
+  P.tiles_n = (int)((n + bn - 1) / bn);
+  P.group_m = P.tiles_m < 8 ? P.tiles_m : 8;
+  dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+#define GO(BM_, BN_)                                                   \
+  if (fast) launch_tt<BM_, BN_, false>(ta, tb, grid, stream, P);        \
+  else launch_tt<BM_, BN_, true>(ta, tb, grid, stream, P);
+  if (bm == 128 && bn == 128) { GO(128, 128) }
+  else if (bm == 128 && bn == 64) { GO(128, 64) }
+  else if (bm == 64 && bn == 128) { GO(64, 128) }
+  else { GO(64, 64) }
+#undef GO
+  hipError_t e = hipGetLastError();
+  THCL_CHECK(e == hipSuccess, "gemm launch failed: %s", hipGetErrorString(e));
+  thcl_after_launch(state, rt);
+}

@@ -1,0 +1,636 @@
+// Reductions: whole tensor -> scalar, and along one dimension (sum, prod,
+// max, min; max/min also report positions).
+//
+// What it replaces (reference): THClTensor_reduceAll's one- or two-pass
+// kernels that run on at most 4 work-groups (src/lib/THClReduceAll.cpp:225-272,
+// src/lib/THClGeneral.cpp:16-17), THClTensor_reduceDim's two kernels
+// (src/lib/THClReduce.cl:30-111) and the (value, index) kernels of
+// src/lib/THClTensorMathTransformReduce.cl:17-102.
+//
+// Numerics follow Torch7's CPU path: sums and products accumulate in fp64 and
+// round to fp32 once; max/min propagate NaN (the first one wins) and resolve
+// ties to the lowest position.  Every combine order is fixed by the launch
+// shape, so results are reproducible run to run; no floating-point atomics.
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+#include <cmath>
+#include <cstring>
+
+#include "apply_device.h"
+#include "internal.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWave = 64;
+
+// scratch block layout (bytes)
+constexpr size_t kTicketOff = 0;            // 1024 uint32 tickets
+constexpr size_t kPartialOff = 4096;        // partials
+constexpr size_t kResultSlot = 256;         // tail reserved for scalar results
+
+// --------------------------------------------------------------- combiners ---
+template <int KIND>
+struct Acc;  // accumulator type + combine rule for value-only reductions
+
+template <>
+struct Acc<RED_SUM> {
+  typedef double T;
+  static __device__ __forceinline__ T init() { return 0.0; }
+  static __device__ __forceinline__ T lift(float x) { return (double)x; }
+  static __device__ __forceinline__ T comb(T a, T b) { return a + b; }
+  static __device__ __forceinline__ float lower(T a) { return (float)a; }
+};
+template <>
+struct Acc<RED_PROD> {
+  typedef double T;
+  static __device__ __forceinline__ T init() { return 1.0; }
+  static __device__ __forceinline__ T lift(float x) { return (double)x; }
+  static __device__ __forceinline__ T comb(T a, T b) { return a * b; }
+  static __device__ __forceinline__ float lower(T a) { return (float)a; }
+};
+template <>
+struct Acc<RED_MAX> {
+  typedef float T;
+  static __device__ __forceinline__ T init() { return -INFINITY; }
+  static __device__ __forceinline__ T lift(float x) { return x; }
+  // NaN on either side gives NaN
+  static __device__ __forceinline__ T comb(T a, T b) { return (b > a || b != b) ? b : a; }
+  static __device__ __forceinline__ float lower(T a) { return a; }
+};
+template <>
+struct Acc<RED_MIN> {
+  typedef float T;
+  static __device__ __forceinline__ T init() { return INFINITY; }
+  static __device__ __forceinline__ T lift(float x) { return x; }
+  static __device__ __forceinline__ T comb(T a, T b) { return (b < a || b != b) ? b : a; }
+  static __device__ __forceinline__ float lower(T a) { return a; }
+};
+
+// (value, position) pairs for max/min along a dim.  Order-independent rule
+// equal to the sequential "replace when !(x <= cur), stop at the first NaN":
+// NaN beats any number, the earlier NaN beats a later one, equal values keep
+// the lower position.
+struct VI {
+  float v;
+  int i;
+};
+template <int KIND>
+__device__ __forceinline__ VI vi_init() {
+  VI r;
+  r.v = (KIND == RED_MAX) ? -INFINITY : INFINITY;
+  r.i = 0x7fffffff;
+  return r;
+}
+template <int KIND>
+__device__ __forceinline__ VI vi_comb(VI cur, VI x) {
+  const bool xn = x.v != x.v, cn = cur.v != cur.v;
+  bool take;
+  if (cn) take = xn && x.i < cur.i;
+  else if (xn) take = true;
+  else if (KIND == RED_MAX) take = (x.v > cur.v) || (x.v == cur.v && x.i < cur.i);
+  else take = (x.v < cur.v) || (x.v == cur.v && x.i < cur.i);
+  return take ? x : cur;
+}
+
+__device__ __forceinline__ double shfl_xor_t(double v, int m) { return __shfl_xor(v, m, kWave); }
+__device__ __forceinline__ float shfl_xor_t(float v, int m) { return __shfl_xor(v, m, kWave); }
+__device__ __forceinline__ VI shfl_xor_t(VI v, int m) {
+  VI r;
+  r.v = __shfl_xor(v.v, m, kWave);
+  r.i = __shfl_xor(v.i, m, kWave);
+  return r;
+}
+
+// butterfly over the `width` lanes (power of two <= 64) a lane belongs to
+template <int KIND, class T>
+__device__ __forceinline__ T group_reduce(T v, int width) {
+  for (int m = width >> 1; m > 0; m >>= 1) v = Acc<KIND>::comb(v, shfl_xor_t(v, m));
+  return v;
+}
+template <int KIND>
+__device__ __forceinline__ VI group_reduce_vi(VI v, int width) {
+  for (int m = width >> 1; m > 0; m >>= 1) v = vi_comb<KIND>(v, shfl_xor_t(v, m));
+  return v;
+}
+
+// whole-block reduce; result valid in thread 0
+template <int KIND, class T>
+__device__ __forceinline__ T block_reduce(T v, T *lds) {
+  v = group_reduce<KIND, T>(v, kWave);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  __syncthreads();  // lds may still be read by a previous round
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    T r = lds[0];
+    for (int w = 1; w < kThreads / kWave; w++) r = Acc<KIND>::comb(r, lds[w]);
+    v = r;
+  }
+  return v;
+}
+
+// loads that bypass the non-coherent per-CU cache (partials written by other blocks)
+__device__ __forceinline__ double load_fresh(const double *p) {
+  return __longlong_as_double((long long)__atomic_load_n((const unsigned long long *)p, __ATOMIC_RELAXED));
+}
+__device__ __forceinline__ float load_fresh(const float *p) {
+  return __uint_as_float(__atomic_load_n((const unsigned *)p, __ATOMIC_RELAXED));
+}
+
+// ------------------------------------------------------------- reduce all ---
+struct ReduceAllParams {
+  const float *in;
+  thcl_u64 n;
+  void *partials;
+  unsigned *ticket;
+  float *out;
+  ThclGenericOperand L;  // strided input only
+};
+
+// Last block to arrive (integer ticket) folds the per-block partials in block
+// order and writes the scalar; the ticket is left at zero for the next launch.
+template <int KIND>
+__device__ __forceinline__ void finish_all(typename Acc<KIND>::T blockval, const ReduceAllParams &P,
+                                           typename Acc<KIND>::T *lds) {
+  typedef typename Acc<KIND>::T T;
+  T *partials = (T *)P.partials;
+  __shared__ unsigned s_last;
+  if (threadIdx.x == 0) {
+    partials[blockIdx.x] = blockval;
+    __threadfence();
+    const unsigned t = atomicAdd(P.ticket, 1u);
+    s_last = (t == gridDim.x - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  T v = Acc<KIND>::init();
+  for (unsigned i = threadIdx.x; i < gridDim.x; i += kThreads)
+    v = Acc<KIND>::comb(v, load_fresh(&partials[i]));
+  v = block_reduce<KIND, T>(v, lds);
+  if (threadIdx.x == 0) {
+    P.out[0] = Acc<KIND>::lower(v);
+    *P.ticket = 0u;
+  }
+}
+
+template <int KIND>
+__global__ __launch_bounds__(kThreads) void reduce_all_dense(ReduceAllParams P) {
+  typedef typename Acc<KIND>::T T;
+  __shared__ T lds[kThreads / kWave];
+  constexpr int U = 4;
+  T acc[U];
+#pragma unroll
+  for (int k = 0; k < U; k++) acc[k] = Acc<KIND>::init();
+  // 16-byte aligned body as float4, unaligned head/tail as scalars
+  const uintptr_t addr = (uintptr_t)P.in;
+  thcl_u64 head = ((16 - (addr & 15)) & 15) / 4;
+  if (head > P.n) head = P.n;
+  const thcl_u64 n4 = (P.n - head) >> 2;
+  const thcl_f4 *in4 = (const thcl_f4 *)(P.in + head);
+  const thcl_u64 tile = (thcl_u64)kThreads * U;
+  for (thcl_u64 base = (thcl_u64)blockIdx.x * tile + threadIdx.x; base < n4; base += (thcl_u64)gridDim.x * tile) {
+    thcl_f4 v[U];
+#pragma unroll
+    for (int k = 0; k < U; k++) {
+      const thcl_u64 i = base + (thcl_u64)k * kThreads;
+      if (i < n4) v[k] = __builtin_nontemporal_load(in4 + i);
+    }
+#pragma unroll
+    for (int k = 0; k < U; k++) {
+      const thcl_u64 i = base + (thcl_u64)k * kThreads;
+      if (i < n4) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[k] = Acc<KIND>::comb(acc[k], Acc<KIND>::lift(v[k][c]));
+      }
+    }
+  }
+  if (blockIdx.x == 0) {
+    const thcl_u64 tail0 = head + (n4 << 2);
+    for (thcl_u64 i = threadIdx.x; i < head; i += kThreads) acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i]));
+    for (thcl_u64 i = tail0 + threadIdx.x; i < P.n; i += kThreads)
+      acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i]));
+  }
+  T v = Acc<KIND>::comb(Acc<KIND>::comb(acc[0], acc[1]), Acc<KIND>::comb(acc[2], acc[3]));
+  v = block_reduce<KIND, T>(v, lds);
+  finish_all<KIND>(v, P, lds);
+}
+
+template <int KIND>
+__global__ __launch_bounds__(kThreads) void reduce_all_strided(ReduceAllParams P) {
+  typedef typename Acc<KIND>::T T;
+  __shared__ T lds[kThreads / kWave];
+  T acc = Acc<KIND>::init();
+  for (thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x; i < P.n; i += (thcl_u64)gridDim.x * kThreads)
+    acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(P.in[thcl_generic_offset((thcl_u32)i, P.L)]));
+  acc = block_reduce<KIND, T>(acc, lds);
+  finish_all<KIND>(acc, P, lds);
+}
+
+// ------------------------------------------------------- reduce along dim ---
+struct ReduceDimParams {
+  const float *in;       // first element of the view
+  float *out;            // dense, one value per slice (NULL while writing partials)
+  float *idx_f32;        // dense 1-based positions as fp32, or NULL
+  long long *idx_i64;    // dense 1-based positions as int64, or NULL
+  void *partials;        // [split][nslices] when the reduction length is split over blocks
+  thcl_u32 nslices;      // output elements
+  thcl_u32 nunits;       // slices / VEC (column kernel)
+  thcl_u32 R;            // reduction length
+  thcl_u32 rstride;      // elements between consecutive reduced elements
+  thcl_u32 split;        // blocks sharing one slice's reduction (column kernel)
+  thcl_u32 rows_per_split;
+  ThclGenericOperand L;  // layout of the slice starts (the view without `dim`)
+};
+
+template <int KIND, bool ARG>
+struct Slot;  // what a thread carries
+template <int KIND>
+struct Slot<KIND, false> {
+  typedef typename Acc<KIND>::T T;
+  static __device__ __forceinline__ T init() { return Acc<KIND>::init(); }
+  static __device__ __forceinline__ T take(T cur, float x, int) { return Acc<KIND>::comb(cur, Acc<KIND>::lift(x)); }
+  static __device__ __forceinline__ T comb(T a, T b) { return Acc<KIND>::comb(a, b); }
+  static __device__ __forceinline__ T reduce(T v, int width) { return group_reduce<KIND, T>(v, width); }
+  static __device__ __forceinline__ void store(const ReduceDimParams &P, thcl_u32 s, T v) { P.out[s] = Acc<KIND>::lower(v); }
+};
+template <int KIND>
+struct Slot<KIND, true> {
+  typedef VI T;
+  static __device__ __forceinline__ T init() { return vi_init<KIND>(); }
+  static __device__ __forceinline__ T take(T cur, float x, int i) {
+    VI n;
+    n.v = x;
+    n.i = i;
+    return vi_comb<KIND>(cur, n);
+  }
+  static __device__ __forceinline__ T comb(T a, T b) { return vi_comb<KIND>(a, b); }
+  static __device__ __forceinline__ T reduce(T v, int width) { return group_reduce_vi<KIND>(v, width); }
+  static __device__ __forceinline__ void store(const ReduceDimParams &P, thcl_u32 s, T v) {
+    P.out[s] = v.v;
+    if (P.idx_f32) P.idx_f32[s] = (float)(v.i + 1);
+    if (P.idx_i64) P.idx_i64[s] = (long long)v.i + 1;
+  }
+};
+
+// Reduced dim is dense in memory: LPR lanes walk one slice, VEC floats each.
+// LPR in {8, 64, 256}; a block holds 256/LPR slices.
+template <int KIND, bool ARG, int LPR, int VEC>
+__global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
+  typedef Slot<KIND, ARG> S;
+  typedef typename S::T T;
+  constexpr int ROWS = kThreads / LPR;
+  __shared__ T lds[kThreads / kWave];
+  const int sub = threadIdx.x % LPR, row_in_block = threadIdx.x / LPR;
+  const thcl_u32 ngroups = (P.nslices + ROWS - 1) / ROWS;
+  for (thcl_u32 g = blockIdx.x; g < ngroups; g += gridDim.x) {
+    const thcl_u32 s = g * ROWS + row_in_block;
+    T acc = S::init();
+    if (s < P.nslices) {
+      const float *row = P.in + thcl_generic_offset(s, P.L);
+      if (VEC == 4) {
+        const thcl_f4 *row4 = (const thcl_f4 *)row;
+        const thcl_u32 r4 = P.R >> 2;
+        for (thcl_u32 i = sub; i < r4; i += LPR) {
+          const thcl_f4 v = __builtin_nontemporal_load(row4 + i);
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc = S::take(acc, v[c], (int)(i * 4 + c));
+        }
+      } else {
+        for (thcl_u32 i = sub; i < P.R; i += LPR) acc = S::take(acc, row[i], (int)i);
+      }
+    }
+    if (LPR <= kWave) {
+      acc = S::reduce(acc, LPR);
+      if (sub == 0 && s < P.nslices) S::store(P, s, acc);
+    } else {
+      acc = S::reduce(acc, kWave);
+      const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+      __syncthreads();
+      if (lane == 0) lds[wave] = acc;
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        T r = lds[0];
+        for (int w = 1; w < kThreads / kWave; w++) r = S::comb(r, lds[w]);
+        S::store(P, s, r);
+      }
+    }
+  }
+}
+
+// Reduced dim is strided: lanes lie along the slices (64 lanes x VEC adjacent
+// slices), the 4 waves of a block interleave over the reduced dim and meet in
+// LDS; blockIdx.y splits long reductions, leaving partials for the finisher.
+template <int KIND, bool ARG, int VEC>
+__global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
+  typedef Slot<KIND, ARG> S;
+  typedef typename S::T T;
+  constexpr int WAVES = kThreads / kWave;
+  __shared__ T lds[WAVES][kWave * VEC];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const thcl_u32 ntiles = (P.nunits + kWave - 1) / kWave;
+  const thcl_u32 r_begin = blockIdx.y * P.rows_per_split;
+  thcl_u32 r_end = r_begin + P.rows_per_split;
+  if (r_end > P.R) r_end = P.R;
+  for (thcl_u32 tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    const thcl_u32 u = tile * kWave + lane;
+    T acc[VEC];
+#pragma unroll
+    for (int c = 0; c < VEC; c++) acc[c] = S::init();
+    if (u < P.nunits) {
+      // a unit is VEC adjacent slices; the innermost slice dim counts units
+      thcl_u64 off;
+      {
+        thcl_u32 i = u;
+        off = 0;
+        for (int d = P.L.dims - 1; d > 0; d--) {
+          const thcl_u32 q = thcl_div(i, P.L.size[d]);
+          const thcl_u32 r = i - q * P.L.size[d].d;
+          off += (thcl_u64)((d == P.L.dims - 1) ? r * VEC : r) * P.L.stride[d];
+          i = q;
+        }
+        off += (thcl_u64)((P.L.dims == 1) ? i * VEC : i) * P.L.stride[0];
+      }
+      const float *col = P.in + off;
+      thcl_u32 r = r_begin + wave;
+      // two rows in flight per lane
+      for (; r + WAVES < r_end; r += 2 * WAVES) {
+        if (VEC == 4) {
+          const thcl_f4 v0 = __builtin_nontemporal_load((const thcl_f4 *)(col + (thcl_u64)r * P.rstride));
+          const thcl_f4 v1 = __builtin_nontemporal_load((const thcl_f4 *)(col + (thcl_u64)(r + WAVES) * P.rstride));
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v0[c], (int)r);
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v1[c], (int)(r + WAVES));
+        } else {
+          const float v0 = col[(thcl_u64)r * P.rstride];
+          const float v1 = col[(thcl_u64)(r + WAVES) * P.rstride];
+          acc[0] = S::take(acc[0], v0, (int)r);
+          acc[0] = S::take(acc[0], v1, (int)(r + WAVES));
+        }
+      }
+      for (; r < r_end; r += WAVES) {
+        if (VEC == 4) {
+          const thcl_f4 v0 = *(const thcl_f4 *)(col + (thcl_u64)r * P.rstride);
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v0[c], (int)r);
+        } else {
+          acc[0] = S::take(acc[0], col[(thcl_u64)r * P.rstride], (int)r);
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < VEC; c++) lds[wave][lane * VEC + c] = acc[c];
+    __syncthreads();
+    if (wave == 0 && u < P.nunits) {
+#pragma unroll
+      for (int c = 0; c < VEC; c++) {
+        T r = lds[0][lane * VEC + c];
+        for (int w = 1; w < WAVES; w++) r = S::comb(r, lds[w][lane * VEC + c]);
+        const thcl_u32 s = u * VEC + c;
+        if (P.split > 1) ((T *)P.partials)[(thcl_u64)blockIdx.y * P.nslices + s] = r;
+        else S::store(P, s, r);
+      }
+    }
+  }
+}
+
+template <int KIND, bool ARG>
+__global__ __launch_bounds__(kThreads) void reduce_cols_finish(ReduceDimParams P) {
+  typedef Slot<KIND, ARG> S;
+  typedef typename S::T T;
+  const T *partials = (const T *)P.partials;
+  for (thcl_u32 s = blockIdx.x * kThreads + threadIdx.x; s < P.nslices; s += gridDim.x * kThreads) {
+    T r = partials[s];
+    for (thcl_u32 k = 1; k < P.split; k++) r = S::comb(r, partials[(thcl_u64)k * P.nslices + s]);
+    S::store(P, s, r);
+  }
+}
+
+// ------------------------------------------------------------ host helpers ---
+
+void fill_operand(ThclGenericOperand &o, const Layout &L) {
+  memset(&o, 0, sizeof(o));
+  o.dims = L.dims;
+  for (int d = 0; d < L.dims; d++) {
+    THCL_CHECK(L.strides[d] >= 0 && L.strides[d] < (1l << 32) && L.sizes[d] < (1l << 31), THCL_DIM_WARNING);
+    o.size[d] = thcl_make_divisor(L.sizes[d]);
+    o.stride[d] = (thcl_u32)L.strides[d];
+  }
+}
+
+float init_value(ThclReduce kind) {
+  switch (kind) {
+    case RED_SUM: return 0.f;
+    case RED_PROD: return 1.f;
+    case RED_MAX: return -INFINITY;
+    default: return INFINITY;
+  }
+}
+
+void check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  THCL_CHECK(e == hipSuccess, "%s launch failed: %s", what, hipGetErrorString(e));
+}
+
+template <int KIND>
+void launch_all(bool dense, unsigned grid, hipStream_t stream, const ReduceAllParams &P) {
+  if (dense) hipLaunchKernelGGL(reduce_all_dense<KIND>, dim3(grid), dim3(kThreads), 0, stream, P);
+  else hipLaunchKernelGGL(reduce_all_strided<KIND>, dim3(grid), dim3(kThreads), 0, stream, P);
+}
+
+template <int KIND, bool ARG>
+void launch_dim(bool rows, int lpr, int vec, dim3 grid, hipStream_t stream, const ReduceDimParams &P) {
+  dim3 block(kThreads);
+  if (rows) {
+#define ROWS_CASE(L, V) \
+  if (lpr == L && vec == V) { hipLaunchKernelGGL((reduce_rows<KIND, ARG, L, V>), grid, block, 0, stream, P); return; }
+    ROWS_CASE(8, 1) ROWS_CASE(8, 4) ROWS_CASE(64, 1) ROWS_CASE(64, 4) ROWS_CASE(256, 1) ROWS_CASE(256, 4)
+#undef ROWS_CASE
+    thcl_throw("internal: no row-reduction kernel for lanes=%d vec=%d", lpr, vec);
+  } else {
+    if (vec == 4) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 4>), grid, block, 0, stream, P);
+    else hipLaunchKernelGGL((reduce_cols<KIND, ARG, 1>), grid, block, 0, stream, P);
+  }
+}
+
+template <int KIND, bool ARG>
+void launch_finish(unsigned grid, hipStream_t stream, const ReduceDimParams &P) {
+  hipLaunchKernelGGL((reduce_cols_finish<KIND, ARG>), dim3(grid), dim3(kThreads), 0, stream, P);
+}
+
+bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+}  // namespace
+
+// ----------------------------------------------------------------- reduce all
+void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out) {
+  const long n = THClTensor_nElement(state, src);
+  THCL_CHECK(src->nDimension <= THCL_MAX_DIMS, THCL_DIM_WARNING);
+  int device = THClTensor_getDevice(state, src);
+  thcl_rt *rt = thcl_ctx(state, device);
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  if (n == 0) {  // nothing to fold: the identity element
+    thcl_fill_contig(rt, out, init_value(kind), 1);
+    thcl_after_launch(state, rt);
+    return;
+  }
+  THCL_CHECK(src->storage && src->storage->wrapper, "tensor has no device storage");
+  size_t sbytes = 0;
+  char *scratch = (char *)thcl_rt_scratch(rt, &sbytes);
+  ReduceAllParams P;
+  memset(&P, 0, sizeof(P));
+  P.in = thcl_dptr(src);
+  P.n = (thcl_u64)n;
+  P.partials = scratch + kPartialOff;
+  P.ticket = (unsigned *)(scratch + kTicketOff);
+  P.out = out;
+  const bool dense = THClTensor_isContiguous(state, src);
+  const int cus = thcl_rt_get_props(rt)->compute_units;
+  long want;
+  if (dense) {
+    want = (n / 4 + kThreads * 4 - 1) / (kThreads * 4);
+  } else {
+    THCL_CHECK(n < (1l << 31), THCL_DIM_WARNING);
+    fill_operand(P.L, thcl_collapse(src));
+    want = (n + kThreads - 1) / kThreads;
+  }
+  long cap = (long)cus * 8;
+  const long max_partials = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
+  if (cap > max_partials) cap = max_partials;
+  unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));
+  switch (kind) {
+    case RED_SUM: launch_all<RED_SUM>(dense, grid, stream, P); break;
+    case RED_PROD: launch_all<RED_PROD>(dense, grid, stream, P); break;
+    case RED_MAX: launch_all<RED_MAX>(dense, grid, stream, P); break;
+    case RED_MIN: launch_all<RED_MIN>(dense, grid, stream, P); break;
+  }
+  check_launch("reduce-all");
+  thcl_after_launch(state, rt);
+}
+
+// ------------------------------------------------------------ reduce along dim
+void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THClTensor *indices_f32,
+                     int64_t *idx_i64_dev, THClTensor *src, long dim) {
+  thcl_check_same_device(state, 3, values, indices_f32, src);
+  THCL_CHECK(src->nDimension <= THCL_MAX_DIMS, THCL_DIM_WARNING);
+  if (src->nDimension <= 0) return;  // nothing to reduce (src/lib/THClReduce.cpp:234-237)
+  THCL_ARGCHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
+  THCL_CHECK(values != src && indices_f32 != src, "result and source must be different tensors");
+  THCL_CHECK(src->storage && src->storage->wrapper, "tensor has no device storage");
+  const bool arg = (kind == RED_MAX || kind == RED_MIN) && (indices_f32 != nullptr || idx_i64_dev != nullptr);
+  const int device = THClTensor_getDevice(state, src);
+  thcl_rt *rt = thcl_ctx(state, device);
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+
+  // outputs take the source's shape with size 1 along dim (src/lib/THClReduce.cpp:258-262)
+  long osz[THCL_MAX_DIMS];
+  long nslices = 1;
+  for (int d = 0; d < src->nDimension; d++) {
+    osz[d] = (d == dim) ? 1 : src->size[d];
+    nslices *= osz[d];
+  }
+  THLongStorage oshape;
+  memset(&oshape, 0, sizeof(oshape));
+  oshape.data = osz;
+  oshape.size = src->nDimension;
+  if (values->nDimension < 0 && !values->storage) values->device = device;
+  THClTensor_resize(state, values, &oshape, nullptr);
+  if (indices_f32) {
+    if (indices_f32->nDimension < 0 && !indices_f32->storage) indices_f32->device = device;
+    THClTensor_resize(state, indices_f32, &oshape, nullptr);
+  }
+  const long R = src->size[dim];
+  THCL_CHECK(nslices < (1l << 31) && R < (1l << 31), THCL_DIM_WARNING);
+  THCL_CHECK(thcl_fits_32bit(src), THCL_DIM_WARNING);
+
+  // kernels write dense outputs; strided destinations get a dense stand-in
+  THClTensor *vdense = values, *idense = indices_f32;
+  if (!THClTensor_isContiguous(state, values)) {
+    vdense = THClTensor_newv2(state, device);
+    THClTensor_resize(state, vdense, &oshape, nullptr);
+  }
+  if (indices_f32 && !THClTensor_isContiguous(state, indices_f32)) {
+    idense = THClTensor_newv2(state, device);
+    THClTensor_resize(state, idense, &oshape, nullptr);
+  }
+
+  ReduceDimParams P;
+  memset(&P, 0, sizeof(P));
+  P.in = thcl_dptr(src);
+  P.out = thcl_dptr(vdense);
+  P.idx_f32 = idense ? thcl_dptr(idense) : nullptr;
+  P.idx_i64 = (long long *)idx_i64_dev;
+  P.nslices = (thcl_u32)nslices;
+  P.R = (thcl_u32)R;
+  P.rstride = (thcl_u32)src->stride[dim];
+  P.split = 1;
+  P.rows_per_split = P.R;
+  Layout L = thcl_collapse(src, (int)dim);
+  fill_operand(P.L, L);
+
+  size_t sbytes = 0;
+  char *scratch = (char *)thcl_rt_scratch(rt, &sbytes);
+  P.partials = scratch + kPartialOff;
+  const long partial_cap = (long)((sbytes - kPartialOff - kResultSlot) / 8);  // 8-byte entries
+  const int cus = thcl_rt_get_props(rt)->compute_units;
+
+  const bool rows = (src->stride[dim] == 1) || R == 1;
+  int lpr = 0, vec = 1;
+  dim3 grid(1, 1, 1);
+  if (rows) {
+    lpr = R >= 2048 ? 256 : (R >= 128 ? 64 : 8);
+    bool v4 = (R % 4 == 0) && aligned16(P.in);
+    for (int d = 0; d < L.dims && v4; d++) v4 = (L.strides[d] % 4 == 0) || L.sizes[d] == 1;
+    vec = v4 ? 4 : 1;
+    const long groups = (nslices + (kThreads / lpr) - 1) / (kThreads / lpr);
+    grid.x = (unsigned)(groups > (1l << 22) ? (1l << 22) : groups);
+  } else {
+    const int last = L.dims - 1;
+    bool v4 = L.strides[last] == 1 && (L.sizes[last] % 4 == 0) && (src->stride[dim] % 4 == 0) && aligned16(P.in);
+    for (int d = 0; d < last && v4; d++) v4 = (L.strides[d] % 4 == 0);
+    vec = v4 ? 4 : 1;
+    if (v4) P.L.size[last] = thcl_make_divisor(L.sizes[last] / 4);
+    P.nunits = (thcl_u32)(nslices / vec);
+    const long tiles = (P.nunits + kWave - 1) / kWave;
+    // enough blocks to fill the chip: split the reduced dim when slices are few
+    long split = 1;
+    const long target = (long)cus * 8;
+    if (tiles < target) {
+      split = (target + tiles - 1) / tiles;
+      const long max_by_rows = (R + 31) / 32;  // at least 32 rows per block
+      if (split > max_by_rows) split = max_by_rows;
+      if (split * nslices > partial_cap) split = partial_cap / nslices;
+      if (split < 1) split = 1;
+    }
+    long rps = (R + split - 1) / split;
+    split = (R + rps - 1) / rps;
+    P.split = (thcl_u32)split;
+    P.rows_per_split = (thcl_u32)rps;
+    grid.x = (unsigned)(tiles > (1l << 20) ? (1l << 20) : tiles);
+    grid.y = (unsigned)split;
+  }
+
+#define DISPATCH(K)                                                       \
+  if (arg) launch_dim<K, true>(rows, lpr, vec, grid, stream, P);          \
+  else launch_dim<K, false>(rows, lpr, vec, grid, stream, P);             \
+  check_launch("reduce-dim");                                             \
+  if (!rows && P.split > 1) {                                             \
+    unsigned fg = (unsigned)((nslices + kThreads - 1) / kThreads);        \
+    if (arg) launch_finish<K, true>(fg, stream, P);                       \
+    else launch_finish<K, false>(fg, stream, P);                          \
+    check_launch("reduce-dim finish");                                    \
+  }
+  switch (kind) {
+    case RED_SUM: DISPATCH(RED_SUM) break;
+    case RED_PROD: DISPATCH(RED_PROD) break;
+    case RED_MAX: DISPATCH(RED_MAX) break;
+    case RED_MIN: DISPATCH(RED_MIN) break;
+  }
+#undef DISPATCH
+  thcl_after_launch(state, rt);
+  if (vdense != values) THClTensor_freeCopyTo(state, vdense, values);
+  if (idense != indices_f32) THClTensor_freeCopyTo(state, idense, indices_f32);
+}

@@ -1,0 +1,308 @@
+// Thin HIP runtime layer behind thcl_rt.h: device contexts, buffers, the
+// in-order stream, the hipRTC kernel cache and event timers.
+#include "thcl_rt.h"
+
+#include <hip/hip_runtime_api.h>
+#include <hip/hiprtc.h>
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+struct thcl_rt_kernel {
+  hipModule_t module = nullptr;
+  hipFunction_t fn = nullptr;
+};
+
+struct thcl_rt {
+  int device = -1;
+  hipStream_t stream = nullptr;
+  void *scratch = nullptr;
+  size_t scratch_bytes = 0;
+  float *host_word = nullptr;
+  thcl_rt_props props{};
+  std::map<std::string, thcl_rt_kernel *> kernels;
+};
+
+struct thcl_rt_timer {
+  thcl_rt *rt;
+  hipEvent_t a, b;
+};
+
+namespace {
+constexpr int kMaxDevices = 64;
+constexpr size_t kScratchBytes = 1u << 20;
+thcl_rt *g_ctx[kMaxDevices] = {nullptr};
+std::mutex g_mu;
+thread_local std::string g_err;
+
+int fail(const char *what, hipError_t e) {
+  g_err = std::string(what) + ": " + hipGetErrorString(e);
+  return -1;
+}
+#define RT_CHECK(call)                                  \
+  do {                                                  \
+    hipError_t e_ = (call);                             \
+    if (e_ != hipSuccess) return fail(#call, e_);       \
+  } while (0)
+
+struct DeviceGuard {
+  int prev = -1;
+  explicit DeviceGuard(int d) {
+    if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+    if (prev != d) (void)hipSetDevice(d);
+  }
+};
+}  // namespace
+
+extern "C" {
+
+const char *thcl_rt_error(void) { return g_err.c_str(); }
+
+int thcl_rt_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+  return n;
+}
+
+thcl_rt *thcl_rt_get(int device) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (device < 0 || device >= kMaxDevices) {
+    g_err = "device index out of range";
+    return nullptr;
+  }
+  if (g_ctx[device]) return g_ctx[device];
+  int n = thcl_rt_device_count();
+  if (device >= n) {
+    g_err = "no such HIP device: " + std::to_string(device) + " (visible: " + std::to_string(n) + ")";
+    return nullptr;
+  }
+  hipError_t e = hipSetDevice(device);
+  if (e != hipSuccess) {
+    fail("hipSetDevice", e);
+    return nullptr;
+  }
+  auto *rt = new thcl_rt();
+  rt->device = device;
+  hipDeviceProp_t p;
+  e = hipGetDeviceProperties(&p, device);
+  if (e != hipSuccess) {
+    fail("hipGetDeviceProperties", e);
+    delete rt;
+    return nullptr;
+  }
+  snprintf(rt->props.name, sizeof(rt->props.name), "%s", p.name);
+  snprintf(rt->props.arch, sizeof(rt->props.arch), "%s", p.gcnArchName);
+  rt->props.compute_units = p.multiProcessorCount;
+  rt->props.wavefront = p.warpSize;
+  rt->props.max_threads_per_block = p.maxThreadsPerBlock;
+  rt->props.clock_khz = p.clockRate;
+  rt->props.lds_bytes_per_block = (int)p.sharedMemPerBlock;
+  rt->props.total_mem = p.totalGlobalMem;
+  e = hipStreamCreateWithFlags(&rt->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    fail("hipStreamCreateWithFlags", e);
+    delete rt;
+    return nullptr;
+  }
+  e = hipMalloc(&rt->scratch, kScratchBytes);
+  if (e == hipSuccess) e = hipMemset(rt->scratch, 0, kScratchBytes);
+  if (e == hipSuccess) e = hipHostMalloc((void **)&rt->host_word, 64 * sizeof(float), hipHostMallocDefault);
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (e != hipSuccess) {
+    fail("scratch allocation", e);
+    delete rt;
+    return nullptr;
+  }
+  rt->scratch_bytes = kScratchBytes;
+  g_ctx[device] = rt;
+  return rt;
+}
+
+void thcl_rt_release_all(void) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  for (int d = 0; d < kMaxDevices; d++) {
+    thcl_rt *rt = g_ctx[d];
+    if (!rt) continue;
+    DeviceGuard g(d);
+    (void)hipStreamSynchronize(rt->stream);
+    for (auto &kv : rt->kernels) {
+      if (kv.second->module) (void)hipModuleUnload(kv.second->module);
+      delete kv.second;
+    }
+    (void)hipFree(rt->scratch);
+    (void)hipHostFree(rt->host_word);
+    (void)hipStreamDestroy(rt->stream);
+    delete rt;
+    g_ctx[d] = nullptr;
+  }
+}
+
+const thcl_rt_props *thcl_rt_get_props(thcl_rt *rt) { return &rt->props; }
+
+void *thcl_rt_malloc(thcl_rt *rt, size_t bytes) {
+  DeviceGuard g(rt->device);
+  void *p = nullptr;
+  hipError_t e = hipMalloc(&p, bytes ? bytes : 4);
+  if (e != hipSuccess) {
+    fail("hipMalloc", e);
+    return nullptr;
+  }
+  return p;
+}
+
+int thcl_rt_free(thcl_rt *rt, void *dptr) {
+  if (!dptr) return 0;
+  DeviceGuard g(rt->device);
+  // queued work may still read the block
+  RT_CHECK(hipStreamSynchronize(rt->stream));
+  RT_CHECK(hipFree(dptr));
+  return 0;
+}
+
+int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
+  if (!bytes) return 0;
+  DeviceGuard g(rt->device);
+  RT_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, rt->stream));
+  RT_CHECK(hipStreamSynchronize(rt->stream));
+  return 0;
+}
+
+int thcl_rt_memcpy_d2h(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
+  if (!bytes) return 0;
+  DeviceGuard g(rt->device);
+  RT_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, rt->stream));
+  RT_CHECK(hipStreamSynchronize(rt->stream));
+  return 0;
+}
+
+int thcl_rt_memcpy_d2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
+  if (!bytes) return 0;
+  DeviceGuard g(rt->device);
+  RT_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, rt->stream));
+  return 0;
+}
+
+void *thcl_rt_stream(thcl_rt *rt) { return (void *)rt->stream; }
+
+int thcl_rt_sync(thcl_rt *rt) {
+  DeviceGuard g(rt->device);
+  RT_CHECK(hipStreamSynchronize(rt->stream));
+  return 0;
+}
+
+void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes) {
+  if (bytes) *bytes = rt->scratch_bytes;
+  return rt->scratch;
+}
+
+float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
+
+static int rtc_compile(const char *source, const char *arch, std::vector<char> &code) {
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, source, "thcl_user_expr.hip", 0, nullptr, nullptr);
+  if (r != HIPRTC_SUCCESS) {
+    g_err = std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r);
+    return -1;
+  }
+  std::string archopt = std::string("--offload-arch=") + arch;
+  // Contraction stays off so a*b+c rounds twice like the host arithmetic it is
+  // compared with; packed fp32 instructions are disabled on this hardware pool.
+  const char *opts[] = {archopt.c_str(), "-O3", "-ffp-contract=off", "-std=c++17",
+                        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  int nopts = (int)(sizeof(opts) / sizeof(opts[0]));
+  r = hiprtcCompileProgram(prog, nopts, opts);
+  if (r != HIPRTC_SUCCESS) {
+    size_t ls = 0;
+    hiprtcGetProgramLogSize(prog, &ls);
+    std::string log(ls + 1, '\0');
+    if (ls) hiprtcGetProgramLog(prog, &log[0]);
+    g_err = std::string("expression failed to compile: ") + hiprtcGetErrorString(r) + "\n" + log.c_str();
+    hiprtcDestroyProgram(&prog);
+    return -1;
+  }
+  size_t cs = 0;
+  hiprtcGetCodeSize(prog, &cs);
+  code.resize(cs);
+  hiprtcGetCode(prog, code.data());
+  hiprtcDestroyProgram(&prog);
+  return 0;
+}
+
+int thcl_rt_compile_check(const char *source, const char *arch, size_t *code_bytes) {
+  std::vector<char> code;
+  int rc = rtc_compile(source, arch, code);
+  if (rc == 0 && code_bytes) *code_bytes = code.size();
+  return rc;
+}
+
+int thcl_rt_kernel_cached(thcl_rt *rt, const char *key) { return rt->kernels.count(key) ? 1 : 0; }
+
+thcl_rt_kernel *thcl_rt_kernel_get(thcl_rt *rt, const char *key, const char *source, const char *entry) {
+  auto it = rt->kernels.find(key);
+  if (it != rt->kernels.end()) return it->second;
+  DeviceGuard g(rt->device);
+  std::vector<char> code;
+  // strip feature suffixes such as ":sramecc+:xnack-" from the device's arch name
+  std::string arch = rt->props.arch;
+  size_t colon = arch.find(':');
+  if (colon != std::string::npos) arch = arch.substr(0, colon);
+  if (rtc_compile(source, arch.c_str(), code) != 0) return nullptr;
+  auto *k = new thcl_rt_kernel();
+  hipError_t e = hipModuleLoadData(&k->module, code.data());
+  if (e == hipSuccess) e = hipModuleGetFunction(&k->fn, k->module, entry);
+  if (e != hipSuccess) {
+    fail("loading runtime-compiled kernel", e);
+    if (k->module) (void)hipModuleUnload(k->module);
+    delete k;
+    return nullptr;
+  }
+  rt->kernels[key] = k;
+  return k;
+}
+
+int thcl_rt_launch(thcl_rt *rt, thcl_rt_kernel *k, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                   unsigned by, unsigned bz, unsigned lds_bytes, void *params, size_t params_bytes) {
+  DeviceGuard g(rt->device);
+  size_t sz = params_bytes;
+  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, params, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz,
+                    HIP_LAUNCH_PARAM_END};
+  RT_CHECK(hipModuleLaunchKernel(k->fn, gx, gy, gz, bx, by, bz, lds_bytes, rt->stream, nullptr, config));
+  return 0;
+}
+
+thcl_rt_timer *thcl_rt_timer_new(thcl_rt *rt) {
+  DeviceGuard g(rt->device);
+  auto *t = new thcl_rt_timer();
+  t->rt = rt;
+  if (hipEventCreate(&t->a) != hipSuccess || hipEventCreate(&t->b) != hipSuccess) {
+    delete t;
+    return nullptr;
+  }
+  return t;
+}
+int thcl_rt_timer_start(thcl_rt_timer *t) {
+  RT_CHECK(hipEventRecord(t->a, t->rt->stream));
+  return 0;
+}
+int thcl_rt_timer_stop(thcl_rt_timer *t) {
+  RT_CHECK(hipEventRecord(t->b, t->rt->stream));
+  return 0;
+}
+float thcl_rt_timer_ms(thcl_rt_timer *t) {
+  float ms = -1.f;
+  if (hipEventSynchronize(t->b) != hipSuccess) return -1.f;
+  if (hipEventElapsedTime(&ms, t->a, t->b) != hipSuccess) return -1.f;
+  return ms;
+}
+void thcl_rt_timer_free(thcl_rt_timer *t) {
+  if (!t) return;
+  (void)hipEventDestroy(t->a);
+  (void)hipEventDestroy(t->b);
+  delete t;
+}
+
+}  // extern "C"

@@ -1,0 +1,461 @@
+"""Host-side mirror of cltorch's Lua ``torch.ClTensor`` for the hot path.
+
+The reference's user-facing layer is Lua (``src/TensorMath.lua`` declares every
+method and overload; cwrap turns them into calls of ``THClTensor_*``).  Lua is
+not available here, so this module plays the role of that generated layer over
+the same C ABI: same method names, same overload resolution
+(``src/TensorMath.lua:655-668,727-736,943-988``), **1-based dimensions and
+1-based returned indices** as in Lua, results returned the way the Lua methods
+return them.  All arithmetic happens in ``libthcl_hip.so``; nothing here
+computes on the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence, Tuple, Union
+
+import numpy as np
+
+from . import _lib
+
+
+class ClError(RuntimeError):
+    """A check inside the library failed (what Torch7 raises as a Lua error)."""
+
+
+class _State:
+    """The global THClState that ``require 'cltorch'`` creates (``src/init.cpp:229-249``)."""
+
+    def __init__(self):
+        self.lib = _lib.load()
+        self.buf = C.create_string_buffer(256)  # larger than sizeof(THClState)
+        self.ptr = C.cast(self.buf, C.c_void_p)
+        self.lib.THCl_initializeState(self.ptr)
+        self.lib.THClInit(self.ptr)
+        err = self.lib.THClLastError()
+        if err:
+            raise ClError(err.decode())
+
+    def check(self):
+        err = self.lib.THClLastError()
+        if err:
+            msg = err.decode()
+            self.lib.THClClearError()
+            raise ClError(msg)
+
+
+_state: Optional[_State] = None
+
+
+def state() -> _State:
+    global _state
+    if _state is None:
+        _state = _State()
+    return _state
+
+
+def _call(name: str, *args):
+    st = state()
+    r = getattr(st.lib, name)(st.ptr, *args)
+    st.check()
+    return r
+
+
+def synchronize() -> None:
+    """``cltorch.synchronize()`` / ``cltorch.finish()``."""
+    _call("THClState_synchronize")
+
+
+finish = synchronize
+
+
+def getDeviceCount() -> int:
+    return int(_call("THClState_getNumDevices"))
+
+
+def setAddFinish(flag: int) -> None:
+    # THClState.addFinish is the 6th int of the struct (src/lib/THClGeneral.h:76-93)
+    ints = C.cast(state().buf, C.POINTER(C.c_int))
+    ints[5] = int(flag)
+
+
+def _long_storage(values: Sequence[int]):
+    lib = state().lib
+    s = lib.THLongStorage_newWithSize(len(values))
+    for i, v in enumerate(values):
+        lib.THLongStorage_set(s, i, int(v))
+    return s
+
+
+class ClTensor:
+    """``torch.ClTensor``: a strided fp32 view of device storage."""
+
+    def __init__(self, *sizes, _handle=None, device: int = 0):
+        self._lib = state().lib
+        if _handle is not None:
+            self._h = _handle
+            return
+        if len(sizes) == 1 and isinstance(sizes[0], (list, tuple, np.ndarray)) and not isinstance(sizes[0], (int,)):
+            arr = np.asarray(sizes[0], dtype=np.float32)
+            self._h = _call("THClTensor_newv2", device)
+            self._resize(arr.shape)
+            self._upload(arr)
+            return
+        self._h = _call("THClTensor_newv2", device)
+        if sizes:
+            self._resize(sizes)
+
+    # ---- lifecycle ------------------------------------------------------
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None) and _state is not None:
+                self._lib.THClTensor_free(_state.ptr, self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    def _resize(self, sizes):
+        s = _long_storage(list(sizes))
+        try:
+            _call("THClTensor_resize", self._h, s, None)
+        finally:
+            self._lib.THLongStorage_free(s)
+
+    def _upload(self, arr: np.ndarray):
+        arr = np.ascontiguousarray(arr, dtype=np.float32)
+        sz = (C.c_long * max(arr.ndim, 1))(*arr.shape)
+        ft = self._lib.THFloatTensor_newWithData(arr.ctypes.data_as(C.c_void_p), arr.size, 0, arr.ndim, sz, None)
+        try:
+            _call("THClTensor_copyFloat", self._h, ft)
+        finally:
+            self._lib.THFloatTensor_free(ft)
+
+    @staticmethod
+    def from_numpy(arr) -> "ClTensor":
+        """``floatTensor:cl()``"""
+        return ClTensor(np.asarray(arr, dtype=np.float32))
+
+    # ---- metadata ---------------------------------------------------------
+    def nDimension(self) -> int:
+        return int(_call("THClTensor_nDimension", self._h))
+
+    dim = nDimension
+
+    def size(self, dim: Optional[int] = None):
+        nd = max(self.nDimension(), 0)
+        if dim is not None:
+            return int(_call("THClTensor_size", self._h, dim - 1))
+        return tuple(int(_call("THClTensor_size", self._h, d)) for d in range(nd))
+
+    def stride(self, dim: Optional[int] = None):
+        nd = max(self.nDimension(), 0)
+        if dim is not None:
+            return int(_call("THClTensor_stride", self._h, dim - 1))
+        return tuple(int(_call("THClTensor_stride", self._h, d)) for d in range(nd))
+
+    def storageOffset(self) -> int:
+        """1-based, as in Lua."""
+        return int(_call("THClTensor_storageOffset", self._h)) + 1
+
+    def nElement(self) -> int:
+        return int(_call("THClTensor_nElement", self._h))
+
+    numel = nElement
+
+    def isContiguous(self) -> bool:
+        return bool(_call("THClTensor_isContiguous", self._h))
+
+    def data_ptr(self) -> int:
+        return int(_call("THClTensor_data", self._h) or 0)
+
+    # ---- views (header only) ---------------------------------------------
+    def _wrap(self, h) -> "ClTensor":
+        if not h:
+            state().check()
+            raise ClError("view creation failed")
+        return ClTensor(_handle=h)
+
+    def narrow(self, dim: int, first: int, size: int) -> "ClTensor":
+        return self._wrap(_call("THClTensor_newNarrow", self._h, dim - 1, first - 1, size))
+
+    def select(self, dim: int, index: int) -> "ClTensor":
+        return self._wrap(_call("THClTensor_newSelect", self._h, dim - 1, index - 1))
+
+    def transpose(self, d1: int, d2: int) -> "ClTensor":
+        return self._wrap(_call("THClTensor_newTranspose", self._h, d1 - 1, d2 - 1))
+
+    def t(self) -> "ClTensor":
+        if self.nDimension() != 2:
+            raise ClError("t() expects a 2D tensor")
+        return self.transpose(1, 2)
+
+    def unfold(self, dim: int, size: int, step: int) -> "ClTensor":
+        return self._wrap(_call("THClTensor_newUnfold", self._h, dim - 1, size, step))
+
+    def strided(self, sizes: Sequence[int], strides: Sequence[int], offset: int = 1) -> "ClTensor":
+        """View of the same storage with explicit sizes/strides (``torch.ClTensor(storage, offset, sizes, strides)``)."""
+        st = _call("THClTensor_storage", self._h)
+        sz, sd = _long_storage(sizes), _long_storage(strides)
+        try:
+            h = _call("THClTensor_newWithStorage", 0, st, offset - 1, sz, sd)
+        finally:
+            self._lib.THLongStorage_free(sz)
+            self._lib.THLongStorage_free(sd)
+        return self._wrap(h)
+
+    def clone(self) -> "ClTensor":
+        return self._wrap(_call("THClTensor_newClone", self._h))
+
+    def contiguous(self) -> "ClTensor":
+        return self._wrap(_call("THClTensor_newContiguous", self._h))
+
+    def resize(self, *sizes) -> "ClTensor":
+        self._resize(sizes)
+        return self
+
+    def resizeAs(self, other: "ClTensor") -> "ClTensor":
+        _call("THClTensor_resizeAs", self._h, other._h)
+        return self
+
+    # ---- host <-> device ---------------------------------------------------
+    def copy(self, src) -> "ClTensor":
+        if isinstance(src, ClTensor):
+            _call("THClTensor_copy", self._h, src._h)
+        else:
+            self._upload(np.asarray(src, dtype=np.float32))
+        return self
+
+    def float(self) -> np.ndarray:
+        """``clTensor:float()``: a host copy shaped like the tensor."""
+        nd = self.nDimension()
+        if nd == 0:
+            return np.array(self.s(), dtype=np.float32)
+        shape = self.size()
+        out = np.empty(shape if nd > 0 else (0,), dtype=np.float32)
+        if out.size:
+            sz = (C.c_long * max(out.ndim, 1))(*out.shape)
+            ft = self._lib.THFloatTensor_newWithData(out.ctypes.data_as(C.c_void_p), out.size, 0, out.ndim, sz, None)
+            try:
+                _call("THFloatTensor_copyCl", ft, self._h)
+            finally:
+                self._lib.THFloatTensor_free(ft)
+        return out
+
+    def double(self) -> np.ndarray:
+        return self.float().astype(np.float64)
+
+    def long(self) -> np.ndarray:
+        return self.float().astype(np.int64)
+
+    def s(self) -> float:
+        """Point tensor -> host scalar (``src/TensorMath.lua:938-941``)."""
+        return float(_call("THClTensor_as_float", self._h))
+
+    # ---- fills --------------------------------------------------------------
+    def fill(self, value) -> "ClTensor":
+        if isinstance(value, ClTensor):
+            _call("THClTensor_fill_gpu", self._h, value._h)
+        else:
+            _call("THClTensor_fill", self._h, C.c_float(value))
+        return self
+
+    def zero(self) -> "ClTensor":
+        _call("THClTensor_zero", self._h)
+        return self
+
+    # ---- pointwise: overloads as declared in src/TensorMath.lua ---------------
+    def add(self, *args) -> "ClTensor":
+        """``x:add(v)``, ``x:add(y)``, ``x:add(v, y)``, ``x:add(a, v)``, ``x:add(a, v, b)``, ``x:add(a, b)``."""
+        src, rest = self, args
+        if len(args) >= 2 and isinstance(args[0], ClTensor):
+            src, rest = args[0], args[1:]
+        if len(rest) == 1 and not isinstance(rest[0], ClTensor):
+            _call("THClTensor_add", self._h, src._h, C.c_float(rest[0]))
+        elif len(rest) == 1:
+            _call("THClTensor_cadd", self._h, src._h, C.c_float(1.0), rest[0]._h)
+        elif len(rest) == 2:
+            _call("THClTensor_cadd", self._h, src._h, C.c_float(rest[0]), rest[1]._h)
+        else:
+            raise ClError("invalid arguments to add")
+        return self
+
+    def csub(self, *args) -> "ClTensor":
+        src, rest = self, args
+        if len(args) >= 2 and isinstance(args[0], ClTensor):
+            src, rest = args[0], args[1:]
+        if len(rest) == 1 and not isinstance(rest[0], ClTensor):
+            _call("THClTensor_sub", self._h, src._h, C.c_float(rest[0]))
+        elif len(rest) == 1:
+            _call("THClTensor_csub", self._h, src._h, C.c_float(1.0), rest[0]._h)
+        elif len(rest) == 2:
+            _call("THClTensor_csub", self._h, src._h, C.c_float(rest[0]), rest[1]._h)
+        else:
+            raise ClError("invalid arguments to csub")
+        return self
+
+    def _scalar_or_point(self, cfn: str, args) -> "ClTensor":
+        src, v = (self, args[0]) if len(args) == 1 else (args[0], args[1])
+        if isinstance(v, ClTensor):
+            _call(f"THClTensor_{cfn}_gpu", self._h, src._h, v._h)
+        else:
+            _call(f"THClTensor_{cfn}", self._h, src._h, C.c_float(v))
+        return self
+
+    def mul(self, *args) -> "ClTensor":
+        return self._scalar_or_point("mul", args)
+
+    def div(self, *args) -> "ClTensor":
+        """``a:div(v)`` or ``a:div(pointTensor)`` (``src/TensorMath.lua:727-736``)."""
+        return self._scalar_or_point("div", args)
+
+    def _binary(self, cfn: str, args) -> "ClTensor":
+        a, b = (self, args[0]) if len(args) == 1 else (args[0], args[1])
+        _call(f"THClTensor_{cfn}", self._h, a._h, b._h)
+        return self
+
+    def cmul(self, *args) -> "ClTensor":
+        return self._binary("cmul", args)
+
+    def cdiv(self, *args) -> "ClTensor":
+        return self._binary("cdiv", args)
+
+    def addcmul(self, *args) -> "ClTensor":
+        t, rest = (self, args) if not isinstance(args[0], ClTensor) or len(args) == 2 else (args[0], args[1:])
+        v, a, b = (1.0, rest[0], rest[1]) if len(rest) == 2 else rest
+        _call("THClTensor_addcmul", self._h, t._h, C.c_float(v), a._h, b._h)
+        return self
+
+    def addcdiv(self, *args) -> "ClTensor":
+        t, rest = (self, args) if not isinstance(args[0], ClTensor) or len(args) == 2 else (args[0], args[1:])
+        v, a, b = (1.0, rest[0], rest[1]) if len(rest) == 2 else rest
+        _call("THClTensor_addcdiv", self._h, t._h, C.c_float(v), a._h, b._h)
+        return self
+
+    def _unary(self, cfn: str, src: Optional["ClTensor"]) -> "ClTensor":
+        _call(f"THClTensor_{cfn}", self._h, (src or self)._h)
+        return self
+
+    def sqrt(self, src=None): return self._unary("sqrt", src)
+    def abs(self, src=None): return self._unary("abs", src)
+    def neg(self, src=None): return self._unary("neg", src)
+    def cinv(self, src=None): return self._unary("cinv", src)
+    def exp(self, src=None): return self._unary("exp", src)
+    def log(self, src=None): return self._unary("log", src)
+    def tanh(self, src=None): return self._unary("tanh", src)
+    def sigmoid(self, src=None): return self._unary("sigmoid", src)
+    def floor(self, src=None): return self._unary("floor", src)
+    def ceil(self, src=None): return self._unary("ceil", src)
+
+    # ---- user expressions ---------------------------------------------------
+    def apply_on_gpu(self, expr: str) -> "ClTensor":
+        _call("THClTensor_apply", self._h, expr.encode())
+        return self
+
+    def map_on_gpu(self, other: "ClTensor", expr: str) -> "ClTensor":
+        _call("THClTensor_map", self._h, other._h, expr.encode())
+        return self
+
+    def map2_on_gpu(self, a: "ClTensor", b: "ClTensor", expr: str) -> "ClTensor":
+        _call("THClTensor_map2", self._h, a._h, b._h, expr.encode())
+        return self
+
+    apply2_on_gpu = map_on_gpu
+    apply3_on_gpu = map2_on_gpu
+
+    # ---- reductions -----------------------------------------------------------
+    def _reduce(self, name: str, args):
+        """``a:sum()`` -> number; ``res:sum(a)`` -> point tensor in res; ``a:sum(dim)`` -> new tensor."""
+        if len(args) == 0:
+            return float(_call(f"THClTensor_{name}all", self._h))
+        if len(args) == 1 and isinstance(args[0], ClTensor):
+            _call(f"THClTensor_{name}all_gpu", self._h, args[0]._h)
+            return self
+        raise ClError(f"invalid arguments to {name}")
+
+    def sum(self, *args):
+        if len(args) == 1 and not isinstance(args[0], ClTensor):
+            res = ClTensor()
+            _call("THClTensor_sum", res._h, self._h, C.c_long(args[0] - 1))
+            return res
+        return self._reduce("sum", args)
+
+    def prod(self, *args):
+        if len(args) == 1 and not isinstance(args[0], ClTensor):
+            res = ClTensor()
+            _call("THClTensor_prod", res._h, self._h, C.c_long(args[0] - 1))
+            return res
+        return self._reduce("prod", args)
+
+    def _minmax(self, name: str, args):
+        if len(args) == 1 and not isinstance(args[0], ClTensor):
+            values, indices = ClTensor(), ClTensor()
+            _call(f"THClTensor_{name}", values._h, indices._h, self._h, C.c_long(args[0] - 1))
+            return values, indices
+        return self._reduce(name, args)
+
+    def max(self, *args):
+        """``a:max()`` -> number; ``a:max(dim)`` -> (values, 1-based indices as ClTensor)."""
+        return self._minmax("max", args)
+
+    def min(self, *args):
+        return self._minmax("min", args)
+
+    def max_long(self, dim: int) -> Tuple["ClTensor", np.ndarray]:
+        """values plus int64 1-based indices (what ``indices:long()`` gives in Lua)."""
+        return self._minmax_long("maxLong", dim)
+
+    def min_long(self, dim: int) -> Tuple["ClTensor", np.ndarray]:
+        return self._minmax_long("minLong", dim)
+
+    def _minmax_long(self, cfn: str, dim: int):
+        shape = [1 if d == dim - 1 else s for d, s in enumerate(self.size())]
+        idx = np.zeros(shape, dtype=np.int64)
+        sz = _long_storage(shape)
+        lt = self._lib.THLongTensor_newWithSize(sz, None)
+        self._lib.THLongStorage_free(sz)
+        values = ClTensor()
+        try:
+            _call(f"THClTensor_{cfn}", values._h, lt, self._h, C.c_long(dim - 1))
+            # THLongTensor: size*, stride*, int nDimension, storage* -> storage->data
+            class _LS(C.Structure):
+                _fields_ = [("data", C.POINTER(C.c_long)), ("size", C.c_long)]
+
+            class _LT(C.Structure):
+                _fields_ = [("size", C.c_void_p), ("stride", C.c_void_p), ("nDimension", C.c_int),
+                            ("storage", C.POINTER(_LS))]
+            t = C.cast(lt, C.POINTER(_LT)).contents
+            n = int(np.prod(shape))
+            idx.reshape(-1)[:] = np.ctypeslib.as_array(t.storage.contents.data, shape=(n,))
+        finally:
+            self._lib.THLongTensor_free(lt)
+        return values, idx
+
+    # ---- blas -------------------------------------------------------------------
+    def addmm(self, *args) -> "ClTensor":
+        """``r:addmm([beta,] [t,] [alpha,] m1, m2)`` (``src/TensorMath.lua:896-929``)."""
+        nums = [a for a in args if not isinstance(a, ClTensor)]
+        tens = [a for a in args if isinstance(a, ClTensor)]
+        if len(tens) == 2:
+            t, m1, m2 = self, tens[0], tens[1]
+        elif len(tens) == 3:
+            t, m1, m2 = tens
+        else:
+            raise ClError("invalid arguments to addmm")
+        if len(nums) == 0:
+            beta, alpha = 1.0, 1.0
+        elif len(nums) == 1:
+            beta, alpha = 1.0, nums[0]
+        else:
+            beta, alpha = nums[0], nums[1]
+        _call("THClTensor_addmm", self._h, C.c_float(beta), t._h, C.c_float(alpha), m1._h, m2._h)
+        return self
+
+    def __repr__(self):
+        return f"ClTensor(size={self.size()}, stride={self.stride()})"
+
+
+def mm(a: ClTensor, b: ClTensor) -> ClTensor:
+    """``torch.mm(a, b)``: zeroed result, then addmm with beta 0 (``src/TensorMath.lua:867-893``)."""
+    r = ClTensor(a.size(1), b.size(2)).zero()
+    _call("THClTensor_addmm", r._h, C.c_float(0.0), r._h, C.c_float(1.0), a._h, b._h)
+    return r

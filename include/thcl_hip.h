@@ -1,0 +1,332 @@
+/*
+ * C ABI of the MI355X tensor backend: the entry points the Lua/C binding layer
+ * of cltorch (cwrap-generated TensorMath.c, Tensor.cpp, Storage.cpp) binds for
+ * the pointwise / copy / reduce / addmm path.  Names, argument order and
+ * argument meaning are those of the reference's `THCL_API` functions; each
+ * declaration cites the reference interface it replaces.  Dimensions are
+ * 0-based here (the Lua layer subtracts 1), sizes/strides are `long` counts of
+ * elements, the element type is fp32.
+ *
+ * Every function is `extern "C"`, takes plain pointers and sizes, and never
+ * lets a C++ exception escape: a failed check calls the installed error
+ * handler (THClSetErrorHandler) and records the message for THClLastError().
+ */
+#ifndef THCL_HIP_H
+#define THCL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------- */
+/* Torch7 `TH` stand-ins.  Field order matches TH's own structs, so objects   */
+/* made by a real libTH can be passed in; with a real Torch7 the definitions  */
+/* come from <TH/TH.h> instead (build with -DTHCL_EXTERNAL_TH).               */
+/* ------------------------------------------------------------------------- */
+#ifndef THCL_EXTERNAL_TH
+typedef struct THLongStorage {
+  long *data;
+  long size;
+  int refcount;
+  char flag;
+  void *allocator;
+  void *allocatorContext;
+  struct THLongStorage *view;
+} THLongStorage;
+
+typedef struct THFloatStorage {
+  float *data;
+  long size;
+  int refcount;
+  char flag;
+  void *allocator;
+  void *allocatorContext;
+  struct THFloatStorage *view;
+} THFloatStorage;
+
+typedef struct THFloatTensor {
+  long *size;
+  long *stride;
+  int nDimension;
+  THFloatStorage *storage;
+  long storageOffset;
+  int refcount;
+  char flag;
+} THFloatTensor;
+
+typedef struct THLongTensor {
+  long *size;
+  long *stride;
+  int nDimension;
+  THLongStorage *storage;
+  long storageOffset;
+  int refcount;
+  char flag;
+} THLongTensor;
+
+THLongStorage *THLongStorage_newWithSize(long size);
+void THLongStorage_free(THLongStorage *s);
+void THLongStorage_set(THLongStorage *s, long i, long v);
+long THLongStorage_get(const THLongStorage *s, long i);
+
+THFloatTensor *THFloatTensor_newWithSize(THLongStorage *size, THLongStorage *stride);
+/* borrows `data` (not freed with the tensor): a strided host view */
+THFloatTensor *THFloatTensor_newWithData(float *data, long storageSize, long storageOffset, int nDimension,
+                                         const long *size, const long *stride);
+void THFloatTensor_free(THFloatTensor *t);
+long THFloatTensor_nElement(const THFloatTensor *t);
+THLongTensor *THLongTensor_newWithSize(THLongStorage *size, THLongStorage *stride);
+void THLongTensor_free(THLongTensor *t);
+long THLongTensor_nElement(const THLongTensor *t);
+#endif
+
+/* ------------------------------------------------------------------------- */
+/* State (reference: src/lib/THClGeneral.h:70-131)                            */
+/* ------------------------------------------------------------------------- */
+struct thcl_rt; /* per-device HIP runtime context, see thcl_rt.h */
+
+typedef struct THClScratchSpace {
+  void *wrapper; /* device pointer of the per-device scratch block */
+  float *data;   /* pinned host word used to hand scalars back     */
+} THClScratchSpace;
+
+typedef struct THClState {
+  int initialized;
+  int allowNonGpus;
+  int allocatedDevices;
+  int currentDevice;
+  int trace;
+  int addFinish; /* 1: synchronise after every launch (debugging) */
+  int detailedTimings;
+  struct THClScratchSpace **scratchSpaceByDevice;
+  void **deviceInfoByDevice;
+  struct thcl_rt **clByDevice;
+} THClState;
+
+/* src/lib/THClGeneral.h:95-98, src/lib/THClGeneral.cpp:29-96 */
+void THCl_initializeState(THClState *state);
+void THClSetAllowNonGpus(THClState *state, int allowNonGpus);
+void THClInit(THClState *state);
+void THClShutdown(THClState *state);
+/* src/lib/THClGeneral.h:101-107 */
+int THClState_getNumDevices(THClState *state);
+void THClState_setDevice(THClState *state, int device);
+int THClState_getDevice(THClState *state);
+struct thcl_rt *THClState_getClv2(THClState *state, int device);
+/* src/lib/THClGeneral.h:128-131 */
+struct THClScratchSpace *THClState_getDeviceScratchSpace(THClState *state, int device, int stream);
+size_t THClState_getDeviceScratchSpaceSize(THClState *state, int device);
+/* `cltorch.synchronize()` / `cltorch.finish()`: src/init.cpp:72-78 */
+void THClState_synchronize(THClState *state);
+
+/* Error reporting: the reference raises through Torch7's THError/THArgCheck
+ * (src/lib/THClKernels.cpp:23-29, src/lib/THClTensorMath.cpp:19-24).  Here a
+ * failed check records its message, calls the handler if one is installed and
+ * returns from the entry point without touching its outputs further. */
+typedef void (*THClErrorHandler)(const char *msg, void *data);
+void THClSetErrorHandler(THClErrorHandler handler, void *data);
+const char *THClLastError(void); /* NULL when the last call succeeded */
+void THClClearError(void);
+
+/* ------------------------------------------------------------------------- */
+/* Storage (reference: src/lib/THClStorage.h:13-59)                           */
+/* ------------------------------------------------------------------------- */
+typedef struct THClStorage {
+  int device;
+  float *data;           /* host mirror; NULL unless a caller asked for one */
+  struct thcl_rt *cl;    /* runtime context of `device`                     */
+  void *wrapper;         /* device pointer (hipMalloc)                      */
+  long size;             /* elements                                        */
+  int refcount;
+  char flag;
+  void *allocator;
+  void *allocatorContext;
+  struct THClStorage *view;
+} THClStorage;
+
+float *THClStorage_data(THClState *state, const THClStorage *s);
+long THClStorage_size(THClState *state, const THClStorage *s);
+void THClStorage_set(THClState *state, THClStorage *s, long index, float value);
+float THClStorage_get(THClState *state, const THClStorage *s, long index);
+THClStorage *THClStorage_newv2(THClState *state, int device);
+THClStorage *THClStorage_newWithSize(THClState *state, int device, long size);
+void THClStorage_retain(THClState *state, THClStorage *s);
+void THClStorage_free(THClState *state, THClStorage *s);
+void THClStorage_resize(THClState *state, THClStorage *s, long size);
+void THClStorage_fill(THClState *state, THClStorage *s, float value);
+/* src/lib/THClStorageCopy.h:9-10,27 */
+void THClStorage_rawCopy(THClState *state, THClStorage *s, float *src);
+void THClStorage_copyFloat(THClState *state, THClStorage *s, THFloatStorage *src);
+void THFloatStorage_copyCl(THClState *state, THFloatStorage *self, THClStorage *src);
+
+/* ------------------------------------------------------------------------- */
+/* Tensor header and views (reference: src/lib/THClTensor.h:14-145)           */
+/* ------------------------------------------------------------------------- */
+typedef struct THClTensor {
+  long *size;
+  long *stride;
+  int nDimension; /* -1: empty header, 0: point tensor (one element of storage) */
+  THClStorage *storage;
+  long storageOffset;
+  int refcount;
+  char flag;
+  int device;
+} THClTensor;
+
+THClStorage *THClTensor_storage(THClState *state, const THClTensor *self);
+long THClTensor_storageOffset(THClState *state, const THClTensor *self);
+int THClTensor_nDimension(THClState *state, const THClTensor *self);
+long THClTensor_size(THClState *state, const THClTensor *self, int dim);
+long THClTensor_stride(THClState *state, const THClTensor *self, int dim);
+THLongStorage *THClTensor_newSizeOf(THClState *state, THClTensor *self);
+THLongStorage *THClTensor_newStrideOf(THClState *state, THClTensor *self);
+/* device address of the first element (the reference returns its host mirror) */
+float *THClTensor_data(THClState *state, const THClTensor *self);
+
+THClTensor *THClTensor_newv2(THClState *state, int device);
+THClTensor *THClTensor_newWithTensor(THClState *state, THClTensor *tensor);
+THClTensor *THClTensor_newWithStorage(THClState *state, int device, THClStorage *storage, long storageOffset,
+                                      THLongStorage *size, THLongStorage *stride);
+THClTensor *THClTensor_newWithSize(THClState *state, int device, THLongStorage *size, THLongStorage *stride);
+THClTensor *THClTensor_newWithSize1d(THClState *state, int device, long size0);
+THClTensor *THClTensor_newWithSize2d(THClState *state, int device, long size0, long size1);
+THClTensor *THClTensor_newWithSize3d(THClState *state, int device, long size0, long size1, long size2);
+THClTensor *THClTensor_newWithSize4d(THClState *state, int device, long size0, long size1, long size2, long size3);
+THClTensor *THClTensor_newClone(THClState *state, THClTensor *self);
+THClTensor *THClTensor_newContiguous(THClState *state, THClTensor *self);
+THClTensor *THClTensor_newSelect(THClState *state, THClTensor *tensor, int dimension, long sliceIndex);
+THClTensor *THClTensor_newNarrow(THClState *state, THClTensor *tensor, int dimension, long firstIndex, long size);
+THClTensor *THClTensor_newTranspose(THClState *state, THClTensor *tensor, int dimension1, int dimension2);
+THClTensor *THClTensor_newUnfold(THClState *state, THClTensor *tensor, int dimension, long size, long step);
+
+void THClTensor_resize(THClState *state, THClTensor *self, THLongStorage *size, THLongStorage *stride);
+void THClTensor_resizeAs(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_resize0d(THClState *state, THClTensor *self);
+void THClTensor_resize1d(THClState *state, THClTensor *self, long size0);
+void THClTensor_resize2d(THClState *state, THClTensor *self, long size0, long size1);
+void THClTensor_resize3d(THClState *state, THClTensor *self, long size0, long size1, long size2);
+void THClTensor_resize4d(THClState *state, THClTensor *self, long size0, long size1, long size2, long size3);
+
+void THClTensor_set(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_setStorage(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset,
+                           THLongStorage *size, THLongStorage *stride);
+void THClTensor_narrow(THClState *state, THClTensor *self, THClTensor *src, int dimension, long firstIndex, long size);
+void THClTensor_select(THClState *state, THClTensor *self, THClTensor *src, int dimension, long sliceIndex);
+void THClTensor_transpose(THClState *state, THClTensor *self, THClTensor *src, int dimension1, int dimension2);
+void THClTensor_unfold(THClState *state, THClTensor *self, THClTensor *src, int dimension, long size, long step);
+void THClTensor_squeeze(THClState *state, THClTensor *self, THClTensor *src);
+
+int THClTensor_isContiguous(THClState *state, const THClTensor *self);
+int THClTensor_isSameSizeAs(THClState *state, const THClTensor *self, const THClTensor *src);
+long THClTensor_nElement(THClState *state, const THClTensor *self);
+void THClTensor_retain(THClState *state, THClTensor *self);
+void THClTensor_free(THClState *state, THClTensor *self);
+void THClTensor_freeCopyTo(THClState *state, THClTensor *self, THClTensor *dst);
+int THClTensor_getDevice(THClState *state, const THClTensor *self);
+
+void THClTensor_set1d(THClState *state, THClTensor *t, long x0, float value);
+void THClTensor_set2d(THClState *state, THClTensor *t, long x0, long x1, float value);
+float THClTensor_get1d(THClState *state, const THClTensor *t, long x0);
+float THClTensor_get2d(THClState *state, const THClTensor *t, long x0, long x1);
+
+/* ------------------------------------------------------------------------- */
+/* Copies (reference: src/lib/THClTensorCopy.h:7-23)                          */
+/* ------------------------------------------------------------------------- */
+void THClTensor_copy(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_copyCl(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_copyFloat(THClState *state, THClTensor *self, THFloatTensor *src);
+void THClTensor_copyLong(THClState *state, THClTensor *self, THLongTensor *src);
+void THFloatTensor_copyCl(THClState *state, THFloatTensor *self, THClTensor *src);
+void THLongTensor_copyCl(THClState *state, THLongTensor *self, THClTensor *src);
+
+/* ------------------------------------------------------------------------- */
+/* Pointwise (reference: src/lib/THClTensorMath.h:7-28,98-155)                */
+/* `self == src` is the in-place form; otherwise `self` is resized to `src`.  */
+/* ------------------------------------------------------------------------- */
+void THClTensor_fill(THClState *state, THClTensor *self, float value);
+void THClTensor_zero(THClState *state, THClTensor *self);
+void THClTensor_fill_gpu(THClState *state, THClTensor *self, THClTensor *value);
+void THClTensor_zeros(THClState *state, THClTensor *r_, THLongStorage *size);
+void THClTensor_ones(THClState *state, THClTensor *r_, THLongStorage *size);
+long THClTensor_numel(THClState *state, THClTensor *t);
+
+void THClTensor_add(THClState *state, THClTensor *self, THClTensor *src, float value);
+void THClTensor_sub(THClState *state, THClTensor *self, THClTensor *src, float value);
+void THClTensor_mul(THClState *state, THClTensor *self, THClTensor *src, float value);
+/* element-wise true division, as Torch7's CPU path computes it (the OpenCL
+ * reference multiplies by 1.0f/value: src/lib/THClTensorMathPairwise.cpp:223-241) */
+void THClTensor_div(THClState *state, THClTensor *self, THClTensor *src, float value);
+
+void THClTensor_cadd(THClState *state, THClTensor *self, THClTensor *src1, float value, THClTensor *src2);
+void THClTensor_csub(THClState *state, THClTensor *self, THClTensor *src1, float value, THClTensor *src2);
+void THClTensor_cmul(THClState *state, THClTensor *self, THClTensor *src1, THClTensor *src2);
+void THClTensor_cdiv(THClState *state, THClTensor *self, THClTensor *src1, THClTensor *src2);
+void THClTensor_addcmul(THClState *state, THClTensor *self, THClTensor *t, float value, THClTensor *src1, THClTensor *src2);
+void THClTensor_addcdiv(THClState *state, THClTensor *self, THClTensor *t, float value, THClTensor *src1, THClTensor *src2);
+
+/* scalar operand held on the device as a point tensor (0-dim, 1 element) */
+void THClTensor_add_gpu(THClState *state, THClTensor *self, THClTensor *src, THClTensor *value);
+void THClTensor_sub_gpu(THClState *state, THClTensor *self, THClTensor *src, THClTensor *value);
+void THClTensor_mul_gpu(THClState *state, THClTensor *self, THClTensor *src, THClTensor *value);
+void THClTensor_div_gpu(THClState *state, THClTensor *self, THClTensor *src, THClTensor *value);
+
+void THClTensor_sqrt(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_abs(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_neg(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_cinv(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_exp(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_log(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_tanh(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_sigmoid(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_floor(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_ceil(THClState *state, THClTensor *self, THClTensor *src);
+
+/* User expressions over x (read-write), y, z -- or *out, *in1, *in2 -- compiled
+ * at run time (reference: src/lib/THClTensorMathPointwise.cpp:79-146; Lua names
+ * apply_on_gpu / map_on_gpu / map2_on_gpu, src/TensorMath.lua:591-620). */
+void THClTensor_apply(THClState *state, THClTensor *self, char const *operation1);
+void THClTensor_map(THClState *state, THClTensor *self, THClTensor *two, char const *operation2);
+void THClTensor_map2(THClState *state, THClTensor *self, THClTensor *in1, THClTensor *in2, char const *operation3);
+
+/* ------------------------------------------------------------------------- */
+/* Reductions (reference: src/lib/THClTensorMath.h:30-39,133-155)             */
+/* ------------------------------------------------------------------------- */
+float THClTensor_sumall(THClState *state, THClTensor *self);
+float THClTensor_prodall(THClState *state, THClTensor *self);
+float THClTensor_maxall(THClState *state, THClTensor *self);
+float THClTensor_minall(THClState *state, THClTensor *self);
+/* result stays on the device in `self`, which becomes a point tensor */
+void THClTensor_sumall_gpu(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_prodall_gpu(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_maxall_gpu(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_minall_gpu(THClState *state, THClTensor *self, THClTensor *src);
+float THClTensor_as_float(THClState *state, THClTensor *self);
+
+void THClTensor_sum(THClState *state, THClTensor *self, THClTensor *src, long dim);
+void THClTensor_prod(THClState *state, THClTensor *self, THClTensor *src, long dim);
+/* `indices` receives 1-based positions as fp32, the reference's convention
+ * (src/lib/THClTensorMathTransformReduce.cl:32,74) */
+void THClTensor_max(THClState *state, THClTensor *values, THClTensor *indices, THClTensor *src, long dim);
+void THClTensor_min(THClState *state, THClTensor *values, THClTensor *indices, THClTensor *src, long dim);
+/* No counterpart in the reference: the same reductions with the positions
+ * written as 1-based int64 into a host LongTensor (what `indices:long()` yields
+ * in Lua), exact for reduction lengths beyond 2^24. */
+void THClTensor_maxLong(THClState *state, THClTensor *values, THLongTensor *indices, THClTensor *src, long dim);
+void THClTensor_minLong(THClState *state, THClTensor *values, THLongTensor *indices, THClTensor *src, long dim);
+
+/* ------------------------------------------------------------------------- */
+/* Dense contraction (reference: src/lib/THClTensorMath.h:47, THClBlas.h:42)  */
+/* ------------------------------------------------------------------------- */
+void THClTensor_addmm(THClState *state, THClTensor *self, float beta, THClTensor *t, float alpha,
+                      THClTensor *mat1, THClTensor *mat2);
+/* column-major sgemm on tensors' storages + offsets, BLAS argument meaning */
+void THClBlas_gemm(THClState *state, char transa, char transb, long m, long n, long k, float alpha,
+                   THClTensor *a, long lda, THClTensor *b, long ldb, float beta, THClTensor *c, long ldc);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

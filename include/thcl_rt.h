@@ -1,0 +1,82 @@
+/*
+ * Thin C-ABI HIP runtime layer: what the host code of the tensor library calls
+ * where the reference called EasyCL (device discovery, buffers, the in-order
+ * queue, the runtime kernel cache and the timers).  Reference call sites this
+ * replaces: `EasyCL::createForIndexedGpu` / `cl->wrap` / `CLWrapper::copyTo*` /
+ * `cl->kernelExists|getKernel` / `TemplatedKernel::buildKernel` /
+ * `CLKernel::run` / `cl->finish` / `StatefulTimer::*`
+ * (src/lib/THClGeneral.cpp:134-165, src/lib/THClStorage.cpp:112-140,
+ *  src/lib/THClApply.cpp:87-141, src/lib/THClKernels.cpp:156-176).
+ *
+ * One context per device, one in-order stream per context.  All functions
+ * return 0 on success or a negative code; thcl_rt_error() gives the message.
+ */
+#ifndef THCL_RT_H
+#define THCL_RT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct thcl_rt thcl_rt;
+typedef struct thcl_rt_kernel thcl_rt_kernel;
+
+typedef struct thcl_rt_props {
+  char name[128];
+  char arch[64];
+  int compute_units;
+  int wavefront;
+  int max_threads_per_block;
+  int clock_khz;
+  int lds_bytes_per_block;
+  size_t total_mem;
+} thcl_rt_props;
+
+int thcl_rt_device_count(void);
+/* lazily creates the context (stream + scratch) of `device`; NULL on failure */
+thcl_rt *thcl_rt_get(int device);
+void thcl_rt_release_all(void);
+const thcl_rt_props *thcl_rt_get_props(thcl_rt *rt);
+const char *thcl_rt_error(void);
+
+/* buffers */
+void *thcl_rt_malloc(thcl_rt *rt, size_t bytes);
+int thcl_rt_free(thcl_rt *rt, void *dptr);
+int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
+int thcl_rt_memcpy_d2h(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
+int thcl_rt_memcpy_d2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* queued            */
+
+/* queue */
+void *thcl_rt_stream(thcl_rt *rt); /* hipStream_t */
+int thcl_rt_sync(thcl_rt *rt);
+
+/* per-device scratch block (partials, tickets), zero-initialised once */
+void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes);
+/* pinned host words for handing scalars back */
+float *thcl_rt_host_word(thcl_rt *rt);
+
+/* Runtime-compiled kernels (hipRTC), cached per context by `key`.  `source`
+ * is complete HIP source; `entry` the extern "C" kernel name.  On a compile
+ * error returns NULL and thcl_rt_error() holds the compiler log. */
+thcl_rt_kernel *thcl_rt_kernel_get(thcl_rt *rt, const char *key, const char *source, const char *entry);
+int thcl_rt_kernel_cached(thcl_rt *rt, const char *key);
+int thcl_rt_launch(thcl_rt *rt, thcl_rt_kernel *k, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                   unsigned by, unsigned bz, unsigned lds_bytes, void *params, size_t params_bytes);
+/* compile only (no device needed): returns 0 and the code-object size */
+int thcl_rt_compile_check(const char *source, const char *arch, size_t *code_bytes);
+
+/* event timers on the context's stream */
+typedef struct thcl_rt_timer thcl_rt_timer;
+thcl_rt_timer *thcl_rt_timer_new(thcl_rt *rt);
+int thcl_rt_timer_start(thcl_rt_timer *t);
+int thcl_rt_timer_stop(thcl_rt_timer *t);
+float thcl_rt_timer_ms(thcl_rt_timer *t); /* waits for the stop event */
+void thcl_rt_timer_free(thcl_rt_timer *t);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
