@@ -295,34 +295,4 @@ unsigned thcl_dbg_divide(unsigned n, long d) {
   return (unsigned)((((unsigned long long)n * dv.magic) >> 32) + n) >> dv.shift;
 }
 
-// kind of kernel a call with these layouts would use; -1 when invalid.
-// ptr_align[i]: byte misalignment to assume for operand i's first element.
-int thcl_dbg_plan_kind(int n, const int *ndims, const long *sizes, const long *strides, const long *offsets,
-                       int *out_dims, long *out_sizes, long *out_strides) {
-  THClTensor hdr[3];
-  THClTensor *tp[3];
-  THClStorage st[3];
-  long sz[3][THCL_MAX_DIMS], sd[3][THCL_MAX_DIMS];
-  for (int i = 0; i < n; i++) {
-    memset(&hdr[i], 0, sizeof(THClTensor));
-    memset(&st[i], 0, sizeof(THClStorage));
-    for (int d = 0; d < ndims[i]; d++) {
-      sz[i][d] = sizes[i * THCL_MAX_DIMS + d];
-      sd[i][d] = strides[i * THCL_MAX_DIMS + d];
-    }
-    hdr[i].size = sz[i];
-    hdr[i].stride = sd[i];
-    hdr[i].nDimension = ndims[i];
-    hdr[i].storageOffset = offsets[i];
-    tp[i] = &hdr[i];
-  }
-  JointLayout J = thcl_joint_collapse(n, tp);
-  if (!J.valid) return -1;
-  *out_dims = J.dims;
-  for (int d = 0; d < J.dims; d++) {
-    out_sizes[d] = J.sizes[d];
-    for (int i = 0; i < n; i++) out_strides[i * THCL_MAX_DIMS + d] = J.strides[i][d];
-  }
-  return J.dims;
-}
 }

@@ -13,8 +13,13 @@
 #include <vector>
 
 struct thcl_rt_kernel {
-  hipModule_t module = nullptr;
   hipFunction_t fn = nullptr;
+};
+
+// one compiled source: its code object and the entry points looked up so far
+struct RtModule {
+  hipModule_t module = nullptr;
+  std::map<std::string, thcl_rt_kernel *> entries;
 };
 
 struct thcl_rt {
@@ -24,7 +29,7 @@ struct thcl_rt {
   size_t scratch_bytes = 0;
   float *host_word = nullptr;
   thcl_rt_props props{};
-  std::map<std::string, thcl_rt_kernel *> kernels;
+  std::map<std::string, RtModule *> modules;
 };
 
 struct thcl_rt_timer {
@@ -129,7 +134,8 @@ void thcl_rt_release_all(void) {
     if (!rt) continue;
     DeviceGuard g(d);
     (void)hipStreamSynchronize(rt->stream);
-    for (auto &kv : rt->kernels) {
+    for (auto &kv : rt->modules) {
+      for (auto &e : kv.second->entries) delete e.second;
       if (kv.second->module) (void)hipModuleUnload(kv.second->module);
       delete kv.second;
     }
@@ -239,28 +245,42 @@ int thcl_rt_compile_check(const char *source, const char *arch, size_t *code_byt
   return rc;
 }
 
-int thcl_rt_kernel_cached(thcl_rt *rt, const char *key) { return rt->kernels.count(key) ? 1 : 0; }
+int thcl_rt_kernel_cached(thcl_rt *rt, const char *key) { return rt->modules.count(key) ? 1 : 0; }
 
+// Modules are cached by `key`, entry points by (key, entry): one source holds
+// several kernels and each call names the one it needs.
 thcl_rt_kernel *thcl_rt_kernel_get(thcl_rt *rt, const char *key, const char *source, const char *entry) {
-  auto it = rt->kernels.find(key);
-  if (it != rt->kernels.end()) return it->second;
   DeviceGuard g(rt->device);
-  std::vector<char> code;
-  // strip feature suffixes such as ":sramecc+:xnack-" from the device's arch name
-  std::string arch = rt->props.arch;
-  size_t colon = arch.find(':');
-  if (colon != std::string::npos) arch = arch.substr(0, colon);
-  if (rtc_compile(source, arch.c_str(), code) != 0) return nullptr;
+  RtModule *mod = nullptr;
+  auto it = rt->modules.find(key);
+  if (it != rt->modules.end()) {
+    mod = it->second;
+  } else {
+    std::vector<char> code;
+    // strip feature suffixes such as ":sramecc+:xnack-" from the device's arch name
+    std::string arch = rt->props.arch;
+    size_t colon = arch.find(':');
+    if (colon != std::string::npos) arch = arch.substr(0, colon);
+    if (rtc_compile(source, arch.c_str(), code) != 0) return nullptr;
+    mod = new RtModule();
+    hipError_t e = hipModuleLoadData(&mod->module, code.data());
+    if (e != hipSuccess) {
+      fail("loading runtime-compiled code", e);
+      delete mod;
+      return nullptr;
+    }
+    rt->modules[key] = mod;
+  }
+  auto fit = mod->entries.find(entry);
+  if (fit != mod->entries.end()) return fit->second;
   auto *k = new thcl_rt_kernel();
-  hipError_t e = hipModuleLoadData(&k->module, code.data());
-  if (e == hipSuccess) e = hipModuleGetFunction(&k->fn, k->module, entry);
+  hipError_t e = hipModuleGetFunction(&k->fn, mod->module, entry);
   if (e != hipSuccess) {
-    fail("loading runtime-compiled kernel", e);
-    if (k->module) (void)hipModuleUnload(k->module);
+    fail((std::string("entry point not found in runtime-compiled code: ") + entry).c_str(), e);
     delete k;
     return nullptr;
   }
-  rt->kernels[key] = k;
+  mod->entries[entry] = k;
   return k;
 }
 

@@ -1,0 +1,201 @@
+"""CPU-side checks of the shipped library: it loads, exports what the headers
+declare, never routes through the oracle, and its host logic (layout rules,
+index division, expression rewrite + run-time compile) is right.  No kernel is
+launched here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle
+from cltorch_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+MAXD = 25
+
+
+@pytest.fixture(scope="module")
+def lib():
+    L = _lib.load()
+    L.thcl_dbg_divide.restype = C.c_uint
+    L.thcl_dbg_divide.argtypes = [C.c_uint, C.c_long]
+    L.thcl_dbg_rewrite_expr.restype = C.c_int
+    L.thcl_dbg_rewrite_expr.argtypes = [C.c_char_p, C.c_int, C.c_char_p, C.c_size_t]
+    L.thcl_dbg_compile_expr.restype = C.c_int
+    L.thcl_dbg_compile_expr.argtypes = [C.c_char_p, C.c_int, C.c_char_p, C.POINTER(C.c_size_t)]
+    return L
+
+
+def test_library_exports_every_declared_symbol():
+    decls = _lib.declared_symbols()
+    assert len(decls) > 120
+    L = C.CDLL(_lib.LIB_PATH)
+    missing = [n for n in decls if not hasattr(L, n)]
+    assert not missing, missing
+    for must in ("THClTensor_cadd", "THClTensor_cmul", "THClTensor_div", "THClTensor_div_gpu", "THClTensor_apply",
+                 "THClTensor_map", "THClTensor_map2", "THClTensor_copy", "THClTensor_sumall", "THClTensor_sumall_gpu",
+                 "THClTensor_maxall", "THClTensor_minall", "THClTensor_sum", "THClTensor_max", "THClTensor_min",
+                 "THClTensor_addmm", "THClBlas_gemm", "THClTensor_as_float", "thcl_rt_kernel_get", "thcl_rt_launch"):
+        assert must in decls, must
+
+
+def test_product_never_touches_the_oracle():
+    pat = re.compile(r"\boracle\b")
+    for base, _, files in os.walk(os.path.join(ROOT, "cltorch_amd")):
+        if os.path.basename(base) == "build":
+            continue
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h", ".inc")):
+                text = open(os.path.join(base, f)).read()
+                assert not pat.search(text), f"{f} mentions the oracle"
+    for f in os.listdir(os.path.join(ROOT, "include")):
+        assert not pat.search(open(os.path.join(ROOT, "include", f)).read())
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libthcl_hip.so")
+    with pytest.raises(_lib.LibraryMissing):
+        _lib.load()
+
+
+def test_no_device_is_an_error_not_a_fallback():
+    L = _lib.load()
+    if L.thcl_rt_device_count() > 0:
+        pytest.skip("a GPU is visible")
+    buf = C.create_string_buffer(256)
+    st = C.cast(buf, C.c_void_p)
+    L.THCl_initializeState(st)
+    L.THClInit(st)
+    err = L.THClLastError()
+    assert err and b"no HIP device" in err
+
+
+def test_multiply_shift_division_is_exact(lib):
+    rng = np.random.RandomState(0)
+    divisors = [1, 2, 3, 4, 5, 7, 10, 63, 64, 65, 127, 128, 255, 256, 1000, 4096, 16384, 65535, 65536, 65537,
+                131072, 2 ** 25, 2 ** 26 - 1, 2 ** 30, 2 ** 31 - 1] + [int(v) for v in rng.randint(1, 2 ** 31 - 1, 40)]
+    for d in divisors:
+        ns = [0, 1, d - 1, d, d + 1, 2 * d - 1, 2 * d, 2 ** 31 - 1, 2 ** 31 - 2] + [int(v) for v in rng.randint(0, 2 ** 31 - 1, 200)]
+        for n in ns:
+            if 0 <= n < 2 ** 31:
+                assert lib.thcl_dbg_divide(n, d) == n // d, (n, d)
+
+
+def _arr(vals, n=MAXD):
+    a = (C.c_long * n)()
+    for i, v in enumerate(vals):
+        a[i] = v
+    return a
+
+
+def test_collapse_matches_oracle_rule(lib):
+    rng = np.random.RandomState(1)
+    for _ in range(400):
+        nd = rng.randint(1, 6)
+        sizes = [int(rng.choice([1, 1, 2, 3, 4, 6])) for _ in range(nd)]
+        strides = [int(rng.choice([0, 1, 2, 3, 4, 6, 8, 12, 24])) for _ in range(nd)]
+        rd = int(rng.randint(-1, nd))
+        osz, ost = (C.c_long * MAXD)(), (C.c_long * MAXD)()
+        k = lib.thcl_dbg_collapse(nd, _arr(sizes), _arr(strides), rd, osz, ost)
+        want = oracle.collapse(sizes, strides, rd)
+        assert (list(osz[:k]), list(ost[:k])) == want
+        assert bool(lib.thcl_dbg_overlapping(nd, _arr(sizes), _arr(strides))) == oracle.overlapping(sizes, strides)
+
+
+def _offsets(sizes, strides):
+    idx = np.indices(sizes).reshape(len(sizes), -1)
+    return (idx * np.array(strides).reshape(-1, 1)).sum(axis=0)
+
+
+def test_joint_collapse_pairs_the_same_elements(lib):
+    """Walking the joint layout must visit exactly the (offset0, offset1, ...) tuples
+    that walking the operands in logical order visits -- in any order."""
+    rng = np.random.RandomState(2)
+    for _ in range(300):
+        nd = rng.randint(1, 5)
+        n = rng.randint(1, 4)
+        sizes = [int(rng.choice([1, 2, 3, 4, 5])) for _ in range(nd)]
+        all_strides = []
+        for i in range(n):
+            perm = rng.permutation(nd)
+            st, z = [0] * nd, 1
+            for d in perm:                       # dense in a random dim order, sometimes with gaps
+                st[d] = z
+                z *= sizes[d] * int(rng.choice([1, 1, 2]))
+            if i > 0 and rng.rand() < 0.2:
+                st[int(rng.randint(nd))] = 0     # broadcast input
+            all_strides.append(st)
+        szs = (C.c_long * (3 * MAXD))()
+        sts = (C.c_long * (3 * MAXD))()
+        for i in range(n):
+            for d in range(nd):
+                szs[i * MAXD + d] = sizes[d]
+                sts[i * MAXD + d] = all_strides[i][d]
+        osz, ost = (C.c_long * MAXD)(), (C.c_long * (3 * MAXD))()
+        k = lib.thcl_dbg_joint_collapse(n, (C.c_int * 3)(*([nd] * n + [0] * (3 - n))), szs, sts, osz, ost)
+        assert k >= 1
+        jsz = list(osz[:k])
+        want = set(zip(*[_offsets(sizes, all_strides[i]).tolist() for i in range(n)]))
+        got = set(zip(*[_offsets(jsz, [ost[i * MAXD + d] for d in range(k)]).tolist() for i in range(n)]))
+        assert got == want
+        assert int(np.prod(jsz)) == int(np.prod(sizes))
+
+
+def test_joint_collapse_makes_identically_transposed_views_dense(lib):
+    szs, sts = (C.c_long * (3 * MAXD))(), (C.c_long * (3 * MAXD))()
+    for i in range(2):
+        for d, (s, t) in enumerate(zip((256, 512, 512), (1, 256, 131072))):
+            szs[i * MAXD + d], sts[i * MAXD + d] = s, t
+    osz, ost = (C.c_long * MAXD)(), (C.c_long * (3 * MAXD))()
+    k = lib.thcl_dbg_joint_collapse(2, (C.c_int * 3)(3, 3, 0), szs, sts, osz, ost)
+    assert k == 1 and osz[0] == 2 ** 26 and ost[0] == 1 and ost[MAXD] == 1
+    # different shapes with equal element counts are not joint-collapsible
+    szs[MAXD + 0], szs[MAXD + 1], szs[MAXD + 2] = 512, 256, 512
+    assert lib.thcl_dbg_joint_collapse(2, (C.c_int * 3)(3, 3, 0), szs, sts, osz, ost) == -1
+
+
+def _rewrite(lib, expr, n):
+    buf = C.create_string_buffer(4096)
+    r = lib.thcl_dbg_rewrite_expr(expr.encode(), n, buf, 4096)
+    assert r >= 0
+    return buf.value.decode()
+
+
+def test_expression_rewrite(lib):
+    # the two spellings the reference's tests use (src/test/unit_tensor.lua:583-635)
+    assert _rewrite(lib, "x = sqrt(x + 3) + exp(x)", 1) == "(*out) = sqrt((*out) + 3) + exp((*out))"
+    assert _rewrite(lib, "*out = sqrt(*out + 3) + exp(*out)", 1) == "*out = sqrt(*out + 3) + exp(*out)"
+    assert _rewrite(lib, "x = sqrt(x * x + y * y + z + 3 + exp(z))", 3) == \
+        "(*out) = sqrt((*out) * (*out) + (*in1) * (*in1) + (*in2) + 3 + exp((*in2)))"
+    # y / z are only operands when the call has that many tensors (src/lib/THClTensorMathPointwise.cpp:79-146)
+    assert _rewrite(lib, "x = y + z", 1) == "(*out) = y + z"
+    assert _rewrite(lib, "x = y + z", 2) == "(*out) = (*in1) + z"
+    # identifiers containing x/y/z survive (the reference only shields exp and max)
+    assert _rewrite(lib, "x = max(x, y) + hypot(x, y) + copysign(x, z)", 3) == \
+        "(*out) = max((*out), (*in1)) + hypot((*out), (*in1)) + copysign((*out), (*in2))"
+    # floating literals become fp32, integer literals and suffixed ones stay
+    assert _rewrite(lib, "x = 1000*x + 0.5 + 1e-3 + 2. + .25 + 3.5f + 7", 1) == \
+        "(*out) = 1000*(*out) + 0.5f + 1e-3f + 2.f + .25f + 3.5f + 7"
+
+
+@pytest.mark.parametrize("expr,n", [
+    ("x = sqrt(1000*x*x + y*10 + z*z)", 3),
+    ("x = 1000*x + y*10", 2),
+    ("*out = sqrt(*out * *out + *in1 * *in1 + 3 + exp(*in1))", 2),
+    ("x = clamp(x, -0.5, 0.5) + pown(x, 3) + sign(x) + fmax(x, 0.1)", 1),
+])
+def test_expressions_compile_for_gfx950(lib, expr, n):
+    size = C.c_size_t(0)
+    rc = lib.thcl_dbg_compile_expr(expr.encode(), n, b"gfx950", C.byref(size))
+    assert rc == 0, lib.thcl_rt_error().decode()
+    assert size.value > 1000
+
+
+def test_bad_expression_reports_compiler_log(lib):
+    size = C.c_size_t(0)
+    rc = lib.thcl_dbg_compile_expr(b"x = this is not C", 1, b"gfx950", C.byref(size))
+    assert rc != 0
+    assert b"error" in lib.thcl_rt_error()

@@ -1,0 +1,146 @@
+"""GPU parity: addmm / gemm against an fp64-accumulated CPU product, 1e-4
+relative (measured against the row's magnitude scale), through the C ABI.
+Layout cases follow src/lib/THClTensorMathBlas.cpp:107-214."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import View
+from gpu_util import Pair
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+RTOL = 1e-4
+
+
+def rel_err(got, want):
+    """max |got - want| relative to the scale of the result (its RMS), which is
+    what a 1e-4 bound on an fp32 dot product of length K can meaningfully mean
+    for entries that cancel to nearly zero."""
+    want = np.asarray(want, dtype=np.float64)
+    scale = max(float(np.sqrt(np.mean(want ** 2))), 1e-30)
+    return float(np.max(np.abs(np.asarray(got, dtype=np.float64) - want))) / scale
+
+
+def test_reference_integer_matrices(cl, golden):
+    g = golden["blas_mm"]
+    assert cl.mm(cl.ClTensor(g["A"]), cl.ClTensor(g["B"])).float().tolist() == g["expect"]
+
+
+def _check(cl, pa: Pair, pb: Pair, pc: Pair, beta, alpha):
+    want = oracle.addmm_f64(beta, pc.view, alpha, pa.view, pb.view)
+    pc.dev.addmm(beta, alpha, pa.dev, pb.dev)
+    got = pc.dev.float()
+    assert rel_err(got, want) < RTOL
+    return got, want
+
+
+@pytest.mark.parametrize("M,N,K", [(2, 2, 3), (1, 1, 1), (5, 7, 3), (64, 64, 16), (128, 128, 32), (128, 256, 64),
+                                   (65, 63, 17), (129, 127, 33), (300, 200, 100), (256, 64, 512), (64, 1024, 48),
+                                   (1, 500, 37), (500, 1, 37), (37, 41, 1)])
+def test_shapes_row_major(cl, M, N, K):
+    a = oracle.normal(1, M * K).reshape(M, K)
+    b = oracle.normal(2, K * N).reshape(K, N)
+    c = oracle.normal(3, M * N).reshape(M, N)
+    _check(cl, Pair.dense(cl, a), Pair.dense(cl, b), Pair.dense(cl, c), 0.5, 1.0)
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("tc", [False, True])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 64), (70, 90, 50)])
+def test_every_operand_layout(cl, ta, tb, tc, M, N, K):
+    """Each operand either dense or the transpose of a dense array: all
+    'n'/'t' combinations of the gemm, with the result row- or column-major."""
+    a = oracle.normal(4, M * K).reshape(M, K)
+    b = oracle.normal(5, K * N).reshape(K, N)
+    c = oracle.normal(6, M * N).reshape(M, N)
+    pa = Pair.dense(cl, a.T.copy()).transpose(0, 1) if ta else Pair.dense(cl, a)
+    pb = Pair.dense(cl, b.T.copy()).transpose(0, 1) if tb else Pair.dense(cl, b)
+    pc = Pair.dense(cl, c.T.copy()).transpose(0, 1) if tc else Pair.dense(cl, c)
+    got, want = _check(cl, pa, pb, pc, 0.5, 1.5)
+    plain = 0.5 * c.astype(np.float64) + 1.5 * (a.astype(np.float64) @ b.astype(np.float64))
+    assert np.allclose(want, plain, rtol=1e-12, atol=1e-12)      # the oracle saw the same matrices
+
+
+def test_operands_with_no_unit_stride_and_gapped_result(cl):
+    M, N, K = 48, 40, 24
+    a = oracle.normal(7, M * K * 2).reshape(M, K * 2)
+    b = oracle.normal(8, K * N * 2).reshape(K, N * 2)
+    c = oracle.normal(9, M * N * 2).reshape(M, N * 2)
+    pa = Pair.dense(cl, a).step(1, 2)          # strides (2K, 2): neither is 1 -> dense clone inside
+    pb = Pair.dense(cl, b).step(1, 2)
+    pc = Pair.dense(cl, c).step(1, 2)          # result with neither stride 1 -> computed aside, copied back
+    before = pc.host_storage.copy()
+    _check(cl, pa, pb, pc, 0.25, 2.0)
+    untouched = pc.device_storage().reshape(M, N * 2)[:, 1::2]
+    assert np.array_equal(untouched, before.reshape(M, N * 2)[:, 1::2])
+
+
+def test_beta_zero_ignores_old_contents_and_out_of_place(cl):
+    M, N, K = 64, 64, 32
+    a = oracle.normal(10, M * K).reshape(M, K)
+    b = oracle.normal(11, K * N).reshape(K, N)
+    c = np.full((M, N), np.nan, dtype=F)
+    got = cl.ClTensor(c).addmm(0.0, 1.0, cl.ClTensor(a), cl.ClTensor(b)).float()
+    assert rel_err(got, a.astype(np.float64) @ b.astype(np.float64)) < RTOL
+    t = oracle.normal(12, M * N).reshape(M, N)
+    T = cl.ClTensor(t)
+    r = cl.ClTensor()
+    r.addmm(0.5, T, 1.0, cl.ClTensor(a), cl.ClTensor(b))    # r_ != t: t is copied, then updated
+    assert rel_err(r.float(), 0.5 * t + a.astype(np.float64) @ b.astype(np.float64)) < RTOL
+    assert np.array_equal(T.float(), t)
+    with pytest.raises(cl.ClError, match="size mismatch"):
+        cl.ClTensor(np.zeros((3, 3), dtype=F)).addmm(cl.ClTensor(a), cl.ClTensor(b))
+    with pytest.raises(cl.ClError, match="matrix and matrix expected"):
+        cl.ClTensor(c).addmm(cl.ClTensor(np.zeros(4, dtype=F)), cl.ClTensor(b))
+
+
+def test_gemm_entry_point_column_major(cl):
+    # THClBlas_gemm with BLAS argument meaning on column-major data
+    m, n, k = 96, 80, 40
+    A = oracle.normal(13, m * k).reshape(k, m)      # column-major m x k  == row-major (k, m)
+    B = oracle.normal(14, k * n).reshape(n, k)      # column-major k x n
+    Cm = oracle.normal(15, m * n).reshape(n, m)     # column-major m x n
+    tA, tB, tC = cl.ClTensor(A), cl.ClTensor(B), cl.ClTensor(Cm)
+    st = cl.state()
+    st.lib.THClBlas_gemm(st.ptr, C.c_char(b"n"), C.c_char(b"n"), m, n, k, C.c_float(1.0), tA._h, m, tB._h, k,
+                         C.c_float(0.5), tC._h, m)
+    st.check()
+    want = 0.5 * Cm.T.astype(np.float64) + A.T.astype(np.float64) @ B.T.astype(np.float64)
+    assert rel_err(tC.float().T, want) < RTOL
+
+
+def test_skinny_config_shape_reduced(cl):
+    # M=64, A given as the transpose of a dense (K x M) array, as in the benchmark configuration
+    M, N, K = 64, 2048, 512
+    at = oracle.normal(16, K * M, 0.0, 1.0 / np.sqrt(K)).reshape(K, M)
+    b = oracle.normal(17, K * N, 0.0, 1.0 / np.sqrt(K)).reshape(K, N)
+    c = oracle.normal(18, M * N, 0.0, 1.0 / np.sqrt(K)).reshape(M, N)
+    pa = Pair.dense(cl, at).transpose(0, 1)
+    assert pa.dev.stride() == (1, 64)
+    _check(cl, pa, Pair.dense(cl, b), Pair.dense(cl, c), 0.5, 1.0)
+
+
+def test_large_square_sampled(cl):
+    """2048^3 checked on sampled entries against fp64 dot products, plus a
+    size-independent property: (A @ I) == A bit for bit, and linearity in alpha."""
+    n = 2048
+    a = oracle.normal(8, n * n, 0.0, 1.0 / np.sqrt(n)).reshape(n, n)
+    b = oracle.normal(9, n * n, 0.0, 1.0 / np.sqrt(n)).reshape(n, n)
+    c = oracle.normal(10, n * n, 0.0, 1.0 / np.sqrt(n)).reshape(n, n)
+    A, B = cl.ClTensor(a), cl.ClTensor(b)
+    got = cl.ClTensor(c).addmm(0.5, 1.0, A, B).float()
+    rng = np.random.RandomState(0)
+    rows, cols = rng.randint(0, n, 4096), rng.randint(0, n, 4096)
+    want = oracle.addmm_f64_sampled(rows, cols, 0.5, View.contiguous(c), 1.0, View.contiguous(a), View.contiguous(b))
+    scale = float(np.sqrt(np.mean(want ** 2)))
+    assert np.max(np.abs(got[rows, cols] - want)) / scale < RTOL
+    eye = cl.ClTensor(np.eye(n, dtype=F))
+    assert np.array_equal(cl.mm(A, eye).float(), a)          # products with 0/1 are exact
+    assert np.array_equal(cl.mm(eye, A).float(), a)
+    two = cl.ClTensor(np.zeros((n, n), dtype=F)).addmm(0.0, 2.0, A, B).float()
+    one = cl.mm(A, B).float()
+    assert np.array_equal(two, 2 * one)                      # scaling by 2 is exact

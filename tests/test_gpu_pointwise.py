@@ -1,0 +1,308 @@
+"""GPU parity: pointwise apply, expressions and copies against the CPU oracle,
+bit for bit, through the C ABI (ctypes mirror of the Lua methods).  Modelled on
+the reference's own cases (src/test/unit_tensor.lua:225-359,583-635,759-775)."""
+import numpy as np
+import pytest
+
+import oracle
+from oracle import View, expr_host
+from gpu_util import Pair, assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+SIZES = [1, 2, 3, 4, 5, 63, 64, 65, 255, 1023, 1024, 1025, 4096 + 3, 100003, (1 << 20) + 1]
+
+
+def _ops():
+    # name, device call, oracle op, oracle scalar
+    return [
+        ("add(y)", lambda X, Y: X.add(Y), "cadd", 1.0),
+        ("add(0.3,y)", lambda X, Y: X.add(0.3, Y), "cadd", float(F(0.3))),
+        ("csub(y)", lambda X, Y: X.csub(Y), "csub", 1.0),
+        ("csub(0.7,y)", lambda X, Y: X.csub(0.7, Y), "csub", float(F(0.7))),
+        ("cmul(y)", lambda X, Y: X.cmul(Y), "cmul", 0.0),
+        ("cdiv(y)", lambda X, Y: X.cdiv(Y), "cdiv", 0.0),
+    ]
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_inplace_binary_dense_all_lengths(cl, n):
+    x, y = oracle.uniform(1, n), oracle.uniform(2, n, 0.5, 1.5)
+    for name, dev, op, v in _ops():
+        px, py = Pair.dense(cl, x), Pair.dense(cl, y)
+        dev(px.dev, py.dev)
+        oracle.pointwise(op, px.view, px.view, py.view, v)
+        assert_bit_equal(px.device_storage(), px.host_storage, f"{name} n={n}")
+        assert_bit_equal(py.device_storage(), y, "input modified")
+
+
+def test_reference_small_matrices(cl, golden):
+    c = np.array(golden["pointwise_pairs"]["c"], dtype=F)
+    d = np.array(golden["pointwise_pairs"]["d"], dtype=F)
+    assert_bit_equal(cl.ClTensor(c).add(cl.ClTensor(d)).float(), c + d)
+    assert_bit_equal(cl.ClTensor(c).cmul(cl.ClTensor(d)).float(), c * d)
+    assert_bit_equal(cl.ClTensor(c).cdiv(cl.ClTensor(d)).float(), c / d)
+    # out-of-place forms resize the result (torch.add(c, d))
+    r = cl.ClTensor()
+    r.add(cl.ClTensor(c), cl.ClTensor(d))
+    assert r.size() == (2, 3)
+    assert_bit_equal(r.float(), c + d)
+    r = cl.ClTensor()
+    r.cmul(cl.ClTensor(c), cl.ClTensor(d))
+    assert_bit_equal(r.float(), c * d)
+    g = golden["user_kernel_add3"]
+    assert cl.ClTensor(g["x"]).apply_on_gpu(g["expr"]).float().tolist() == g["expect"]
+
+
+def test_scalar_forms(cl, golden):
+    c = np.array(golden["scalar_ops"]["c"], dtype=F)
+    v = golden["scalar_ops"]["value"]
+    fv = F(v)
+    assert_bit_equal(cl.ClTensor(c).add(v).float(), c + fv)
+    assert_bit_equal(cl.ClTensor(c).csub(v).float(), c + (-fv))
+    assert_bit_equal(cl.ClTensor(c).mul(v).float(), c * fv)
+    assert_bit_equal(cl.ClTensor(c).div(v).float(), c / fv)        # true division, Torch7's CPU result
+    r = cl.ClTensor()
+    r.mul(cl.ClTensor(c), v)
+    assert_bit_equal(r.float(), c * fv)
+    x = oracle.uniform(4, 100001)
+    assert_bit_equal(cl.ClTensor(x).div(3.4).float(), x / F(3.4))
+    assert_bit_equal(cl.ClTensor(x).fill(1.345).float(), np.full_like(x, F(1.345)))
+    assert_bit_equal(cl.ClTensor(x).zero().float(), np.zeros_like(x))
+
+
+def test_unary_fixed_ops(cl, golden):
+    c = np.array(golden["pointwise_unary"]["c"], dtype=F)
+    with np.errstate(invalid="ignore"):
+        assert_bit_equal(cl.ClTensor(c).sqrt().float(), np.sqrt(c))
+    assert_bit_equal(cl.ClTensor(c).abs().float(), np.abs(c))
+    assert_bit_equal(cl.ClTensor(c).neg().float(), -c)
+    assert_bit_equal(cl.ClTensor(c).cinv().float(), F(1) / c)
+    r = cl.ClTensor()
+    r.abs(cl.ClTensor(c))
+    assert_bit_equal(r.float(), np.abs(c))
+    # transcendental operators: the reference's own tolerance (abs 2e-4, src/test/unit_tensor.lua:73-93)
+    tol = golden["tolerances"]["float_abs"]
+    pos = np.abs(c) + F(0.5)
+    assert np.allclose(cl.ClTensor(c).exp().float(), np.exp(c), atol=tol, rtol=1e-6)
+    assert np.allclose(cl.ClTensor(pos).log().float(), np.log(pos), atol=tol)
+    assert np.allclose(cl.ClTensor(c).tanh().float(), np.tanh(c), atol=tol)
+    assert np.allclose(cl.ClTensor(c).sigmoid().float(), 1 / (1 + np.exp(-c)), atol=tol)
+    assert_bit_equal(cl.ClTensor(c).floor().float(), np.floor(c))
+    assert_bit_equal(cl.ClTensor(c).ceil().float(), np.ceil(c))
+
+
+def test_three_tensor_forms(cl):
+    n = 70001
+    a, b, t = oracle.uniform(1, n), oracle.uniform(2, n, 0.5, 1.5), oracle.uniform(3, n)
+    A, B = cl.ClTensor(a), cl.ClTensor(b)
+    assert_bit_equal(cl.ClTensor().add(A, 0.25, B).float(), a + F(0.25) * b)
+    assert_bit_equal(cl.ClTensor().csub(A, B).float(), a - b)
+    assert_bit_equal(cl.ClTensor().cdiv(A, B).float(), a / b)
+    assert_bit_equal(cl.ClTensor(t).addcmul(0.5, A, B).float(), t + F(0.5) * a * b)
+    assert_bit_equal(cl.ClTensor(t).addcdiv(0.5, A, B).float(), t + F(0.5) * a / b)
+    r = cl.ClTensor()
+    r.addcmul(cl.ClTensor(t), 2.0, A, B)
+    assert_bit_equal(r.float(), t + F(2.0) * a * b)
+
+
+@pytest.mark.parametrize("misalign", [1, 2, 3])
+def test_dense_but_misaligned_views(cl, misalign):
+    n = 50000
+    x, y = oracle.uniform(1, n + 8), oracle.uniform(2, n + 8)
+    px = Pair(cl, x, misalign, (n,), (1,))
+    py = Pair(cl, y, (misalign * 2) % 4, (n,), (1,))
+    px.dev.add(py.dev)
+    oracle.pointwise("cadd", px.view, px.view, py.view, 1.0)
+    assert_bit_equal(px.device_storage(), px.host_storage, "outside the view must stay untouched")
+
+
+def _strided_cases(cl):
+    """(name, Pair x, Pair y) with equal shapes, covering each kernel family."""
+    rng_x = oracle.uniform(4, 24 * 40 * 16)
+    rng_y = oracle.uniform(5, 24 * 40 * 16)
+    base_x = Pair.dense(cl, rng_x.reshape(24, 40, 16))
+    base_y = Pair.dense(cl, rng_y.reshape(24, 40, 16))
+    yield "both transposed alike", base_x.transpose(0, 2), base_y.transpose(0, 2)
+    yield "x transposed, y dense", base_x.transpose(0, 2), Pair.dense(cl, rng_y.reshape(16, 40, 24))
+    yield "x dense, y transposed", Pair.dense(cl, rng_x.reshape(16, 40, 24)), base_y.transpose(0, 2)
+    yield "stride 2 inner", base_x.step(2, 2), base_y.step(2, 2)
+    yield "narrow inner aligned", base_x.narrow(2, 4, 8), base_y.narrow(2, 8, 8)
+    yield "narrow inner misaligned", base_x.narrow(2, 1, 7), base_y.narrow(2, 3, 7)
+    yield "narrow middle", base_x.narrow(1, 3, 21), base_y.narrow(1, 5, 21)
+    yield "select-like", base_x.narrow(0, 5, 1), base_y.narrow(0, 7, 1)
+    yield "transpose(1,2)", base_x.transpose(1, 2), base_y.transpose(1, 2).narrow(0, 0, 24)
+
+
+def test_strided_binary_ops_joint_layouts(cl):
+    for name, px, py in _strided_cases(cl):
+        before_y = py.host_storage.copy()
+        px.dev.add(py.dev)
+        oracle.pointwise("cadd", px.view, px.view, py.view, 1.0)
+        assert_bit_equal(px.device_storage(), px.host_storage, name)
+        px.dev.map_on_gpu(py.dev, "x = 1000*x + y*10")
+        oracle.pointwise("map_c2", px.view, py.view)
+        assert_bit_equal(px.device_storage(), px.host_storage, name + " (expression)")
+        assert_bit_equal(py.device_storage(), before_y, name + " input")
+
+
+def test_operands_of_different_shapes_pair_by_position(cl):
+    # only the element counts agree (src/lib/THClApply.cpp:152-159)
+    x = oracle.uniform(6, 30 * 28)
+    y = oracle.uniform(7, 30 * 28 * 2)
+    px = Pair.dense(cl, x.reshape(30, 28))
+    py = Pair(cl, y, 0, (28, 30), (1, 56))          # transposed, gapped, different shape
+    px.dev.add(py.dev)
+    oracle.pointwise("cadd", px.view, px.view, py.view, 1.0)
+    assert_bit_equal(px.device_storage(), px.host_storage)
+    pz = Pair(cl, y, 1, (4, 7, 30), (2, 8, 56))     # last element at 1 + 6 + 48 + 1624 = 1679, inside the storage
+    px.dev.map2_on_gpu(py.dev, pz.dev, "x = x*y + z")
+    want = expr_host.evaluate("x = x*y + z", px.view.gather().reshape(-1), py.view.gather().reshape(-1),
+                              pz.view.gather().reshape(-1))
+    assert_bit_equal(px.device_storage(), want)
+
+
+def test_many_dimensions(cl):
+    sizes = (2, 3, 2, 2, 3, 2, 2, 2, 3, 2)
+    n = int(np.prod(sizes))
+    x, y = oracle.uniform(8, n * 2), oracle.uniform(9, n)
+    strides, z = [], 2
+    for s in reversed(sizes):
+        strides.append(z)
+        z *= s
+    strides = tuple(reversed(strides))              # every element 2 apart: collapses to one strided dim
+    px = Pair(cl, x, 1, sizes, strides)
+    py = Pair.dense(cl, y.reshape(sizes))
+    px.dev.cmul(py.dev)
+    oracle.pointwise("cmul", px.view, px.view, py.view)
+    assert_bit_equal(px.device_storage(), px.host_storage)
+    # non-collapsible: reverse the dims of a dense tensor
+    rev = tuple(range(len(sizes) - 1, -1, -1))
+    base = Pair.dense(cl, y.reshape(sizes))
+    v = View(base.host_storage, 0, tuple(sizes[i] for i in rev), tuple(base.view.strides[i] for i in rev))
+    pr = base.derive(v)
+    out = Pair.dense(cl, np.zeros(v.sizes, dtype=F))
+    out.dev.copy(pr.dev)
+    oracle.pointwise("copy", out.view, pr.view)
+    assert_bit_equal(out.device_storage(), out.host_storage)
+    with pytest.raises(cl.ClError):
+        cl.ClTensor(4).add(cl.ClTensor(5))
+
+
+def test_written_operand_that_overlaps_itself(cl):
+    # expanded (stride 0) destination: staged through a dense temporary, then
+    # scattered back; every alias ends up with one of the written values
+    x = oracle.uniform(10, 8)
+    px = Pair(cl, x, 0, (4, 8), (0, 1))
+    y = oracle.uniform(11, 32).reshape(4, 8)
+    px.dev.add(cl.ClTensor(y))
+    got = px.device_storage()
+    candidates = x.reshape(1, 8) + y
+    assert all(any(got[j] == candidates[i, j] for i in range(4)) for j in range(8))
+
+
+def test_point_tensor_operands(cl):
+    n = 100003
+    a = oracle.uniform(7, n, 0.0, 1.0)
+    A = cl.ClTensor(a)
+    s = cl.ClTensor()
+    s.sum(A)                                   # stays on the device
+    assert s.nDimension() == 0
+    sv = F(s.s())
+    assert_bit_equal(cl.ClTensor(a).div(s).float(), a / sv)
+    assert_bit_equal(cl.ClTensor(a).mul(s).float(), a * sv)
+    assert_bit_equal(cl.ClTensor(a).add(s).float(), a + sv)     # cadd with a point tensor on the right
+    assert_bit_equal(cl.ClTensor(a).csub(s).float(), a - sv)
+    assert_bit_equal(cl.ClTensor(n).fill(s).float(), np.full(n, sv, dtype=F))
+    r = cl.ClTensor()
+    r.div(A, s)
+    assert_bit_equal(r.float(), a / sv)
+
+
+EXPRS = [
+    ("x = sqrt(1000*x*x + y*10 + z*z)", 3, True),
+    ("*out = sqrt(*out * *out + *in1 * *in1 + *in2 + 3 + exp(*in2))", 3, False),
+    ("x = sqrt(x * x + y * y + z + 3 + exp(z))", 3, False),
+    ("x = 1000*x + y*10", 2, True),
+    ("*out = sqrt(*out * *out + *in1 * *in1 + 3 + exp(*in1))", 2, False),
+    ("x = sqrt(x + 3) + exp(x)", 1, False),
+    ("x = x * 0.5 + 1e-3", 1, True),
+    ("x = (x > 0.25) ? x : 2*x", 1, True),
+    ("x = max(x, y) - min(x, y)", 2, True),
+]
+
+
+@pytest.mark.parametrize("expr,nt,exact", EXPRS)
+def test_user_expressions(cl, golden, expr, nt, exact):
+    n = 60 * 50
+    arrs = [oracle.uniform(20 + i, n, -0.5, 0.5) for i in range(3)][:nt]
+    T = [cl.ClTensor(a.reshape(60, 50)) for a in arrs]
+    if nt == 1:
+        T[0].apply_on_gpu(expr)
+    elif nt == 2:
+        T[0].map_on_gpu(T[1], expr)
+    else:
+        T[0].map2_on_gpu(T[1], T[2], expr)
+    want = expr_host.evaluate(expr, *arrs)
+    got = T[0].float().reshape(-1)
+    if exact:
+        assert_bit_equal(got, want, expr)
+    else:
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        ok = ~np.isnan(want)
+        assert np.max(np.abs(got[ok] - want[ok])) <= golden["tolerances"]["float_abs"], expr
+
+
+def test_expression_aliases_and_errors(cl):
+    x, y = oracle.uniform(1, 1000), oracle.uniform(2, 1000)
+    a = cl.ClTensor(x).apply2_on_gpu(cl.ClTensor(y), "x = x - y").float()
+    b = cl.ClTensor(x).map_on_gpu(cl.ClTensor(y), "*out = *out - *in1").float()
+    assert_bit_equal(a, x - y)
+    assert_bit_equal(b, x - y)
+    with pytest.raises(cl.ClError, match="compile"):
+        cl.ClTensor(x).apply_on_gpu("x = undefined_function_zzz(x)")
+    with pytest.raises(cl.ClError):
+        cl.ClTensor(x).div(0.0)
+    # the library is still usable after an error
+    assert_bit_equal(cl.ClTensor(x).add(1.0).float(), x + F(1))
+
+
+# ------------------------------------------------------------------ copies ---
+def test_copies_are_bit_exact_for_every_layout(cl):
+    for name, px, _ in _strided_cases(cl):
+        dst = Pair.dense(cl, np.zeros(px.view.sizes, dtype=F))
+        dst.dev.copy(px.dev)
+        assert_bit_equal(dst.device_storage(), px.view.gather(), name + " -> dense")
+        back = Pair.dense(cl, np.full(px.view.sizes, F(7)))
+        px.dev.copy(back.dev)                   # dense -> strided scatter
+        oracle.pointwise("copy", px.view, back.view)
+        assert_bit_equal(px.device_storage(), px.host_storage, "dense -> " + name)
+    # special values travel unchanged
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38], dtype=F)
+    assert np.array_equal(cl.ClTensor(special).clone().float().view(np.uint32), special.view(np.uint32))
+    t = Pair.dense(cl, np.tile(special, 8).reshape(8, 8)).transpose(0, 1)
+    assert np.array_equal(t.dev.contiguous().float().view(np.uint32),
+                          np.tile(special, 8).reshape(8, 8).T.copy().view(np.uint32))
+
+
+def test_copy_within_one_storage_and_size_checks(cl):
+    x = oracle.uniform(3, 64)
+    p = Pair(cl, x, 0, (32,), (1,))
+    q = p.derive(View(p.host_storage, 32, (32,), (1,)))
+    q.dev.copy(p.dev)                           # same storage: goes through the kernel, not a block copy
+    assert_bit_equal(p.device_storage(), np.concatenate([x[:32], x[:32]]))
+    with pytest.raises(cl.ClError, match="sizes do not match"):
+        cl.ClTensor(5).copy(cl.ClTensor(6))
+    e = cl.ClTensor()
+    e.copy(cl.ClTensor())                       # empty to empty: nothing happens
+
+
+def test_host_roundtrip_of_strided_views(cl):
+    base = oracle.uniform(12, 6 * 8 * 10).reshape(6, 8, 10)
+    p = Pair.dense(cl, base)
+    assert_bit_equal(p.transpose(0, 2).dev.float(), base.transpose(2, 1, 0))
+    assert_bit_equal(p.narrow(1, 2, 3).dev.float(), base[:, 2:5, :])
+    t = p.transpose(0, 1)
+    t.dev.copy(np.arange(8 * 6 * 10, dtype=F).reshape(8, 6, 10))     # host -> strided device view
+    assert_bit_equal(p.dev.float(), np.arange(480, dtype=F).reshape(8, 6, 10).transpose(1, 0, 2))

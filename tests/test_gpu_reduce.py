@@ -1,0 +1,197 @@
+"""GPU parity: reduce-all (host scalar and point tensor), reduce along a
+dimension, max/min with positions -- against the CPU oracle, through the C ABI.
+Sums: 1e-5 relative (the device accumulates in fp64 like Torch7's CPU path, so
+they are in practice equal or one ulp apart); max/min values and all positions:
+exact.  Cases follow src/test/unit_tensor.lua:488-496,637-657,735-832."""
+import numpy as np
+import pytest
+
+import oracle
+from oracle import View
+from gpu_util import Pair, assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+SUM_RTOL = 1e-5
+
+
+def close_sum(got, want64):
+    want = np.asarray(want64, dtype=np.float64)
+    got = np.asarray(got, dtype=np.float64)
+    assert np.all(np.abs(got - want) <= SUM_RTOL * np.abs(want) + 1e-30), (got, want)
+    # much tighter in practice: fp64 accumulation leaves at most the final rounding
+    assert np.all(np.abs(got - want) <= 1.5 * np.spacing(np.abs(want).astype(F)).astype(np.float64))
+
+
+def test_reference_matrix(cl, golden):
+    g = golden["matrixwide"]
+    C = cl.ClTensor(g["C"])
+    assert C.max() == g["max"] and C.min() == g["min"] and C.sum() == g["sum"]
+    assert C.sum(1).float().tolist() == g["sum_dim1"] and C.sum(2).float().tolist() == g["sum_dim2"]
+    for kind in ("max", "min"):
+        for dim in (1, 2):
+            vals, idx = getattr(C, kind)(dim)
+            assert vals.float().tolist() == g[f"{kind}_dim{dim}"]
+            assert idx.long().tolist() == g[f"arg{kind}_dim{dim}"]
+            vals2, idx2 = getattr(C, f"{kind}_long")(dim)
+            assert idx2.tolist() == g[f"arg{kind}_dim{dim}"] and idx2.dtype == np.int64
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 63, 64, 65, 1023, 1024, 1025, 4099, 65537, 1 << 20, (1 << 22) + 7])
+def test_reduce_all_lengths(cl, n):
+    x = oracle.uniform(5, n, -0.5, 0.5)
+    X, v = cl.ClTensor(x), View.contiguous(x)
+    close_sum(X.sum(), oracle.sumall(v))
+    assert X.max() == oracle.maxall(v) and X.min() == oracle.minall(v)
+    pt = cl.ClTensor()
+    pt.sum(X)
+    assert pt.nDimension() == 0 and pt.nElement() == 0
+    close_sum(pt.s(), oracle.sumall(v))
+    pt.max(X)
+    assert pt.s() == oracle.maxall(v)
+    pt.min(X)
+    assert pt.s() == oracle.minall(v)
+
+
+def test_reduce_all_reference_sizes(cl, golden):
+    # the two shapes of test_reduceAll, with the reference's (loose) bounds and ours
+    t = golden["tolerances"]
+    for shape, bound in ((t["reduceall_two_pass_shape"], t["reduceall_two_pass_abs"]),
+                         (t["reduceall_one_pass_shape"], t["reduceall_one_pass_abs"])):
+        n = int(np.prod(shape))
+        x = oracle.uniform(9, n, -0.5, 0.5)
+        got = cl.ClTensor(x.reshape(shape)).sum()
+        want = oracle.sumall(View.contiguous(x))
+        assert abs(got - want) < bound
+        close_sum(got, want)
+
+
+def test_reduce_all_closed_forms_and_determinism(cl):
+    assert cl.ClTensor(np.ones(1 << 21, dtype=F)).sum() == float(1 << 21)
+    ar = np.arange(1, 4097, dtype=F)
+    assert cl.ClTensor(ar).sum() == 4096 * 4097 / 2
+    assert cl.ClTensor(np.array([1, 2, 3, 4, 0.5], dtype=F)).prod() == 12.0
+    x = oracle.uniform(13, (1 << 21) + 3)
+    X = cl.ClTensor(x)
+    first = X.sum()
+    assert all(X.sum() == first for _ in range(5))
+    # linearity: doubling every element doubles the sum exactly (same combine order, exact scaling)
+    assert cl.ClTensor(x).mul(2.0).sum() == 2 * first
+
+
+def test_reduce_all_special_values(cl):
+    x = oracle.uniform(14, 100000)
+    x[777] = np.nan
+    X = cl.ClTensor(x)
+    assert np.isnan(X.sum()) and np.isnan(X.max()) and np.isnan(X.min())     # Torch7's CPU rule: NaN propagates
+    y = np.full(5000, -np.inf, dtype=F)
+    assert cl.ClTensor(y).max() == -np.inf
+    y[4321] = -3.0
+    assert cl.ClTensor(y).max() == -3.0 and cl.ClTensor(y).min() == -np.inf
+    assert cl.ClTensor(np.array([-0.0, 0.0], dtype=F)).sum() == 0.0
+
+
+def test_reduce_all_on_views(cl):
+    base = oracle.uniform(15, 40 * 30 * 20).reshape(40, 30, 20)
+    p = Pair.dense(cl, base)
+    for q in (p.transpose(0, 2), p.narrow(2, 3, 9), p.step(2, 2), p.narrow(0, 7, 1), p.transpose(0, 1).narrow(1, 2, 11)):
+        close_sum(q.dev.sum(), oracle.sumall(q.view))
+        assert q.dev.max() == oracle.maxall(q.view) and q.dev.min() == oracle.minall(q.view)
+    mis = Pair(cl, base.reshape(-1), 3, (5001,), (1,))
+    close_sum(mis.dev.sum(), oracle.sumall(mis.view))
+    assert cl.ClTensor().sum() == 0.0            # empty tensor: the identity
+
+
+def _check_dim(cl, pair, dim0):
+    """All three reductions along 0-based dim of a Pair, values + positions."""
+    dim = dim0 + 1
+    want, _ = oracle.reduce_dim("sum", pair.view, dim0)
+    got = pair.dev.sum(dim)
+    assert got.size() == want.shape
+    exact64 = pair.view.gather().astype(np.float64).sum(axis=dim0, keepdims=True)
+    close_sum(got.float(), exact64)
+    for kind in ("max", "min"):
+        wv, wi = oracle.reduce_dim(kind, pair.view, dim0)
+        gv, gi = getattr(pair.dev, kind)(dim)
+        assert_bit_equal(gv.float(), wv, f"{kind} values dim {dim}")
+        assert np.array_equal(gi.long(), wi), f"{kind} positions dim {dim}"
+        gv2, gi2 = getattr(pair.dev, f"{kind}_long")(dim)
+        assert np.array_equal(gi2, wi) and np.array_equal(gv2.float(), wv)
+
+
+@pytest.mark.parametrize("shape", [(5, 2), (60, 50), (3, 2000), (2000, 3), (7, 128), (129, 64), (33, 4096), (4096, 33),
+                                   (17, 9, 13), (4, 300, 8), (2, 3, 4, 5), (1, 77), (77, 1), (256, 2048)])
+def test_reduce_dim_shapes(cl, shape):
+    x = oracle.normal(6, int(np.prod(shape))).reshape(shape)
+    p = Pair.dense(cl, x)
+    for d in range(len(shape)):
+        _check_dim(cl, p, d)
+
+
+def test_reduce_dim_on_views_like_the_reference_tests(cl):
+    # A:t():sum(d), A:narrow(..):t():sum(d)  (src/test/unit_tensor.lua:759-775)
+    x = oracle.uniform(16, 60 * 50, -0.5, 0.5).reshape(60, 50)
+    p = Pair.dense(cl, x)
+    for q in (p.transpose(0, 1), p.narrow(0, 9, 30).transpose(0, 1), p.narrow(1, 9, 30).transpose(0, 1),
+              p.step(1, 2), p.narrow(1, 1, 33)):
+        for d in (0, 1):
+            _check_dim(cl, q, d)
+    y = oracle.uniform(17, 12 * 10 * 16).reshape(12, 10, 16)
+    p3 = Pair.dense(cl, y)
+    for q in (p3.transpose(0, 2), p3.transpose(1, 2), p3.narrow(2, 4, 8), p3.step(0, 3)):
+        for d in range(3):
+            _check_dim(cl, q, d)
+
+
+def test_positions_ties_and_nans(cl):
+    row = np.array([[1, 5, 5, 2, 5], [3, 3, 3, 3, 3]], dtype=F)
+    R = cl.ClTensor(row)
+    assert R.max(2)[1].long().ravel().tolist() == [2, 1]
+    assert R.min(2)[1].long().ravel().tolist() == [1, 1]
+    assert R.max(1)[1].long().ravel().tolist() == [2, 1, 1, 2, 1]
+    # long constant rows: every tree shape must still report position 1
+    for n in (64, 257, 5000):
+        c = cl.ClTensor(np.full((3, n), F(2.5)))
+        assert c.max(2)[1].long().ravel().tolist() == [1, 1, 1] and c.min(2)[1].long().ravel().tolist() == [1, 1, 1]
+        ct = cl.ClTensor(np.full((n, 3), F(2.5)))
+        assert ct.max(1)[1].long().ravel().tolist() == [1, 1, 1]
+    # planted ties far apart, and NaNs: first NaN wins (Torch7's CPU rule)
+    x = oracle.uniform(18, 4 * 3000).reshape(4, 3000)
+    x[0, 2500] = x[0, 17] = 9.0
+    x[1, 100] = np.nan
+    x[1, 2000] = np.nan
+    x[2, 2999] = -9.0
+    x[2, 1] = -9.0
+    p = Pair.dense(cl, x)
+    for d in (0, 1):
+        for kind in ("max", "min"):
+            wv, wi = oracle.reduce_dim(kind, p.view, d)
+            gv, gi = getattr(p.dev, kind)(d + 1)
+            assert_bit_equal(gv.float(), wv)
+            assert np.array_equal(gi.long(), wi)
+    assert p.dev.max(2)[1].long()[0, 0] == 18 and p.dev.max(2)[1].long()[1, 0] == 101
+    assert p.dev.min(2)[1].long()[2, 0] == 2
+
+
+def test_results_into_existing_strided_tensors(cl):
+    x = oracle.uniform(19, 40 * 24).reshape(40, 24)
+    X = cl.ClTensor(x)
+    holder = Pair.dense(cl, np.zeros((24, 2), dtype=F))
+    col = holder.narrow(1, 0, 1).transpose(0, 1)            # sizes (1,24), strides (1,2): right shape, not dense
+    st = cl.state()
+    import ctypes as C
+    st.lib.THClTensor_sum(st.ptr, col.dev._h, X._h, C.c_long(0))
+    st.check()
+    want = x.astype(np.float64).sum(axis=0).astype(F)
+    got = holder.device_storage().reshape(24, 2)
+    assert np.array_equal(got[:, 0], want) and np.all(got[:, 1] == 0)
+
+
+def test_dim_argument_checks(cl):
+    X = cl.ClTensor(np.zeros((3, 4), dtype=F))
+    with pytest.raises(cl.ClError, match="dimension out of range"):
+        X.sum(3)
+    with pytest.raises(cl.ClError, match="dimension out of range"):
+        X.max(0)
+    with pytest.raises(cl.ClError):
+        cl.ClTensor(np.zeros(3, dtype=F)).s()              # not a point tensor

@@ -1,0 +1,267 @@
+"""Pins the CPU oracle (oracle/th_oracle.c) before anything is compared with it.
+
+Each check is chosen so that a plausible slip -- a dropped term, operands
+swapped, a wrong index, a transposed stride -- makes it fail: IEEE fp32
+arithmetic redone by numpy, exactly rounded sums (math.fsum), brute-force
+index walks, closed forms, and the vectors of the reference's own tests
+(tests/golden/reference_vectors.json).
+"""
+import math
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import View
+
+F = np.float32
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).reshape(-1).view(np.uint32)
+
+
+# --------------------------------------------------------------- MT19937 ---
+def test_mt19937_known_answers():
+    # first outputs of the reference implementation (mt19937ar.c) for the default seed 5489
+    assert list(oracle.mt_raw(5489, 3)) == [3499211612, 581869302, 3890346734]
+
+
+def test_mt19937_matches_numpy_legacy_stream():
+    for seed in (1, 7, 12345):
+        rs = np.random.RandomState(seed)
+        want = rs.randint(0, 2 ** 32, size=2000, dtype=np.uint64).astype(np.uint32)
+        # RandomState.randint on the full 32-bit range consumes one raw word per draw
+        got = oracle.mt_raw(seed, 2000)
+        assert np.array_equal(got, want)
+
+
+def test_uniform_and_normal_ranges():
+    u = oracle.uniform(3, 200000, -1.0, 1.0)
+    assert u.dtype == np.float32 and u.min() >= -1.0 and u.max() < 1.0
+    assert abs(float(u.mean())) < 0.01 and abs(float(u.var()) - 1 / 3) < 0.01
+    raw = oracle.mt_raw(3, 5)
+    assert np.array_equal(u[:5], (raw.astype(np.float64) / 2 ** 32 * 2 - 1).astype(np.float32))
+    g = oracle.normal(6, 200000, 0.0, 1.0)
+    assert abs(float(g.mean())) < 0.01 and abs(float(g.std()) - 1) < 0.01
+    assert np.all(np.isfinite(g))
+
+
+# ------------------------------------------------------------- pointwise ---
+def test_pointwise_reference_pairs(golden):
+    c = np.array(golden["pointwise_pairs"]["c"], dtype=F)
+    d = np.array(golden["pointwise_pairs"]["d"], dtype=F)
+    for op, want in [("cadd", c + d), ("cmul", c * d), ("cdiv", c / d), ("csub", c - d)]:
+        r = View.contiguous(c.copy())
+        oracle.pointwise(op, r, r, View.contiguous(d), 1.0)
+        assert np.array_equal(bits(r.storage), bits(want)), op
+
+
+def test_pointwise_scalar_forms(golden):
+    c = np.array(golden["scalar_ops"]["c"], dtype=F)
+    v = F(golden["scalar_ops"]["value"])
+    for op, want in [("add_s", c + v), ("mul_s", c * v), ("div_s", c / v), ("sub_s", c + (-v)),
+                     ("mulrecip_s", c * (F(1) / v))]:
+        r = View.contiguous(c.copy())
+        oracle.pointwise(op, r, r, None, float(v))
+        assert np.array_equal(bits(r.storage), bits(want)), op
+    # dividing and multiplying by the reciprocal really are different roundings somewhere
+    x = oracle.uniform(11, 4096)
+    a, b = View.contiguous(x.copy()), View.contiguous(x.copy())
+    oracle.pointwise("div_s", a, a, None, 3.4)
+    oracle.pointwise("mulrecip_s", b, b, None, 3.4)
+    assert np.array_equal(a.storage, x / F(3.4)) and not np.array_equal(a.storage, b.storage)
+
+
+def test_cadd_rounds_product_then_sum():
+    # a + v*b with two roundings; a fused multiply-add would differ on some inputs
+    rng = np.random.RandomState(0)
+    a = rng.uniform(-1, 1, 50000).astype(F)
+    b = rng.uniform(-1, 1, 50000).astype(F)
+    v = F(0.3)
+    r = View.contiguous(a.copy())
+    oracle.pointwise("cadd", r, r, View.contiguous(b), float(v))
+    two_roundings = a + (v * b)
+    fused = (a.astype(np.float64) + np.float64(v) * b.astype(np.float64)).astype(F)
+    assert np.array_equal(bits(r.storage), bits(two_roundings))
+    assert not np.array_equal(two_roundings, fused)  # the check can tell the two apart
+
+
+def test_config_expressions_closed_form():
+    x, y, z = (oracle.uniform(s, 10000) for s in (1, 2, 3))
+    r = View.contiguous(x.copy())
+    oracle.pointwise("map2_c1", r, View.contiguous(y), View.contiguous(z))
+    with np.errstate(invalid="ignore"):
+        want = np.sqrt(F(1000) * x * x + y * F(10) + z * z)
+    assert np.array_equal(np.isnan(r.storage), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(bits(r.storage[ok]), bits(want[ok]))
+    r = View.contiguous(x.copy())
+    oracle.pointwise("map_c2", r, View.contiguous(y))
+    assert np.array_equal(bits(r.storage), bits(F(1000) * x + y * F(10)))
+
+
+def test_pointwise_walks_strided_views_in_logical_order():
+    base = np.arange(4 * 6 * 5, dtype=F)
+    a = View.contiguous(base.reshape(4, 6, 5).copy())
+    t = a.transpose(0, 2)                      # sizes (5,6,4), strides (1,5,30)
+    dst = View.contiguous(np.zeros((5, 6, 4), dtype=F))
+    oracle.pointwise("copy", dst, t)
+    assert np.array_equal(dst.storage.reshape(5, 6, 4), base.reshape(4, 6, 5).transpose(2, 1, 0))
+    n = a.narrow(2, 1, 3)                      # offset 1
+    assert np.array_equal(n.gather(), base.reshape(4, 6, 5)[:, :, 1:4])
+    s = a.step(2, 2)
+    assert np.array_equal(s.gather(), base.reshape(4, 6, 5)[:, :, ::2])
+    # same element count, different shapes: pairing is by logical position
+    flat = View.contiguous(np.zeros(5 * 6 * 4, dtype=F))
+    oracle.pointwise("copy", flat, t)
+    assert np.array_equal(flat.storage, base.reshape(4, 6, 5).transpose(2, 1, 0).reshape(-1))
+    with pytest.raises(ValueError):
+        oracle.pointwise("copy", View.contiguous(np.zeros(7, dtype=F)), t)
+
+
+# ---------------------------------------------------------------- reduce ---
+def test_sumall_is_double_accumulated():
+    x = oracle.uniform(5, 300001, 0.0, 1.0)
+    got = oracle.sumall(View.contiguous(x))
+    exact = math.fsum(float(v) for v in x)
+    assert abs(got - exact) < 1e-7 * exact
+    # an fp32 accumulator would be far off at this length: the check notices
+    f32 = F(0)
+    for v in x[:100000]:
+        f32 = F(f32 + v)
+    assert abs(float(f32) - math.fsum(float(v) for v in x[:100000])) > 1e-3
+    assert oracle.sumall(View.contiguous(np.ones(12345, dtype=F))) == 12345.0
+    ar = np.arange(1, 2001, dtype=F)
+    assert oracle.sumall(View.contiguous(ar)) == 2000 * 2001 / 2
+    assert oracle.prodall(View.contiguous(np.array([1, 2, 3, 4, 0.5], dtype=F))) == 12.0
+
+
+def test_reduce_reference_vectors(golden):
+    g = golden["matrixwide"]
+    C = np.array(g["C"], dtype=F)
+    v = View.contiguous(C)
+    assert oracle.maxall(v) == g["max"] and oracle.minall(v) == g["min"] and oracle.sumall(v) == g["sum"]
+    assert np.array_equal(oracle.reduce_dim("sum", v, 0)[0], np.array(g["sum_dim1"], dtype=F))
+    assert np.array_equal(oracle.reduce_dim("sum", v, 1)[0], np.array(g["sum_dim2"], dtype=F))
+    for kind in ("max", "min"):
+        for dim in (0, 1):
+            vals, idx = oracle.reduce_dim(kind, v, dim)
+            assert np.array_equal(vals, np.array(g[f"{kind}_dim{dim + 1}"], dtype=F))
+            assert np.array_equal(idx, np.array(g[f"arg{kind}_dim{dim + 1}"], dtype=np.int64))
+
+
+def test_reduce_dim_brute_force_on_views():
+    rng = np.random.RandomState(1)
+    base = rng.uniform(-1, 1, (7, 9, 5)).astype(F)
+    a = View.contiguous(base)
+    for view, ref in [(a, base), (a.transpose(0, 2), base.transpose(2, 1, 0)),
+                      (a.narrow(1, 2, 4), base[:, 2:6, :]), (a.step(2, 2), base[:, :, ::2])]:
+        for dim in range(3):
+            s, _ = oracle.reduce_dim("sum", view, dim)
+            want = ref.astype(np.float64).sum(axis=dim, keepdims=True).astype(F)
+            assert np.array_equal(s, want)
+            for kind, fn, arg in (("max", np.max, np.argmax), ("min", np.min, np.argmin)):
+                vals, idx = oracle.reduce_dim(kind, view, dim)
+                assert np.array_equal(vals, fn(ref, axis=dim, keepdims=True))
+                assert np.array_equal(idx, np.expand_dims(arg(ref, axis=dim), dim) + 1)
+
+
+def test_max_min_ties_and_nan_rules():
+    # ties keep the first position; the first NaN wins and stops the scan
+    row = np.array([[1, 5, 5, 2, 5], [3, 3, 3, 3, 3]], dtype=F)
+    vals, idx = oracle.reduce_dim("max", View.contiguous(row), 1)
+    assert idx.ravel().tolist() == [2, 1]
+    vals, idx = oracle.reduce_dim("min", View.contiguous(row), 1)
+    assert idx.ravel().tolist() == [1, 1]
+    nanrow = np.array([[1, np.nan, 7, np.nan, 9]], dtype=F)
+    for kind in ("max", "min"):
+        vals, idx = oracle.reduce_dim(kind, View.contiguous(nanrow), 1)
+        assert np.isnan(vals[0, 0]) and idx[0, 0] == 2
+    assert np.isnan(oracle.maxall(View.contiguous(nanrow))) and np.isnan(oracle.minall(View.contiguous(nanrow)))
+    assert oracle.maxall(View.contiguous(np.array([-np.inf, -3, -np.inf], dtype=F))) == -3
+    lead = np.array([[np.nan, 4, 5]], dtype=F)
+    assert oracle.reduce_dim("max", View.contiguous(lead), 1)[1][0, 0] == 1
+
+
+# ----------------------------------------------------------------- addmm ---
+def test_addmm_reference_vector_and_numpy(golden):
+    g = golden["blas_mm"]
+    A, B = np.array(g["A"], dtype=F), np.array(g["B"], dtype=F)
+    Z = np.zeros((2, 2), dtype=F)
+    r = oracle.addmm_f64(0.0, View.contiguous(Z), 1.0, View.contiguous(A), View.contiguous(B))
+    assert np.array_equal(r, np.array(g["expect"], dtype=np.float64))
+    rng = np.random.RandomState(2)
+    A = rng.normal(size=(37, 53)).astype(F)
+    B = rng.normal(size=(53, 29)).astype(F)
+    C = rng.normal(size=(37, 29)).astype(F)
+    want = 0.5 * C.astype(np.float64) + 1.5 * (A.astype(np.float64) @ B.astype(np.float64))
+    got = oracle.addmm_f64(0.5, View.contiguous(C), 1.5, View.contiguous(A), View.contiguous(B))
+    assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
+    # asymmetric operands: a transposed or swapped product would not match
+    assert not np.allclose(got, 0.5 * C + 1.5 * (B.T.astype(np.float64) @ A.T.astype(np.float64)).T[:, ::-1])
+    # strided operands: A given as the transpose of a dense (K x M) array
+    At = np.ascontiguousarray(A.T)
+    got_t = oracle.addmm_f64(0.5, View.contiguous(C), 1.5, View.contiguous(At).transpose(0, 1), View.contiguous(B))
+    assert np.array_equal(got_t, got)
+    rows, cols = np.array([0, 5, 36]), np.array([28, 3, 0])
+    samp = oracle.addmm_f64_sampled(rows, cols, 0.5, View.contiguous(C), 1.5, View.contiguous(A), View.contiguous(B))
+    assert np.allclose(samp, want[rows, cols], rtol=1e-12)
+
+
+# ---------------------------------------------------------------- layout ---
+def _offsets(sizes, strides):
+    idx = np.indices(sizes).reshape(len(sizes), -1)
+    return (idx * np.array(strides).reshape(-1, 1)).sum(axis=0)
+
+
+def test_collapse_preserves_every_offset():
+    rng = np.random.RandomState(3)
+    for _ in range(300):
+        nd = rng.randint(1, 6)
+        sizes = [int(rng.choice([1, 1, 2, 3, 4, 5])) for _ in range(nd)]
+        # start dense, then perturb: transpose, widen a stride, or keep
+        strides, z = [0] * nd, 1
+        for d in reversed(range(nd)):
+            strides[d] = z
+            z *= sizes[d] * int(rng.choice([1, 1, 1, 2]))
+        if nd > 1 and rng.rand() < 0.4:
+            i, j = rng.choice(nd, 2, replace=False)
+            sizes[i], sizes[j] = sizes[j], sizes[i]
+            strides[i], strides[j] = strides[j], strides[i]
+        csz, cst = oracle.collapse(sizes, strides)
+        assert np.array_equal(_offsets(sizes, strides), _offsets(csz, cst))
+        assert all(s > 1 for s in csz) or csz == [1]
+        assert oracle.is_contiguous(sizes, strides) == (len(csz) == 1 and cst[0] == 1) or csz == [1]
+
+
+def test_collapse_worked_layouts_of_the_strided_config():
+    # 512x512x256 dense; transpose(0,2), stride-2 and narrow views
+    assert oracle.collapse([256, 512, 512], [1, 256, 131072]) == ([256, 512, 512], [1, 256, 131072])
+    assert oracle.collapse([512, 512, 128], [131072, 256, 2]) == ([2 ** 25], [2])
+    assert oracle.collapse([512, 512, 128], [131072, 256, 1]) == ([262144, 128], [256, 1])
+    assert oracle.collapse([512, 512, 256], [131072, 256, 1]) == ([2 ** 26], [1])
+    # reduce dim is treated as size 1
+    assert oracle.collapse([4096, 16384], [16384, 1], reduce_dim=0) == ([16384], [1])
+    assert oracle.collapse([4096, 16384], [16384, 1], reduce_dim=1) == ([4096], [16384])
+    assert oracle.collapse([1, 1], [1, 1]) == ([1], [1])
+
+
+def test_overlap_rule():
+    assert not oracle.overlapping([4, 5], [5, 1])
+    assert not oracle.overlapping([5, 4], [1, 5])          # transposed: no overlap
+    assert not oracle.overlapping([4, 5], [10, 2])         # holes
+    assert oracle.overlapping([4, 5], [0, 1])              # expanded
+    assert oracle.overlapping([4, 5], [3, 1])              # rows overlap
+    assert oracle.overlapping([3, 4], [1, 1])              # unfold-like
+    assert not oracle.overlapping([1, 1], [0, 0])
+    rng = np.random.RandomState(4)
+    for _ in range(200):
+        nd = rng.randint(1, 4)
+        sizes = [int(rng.randint(1, 5)) for _ in range(nd)]
+        strides = [int(rng.randint(0, 7)) for _ in range(nd)]
+        offs = _offsets(sizes, strides)
+        brute = len(set(offs.tolist())) != len(offs)
+        if oracle.overlapping(sizes, strides) != brute:
+            # the rule is conservative: it may report overlap for interleaved but disjoint views
+            assert oracle.overlapping(sizes, strides) and not brute
