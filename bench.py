@@ -1,0 +1,243 @@
+#!/usr/bin/env python
+"""Benchmark of the hot path on one MI355X.
+
+A *step* is one pass of the pointwise/reduce sequence of the first benchmark
+configuration over resident fp32 tensors of 2^28 elements (the size the
+bandwidth target is quoted on):
+
+    x:add(y); x:cmul(y); x:map2_on_gpu(y, z, "x = sqrt(1000*x*x + y*10 + z*z)"); x:sum(); x:max()
+
+Algorithmic bytes per element: 12 + 12 + 16 + 4 + 4 = 48.  ``value`` is those
+bytes divided by the wall time of a step (inputs already in HBM).  Each kernel
+is also timed with HIP events on the library's stream inside the timed region;
+the ``roofline`` object describes the kernel that takes the largest share (the
+three-operand expression kernel).  ``detail`` carries the other configurations
+(strided map/copy, reductions along a dim, the point-tensor chain, addmm), each
+with its own effective GB/s or TFLOP/s.  The CPU baseline is the TH-semantics
+restatement (oracle/) on the host's cores over a bounded sample.
+
+Prints ONE JSON line.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FP32_MFMA_PEAK_TFLOPS = 157.3
+EXPR = "x = sqrt(1000*x*x + y*10 + z*z)"
+
+
+class Timers:
+    """HIP-event pairs on the library's stream; read only after the final sync."""
+
+    def __init__(self, cl):
+        self.cl = cl
+        self.st = cl.state()
+        self.lib = self.st.lib
+        self.rt = self.lib.THClState_getClv2(self.st.ptr, 0)
+        self.items = []
+
+    def timed(self, name, fn):
+        t = self.lib.thcl_rt_timer_new(self.rt)
+        self.lib.thcl_rt_timer_start(t)
+        r = fn()
+        self.lib.thcl_rt_timer_stop(t)
+        self.items.append((name, t))
+        return r
+
+    def collect(self):
+        out = {}
+        for name, t in self.items:
+            out.setdefault(name, []).append(self.lib.thcl_rt_timer_ms(t))
+            self.lib.thcl_rt_timer_free(t)
+        self.items = []
+        return out
+
+
+def stats(ms_list, bytes_or_flops, unit):
+    ms = np.array(ms_list, dtype=np.float64)
+    avg, med, mn = float(ms.mean()), float(np.median(ms)), float(ms.min())
+    scale = 1e-9 if unit == "GB/s" else 1e-12
+    return {"avg_ms": round(avg, 4), "median_ms": round(med, 4), "min_ms": round(mn, 4),
+            "achieved": round(bytes_or_flops / (avg * 1e-3) * scale, 1), "unit": unit}
+
+
+def cpu_baseline(n_sample, seed_base=1):
+    """The same step on the host with the TH-semantics restatement: contiguous
+    cadd/cmul/map2 with all OpenMP threads (TH parallelises those), sum and max
+    on one thread in element order (TH's are serial)."""
+    import oracle
+    L = oracle.lib()
+    x, y, z = (oracle.uniform(seed_base + i, n_sample) for i in range(3))
+    vx = oracle.View.contiguous(x)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    t0 = time.perf_counter()
+    L.th_pointwise_contig_omp(C.c_int(oracle.OPS["cadd"]), C.c_float(1.0), p(vx.storage), p(vx.storage), p(y), C.c_long(n_sample))
+    L.th_pointwise_contig_omp(C.c_int(oracle.OPS["cmul"]), C.c_float(0.0), p(vx.storage), p(vx.storage), p(y), C.c_long(n_sample))
+    L.th_pointwise_contig_omp(C.c_int(oracle.OPS["map2_c1"]), C.c_float(0.0), p(vx.storage), p(y), p(z), C.c_long(n_sample))
+    s = oracle.sumall(vx)
+    m = oracle.maxall(vx)
+    dt = time.perf_counter() - t0
+    return {"value": round(48.0 * n_sample / dt * 1e-9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"one step on 2^{int(np.log2(n_sample))} elements per tensor ({dt:.2f} s): cadd/cmul/map2 as dense "
+                      f"OpenMP loops on {oracle.num_threads()} threads, sum (fp64 accumulator) and max serial, "
+                      f"as Torch7's TH does; Torch7's own map2 calls a Lua closure per element and is far slower",
+            "seconds": round(dt, 3), "check": [float(np.float32(s)) if np.isfinite(s) else str(s), float(m) if np.isfinite(m) else str(m)]}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--log2n", type=int, default=28, help="elements per tensor (2^k) of the headline step")
+    ap.add_argument("--no-detail", action="store_true", help="skip the other configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-log2n", type=int, default=27)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import cltorch_amd as cl
+    import oracle
+    T = Timers(cl)
+    n = 1 << args.log2n
+    X, Y, Z = (cl.ClTensor(oracle.uniform(s, n)) for s in (1, 2, 3))
+
+    pt_sum, pt_max = cl.ClTensor(), cl.ClTensor()   # point tensors: results stay on the device, no stall in a step
+
+    def step(tm=None):
+        run = tm.timed if tm else (lambda name, fn: fn())
+        run("add", lambda: X.add(Y))
+        run("cmul", lambda: X.cmul(Y))
+        run("map2", lambda: X.map2_on_gpu(Y, Z, EXPR))
+        run("sum", lambda: pt_sum.sum(X))
+        run("max", lambda: pt_max.max(X))
+
+    for _ in range(args.warmup):
+        step()
+    cl.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(T)
+    cl.synchronize()
+    wall = time.perf_counter() - t0
+    per_kernel = T.collect()
+    ms_per_step = wall / args.steps * 1e3
+    bytes_per_elem = {"add": 12, "cmul": 12, "map2": 16, "sum": 4, "max": 4}
+    kernels = {k: stats(v, bytes_per_elem[k] * n, "GB/s") for k, v in per_kernel.items()}
+    for k in kernels.values():
+        k["frac_of_peak"] = round(k["achieved"] / HBM_PEAK_GBS, 4)
+    value = 48.0 * n / (ms_per_step * 1e-3) * 1e-9
+    dom = kernels["map2"]
+    out = {
+        "metric": "effective HBM GB/s (% of peak) for apply/reduce; fp32 addmm TFLOP/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"config 1 sequence (add, cmul, map2 '{EXPR}', sum, max) on contiguous fp32 1-D tensors of "
+                               f"2^{args.log2n} elements, uniform[-1,1) MT19937 seeds 1,2,3; 48 algorithmic bytes/element/step",
+                   "elements": n},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "roofline": {"bound": "hbm", "kernel": "thcl_user_contig_v4 (map2 expression, 3 operands)",
+                     "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom["achieved"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": 16 * n, "avg_launch_ms": dom["avg_ms"]},
+        "kernels": kernels,
+    }
+
+    if not args.no_detail:
+        out["detail"] = detail(cl, oracle, T, X, Y, Z, n)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(1 << args.cpu_log2n)
+    print(json.dumps(out))
+
+
+def detail(cl, oracle, T, X, Y, Z, n):
+    """The other benchmark configurations, a few launches each."""
+    d = {}
+    reps = 10
+
+    def measure(name, fn, work, unit="GB/s", reps=reps, peak=HBM_PEAK_GBS):
+        fn()
+        cl.synchronize()
+        for _ in range(reps):
+            T.timed(name, fn)
+        cl.synchronize()
+        s = stats(T.collect()[name], work, unit)
+        s["frac_of_peak"] = round(s["achieved"] / peak, 4)
+        d[name] = s
+
+    # config 4: reduce-all into a point tensor, then pointwise ops fed by it, no host sync in between
+    pt = cl.ClTensor()
+    A = X
+    A.copy(cl.ClTensor(oracle.uniform(7, n, 0.0, 1.0)))
+    measure("c4_sumall_gpu_2^%d" % int(np.log2(n)), lambda: pt.sum(A), 4 * n)
+    measure("c4_div_point_tensor", lambda: A.div(pt) and pt.sum(A), 12 * n)   # div (8 B) + the sum that feeds the next div (4 B)
+    chain = [lambda: A.mul(1.0001), lambda: A.add(0.5), lambda: A.cmul(A), lambda: A.sqrt(), lambda: A.add(pt),
+             lambda: A.mul(pt), lambda: A.abs(), lambda: A.csub(0.25)]
+    cl.synchronize()
+    t0 = time.perf_counter()
+    T.timed("c4_chain_10_launches", lambda: [pt.sum(A), A.div(pt)] + [f() for f in chain])
+    cl.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    ms = T.collect()["c4_chain_10_launches"]
+    d["c4_chain_10_launches"] = {"gpu_ms": round(ms[0], 3), "wall_ms": round(wall, 3),
+                                 "achieved": round((4 + 8 * 9) * n / (ms[0] * 1e-3) * 1e-9, 1), "unit": "GB/s",
+                                 "note": "sumall_gpu + div_gpu + 8 in-place ops, one sync at the end"}
+    measure("c1_fill", lambda: A.fill(0.5), 4 * n)
+
+    # config 2: strided views of a 512x512x256 tensor
+    m = 512 * 512 * 256
+    a = cl.ClTensor(oracle.uniform(4, m)).resize(512, 512, 256)
+    b = cl.ClTensor(oracle.uniform(5, m)).resize(512, 512, 256)
+    aT, bT = a.transpose(1, 3), b.transpose(1, 3)
+    measure("c2_map_transposed_views", lambda: aT.map_on_gpu(bT, "x = 1000*x + y*10"), 12 * m)
+    dst = cl.ClTensor(256, 512, 512)
+    measure("c2_copy_transposed_to_dense", lambda: dst.copy(aT), 8 * m)
+    aS = a.strided((512, 512, 128), (131072, 256, 2))
+    bS = b.strided((512, 512, 128), (131072, 256, 2))
+    measure("c2_map_stride2_views", lambda: aS.map_on_gpu(bS, "x = 1000*x + y*10"), 12 * (m // 2))
+    dS = cl.ClTensor(512, 512, 128)
+    measure("c2_copy_stride2_to_dense", lambda: dS.copy(aS), 8 * (m // 2))
+    aN, bN = a.narrow(3, 65, 128), b.narrow(3, 65, 128)
+    measure("c2_map_narrow_views", lambda: aN.map_on_gpu(bN, "x = 1000*x + y*10"), 12 * (m // 2))
+    del a, b, aT, bT, aS, bS, aN, bN, dst, dS
+
+    # config 3: reductions along each dim of 4096 x 16384
+    r, c = 4096, 16384
+    G = cl.ClTensor(oracle.normal(6, r * c)).resize(r, c)
+    for dim, nout in ((1, c), (2, r)):
+        measure(f"c3_sum_dim{dim}", lambda: G.sum(dim), 4 * r * c + 4 * nout)
+        measure(f"c3_max_dim{dim}", lambda: G.max(dim), 4 * r * c + 8 * nout)
+        measure(f"c3_min_dim{dim}", lambda: G.min(dim), 4 * r * c + 8 * nout)
+    del G
+
+    # config 5: addmm
+    k = 8192
+    sd = 1.0 / np.sqrt(k)
+    Am, Bm, Cm = (cl.ClTensor(oracle.normal(s, k * k, 0.0, sd)).resize(k, k) for s in (8, 9, 10))
+    measure("c5_addmm_8192", lambda: Cm.addmm(0.5, 1.0, Am, Bm), 2.0 * k ** 3, "TFLOP/s", reps=5, peak=FP32_MFMA_PEAK_TFLOPS)
+    del Am, Bm, Cm
+    M, N, K = 64, 16384, 4096
+    At = cl.ClTensor(oracle.normal(11, K * M, 0.0, sd)).resize(K, M)
+    Bs = cl.ClTensor(oracle.normal(12, K * N, 0.0, sd)).resize(K, N)
+    Cs = cl.ClTensor(oracle.normal(13, M * N, 0.0, sd)).resize(M, N)
+    measure("c5_addmm_skinny_64x16384x4096", lambda: Cs.addmm(0.5, 1.0, At.t(), Bs), 2.0 * M * N * K, "TFLOP/s",
+            peak=FP32_MFMA_PEAK_TFLOPS)
+    d["c5_addmm_skinny_64x16384x4096"]["hbm_GBs"] = round(
+        4.0 * (M * K + K * N + 2 * M * N) / (d["c5_addmm_skinny_64x16384x4096"]["avg_ms"] * 1e-3) * 1e-9, 1)
+    return d
+
+
+if __name__ == "__main__":
+    main()

@@ -197,7 +197,7 @@ void launch_fixed(const KernelSet &ks, ApplyPlan &plan) {
 
 void launch_expr(THClState *state, const std::string &expr, int nt, ApplyPlan &plan) {
   std::string key = std::to_string(nt) + "|" + expr;
-  std::string entry = std::string("thcl_user") + kKindSuffix[plan.kind];
+  std::string entry = thcl_expr_tag(expr, nt) + kKindSuffix[plan.kind];
   std::string source;
   if (!thcl_rt_kernel_cached(plan.rt, key.c_str())) source = thcl_expr_source(expr, nt);
   thcl_rt_kernel *k = thcl_rt_kernel_get(plan.rt, key.c_str(), source.c_str(), entry.c_str());

@@ -8,6 +8,7 @@
 // accepted spellings -- x/y/z and *out/*in1/*in2
 // (src/test/unit_tensor.lua:583-635) -- give the same kernel.
 #include <cctype>
+#include <cstdio>
 #include <cstring>
 #include <string>
 
@@ -112,6 +113,17 @@ std::string thcl_rewrite_expr(const char *expr, int ntensors) {
   return out;
 }
 
+// Kernel-name prefix of an expression: the names carry a hash of the text so
+// that profiles tell one expression's kernels from another's.
+std::string thcl_expr_tag(const std::string &rewritten, int ntensors) {
+  unsigned h = 2166136261u;  // FNV-1a
+  for (unsigned char c : rewritten) h = (h ^ c) * 16777619u;
+  h = (h ^ (unsigned)ntensors) * 16777619u;
+  char buf[32];
+  snprintf(buf, sizeof(buf), "thcl_expr%d_%08x", ntensors, h);
+  return buf;
+}
+
 std::string thcl_expr_source(const std::string &rewritten, int ntensors) {
   THCL_CHECK(ntensors >= 1 && ntensors <= 3, "expression kernels take 1 to 3 tensors");
   std::string src;
@@ -127,7 +139,7 @@ std::string thcl_expr_source(const std::string &rewritten, int ntensors) {
   src += "    (void)out; (void)in1; (void)in2; (void)val1; (void)val2; (void)pointTensor1; (void)pointTensor2;\n";
   src += "    " + rewritten + ";\n";
   src += "  }\n};\n";
-  src += "THCL_DEFINE_APPLY_KERNELS(thcl_user, ThclUserOp, " + std::to_string(ntensors) + ")\n";
+  src += "THCL_DEFINE_APPLY_KERNELS(" + thcl_expr_tag(rewritten, ntensors) + ", ThclUserOp, " + std::to_string(ntensors) + ")\n";
   return src;
 }
 

@@ -107,6 +107,7 @@ void thcl_apply_expr(THClState *state, const std::string &expr, ApplyCall &call)
 // float literals suffixed); exposed for host-side tests.
 std::string thcl_rewrite_expr(const char *expr, int ntensors);
 std::string thcl_expr_source(const std::string &rewritten, int ntensors);
+std::string thcl_expr_tag(const std::string &rewritten, int ntensors);
 
 // ------------------------------------------------------------- reductions ---
 enum ThclReduce : int { RED_SUM = 0, RED_PROD = 1, RED_MAX = 2, RED_MIN = 3 };
