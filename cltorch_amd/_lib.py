@@ -13,7 +13,8 @@ from typing import Dict, List, Tuple
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-LIB_PATH = os.path.join(HERE, "libthcl_hip.so")
+# THCL_HIP_LIBRARY may name another build of the same library (never another implementation)
+LIB_PATH = os.environ.get("THCL_HIP_LIBRARY") or os.path.join(HERE, "libthcl_hip.so")
 HEADERS = [os.path.join(ROOT, "include", "thcl_hip.h"), os.path.join(ROOT, "include", "thcl_rt.h")]
 
 

@@ -15,8 +15,8 @@
 
 namespace {
 
-enum PlanKind { K_CONTIG_V4 = 0, K_CONTIG_S, K_JOINT_V4, K_JOINT_S, K_GENERIC, K_NONE };
-const char *const kKindSuffix[] = {"_contig_v4", "_contig_s", "_joint_v4", "_joint_s", "_generic"};
+enum PlanKind { K_CONTIG_V4 = 0, K_CONTIG_S, K_JOINT_V4, K_JOINT_S, K_GENERIC, K_TILED, K_NONE };
+const char *const kKindSuffix[] = {"_contig_v4", "_contig_s", "_joint_v4", "_joint_s", "_generic", "_tiled"};
 
 struct ApplyPlan {
   PlanKind kind = K_NONE;
@@ -25,10 +25,19 @@ struct ApplyPlan {
   ThclContigParams c;
   ThclJointParams j;
   ThclGenericParams g;
+  ThclTileParams t;
 };
 
-constexpr unsigned kMaxGrid = 1u << 22;
-constexpr long kUnitsPerTile = THCL_APPLY_THREADS * THCL_APPLY_UNROLL;
+constexpr unsigned kMaxGrid = 1u << 23;  // x 256 threads stays below 2^32 work-items; larger inputs loop
+long units_per_tile(PlanKind k) {
+  switch (k) {
+    case K_CONTIG_V4:
+    case K_CONTIG_S: return THCL_APPLY_THREADS * THCL_CONTIG_UNROLL;
+    case K_JOINT_V4: return THCL_APPLY_THREADS * THCL_JOINT_V4_UNROLL;
+    case K_JOINT_S: return THCL_APPLY_THREADS * THCL_JOINT_S_UNROLL;
+    default: return THCL_APPLY_THREADS * THCL_GENERIC_UNROLL;
+  }
+}
 
 
 bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
@@ -77,7 +86,8 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan) {
     c.val[1] = call.val[1];
     c.n = (thcl_u64)total;
     const long units = al ? (total >> 2) : total;
-    const long tiles = (units + kUnitsPerTile - 1) / kUnitsPerTile;
+    const long upt = units_per_tile(plan.kind);
+    const long tiles = (units + upt - 1) / upt;
     c.ntiles = (thcl_u64)tiles;
     plan.grid = (unsigned)(tiles < 1 ? 1 : (tiles > kMaxGrid ? kMaxGrid : tiles));
     return true;
@@ -91,6 +101,56 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan) {
     for (int i = 0; i < n && joint_ok; i++)
       for (int d = 0; d < J.dims; d++)
         if (J.strides[i][d] < 0 || J.strides[i][d] >= (1l << 32)) joint_ok = false;
+
+  // transposed inputs meeting a unit-stride destination: tile through LDS
+  if (joint_ok && n >= 2 && J.dims >= 2 && J.dims - 2 <= THCL_TILE_MAX_OUTER) {
+    const int A = J.dims - 1;
+    int B = -1;
+    if (J.strides[0][A] == 1 && J.sizes[A] >= 16) {
+      for (int i = 1; i < n && B < 0; i++) {
+        if (J.strides[i][A] == 1) continue;
+        for (int d = A - 1; d >= 0; d--)
+          if (J.strides[i][d] == 1 && J.sizes[d] >= 16) {
+            B = d;
+            break;
+          }
+      }
+    }
+    if (B >= 0) {
+      ThclTileParams &t = plan.t;
+      memset(&t, 0, sizeof(t));
+      for (int i = 0; i < 3; i++) t.p[i] = p[i];
+      t.pt[0] = call.pt[0];
+      t.pt[1] = call.pt[1];
+      t.val[0] = call.val[0];
+      t.val[1] = call.val[1];
+      t.sizeA = (thcl_u32)J.sizes[A];
+      t.sizeB = (thcl_u32)J.sizes[B];
+      const long tilesA = (J.sizes[A] + THCL_TILE_A - 1) / THCL_TILE_A, tilesB = (J.sizes[B] + THCL_TILE_B - 1) / THCL_TILE_B;
+      t.tilesA = thcl_make_divisor(tilesA);
+      t.tilesB = thcl_make_divisor(tilesB);
+      long blocks = tilesA * tilesB;
+      for (int i = 0; i < n; i++) {
+        t.strideA[i] = (thcl_u32)J.strides[i][A];
+        t.strideB[i] = (thcl_u32)J.strides[i][B];
+        t.via_lds[i] = (i > 0 && J.strides[i][B] == 1 && J.strides[i][A] != 1) ? 1u : 0u;
+      }
+      int no = 0;
+      for (int d = 0; d < J.dims; d++) {
+        if (d == A || d == B) continue;
+        t.osize[no] = thcl_make_divisor(J.sizes[d]);
+        for (int i = 0; i < n; i++) t.ostride[i][no] = (thcl_u32)J.strides[i][d];
+        blocks *= J.sizes[d];
+        no++;
+      }
+      t.nouter = no;
+      if (blocks < (1l << 31)) {
+        plan.kind = K_TILED;
+        plan.grid = (unsigned)blocks;
+        return true;
+      }
+    }
+  }
 
   if (joint_ok) {
     const int last = J.dims - 1;
@@ -116,7 +176,8 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan) {
       j.size[d] = thcl_make_divisor(s);
       for (int i = 0; i < n; i++) j.stride[i][d] = (thcl_u32)J.strides[i][d];
     }
-    const long tiles = (units + kUnitsPerTile - 1) / kUnitsPerTile;
+    const long upt = units_per_tile(plan.kind);
+    const long tiles = (units + upt - 1) / upt;
     j.ntiles = (thcl_u32)tiles;
     plan.grid = (unsigned)(tiles > kMaxGrid ? kMaxGrid : tiles);
     return true;
@@ -140,7 +201,8 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan) {
       g.op[i].stride[d] = (thcl_u32)L.strides[d];
     }
   }
-  const long tiles = (total + kUnitsPerTile - 1) / kUnitsPerTile;
+  const long upt = units_per_tile(plan.kind);
+  const long tiles = (total + upt - 1) / upt;
   g.ntiles = (thcl_u32)tiles;
   plan.grid = (unsigned)(tiles > kMaxGrid ? kMaxGrid : tiles);
   return true;
@@ -172,10 +234,11 @@ struct KernelSet {
   void (*joint_v4)(ThclJointParams);
   void (*joint_s)(ThclJointParams);
   void (*generic)(ThclGenericParams);
+  void (*tiled)(ThclTileParams);
 };
 const KernelSet kFixed[OP_COUNT] = {
 #define X(name, nt, stmt) \
-  {nt, thcl_k_##name##_contig_v4, thcl_k_##name##_contig_s, thcl_k_##name##_joint_v4, thcl_k_##name##_joint_s, thcl_k_##name##_generic},
+  {nt, thcl_k_##name##_contig_v4, thcl_k_##name##_contig_s, thcl_k_##name##_joint_v4, thcl_k_##name##_joint_s, thcl_k_##name##_generic, thcl_k_##name##_tiled},
     THCL_FIXED_OPS(X)
 #undef X
 };
@@ -189,6 +252,7 @@ void launch_fixed(const KernelSet &ks, ApplyPlan &plan) {
     case K_JOINT_V4: hipLaunchKernelGGL(ks.joint_v4, grid, block, 0, stream, plan.j); break;
     case K_JOINT_S: hipLaunchKernelGGL(ks.joint_s, grid, block, 0, stream, plan.j); break;
     case K_GENERIC: hipLaunchKernelGGL(ks.generic, grid, block, 0, stream, plan.g); break;
+    case K_TILED: hipLaunchKernelGGL(ks.tiled, grid, dim3(THCL_TILE_THREADS), 0, stream, plan.t); break;
     default: return;
   }
   hipError_t e = hipGetLastError();
@@ -209,9 +273,11 @@ void launch_expr(THClState *state, const std::string &expr, int nt, ApplyPlan &p
     case K_CONTIG_S: params = &plan.c; bytes = sizeof(plan.c); break;
     case K_JOINT_V4:
     case K_JOINT_S: params = &plan.j; bytes = sizeof(plan.j); break;
+    case K_TILED: params = &plan.t; bytes = sizeof(plan.t); break;
     default: params = &plan.g; bytes = sizeof(plan.g); break;
   }
-  THCL_CHECK(thcl_rt_launch(plan.rt, k, plan.grid, 1, 1, THCL_APPLY_THREADS, 1, 1, 0, params, bytes) == 0, "%s",
+  const unsigned threads = plan.kind == K_TILED ? THCL_TILE_THREADS : THCL_APPLY_THREADS;
+  THCL_CHECK(thcl_rt_launch(plan.rt, k, plan.grid, 1, 1, threads, 1, 1, 0, params, bytes) == 0, "%s",
              thcl_rt_error());
   (void)state;
 }
@@ -281,7 +347,8 @@ void thcl_fill_contig(thcl_rt *rt, float *dst, float value, long n) {
   const bool al = aligned16(dst);
   plan.kind = al ? K_CONTIG_V4 : K_CONTIG_S;
   const long units = al ? (n >> 2) : n;
-  const long tiles = (units + kUnitsPerTile - 1) / kUnitsPerTile;
+  const long upt = units_per_tile(plan.kind);
+  const long tiles = (units + upt - 1) / upt;
   c.ntiles = (thcl_u64)tiles;
   plan.grid = (unsigned)(tiles < 1 ? 1 : (tiles > kMaxGrid ? kMaxGrid : tiles));
   launch_fixed(kFixed[OP_FILL], plan);

@@ -22,7 +22,13 @@
 #define THCL_APPLY_DEVICE_H
 
 #define THCL_APPLY_THREADS 256
-#define THCL_APPLY_UNROLL 4
+// units per lane and tile, per kernel family (measured on MI355X: dense kernels stream
+// fastest with one 128-bit unit per lane and a very large grid; strided scalar
+// kernels gain from several independent loads in flight)
+#define THCL_CONTIG_UNROLL 1
+#define THCL_JOINT_V4_UNROLL 1
+#define THCL_JOINT_S_UNROLL 4
+#define THCL_GENERIC_UNROLL 4
 #define THCL_JOINT_MAX_DIMS 8
 #define THCL_GENERIC_MAX_DIMS 25
 
@@ -107,18 +113,18 @@ __device__ __forceinline__ void thcl_apply_contig_v4(const ThclContigParams &P) 
   const thcl_f4 *a4 = (const thcl_f4 *)P.p[1];
   const thcl_f4 *b4 = (const thcl_f4 *)P.p[2];
   for (thcl_u64 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
-    const thcl_u64 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
-    thcl_f4 o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
-    if (base + (THCL_APPLY_UNROLL - 1) * THCL_APPLY_THREADS < n4) {
+    const thcl_u64 base = tile * (THCL_APPLY_THREADS * THCL_CONTIG_UNROLL) + threadIdx.x;
+    thcl_f4 o[THCL_CONTIG_UNROLL], a[THCL_CONTIG_UNROLL], b[THCL_CONTIG_UNROLL];
+    if (base + (THCL_CONTIG_UNROLL - 1) * THCL_APPLY_THREADS < n4) {
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      for (int k = 0; k < THCL_CONTIG_UNROLL; k++) {
         const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
         o[k] = __builtin_nontemporal_load(o4 + i);
         if (NT > 1) a[k] = __builtin_nontemporal_load(a4 + i);
         if (NT > 2) b[k] = __builtin_nontemporal_load(b4 + i);
       }
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      for (int k = 0; k < THCL_CONTIG_UNROLL; k++) {
 #pragma unroll
         for (int c = 0; c < 4; c++) {
           float oo = o[k][c];
@@ -127,11 +133,11 @@ __device__ __forceinline__ void thcl_apply_contig_v4(const ThclContigParams &P) 
         }
       }
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++)
+      for (int k = 0; k < THCL_CONTIG_UNROLL; k++)
         __builtin_nontemporal_store(o[k], o4 + base + (thcl_u64)k * THCL_APPLY_THREADS);
     } else {
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      for (int k = 0; k < THCL_CONTIG_UNROLL; k++) {
         const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
         if (i < n4) {
           thcl_f4 ov = o4[i], av, bv;
@@ -166,10 +172,10 @@ __device__ __forceinline__ void thcl_apply_contig_s(const ThclContigParams &P) {
   const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
   const float v1 = P.val[0], v2 = P.val[1];
   for (thcl_u64 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
-    const thcl_u64 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
-    float o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
+    const thcl_u64 base = tile * (THCL_APPLY_THREADS * THCL_CONTIG_UNROLL) + threadIdx.x;
+    float o[THCL_CONTIG_UNROLL], a[THCL_CONTIG_UNROLL], b[THCL_CONTIG_UNROLL];
 #pragma unroll
-    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+    for (int k = 0; k < THCL_CONTIG_UNROLL; k++) {
       const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
       if (i < P.n) {
         o[k] = P.p[0][i];
@@ -178,7 +184,7 @@ __device__ __forceinline__ void thcl_apply_contig_s(const ThclContigParams &P) {
       }
     }
 #pragma unroll
-    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+    for (int k = 0; k < THCL_CONTIG_UNROLL; k++) {
       const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
       if (i < P.n) {
         float oo = o[k];
@@ -193,16 +199,16 @@ __device__ __forceinline__ void thcl_apply_contig_s(const ThclContigParams &P) {
 // Operands share sizes; dims were ordered by the written operand's stride and
 // merged on the host.  A unit is VEC consecutive elements of the innermost
 // dim (VEC = 4 needs unit stride there plus 16-byte aligned rows).
-template <class Op, int NT, int VEC>
+template <class Op, int NT, int VEC, int U>
 __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
   const float p1 = P.pt[0] ? *P.pt[0] : 0.f;
   const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
   const float v1 = P.val[0], v2 = P.val[1];
   for (thcl_u32 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
-    const thcl_u32 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
-    thcl_u64 off[THCL_APPLY_UNROLL][3];
+    const thcl_u32 base = tile * (THCL_APPLY_THREADS * U) + threadIdx.x;
+    thcl_u64 off[U][3];
 #pragma unroll
-    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+    for (int k = 0; k < U; k++) {
       thcl_u32 u = base + k * THCL_APPLY_THREADS;
       thcl_u64 o0 = 0, o1 = 0, o2 = 0;
       for (int d = P.dims - 1; d > 0; d--) {
@@ -220,9 +226,9 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
       off[k][2] = o2 + (thcl_u64)r0 * P.stride[2][0];
     }
     if (VEC == 4) {
-      thcl_f4 o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
+      thcl_f4 o[U], a[U], b[U];
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      for (int k = 0; k < U; k++) {
         if (base + k * THCL_APPLY_THREADS < P.nunits) {
           o[k] = *(const thcl_f4 *)(P.p[0] + off[k][0]);
           if (NT > 1) a[k] = *(const thcl_f4 *)(P.p[1] + off[k][1]);
@@ -230,7 +236,7 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
         }
       }
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      for (int k = 0; k < U; k++) {
         if (base + k * THCL_APPLY_THREADS < P.nunits) {
 #pragma unroll
           for (int c = 0; c < 4; c++) {
@@ -242,9 +248,9 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
         }
       }
     } else {
-      float o[THCL_APPLY_UNROLL], a[THCL_APPLY_UNROLL], b[THCL_APPLY_UNROLL];
+      float o[U], a[U], b[U];
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      for (int k = 0; k < U; k++) {
         if (base + k * THCL_APPLY_THREADS < P.nunits) {
           o[k] = P.p[0][off[k][0]];
           if (NT > 1) a[k] = P.p[1][off[k][1]];
@@ -252,7 +258,7 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
         }
       }
 #pragma unroll
-      for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+      for (int k = 0; k < U; k++) {
         if (base + k * THCL_APPLY_THREADS < P.nunits) {
           float oo = o[k];
           thcl_apply_one<Op>(oo, NT > 1 ? a[k] : 0.f, NT > 2 ? b[k] : 0.f, v1, v2, p1, p2);
@@ -282,9 +288,9 @@ __device__ __forceinline__ void thcl_apply_generic(const ThclGenericParams &P) {
   const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
   const float v1 = P.val[0], v2 = P.val[1];
   for (thcl_u32 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
-    const thcl_u32 base = tile * (THCL_APPLY_THREADS * THCL_APPLY_UNROLL) + threadIdx.x;
+    const thcl_u32 base = tile * (THCL_APPLY_THREADS * THCL_GENERIC_UNROLL) + threadIdx.x;
 #pragma unroll
-    for (int k = 0; k < THCL_APPLY_UNROLL; k++) {
+    for (int k = 0; k < THCL_GENERIC_UNROLL; k++) {
       const thcl_u32 i = base + k * THCL_APPLY_THREADS;
       if (i < P.n) {
         const thcl_u64 o0 = thcl_generic_offset(i, P.op[0]);
@@ -299,6 +305,128 @@ __device__ __forceinline__ void thcl_apply_generic(const ThclGenericParams &P) {
   }
 }
 
+// ---------------------------------------------------------------- tiled ---
+// Same-shaped operands whose unit-stride dims differ (a transposed view meeting
+// a dense tensor).  A block owns a TILE_A x TILE_B tile of the plane spanned by dim A
+// (unit stride in the written operand) and dim B (unit stride in the
+// transposed inputs): those inputs are read with lanes along B into LDS, then
+// everything is processed with lanes along A, so every global access is a run
+// of 256 contiguous bytes per wave.
+// tile shape and block size measured best on MI355X among 32..128 squares/rectangles
+#ifndef THCL_TILE_A
+#define THCL_TILE_A 64
+#endif
+#ifndef THCL_TILE_B
+#define THCL_TILE_B 128
+#endif
+#ifndef THCL_TILE_UNROLL
+#define THCL_TILE_UNROLL 8
+#endif
+#ifndef THCL_TILE_THREADS
+#define THCL_TILE_THREADS 512
+#endif
+#define THCL_TILE_MAX_OUTER 6
+struct ThclTileParams {
+  float *p[3];
+  const float *pt[2];
+  float val[2];
+  thcl_u32 sizeA, sizeB;
+  thcl_u32 strideA[3], strideB[3];
+  thcl_u32 via_lds[3];                  // input t is staged through LDS (its strideB is 1)
+  ThclDivisor tilesA, tilesB;
+  int nouter;
+  ThclDivisor osize[THCL_TILE_MAX_OUTER];
+  thcl_u32 ostride[3][THCL_TILE_MAX_OUTER];
+};
+
+template <class Op, int NT>
+__device__ __forceinline__ void thcl_apply_tiled(const ThclTileParams &P) {
+  constexpr int TA = THCL_TILE_A, TB = THCL_TILE_B;
+  __shared__ float tile[NT > 2 ? 2 : 1][TA][TB + 1];
+  const float p1 = P.pt[0] ? *P.pt[0] : 0.f;
+  const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
+  const float v1 = P.val[0], v2 = P.val[1];
+  // block -> (tile along A fastest, tile along B, outer indices)
+  thcl_u32 bid = blockIdx.x;
+  thcl_u32 q = thcl_div(bid, P.tilesA);
+  const thcl_u32 a0 = (bid - q * P.tilesA.d) * TA;
+  bid = q;
+  q = thcl_div(bid, P.tilesB);
+  const thcl_u32 b0 = (bid - q * P.tilesB.d) * TB;
+  bid = q;
+  thcl_u64 base[3] = {0, 0, 0};
+  for (int d = P.nouter - 1; d >= 0; d--) {
+    q = thcl_div(bid, P.osize[d]);
+    const thcl_u32 r = bid - q * P.osize[d].d;
+    base[0] += (thcl_u64)r * P.ostride[0][d];
+    if (NT > 1) base[1] += (thcl_u64)r * P.ostride[1][d];
+    if (NT > 2) base[2] += (thcl_u64)r * P.ostride[2][d];
+    bid = q;
+  }
+  // Addresses advance by a constant step per pass, so each access costs one
+  // 64-bit add; full tiles skip the bounds tests.
+  const bool full = (a0 + TA <= P.sizeA) && (b0 + TB <= P.sizeB);
+  // phase 1: lanes along B
+  {
+    constexpr int ROWS = THCL_TILE_THREADS / TB;  // rows of the tile covered per pass
+    const thcl_u32 lane = threadIdx.x % TB, row = threadIdx.x / TB;
+#pragma unroll
+    for (int t = 1; t < NT; t++) {
+      if (P.via_lds[t]) {
+        const float *src = P.p[t] + base[t] + (thcl_u64)(a0 + row) * P.strideA[t] + (thcl_u64)(b0 + lane) * P.strideB[t];
+        const thcl_u64 step = (thcl_u64)ROWS * P.strideA[t];
+        if (full) {
+#pragma unroll
+          for (int i = 0; i < TA / ROWS; i++) {
+            tile[t - 1][row + ROWS * i][lane] = *src;
+            src += step;
+          }
+        } else {
+          const bool bok = b0 + lane < P.sizeB;
+#pragma unroll 4
+          for (int i = 0; i < TA / ROWS; i++) {
+            if (bok && a0 + row + ROWS * i < P.sizeA) tile[t - 1][row + ROWS * i][lane] = *src;
+            src += step;
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // phase 2: lanes along A
+  {
+    constexpr int ROWS = THCL_TILE_THREADS / TA;
+    const thcl_u32 lane = threadIdx.x % TA, row = threadIdx.x / TA;
+    float *op = P.p[0] + base[0] + (thcl_u64)(a0 + lane) * P.strideA[0] + (thcl_u64)(b0 + row) * P.strideB[0];
+    const thcl_u64 ostep = (thcl_u64)ROWS * P.strideB[0];
+    const float *q1 = nullptr, *q2 = nullptr;
+    thcl_u64 step1 = 0, step2 = 0;
+    if (NT > 1 && !P.via_lds[1]) {
+      q1 = P.p[1] + base[1] + (thcl_u64)(a0 + lane) * P.strideA[1] + (thcl_u64)(b0 + row) * P.strideB[1];
+      step1 = (thcl_u64)ROWS * P.strideB[1];
+    }
+    if (NT > 2 && !P.via_lds[2]) {
+      q2 = P.p[2] + base[2] + (thcl_u64)(a0 + lane) * P.strideA[2] + (thcl_u64)(b0 + row) * P.strideB[2];
+      step2 = (thcl_u64)ROWS * P.strideB[2];
+    }
+    const bool aok = a0 + lane < P.sizeA;
+#pragma unroll THCL_TILE_UNROLL
+    for (int i = 0; i < TB / ROWS; i++) {
+      const thcl_u32 bl = row + ROWS * i;
+      if (full || (aok && b0 + bl < P.sizeB)) {
+        float oo = *op, x = 0.f, y = 0.f;
+        if (NT > 1) x = P.via_lds[1] ? tile[0][lane][bl] : *q1;
+        if (NT > 2) y = P.via_lds[2] ? tile[NT > 2 ? 1 : 0][lane][bl] : *q2;
+        thcl_apply_one<Op>(oo, x, y, v1, v2, p1, p2);
+        *op = oo;
+      }
+      op += ostep;
+      if (NT > 1) q1 += step1;
+      if (NT > 2) q2 += step2;
+    }
+  }
+}
+
 // Entry points for one operator; K is a name prefix.
 #define THCL_DEFINE_APPLY_KERNELS(K, Op, NT)                                                             \
   extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_contig_v4(ThclContigParams P) {  \
@@ -308,13 +436,16 @@ __device__ __forceinline__ void thcl_apply_generic(const ThclGenericParams &P) {
     thcl_apply_contig_s<Op, NT>(P);                                                                      \
   }                                                                                                      \
   extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_v4(ThclJointParams P) {    \
-    thcl_apply_joint<Op, NT, 4>(P);                                                                      \
+    thcl_apply_joint<Op, NT, 4, THCL_JOINT_V4_UNROLL>(P);                                                                      \
   }                                                                                                      \
   extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_s(ThclJointParams P) {     \
-    thcl_apply_joint<Op, NT, 1>(P);                                                                      \
+    thcl_apply_joint<Op, NT, 1, THCL_JOINT_S_UNROLL>(P);                                                                      \
   }                                                                                                      \
   extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_generic(ThclGenericParams P) {   \
     thcl_apply_generic<Op, NT>(P);                                                                       \
+  }                                                                                                      \
+  extern "C" __global__ __launch_bounds__(THCL_TILE_THREADS) void K##_tiled(ThclTileParams P) {         \
+    thcl_apply_tiled<Op, NT>(P);                                                                         \
   }
 
 #endif  // THCL_APPLY_DEVICE_H

@@ -149,8 +149,22 @@ struct ReduceAllParams {
   ThclGenericOperand L;  // strided input only
 };
 
+// Publishing a block's partial: a device-scope atomic exchange lands at the
+// level every XCD sees, and its return value tells this thread it has landed.
+// That avoids a release fence, which on this chip writes back the whole L2 of
+// the XCD and cost ~45 ns per block when measured.
+__device__ __forceinline__ unsigned publish(double *slot, double v) {
+  return (unsigned)atomicExch((unsigned long long *)slot, (unsigned long long)__double_as_longlong(v));
+}
+__device__ __forceinline__ unsigned publish(float *slot, float v) {
+  return atomicExch((unsigned *)slot, __float_as_uint(v));
+}
+
 // Last block to arrive (integer ticket) folds the per-block partials in block
 // order and writes the scalar; the ticket is left at zero for the next launch.
+// Order of events per block: partial exchanged -> its return observed -> ticket
+// taken.  The last block therefore takes its ticket after every partial has
+// landed, and reads them with device-scope atomic loads.
 template <int KIND>
 __device__ __forceinline__ void finish_all(typename Acc<KIND>::T blockval, const ReduceAllParams &P,
                                            typename Acc<KIND>::T *lds) {
@@ -158,14 +172,14 @@ __device__ __forceinline__ void finish_all(typename Acc<KIND>::T blockval, const
   T *partials = (T *)P.partials;
   __shared__ unsigned s_last;
   if (threadIdx.x == 0) {
-    partials[blockIdx.x] = blockval;
-    __threadfence();
-    const unsigned t = atomicAdd(P.ticket, 1u);
+    const unsigned landed = publish(&partials[blockIdx.x], blockval);
+    unsigned inc = 1u;
+    asm volatile("" : "+v"(inc) : "v"(landed));  // the increment depends on the exchange's return
+    const unsigned t = atomicAdd(P.ticket, inc);
     s_last = (t == gridDim.x - 1) ? 1u : 0u;
   }
   __syncthreads();
   if (!s_last) return;
-  __threadfence();
   T v = Acc<KIND>::init();
   for (unsigned i = threadIdx.x; i < gridDim.x; i += kThreads)
     v = Acc<KIND>::comb(v, load_fresh(&partials[i]));
@@ -497,7 +511,7 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
     fill_operand(P.L, thcl_collapse(src));
     want = (n + kThreads - 1) / kThreads;
   }
-  long cap = (long)cus * 8;
+  long cap = (long)cus * 2;  // two resident blocks per CU keep HBM busy; fewer blocks, fewer tickets
   const long max_partials = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
   if (cap > max_partials) cap = max_partials;
   unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));

@@ -306,3 +306,63 @@ def test_host_roundtrip_of_strided_views(cl):
     t = p.transpose(0, 1)
     t.dev.copy(np.arange(8 * 6 * 10, dtype=F).reshape(8, 6, 10))     # host -> strided device view
     assert_bit_equal(p.dev.float(), np.arange(480, dtype=F).reshape(8, 6, 10).transpose(1, 0, 2))
+
+
+# ------------------------------------------------- transposed operands (LDS tiles) ---
+@pytest.mark.parametrize("shape", [(130, 70), (64, 128), (200, 300), (3, 150, 90), (5, 17, 260), (2, 3, 70, 129)])
+def test_transposed_operand_meets_dense_one(cl, shape):
+    """Operands whose unit-stride dims differ: the library stages the transposed
+    ones through LDS tiles; full tiles, ragged edges and outer dims."""
+    n = int(np.prod(shape))
+    nd = len(shape)
+    x, y, z = oracle.uniform(31, n), oracle.uniform(32, n), oracle.uniform(33, n)
+    tshape = shape[:-2] + (shape[-1], shape[-2])
+    # dense destination, source = last two dims transposed
+    dst = Pair.dense(cl, np.zeros(shape, dtype=F))
+    srcT = Pair.dense(cl, y.reshape(tshape)).transpose(nd - 2, nd - 1)
+    dst.dev.copy(srcT.dev)
+    assert_bit_equal(dst.device_storage(), srcT.view.gather(), f"copy T->dense {shape}")
+    # transposed destination, dense source (scatter through the same kernel)
+    dstT = Pair.dense(cl, np.zeros(tshape, dtype=F)).transpose(nd - 2, nd - 1)
+    src = Pair.dense(cl, x.reshape(shape))
+    dstT.dev.copy(src.dev)
+    oracle.pointwise("copy", dstT.view, src.view)
+    assert_bit_equal(dstT.device_storage(), dstT.host_storage, f"copy dense->T {shape}")
+    # read-write destination
+    acc = Pair.dense(cl, x.reshape(shape))
+    acc.dev.add(0.5, srcT.dev)
+    oracle.pointwise("cadd", acc.view, acc.view, srcT.view, 0.5)
+    assert_bit_equal(acc.device_storage(), acc.host_storage, f"cadd {shape}")
+    # three operands: one transposed input, one dense; then both transposed
+    z_d = Pair.dense(cl, z.reshape(shape))
+    acc.dev.map2_on_gpu(srcT.dev, z_d.dev, "x = x*y + z")
+    want = expr_host.evaluate("x = x*y + z", acc.view.gather(), srcT.view.gather(), z_d.view.gather())
+    assert_bit_equal(acc.device_storage(), want, f"map2 T,dense {shape}")
+    zT = Pair.dense(cl, z.reshape(tshape)).transpose(nd - 2, nd - 1)
+    acc2 = Pair.dense(cl, x.reshape(shape))
+    acc2.dev.addcmul(2.0, srcT.dev, zT.dev)
+    oracle.pointwise("addcmul", acc2.view, srcT.view, zT.view, 2.0)
+    assert_bit_equal(acc2.device_storage(), acc2.host_storage, f"addcmul T,T {shape}")
+    assert_bit_equal(srcT.device_storage(), y, "input modified")
+
+
+def test_same_expression_on_every_kernel_family(cl):
+    """One expression string, five layouts: the run-time kernel cache must hand
+    back the kernel that matches each layout."""
+    expr = "x = x*0.5 + y"
+    base = oracle.uniform(41, 96 * 80)
+    other = oracle.uniform(42, 96 * 80 * 2)
+
+    def run(px, py):
+        px.dev.map_on_gpu(py.dev, expr)
+        want = expr_host.evaluate(expr, px.view.gather(), py.view.gather())
+        oracle.pointwise("copy", px.view, View.contiguous(want))
+        assert_bit_equal(px.device_storage(), px.host_storage)
+
+    for _ in range(2):
+        run(Pair.dense(cl, base.reshape(96, 80)), Pair.dense(cl, other[:7680].reshape(96, 80)))            # dense 128-bit
+        run(Pair(cl, base, 1, (7000,), (1,)), Pair(cl, other, 2, (7000,), (1,)))                            # dense, misaligned
+        run(Pair.dense(cl, base.reshape(96, 80)).narrow(1, 8, 32), Pair.dense(cl, other[:7680].reshape(96, 80)).narrow(1, 4, 32))  # joint 128-bit
+        run(Pair.dense(cl, base.reshape(96, 80)).step(1, 2), Pair.dense(cl, other[:7680].reshape(96, 80)).step(1, 2))              # joint scalar
+        run(Pair.dense(cl, base.reshape(96, 80)), Pair.dense(cl, other[:7680].reshape(80, 96)).transpose(0, 1))                    # tiled
+        run(Pair.dense(cl, base.reshape(96, 80)), Pair(cl, other, 0, (80, 96), (1, 160)))                   # different shapes: generic
