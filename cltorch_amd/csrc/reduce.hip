@@ -56,7 +56,7 @@ struct Acc<RED_MAX> {
   static __device__ __forceinline__ T init() { return -INFINITY; }
   static __device__ __forceinline__ T lift(float x) { return x; }
   // NaN on either side gives NaN
-  static __device__ __forceinline__ T comb(T a, T b) { return (b > a || b != b) ? b : a; }
+  static __device__ __forceinline__ T comb(T a, T b) { return ((b > a) | (b != b)) ? b : a; }
   static __device__ __forceinline__ float lower(T a) { return a; }
 };
 template <>
@@ -64,7 +64,7 @@ struct Acc<RED_MIN> {
   typedef float T;
   static __device__ __forceinline__ T init() { return INFINITY; }
   static __device__ __forceinline__ T lift(float x) { return x; }
-  static __device__ __forceinline__ T comb(T a, T b) { return (b < a || b != b) ? b : a; }
+  static __device__ __forceinline__ T comb(T a, T b) { return ((b < a) | (b != b)) ? b : a; }
   static __device__ __forceinline__ float lower(T a) { return a; }
 };
 
@@ -85,13 +85,16 @@ __device__ __forceinline__ VI vi_init() {
 }
 template <int KIND>
 __device__ __forceinline__ VI vi_comb(VI cur, VI x) {
+  // straight-line form (no short-circuit): the compiler turns && / || chains
+  // into exec-mask branches, which cost more than the arithmetic
   const bool xn = x.v != x.v, cn = cur.v != cur.v;
-  bool take;
-  if (cn) take = xn && x.i < cur.i;
-  else if (xn) take = true;
-  else if (KIND == RED_MAX) take = (x.v > cur.v) || (x.v == cur.v && x.i < cur.i);
-  else take = (x.v < cur.v) || (x.v == cur.v && x.i < cur.i);
-  return take ? x : cur;
+  const bool better = (KIND == RED_MAX) ? (x.v > cur.v) : (x.v < cur.v);
+  const bool same = (x.v == cur.v) | (xn & cn);
+  const bool take = (!cn & (xn | better)) | (same & (x.i < cur.i));
+  VI r;
+  r.v = take ? x.v : cur.v;
+  r.i = take ? x.i : cur.i;
+  return r;
 }
 
 __device__ __forceinline__ double shfl_xor_t(double v, int m) { return __shfl_xor(v, m, kWave); }
@@ -307,13 +310,33 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
       if (VEC == 4) {
         const thcl_f4 *row4 = (const thcl_f4 *)row;
         const thcl_u32 r4 = P.R >> 2;
-        for (thcl_u32 i = sub; i < r4; i += LPR) {
+        constexpr int FLY = 4;  // independent loads issued before any is consumed
+        thcl_u32 i = sub;
+        for (; i + (FLY - 1) * LPR < r4; i += FLY * LPR) {
+          thcl_f4 v[FLY];
+#pragma unroll
+          for (int f = 0; f < FLY; f++) v[f] = __builtin_nontemporal_load(row4 + i + f * LPR);
+#pragma unroll
+          for (int f = 0; f < FLY; f++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc = S::take(acc, v[f][c], (int)((i + f * LPR) * 4 + c));
+        }
+        for (; i < r4; i += LPR) {
           const thcl_f4 v = __builtin_nontemporal_load(row4 + i);
 #pragma unroll
           for (int c = 0; c < 4; c++) acc = S::take(acc, v[c], (int)(i * 4 + c));
         }
       } else {
-        for (thcl_u32 i = sub; i < P.R; i += LPR) acc = S::take(acc, row[i], (int)i);
+        constexpr int FLY = 4;
+        thcl_u32 i = sub;
+        for (; i + (FLY - 1) * LPR < P.R; i += FLY * LPR) {
+          float v[FLY];
+#pragma unroll
+          for (int f = 0; f < FLY; f++) v[f] = row[i + f * LPR];
+#pragma unroll
+          for (int f = 0; f < FLY; f++) acc = S::take(acc, v[f], (int)(i + f * LPR));
+        }
+        for (; i < P.R; i += LPR) acc = S::take(acc, row[i], (int)i);
       }
     }
     if (LPR <= kWave) {
@@ -367,32 +390,44 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
         }
         off += (thcl_u64)((P.L.dims == 1) ? i * VEC : i) * P.L.stride[0];
       }
-      const float *col = P.in + off;
+      // this wave takes rows r_begin + wave, + WAVES, ...; FLY of them are loaded
+      // before any is consumed, the address advances by a constant step
+      constexpr int FLY = 4;
       thcl_u32 r = r_begin + wave;
-      // two rows in flight per lane
-      for (; r + WAVES < r_end; r += 2 * WAVES) {
+      const float *ptr = P.in + off + (thcl_u64)r * P.rstride;
+      const thcl_u64 step = (thcl_u64)WAVES * P.rstride;
+      for (; r + (FLY - 1) * WAVES < r_end; r += FLY * WAVES) {
         if (VEC == 4) {
-          const thcl_f4 v0 = __builtin_nontemporal_load((const thcl_f4 *)(col + (thcl_u64)r * P.rstride));
-          const thcl_f4 v1 = __builtin_nontemporal_load((const thcl_f4 *)(col + (thcl_u64)(r + WAVES) * P.rstride));
+          thcl_f4 v[FLY];
 #pragma unroll
-          for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v0[c], (int)r);
+          for (int f = 0; f < FLY; f++) {
+            v[f] = __builtin_nontemporal_load((const thcl_f4 *)ptr);
+            ptr += step;
+          }
 #pragma unroll
-          for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v1[c], (int)(r + WAVES));
+          for (int f = 0; f < FLY; f++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v[f][c], (int)(r + f * WAVES));
         } else {
-          const float v0 = col[(thcl_u64)r * P.rstride];
-          const float v1 = col[(thcl_u64)(r + WAVES) * P.rstride];
-          acc[0] = S::take(acc[0], v0, (int)r);
-          acc[0] = S::take(acc[0], v1, (int)(r + WAVES));
+          float v[FLY];
+#pragma unroll
+          for (int f = 0; f < FLY; f++) {
+            v[f] = *ptr;
+            ptr += step;
+          }
+#pragma unroll
+          for (int f = 0; f < FLY; f++) acc[0] = S::take(acc[0], v[f], (int)(r + f * WAVES));
         }
       }
       for (; r < r_end; r += WAVES) {
         if (VEC == 4) {
-          const thcl_f4 v0 = *(const thcl_f4 *)(col + (thcl_u64)r * P.rstride);
+          const thcl_f4 v0 = *(const thcl_f4 *)ptr;
 #pragma unroll
           for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v0[c], (int)r);
         } else {
-          acc[0] = S::take(acc[0], col[(thcl_u64)r * P.rstride], (int)r);
+          acc[0] = S::take(acc[0], *ptr, (int)r);
         }
+        ptr += step;
       }
     }
     __syncthreads();
@@ -412,15 +447,29 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
   }
 }
 
+// Folds the [split][nslices] partials.  A block owns 16 adjacent slices; its 16
+// thread groups walk the split index 16 apart (each read is a 128-byte run),
+// then the groups meet in LDS and are folded in split order.
+constexpr int kFinSlices = 16, kFinParts = kThreads / kFinSlices;
 template <int KIND, bool ARG>
 __global__ __launch_bounds__(kThreads) void reduce_cols_finish(ReduceDimParams P) {
   typedef Slot<KIND, ARG> S;
   typedef typename S::T T;
+  __shared__ T lds[kFinParts][kFinSlices];
   const T *partials = (const T *)P.partials;
-  for (thcl_u32 s = blockIdx.x * kThreads + threadIdx.x; s < P.nslices; s += gridDim.x * kThreads) {
-    T r = partials[s];
-    for (thcl_u32 k = 1; k < P.split; k++) r = S::comb(r, partials[(thcl_u64)k * P.nslices + s]);
-    S::store(P, s, r);
+  const int sl = threadIdx.x % kFinSlices, part = threadIdx.x / kFinSlices;
+  const thcl_u32 s = blockIdx.x * kFinSlices + sl;
+  T r = S::init();
+  if (s < P.nslices)
+    for (thcl_u32 k = part; k < P.split; k += kFinParts) r = S::comb(r, partials[(thcl_u64)k * P.nslices + s]);
+  lds[part][sl] = r;
+  __syncthreads();
+  if (part == 0 && s < P.nslices) {
+    // group g holds splits g, g+16, ...: folding groups in order keeps sums
+    // reproducible and, for positions, the combine rule is order-independent
+    T t = lds[0][sl];
+    for (int g = 1; g < kFinParts; g++) t = S::comb(t, lds[g][sl]);
+    S::store(P, s, t);
   }
 }
 
@@ -616,6 +665,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
       split = (target + tiles - 1) / tiles;
       const long max_by_rows = (R + 31) / 32;  // at least 32 rows per block
       if (split > max_by_rows) split = max_by_rows;
+      if (split > 256) split = 256;
       if (split * nslices > partial_cap) split = partial_cap / nslices;
       if (split < 1) split = 1;
     }
@@ -632,7 +682,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   else launch_dim<K, false>(rows, lpr, vec, grid, stream, P);             \
   check_launch("reduce-dim");                                             \
   if (!rows && P.split > 1) {                                             \
-    unsigned fg = (unsigned)((nslices + kThreads - 1) / kThreads);        \
+    unsigned fg = (unsigned)((nslices + kFinSlices - 1) / kFinSlices);    \
     if (arg) launch_finish<K, true>(fg, stream, P);                       \
     else launch_finish<K, false>(fg, stream, P);                          \
     check_launch("reduce-dim finish");                                    \

@@ -39,7 +39,7 @@ struct thcl_rt_timer {
 
 namespace {
 constexpr int kMaxDevices = 64;
-constexpr size_t kScratchBytes = 1u << 20;
+constexpr size_t kScratchBytes = 8u << 20;
 thcl_rt *g_ctx[kMaxDevices] = {nullptr};
 std::mutex g_mu;
 thread_local std::string g_err;
