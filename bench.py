@@ -70,27 +70,36 @@ def stats(ms_list, bytes_or_flops, unit):
             "achieved": round(bytes_or_flops / (avg * 1e-3) * scale, 1), "unit": unit}
 
 
-def cpu_baseline(n_sample, seed_base=1):
+def cpu_baseline(n_sample, seed_base=1, min_seconds=12.0):
     """The same step on the host with the TH-semantics restatement: contiguous
     cadd/cmul/map2 with all OpenMP threads (TH parallelises those), sum and max
-    on one thread in element order (TH's are serial)."""
+    on one thread in element order (TH's are serial).  Steps are repeated on the
+    same arrays until about `min_seconds` of CPU work has been timed."""
     import oracle
     L = oracle.lib()
     x, y, z = (oracle.uniform(seed_base + i, n_sample) for i in range(3))
     vx = oracle.View.contiguous(x)
     p = lambda a: a.ctypes.data_as(C.c_void_p)
+    steps, first = 0, None
     t0 = time.perf_counter()
-    L.th_pointwise_contig_omp(C.c_int(oracle.OPS["cadd"]), C.c_float(1.0), p(vx.storage), p(vx.storage), p(y), C.c_long(n_sample))
-    L.th_pointwise_contig_omp(C.c_int(oracle.OPS["cmul"]), C.c_float(0.0), p(vx.storage), p(vx.storage), p(y), C.c_long(n_sample))
-    L.th_pointwise_contig_omp(C.c_int(oracle.OPS["map2_c1"]), C.c_float(0.0), p(vx.storage), p(y), p(z), C.c_long(n_sample))
-    s = oracle.sumall(vx)
-    m = oracle.maxall(vx)
-    dt = time.perf_counter() - t0
-    return {"value": round(48.0 * n_sample / dt * 1e-9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"one step on 2^{int(np.log2(n_sample))} elements per tensor ({dt:.2f} s): cadd/cmul/map2 as dense "
-                      f"OpenMP loops on {oracle.num_threads()} threads, sum (fp64 accumulator) and max serial, "
-                      f"as Torch7's TH does; Torch7's own map2 calls a Lua closure per element and is far slower",
-            "seconds": round(dt, 3), "check": [float(np.float32(s)) if np.isfinite(s) else str(s), float(m) if np.isfinite(m) else str(m)]}
+    while True:
+        L.th_pointwise_contig_omp(C.c_int(oracle.OPS["cadd"]), C.c_float(1.0), p(vx.storage), p(vx.storage), p(y), C.c_long(n_sample))
+        L.th_pointwise_contig_omp(C.c_int(oracle.OPS["cmul"]), C.c_float(0.0), p(vx.storage), p(vx.storage), p(y), C.c_long(n_sample))
+        L.th_pointwise_contig_omp(C.c_int(oracle.OPS["map2_c1"]), C.c_float(0.0), p(vx.storage), p(y), p(z), C.c_long(n_sample))
+        s = oracle.sumall(vx)
+        m = oracle.maxall(vx)
+        steps += 1
+        if first is None:
+            first = (s, m)
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds or steps >= 200:
+            break
+    fmt = lambda v: float(np.float32(v)) if np.isfinite(v) else str(v)
+    return {"value": round(48.0 * n_sample * steps / dt * 1e-9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{steps} steps on 2^{int(np.log2(n_sample))} elements per tensor ({dt:.1f} s of CPU work): cadd/cmul/map2 as dense "
+                      f"OpenMP loops on {oracle.num_threads()} threads, sum (fp64 accumulator) and max serial in element order "
+                      f"(max stops at the first NaN, as TH does); Torch7's own map2 calls a Lua closure per element and is far slower",
+            "seconds": round(dt, 3), "steps": steps, "first_step_sum_max": [fmt(first[0]), fmt(first[1])]}
 
 
 def main():
@@ -102,6 +111,9 @@ def main():
     ap.add_argument("--no-detail", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-log2n", type=int, default=27)
+    ap.add_argument("--pmc-workload", action="store_true",
+                    help="run each headline kernel twice plus a same-size copy (counter calibration) and exit; "
+                         "meant to run under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --kernel-trace`")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -109,6 +121,8 @@ def main():
 
     import cltorch_amd as cl
     import oracle
+    if args.pmc_workload:
+        return pmc_workload(cl, 1 << args.log2n)
     T = Timers(cl)
     n = 1 << args.log2n
     X, Y, Z = (cl.ClTensor(oracle.uniform(s, n)) for s in (1, 2, 3))
@@ -148,9 +162,12 @@ def main():
                                f"2^{args.log2n} elements, uniform[-1,1) MT19937 seeds 1,2,3; 48 algorithmic bytes/element/step",
                    "elements": n},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "roofline": {"bound": "hbm", "kernel": "thcl_user_contig_v4 (map2 expression, 3 operands)",
+        "roofline": {"bound": "hbm", "kernel": "thcl_expr3_d6642be2_contig_v4 (the map2 expression, 3 operands)",
                      "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom["achieved"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(dom["achieved"] / HBM_PEAK_GBS, 4),
+                     # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, calibrated on a copy kernel
+                     # (profiles/headline_kernels_2p28_pmc_traffic.txt): 15.996 bytes/element at 2^28 elements
+                     "traffic": int(round(15.996 * n)) if args.log2n == 28 else None,
                      "algorithmic_bytes_per_launch": 16 * n, "avg_launch_ms": dom["avg_ms"]},
         "kernels": kernels,
     }
@@ -160,6 +177,29 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(1 << args.cpu_log2n)
     print(json.dumps(out))
+
+
+def pmc_workload(cl, n):
+    """Launches for hardware-counter runs: a copy between the two halves of one
+    storage (runs the library's dense copy kernel: reads 4n bytes, writes 4n
+    bytes -- the calibration point for FETCH_SIZE / WRITE_SIZE) and the five
+    kernels of the headline step, twice."""
+    rng = np.random.RandomState(0)
+    x = rng.uniform(-1, 1, n).astype(np.float32)
+    X, Y, Z = cl.ClTensor(x), cl.ClTensor(x[::-1].copy()), cl.ClTensor(np.abs(x))
+    W = cl.ClTensor(2 * n)
+    lo, hi = W.narrow(1, 1, n), W.narrow(1, n + 1, n)
+    lo.copy(X)
+    pt = cl.ClTensor()
+    for _ in range(2):
+        hi.copy(lo)
+        X.add(Y)
+        X.cmul(Y)
+        X.map2_on_gpu(Y, Z, EXPR)
+        pt.sum(X)
+        pt.max(X)
+    cl.synchronize()
+    print(json.dumps({"pmc_workload": "done", "elements": n}))
 
 
 def detail(cl, oracle, T, X, Y, Z, n):

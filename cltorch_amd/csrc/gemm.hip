@@ -36,6 +36,9 @@ struct GemmParams {
   float alpha, beta;
   int tiles_m, tiles_n;
   int group_m;  // tiles along m per scheduling group
+  int ksplit;   // blockIdx.y slices of K; > 1: raw partial products go to `work`
+  int kchunk;   // K per slice (multiple of BK)
+  float *work;  // [ksplit][n][m] dense partials
 };
 
 // One operand tile in LDS.  KC: contiguous along k in global memory.
@@ -154,10 +157,12 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
 
   TileLoader<BM, AKC, EDGE> la;
   TileLoader<BN, BKC, EDGE> lb;
-  const int KT = (P.k + BK - 1) / BK;
+  const int k_begin = blockIdx.y * P.kchunk;
+  const int k_end = (k_begin + P.kchunk < P.k) ? (k_begin + P.kchunk) : P.k;
+  const int KT = (k_end - k_begin + BK - 1) / BK;
 
-  la.load(P.a, P.lda, m0, 0, P.m, P.k);
-  lb.load(P.b, P.ldb, n0, 0, P.n, P.k);
+  la.load(P.a, P.lda, m0, k_begin, P.m, k_end);
+  lb.load(P.b, P.ldb, n0, k_begin, P.n, k_end);
   la.store(lds);
   lb.store(lds + AF);
   __syncthreads();
@@ -167,8 +172,8 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
     float *As = lds + cur * (AF + BF);
     float *Bs = As + AF;
     if (kt + 1 < KT) {
-      la.load(P.a, P.lda, m0, (kt + 1) * BK, P.m, P.k);
-      lb.load(P.b, P.ldb, n0, (kt + 1) * BK, P.n, P.k);
+      la.load(P.a, P.lda, m0, k_begin + (kt + 1) * BK, P.m, k_end);
+      lb.load(P.b, P.ldb, n0, k_begin + (kt + 1) * BK, P.n, k_end);
     }
 #pragma unroll
     for (int kg = 0; kg < BK / 8; kg++) {
@@ -193,6 +198,32 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
 
   // epilogue: lane holds rows 8*(r/4) + 4*(lane/32) + (r%4) of column lane%32
   const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+  if (P.ksplit > 1) {
+    // raw partial product of this K slice, dense [n][m]; scaled and summed by splitk_reduce
+    float *w = P.work + (size_t)blockIdx.y * P.m * P.n;
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+      for (int j = 0; j < NT; j++) {
+        const int col = n0 + wn0 + j * 32 + l32;
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+          const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
+          float *wp = w + (size_t)col * P.m + row;
+          if (!EDGE) {
+            f4 v;
+#pragma unroll
+            for (int c = 0; c < 4; c++) v[c] = acc[i][j][rq * 4 + c];
+            *(f4 *)wp = v;
+          } else if (col < P.n) {
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+              if (row + c < P.m) wp[c] = acc[i][j][rq * 4 + c];
+          }
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < MT; i++) {
 #pragma unroll
@@ -226,6 +257,20 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
         }
       }
     }
+  }
+}
+
+// C = alpha * (sum over K slices, in slice order) + beta * C
+__global__ __launch_bounds__(256) void splitk_reduce(GemmParams P) {
+  const size_t total = (size_t)P.m * P.n;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
+    float s = P.work[e];
+    for (int k = 1; k < P.ksplit; k++) s += P.work[(size_t)k * total + e];
+    const size_t col = e / P.m, row = e - col * P.m;
+    float *cp = P.c + col * P.ldc + row;
+    float v = P.alpha * s;
+    if (P.beta != 0.f) v += P.beta * *cp;
+    *cp = v;
   }
 }
 
@@ -272,7 +317,32 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   P.tiles_m = (int)((m + bm - 1) / bm);
   P.tiles_n = (int)((n + bn - 1) / bn);
   P.group_m = P.tiles_m < 8 ? P.tiles_m : 8;
-  dim3 grid((unsigned)(P.tiles_m * P.tiles_n));
+  // Few tiles and a long K: slice K over blockIdx.y so every CU has work; the
+  // slices' partial products are summed in slice order by a second kernel.
+  P.ksplit = 1;
+  P.kchunk = P.k;
+  {
+    const int cus = thcl_rt_get_props(rt)->compute_units;
+    const long tiles = (long)P.tiles_m * P.tiles_n;
+    if (tiles < cus && k >= 1024) {
+      long want = (2L * cus + tiles - 1) / tiles;
+      long max_by_k = k / 256;  // at least 16 slabs per slice
+      if (want > max_by_k) want = max_by_k;
+      if (want > 32) want = 32;
+      if (want > 1) {
+        long chunk = ((k + want - 1) / want + BK - 1) / BK * BK;
+        P.kchunk = (int)chunk;
+        P.ksplit = (int)((k + chunk - 1) / chunk);
+        if (P.ksplit > 1) {
+          P.work = (float *)thcl_rt_workspace(rt, (size_t)P.ksplit * m * n * sizeof(float));
+          THCL_CHECK(P.work != nullptr, "gemm workspace: %s", thcl_rt_error());
+        } else {
+          P.kchunk = P.k;
+        }
+      }
+    }
+  }
+  dim3 grid((unsigned)(P.tiles_m * P.tiles_n), (unsigned)P.ksplit);
 #define GO(BM_, BN_)                                                   \
   if (fast) launch_tt<BM_, BN_, false>(ta, tb, grid, stream, P);        \
   else launch_tt<BM_, BN_, true>(ta, tb, grid, stream, P);
@@ -281,6 +351,11 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   else if (bm == 64 && bn == 128) { GO(64, 128) }
   else { GO(64, 64) }
 #undef GO
+  if (P.ksplit > 1) {
+    const size_t total = (size_t)m * n;
+    unsigned rg = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+    hipLaunchKernelGGL(splitk_reduce, dim3(rg), dim3(256), 0, stream, P);
+  }
   hipError_t e = hipGetLastError();
   THCL_CHECK(e == hipSuccess, "gemm launch failed: %s", hipGetErrorString(e));
   thcl_after_launch(state, rt);

@@ -28,6 +28,8 @@ struct thcl_rt {
   void *scratch = nullptr;
   size_t scratch_bytes = 0;
   float *host_word = nullptr;
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
   thcl_rt_props props{};
   std::map<std::string, RtModule *> modules;
 };
@@ -140,6 +142,7 @@ void thcl_rt_release_all(void) {
       delete kv.second;
     }
     (void)hipFree(rt->scratch);
+    (void)hipFree(rt->workspace);
     (void)hipHostFree(rt->host_word);
     (void)hipStreamDestroy(rt->stream);
     delete rt;
@@ -206,6 +209,29 @@ void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes) {
 }
 
 float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
+
+void *thcl_rt_workspace(thcl_rt *rt, size_t bytes) {
+  if (bytes <= rt->workspace_bytes) return rt->workspace;
+  DeviceGuard g(rt->device);
+  if (rt->workspace) {
+    // queued kernels may still use the old block
+    if (hipStreamSynchronize(rt->stream) != hipSuccess || hipFree(rt->workspace) != hipSuccess) {
+      g_err = "releasing the workspace failed";
+      return nullptr;
+    }
+    rt->workspace = nullptr;
+    rt->workspace_bytes = 0;
+  }
+  size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+  hipError_t e = hipMalloc(&rt->workspace, want);
+  if (e != hipSuccess) {
+    fail("hipMalloc(workspace)", e);
+    rt->workspace = nullptr;
+    return nullptr;
+  }
+  rt->workspace_bytes = want;
+  return rt->workspace;
+}
 
 static int rtc_compile(const char *source, const char *arch, std::vector<char> &code) {
   hiprtcProgram prog;

@@ -55,6 +55,9 @@ int thcl_rt_sync(thcl_rt *rt);
 
 /* per-device scratch block (partials, tickets), zero-initialised once */
 void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes);
+/* a device buffer of at least `bytes` that lives until a larger one is asked
+ * for; work queued on the stream keeps using it in order */
+void *thcl_rt_workspace(thcl_rt *rt, size_t bytes);
 /* pinned host words for handing scalars back */
 float *thcl_rt_host_word(thcl_rt *rt);
 

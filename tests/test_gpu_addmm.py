@@ -39,7 +39,9 @@ def _check(cl, pa: Pair, pb: Pair, pc: Pair, beta, alpha):
 
 @pytest.mark.parametrize("M,N,K", [(2, 2, 3), (1, 1, 1), (5, 7, 3), (64, 64, 16), (128, 128, 32), (128, 256, 64),
                                    (65, 63, 17), (129, 127, 33), (300, 200, 100), (256, 64, 512), (64, 1024, 48),
-                                   (1, 500, 37), (500, 1, 37), (37, 41, 1)])
+                                   (1, 500, 37), (500, 1, 37), (37, 41, 1),
+                                   # few tiles and a long K: the K dimension is sliced over blocks
+                                   (64, 1024, 2048), (128, 128, 4096), (70, 300, 1500), (33, 65, 5000), (256, 512, 1024)])
 def test_shapes_row_major(cl, M, N, K):
     a = oracle.normal(1, M * K).reshape(M, K)
     b = oracle.normal(2, K * N).reshape(K, N)
