@@ -1,0 +1,186 @@
+"""The five benchmark configurations at their full sizes, through the C ABI.
+
+Where the CPU oracle finishes in seconds the comparison is direct (bit-exact
+for pointwise/copy/positions, 1e-5 relative for sums, 1e-4 for addmm on sampled
+entries); the 2^28-element cases add size-independent properties (closed forms,
+linearity, idempotence, round trips)."""
+import numpy as np
+import pytest
+
+import oracle
+from oracle import View
+from gpu_util import Pair, assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+EXPR1 = "x = sqrt(1000*x*x + y*10 + z*z)"
+EXPR2 = "x = 1000*x + y*10"
+
+
+def test_config1_contiguous_sequence_2p24(cl):
+    n = 1 << 24
+    x, y, z = (oracle.uniform(s, n) for s in (1, 2, 3))
+    X, Y, Z = cl.ClTensor(x), cl.ClTensor(y), cl.ClTensor(z)
+    ref = View.contiguous(x.copy())
+    vy, vz = View.contiguous(y), View.contiguous(z)
+    X.add(Y)
+    oracle.pointwise("cadd", ref, ref, vy, 1.0)
+    assert_bit_equal(X.float(), ref.storage, "add")
+    X.cmul(Y)
+    oracle.pointwise("cmul", ref, ref, vy)
+    assert_bit_equal(X.float(), ref.storage, "cmul")
+    X.map2_on_gpu(Y, Z, EXPR1)
+    oracle.pointwise("map2_c1", ref, vy, vz)
+    assert_bit_equal(X.float(), ref.storage, "map2")          # sqrt of negative arguments: NaN on both sides
+    assert np.isnan(ref.storage).any()
+    # the NaNs make sum and max NaN on both sides (Torch7's CPU rule)
+    assert np.isnan(X.sum()) and np.isnan(oracle.sumall(ref))
+    assert np.isnan(X.max()) and np.isnan(oracle.maxall(ref))
+    # and on NaN-free data they agree numerically
+    clean = np.where(np.isnan(ref.storage), F(0), ref.storage)
+    C = cl.ClTensor(clean)
+    want = oracle.sumall(View.contiguous(clean))
+    assert abs(C.sum() - want) <= 1e-5 * abs(want)
+    assert C.max() == oracle.maxall(View.contiguous(clean)) and C.min() == oracle.minall(View.contiguous(clean))
+
+
+def test_config2_strided_views_full_size(cl):
+    shape = (512, 512, 256)
+    a = Pair.dense(cl, oracle.uniform(4, int(np.prod(shape))).reshape(shape))
+    b = Pair.dense(cl, oracle.uniform(5, int(np.prod(shape))).reshape(shape))
+    # transpose(1,3) views: sizes (256,512,512), strides (1,256,131072)
+    aT, bT = a.transpose(0, 2), b.transpose(0, 2)
+    assert aT.dev.size() == (256, 512, 512) and aT.dev.stride() == (1, 256, 131072)
+    aT.dev.map_on_gpu(bT.dev, EXPR2)
+    oracle.pointwise("map_c2", aT.view, bT.view)
+    assert_bit_equal(a.device_storage(), a.host_storage, "map on transposed views")
+    # strided copy into a fresh dense destination
+    dst = cl.ClTensor(256, 512, 512)
+    dst.copy(aT.dev)
+    assert_bit_equal(dst.float(), aT.view.gather(), "copy transposed -> dense")
+    # stride-2 view: sizes (512,512,128), strides (131072,256,2)
+    aS, bS = a.step(2, 2), b.step(2, 2)
+    assert aS.dev.stride() == (131072, 256, 2)
+    aS.dev.map_on_gpu(bS.dev, EXPR2)
+    oracle.pointwise("map_c2", aS.view, bS.view)
+    assert_bit_equal(a.device_storage(), a.host_storage, "map on stride-2 views (odd elements untouched)")
+    d2 = cl.ClTensor(512, 512, 128)
+    d2.copy(aS.dev)
+    assert_bit_equal(d2.float(), aS.view.gather(), "copy stride-2 -> dense")
+    # narrow view: offset 64, strides (131072,256,1)
+    aN, bN = a.narrow(2, 64, 128), b.narrow(2, 64, 128)
+    assert aN.dev.storageOffset() == 65
+    aN.dev.map_on_gpu(bN.dev, EXPR2)
+    oracle.pointwise("map_c2", aN.view, bN.view)
+    assert_bit_equal(a.device_storage(), a.host_storage, "map on narrow views")
+    # round trip: scatter the dense copy back through the transposed view
+    back = Pair.dense(cl, np.zeros(shape, dtype=F))
+    back.transpose(0, 2).dev.copy(dst)
+    aT_now = dst.float()
+    assert_bit_equal(back.transpose(0, 2).dev.float(), aT_now, "dense -> transposed -> read back")
+    assert_bit_equal(b.device_storage(), b.host_storage, "inputs untouched")
+
+
+def test_config3_reductions_along_each_dim_full_size(cl):
+    r, c = 4096, 16384
+    g = oracle.normal(6, r * c).reshape(r, c)
+    p = Pair.dense(cl, g)
+    g64 = g.astype(np.float64)
+    for dim0 in (0, 1):
+        got = p.dev.sum(dim0 + 1).float()
+        want = g64.sum(axis=dim0, keepdims=True)
+        assert got.shape == want.shape
+        # fp64 accumulation on both sides: at most the final rounding to fp32 apart
+        assert np.all(np.abs(got - want) <= 1.5 * np.spacing(np.abs(want).astype(F)).astype(np.float64))
+        assert np.all(np.abs(got - oracle.reduce_dim("sum", p.view, dim0)[0]) <= np.spacing(np.abs(want).astype(F)))
+        for kind in ("max", "min"):
+            wv, wi = oracle.reduce_dim(kind, p.view, dim0)
+            gv, gi = getattr(p.dev, kind)(dim0 + 1)
+            assert_bit_equal(gv.float(), wv, f"{kind} dim {dim0 + 1}")
+            assert np.array_equal(gi.long(), wi)
+            gv2, gi2 = getattr(p.dev, f"{kind}_long")(dim0 + 1)
+            assert np.array_equal(gi2, wi) and gi2.dtype == np.int64
+            # the reported position really holds the reported value
+            picked = np.take_along_axis(g, gi2 - 1, axis=dim0)
+            assert np.array_equal(picked, wv)
+
+
+def test_config4_point_tensor_chain_2p28(cl):
+    n = 1 << 28
+    a = oracle.uniform(7, n, 0.0, 1.0)
+    A = cl.ClTensor(a)
+    s = cl.ClTensor()
+    s.sum(A)                                    # stays on the device
+    want_sum = oracle.sumall(View.contiguous(a))
+    sv = s.s()
+    assert abs(sv - want_sum) <= 1e-5 * want_sum
+    A.div(s)
+    first = A.narrow(1, 1, 1 << 20).float()
+    assert_bit_equal(first, a[:1 << 20] / F(sv), "div by the point tensor")
+    # after normalisation the elements sum to 1 (to fp32 rounding of each quotient)
+    total = A.sum()
+    assert abs(total - 1.0) < 1e-5
+    # 8 further in-place ops, no host sync in between; mirrored on a slice with numpy fp32 arithmetic
+    ref = (a[:1 << 20] / F(sv)).astype(F)
+    A.mul(1.0001)
+    ref = ref * F(1.0001)
+    A.add(0.5)
+    ref = ref + F(0.5)
+    A.cmul(A)
+    ref = ref * ref
+    A.sqrt()
+    ref = np.sqrt(ref)
+    s2 = cl.ClTensor()
+    s2.max(A)
+    A.div(s2)
+    mx = F(s2.s())
+    ref = ref / mx
+    A.add(s2)
+    ref = ref + mx
+    A.csub(0.25)
+    ref = ref + F(-0.25)
+    A.abs()
+    ref = np.abs(ref)
+    cl.synchronize()
+    assert_bit_equal(A.narrow(1, 1, 1 << 20).float(), ref, "chained ops")
+    # closed forms at full size
+    A.fill(1.0)
+    assert A.sum() == float(n)
+    A.fill(0.25)
+    assert A.sum() == float(n) * 0.25 and A.max() == 0.25 and A.min() == 0.25
+    # idempotence of abs, and max/min bracket every element
+    A.copy(cl.ClTensor(a))
+    lo, hi = A.min(), A.max()
+    assert lo == float(a.min()) and hi == float(a.max())
+
+
+def test_config5_addmm_square_8192_sampled_and_skinny(cl):
+    n = 8192
+    sd = 1.0 / np.sqrt(n)
+    a = oracle.normal(8, n * n, 0.0, sd).reshape(n, n)
+    b = oracle.normal(9, n * n, 0.0, sd).reshape(n, n)
+    c = oracle.normal(10, n * n, 0.0, sd).reshape(n, n)
+    got = cl.ClTensor(c).addmm(0.5, 1.0, cl.ClTensor(a), cl.ClTensor(b)).float()
+    rng = np.random.RandomState(1)
+    rows = np.concatenate([rng.randint(0, n, 4000), [0, 0, n - 1, n - 1, 127, 128]])
+    cols = np.concatenate([rng.randint(0, n, 4000), [0, n - 1, 0, n - 1, 128, 127]])
+    want = oracle.addmm_f64_sampled(rows, cols, 0.5, View.contiguous(c), 1.0, View.contiguous(a), View.contiguous(b))
+    scale = float(np.sqrt(np.mean(want ** 2)))
+    assert np.max(np.abs(got[rows, cols] - want)) / scale < 1e-4
+    # checksum of checksums: ones^T (A B) ones == (ones^T A)(B ones), in fp64 from the device result
+    lhs = got.astype(np.float64).sum() - 0.5 * c.astype(np.float64).sum()
+    rhs = float(a.astype(np.float64).sum(axis=0) @ b.astype(np.float64).sum(axis=1))
+    assert abs(lhs - rhs) < 0.05, (lhs, rhs)
+    del got
+    # skinny: M=64, N=16384, K=4096, A = (K x M dense)^T
+    M, N, K = 64, 16384, 4096
+    at = oracle.normal(11, K * M, 0.0, sd).reshape(K, M)
+    bs = oracle.normal(12, K * N, 0.0, sd).reshape(K, N)
+    cs = oracle.normal(13, M * N, 0.0, sd).reshape(M, N)
+    pa = Pair.dense(cl, at).transpose(0, 1)
+    assert pa.dev.size() == (64, 4096) and pa.dev.stride() == (1, 64)
+    pb, pc = Pair.dense(cl, bs), Pair.dense(cl, cs)
+    pc.dev.addmm(0.5, 1.0, pa.dev, pb.dev)
+    want = oracle.addmm_f64(0.5, pc.view, 1.0, pa.view, pb.view)
+    scale = float(np.sqrt(np.mean(want ** 2)))
+    assert np.max(np.abs(pc.dev.float() - want)) / scale < 1e-4
