@@ -43,7 +43,8 @@ long units_per_tile(PlanKind k) {
 bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 
 // Fills `plan`; returns false when there is nothing to launch.
-bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan) {
+// `dry`: classify only (no device context is opened) -- used by the host-side tests.
+bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dry = false) {
   const int n = call.n;
   THClTensor *const *t = call.t;
   const long total = THClTensor_nElement(state, t[0]);
@@ -55,7 +56,7 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan) {
   for (int i = 0; i < n; i++)
     THCL_CHECK(t[i]->storage && t[i]->storage->wrapper, "tensor %d has no device storage", i + 1);
   thcl_check_same_device(state, 3, t[0], n > 1 ? t[1] : nullptr, n > 2 ? t[2] : nullptr);
-  plan.rt = thcl_ctx(state, t[0]->storage->device);
+  plan.rt = dry ? nullptr : thcl_ctx(state, t[0]->storage->device);
 
   float *p[3] = {nullptr, nullptr, nullptr};
   for (int i = 0; i < n; i++) p[i] = thcl_dptr(t[i]);
@@ -357,6 +358,38 @@ void thcl_fill_contig(thcl_rt *rt, float *dst, float value, long n) {
 // ------------------------------------------------------------ test hooks ---
 // Host-only helpers so the layout logic can be checked without a device.
 extern "C" {
+// Which kernel family a call with these views would launch, and its grid:
+// 0 dense 128-bit, 1 dense scalar, 2 joint 128-bit, 3 joint scalar, 4 generic,
+// 5 tiled, 6 nothing to do, -1 rejected.  Views are rows of [n][25] arrays;
+// misalign[i] = bytes by which operand i's storage misses a 16-byte boundary.
+int thcl_dbg_plan_kind(int n, const int *nd, long *sizes, long *strides, const long *offsets, const int *misalign,
+                       unsigned *grid) {
+  THClTensor hdr[3];
+  THClStorage st[3];
+  ApplyCall call;
+  call.n = n;
+  for (int i = 0; i < n; i++) {
+    hdr[i] = THClTensor{};
+    st[i] = THClStorage{};
+    st[i].wrapper = (void *)(uintptr_t)(0x10000000ull * (i + 1) + (unsigned)misalign[i]);
+    st[i].size = 1l << 40;
+    hdr[i].size = sizes + i * THCL_MAX_DIMS;
+    hdr[i].stride = strides + i * THCL_MAX_DIMS;
+    hdr[i].nDimension = nd[i];
+    hdr[i].storageOffset = offsets[i];
+    hdr[i].storage = &st[i];
+    call.t[i] = &hdr[i];
+  }
+  try {
+    ApplyPlan plan;
+    if (!make_plan(nullptr, call, plan, true)) return 6;
+    if (grid) *grid = plan.grid;
+    return (int)plan.kind;
+  } catch (const std::exception &) {
+    return -1;
+  }
+}
+
 unsigned thcl_dbg_divide(unsigned n, long d) {
   ThclDivisor dv = thcl_make_divisor(d);
   return (unsigned)((((unsigned long long)n * dv.magic) >> 32) + n) >> dv.shift;

@@ -199,3 +199,46 @@ def test_bad_expression_reports_compiler_log(lib):
     rc = lib.thcl_dbg_compile_expr(b"x = this is not C", 1, b"gfx950", C.byref(size))
     assert rc != 0
     assert b"error" in lib.thcl_rt_error()
+
+
+# ------------------------------------------------------------ kernel planning ---
+KINDS = {0: "dense128", 1: "dense32", 2: "joint128", 3: "joint32", 4: "generic", 5: "tiled", 6: "nothing", -1: "rejected"}
+
+
+def _plan(lib, views, misalign=None):
+    """views: list of (sizes, strides, offset).  Returns (kind name, grid)."""
+    n = len(views)
+    lib.thcl_dbg_plan_kind.restype = C.c_int
+    szs, sts = (C.c_long * (3 * MAXD))(), (C.c_long * (3 * MAXD))()
+    nd, off, mis = (C.c_int * 3)(), (C.c_long * 3)(), (C.c_int * 3)()
+    for i, (sz, st, o) in enumerate(views):
+        nd[i], off[i] = len(sz), o
+        mis[i] = (misalign or [0] * n)[i]
+        for d in range(len(sz)):
+            szs[i * MAXD + d], sts[i * MAXD + d] = sz[d], st[d]
+    grid = C.c_uint(0)
+    k = lib.thcl_dbg_plan_kind(n, nd, szs, sts, off, mis, C.byref(grid))
+    return KINDS[k], grid.value
+
+
+def test_planner_picks_the_kernel_family_for_each_layout(lib):
+    dense = ((512, 512, 256), (131072, 256, 1), 0)
+    assert _plan(lib, [dense, dense]) == ("dense128", 2 ** 26 // 4 // 256)
+    assert _plan(lib, [dense, dense], [0, 4])[0] == "dense32"                       # one operand 4 bytes off
+    assert _plan(lib, [((100,), (1,), 1), ((100,), (1,), 0)])[0] == "dense32"       # odd element offset
+    tr = ((256, 512, 512), (1, 256, 131072), 0)
+    assert _plan(lib, [tr, tr])[0] == "dense128"                                    # identically transposed: dense walk
+    dst = ((256, 512, 512), (262144, 512, 1), 0)
+    kind, grid = _plan(lib, [dst, tr])
+    assert kind == "tiled" and grid == 512 * (512 // 64) * (256 // 128)             # 64 x 128 tiles, 512 outer slices
+    assert _plan(lib, [tr, dst])[0] == "tiled"                                      # scatter into the transposed view
+    s2 = ((512, 512, 128), (131072, 256, 2), 0)
+    assert _plan(lib, [s2, s2])[0] == "joint32"
+    nar = ((512, 512, 128), (131072, 256, 1), 64)
+    assert _plan(lib, [nar, nar])[0] == "joint128"
+    assert _plan(lib, [nar, ((512, 512, 128), (131072, 256, 1), 65)])[0] == "joint32"   # rows not 16-byte aligned
+    assert _plan(lib, [((30, 28), (28, 1), 0), ((28, 30), (1, 56), 0)])[0] == "generic"  # shapes differ
+    assert _plan(lib, [((4, 5), (5, 1), 0), ((21,), (1,), 0)])[0] == "rejected"     # element counts differ
+    assert _plan(lib, [((3, 4), (4, 1), 0)])[0] == "dense128"
+    # tiny transposed operands are not worth a tile
+    assert _plan(lib, [((8, 8), (8, 1), 0), ((8, 8), (1, 8), 0)])[0] == "joint32"
