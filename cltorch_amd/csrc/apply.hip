@@ -29,9 +29,9 @@ struct ApplyPlan {
 };
 
 constexpr unsigned kMaxGrid = 1u << 23;  // x 256 threads stays below 2^32 work-items; larger inputs loop
-long units_per_tile(PlanKind k) {
+long units_per_tile(PlanKind k, int nt) {
   switch (k) {
-    case K_CONTIG_V4:
+    case K_CONTIG_V4: return THCL_CONTIG_THREADS_FOR(nt) * THCL_CONTIG_UNROLL;
     case K_CONTIG_S: return THCL_APPLY_THREADS * THCL_CONTIG_UNROLL;
     case K_JOINT_V4: return THCL_APPLY_THREADS * THCL_JOINT_V4_UNROLL;
     case K_JOINT_S: return THCL_APPLY_THREADS * THCL_JOINT_S_UNROLL;
@@ -41,6 +41,7 @@ long units_per_tile(PlanKind k) {
 
 
 bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+bool aligned_vec(const void *p, int nt) { return (((uintptr_t)p) & (THCL_CONTIG_W_FOR(nt) * 4 - 1)) == 0; }
 
 // Fills `plan`; returns false when there is nothing to launch.
 // `dry`: classify only (no device context is opened) -- used by the host-side tests.
@@ -76,7 +77,7 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
 
   if (all_contig) {
     bool al = true;
-    for (int i = 0; i < n; i++) al = al && aligned16(p[i]);
+    for (int i = 0; i < n; i++) al = al && aligned_vec(p[i], n);
     plan.kind = al ? K_CONTIG_V4 : K_CONTIG_S;
     ThclContigParams &c = plan.c;
     memset(&c, 0, sizeof(c));
@@ -86,8 +87,8 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
     c.val[0] = call.val[0];
     c.val[1] = call.val[1];
     c.n = (thcl_u64)total;
-    const long units = al ? (total >> 2) : total;
-    const long upt = units_per_tile(plan.kind);
+    const long units = al ? (total / THCL_CONTIG_W_FOR(n)) : total;
+    const long upt = units_per_tile(plan.kind, n);
     const long tiles = (units + upt - 1) / upt;
     c.ntiles = (thcl_u64)tiles;
     plan.grid = (unsigned)(tiles < 1 ? 1 : (tiles > kMaxGrid ? kMaxGrid : tiles));
@@ -177,7 +178,7 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
       j.size[d] = thcl_make_divisor(s);
       for (int i = 0; i < n; i++) j.stride[i][d] = (thcl_u32)J.strides[i][d];
     }
-    const long upt = units_per_tile(plan.kind);
+    const long upt = units_per_tile(plan.kind, n);
     const long tiles = (units + upt - 1) / upt;
     j.ntiles = (thcl_u32)tiles;
     plan.grid = (unsigned)(tiles > kMaxGrid ? kMaxGrid : tiles);
@@ -202,7 +203,7 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
       g.op[i].stride[d] = (thcl_u32)L.strides[d];
     }
   }
-  const long upt = units_per_tile(plan.kind);
+  const long upt = units_per_tile(plan.kind, n);
   const long tiles = (total + upt - 1) / upt;
   g.ntiles = (thcl_u32)tiles;
   plan.grid = (unsigned)(tiles > kMaxGrid ? kMaxGrid : tiles);
@@ -248,7 +249,7 @@ void launch_fixed(const KernelSet &ks, ApplyPlan &plan) {
   hipStream_t stream = (hipStream_t)thcl_rt_stream(plan.rt);
   dim3 grid(plan.grid), block(THCL_APPLY_THREADS);
   switch (plan.kind) {
-    case K_CONTIG_V4: hipLaunchKernelGGL(ks.contig_v4, grid, block, 0, stream, plan.c); break;
+    case K_CONTIG_V4: hipLaunchKernelGGL(ks.contig_v4, grid, dim3(THCL_CONTIG_THREADS_FOR(ks.nt)), 0, stream, plan.c); break;
     case K_CONTIG_S: hipLaunchKernelGGL(ks.contig_s, grid, block, 0, stream, plan.c); break;
     case K_JOINT_V4: hipLaunchKernelGGL(ks.joint_v4, grid, block, 0, stream, plan.j); break;
     case K_JOINT_S: hipLaunchKernelGGL(ks.joint_s, grid, block, 0, stream, plan.j); break;
@@ -277,7 +278,8 @@ void launch_expr(THClState *state, const std::string &expr, int nt, ApplyPlan &p
     case K_TILED: params = &plan.t; bytes = sizeof(plan.t); break;
     default: params = &plan.g; bytes = sizeof(plan.g); break;
   }
-  const unsigned threads = plan.kind == K_TILED ? THCL_TILE_THREADS : THCL_APPLY_THREADS;
+  const unsigned threads = plan.kind == K_TILED ? THCL_TILE_THREADS
+                           : plan.kind == K_CONTIG_V4 ? THCL_CONTIG_THREADS_FOR(nt) : THCL_APPLY_THREADS;
   THCL_CHECK(thcl_rt_launch(plan.rt, k, plan.grid, 1, 1, threads, 1, 1, 0, params, bytes) == 0, "%s",
              thcl_rt_error());
   (void)state;
@@ -315,6 +317,20 @@ void with_overlap_fixup(THClState *state, ApplyCall &call, F body) {
 }
 }  // namespace
 
+// The tunable shape constants this build was compiled with, as #define lines:
+// prepended to run-time compiled sources so both kinds of kernels agree with
+// the host-side planning.
+std::string thcl_apply_config_defines() {
+#define THCL_STR2(x) #x
+#define THCL_STR(x) THCL_STR2(x)
+  return "#define THCL_TILE_A " THCL_STR(THCL_TILE_A) "\n"
+         "#define THCL_TILE_B " THCL_STR(THCL_TILE_B) "\n"
+         "#define THCL_TILE_THREADS " THCL_STR(THCL_TILE_THREADS) "\n"
+         "#define THCL_TILE_UNROLL " THCL_STR(THCL_TILE_UNROLL) "\n";
+#undef THCL_STR
+#undef THCL_STR2
+}
+
 void thcl_apply_fixed(THClState *state, ThclOp op, ApplyCall &call) {
   THCL_CHECK(op >= 0 && op < OP_COUNT, "unknown operator %d", (int)op);
   const KernelSet &ks = kFixed[op];
@@ -345,10 +361,10 @@ void thcl_fill_contig(thcl_rt *rt, float *dst, float value, long n) {
   c.p[0] = dst;
   c.val[0] = value;
   c.n = (thcl_u64)n;
-  const bool al = aligned16(dst);
+  const bool al = aligned_vec(dst, 1);
   plan.kind = al ? K_CONTIG_V4 : K_CONTIG_S;
-  const long units = al ? (n >> 2) : n;
-  const long upt = units_per_tile(plan.kind);
+  const long units = al ? (n / THCL_CONTIG_W_FOR(1)) : n;
+  const long upt = units_per_tile(plan.kind, 1);
   const long tiles = (units + upt - 1) / upt;
   c.ntiles = (thcl_u64)tiles;
   plan.grid = (unsigned)(tiles < 1 ? 1 : (tiles > kMaxGrid ? kMaxGrid : tiles));

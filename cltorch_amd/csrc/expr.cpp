@@ -128,6 +128,7 @@ std::string thcl_expr_source(const std::string &rewritten, int ntensors) {
   THCL_CHECK(ntensors >= 1 && ntensors <= 3, "expression kernels take 1 to 3 tensors");
   std::string src;
   src.reserve(sizeof(kSkeleton) + sizeof(kPrelude) + rewritten.size() + 1024);
+  src += thcl_apply_config_defines();
   src += kSkeleton;
   src += kPrelude;
   src += "struct ThclUserOp {\n";

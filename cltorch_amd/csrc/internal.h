@@ -108,6 +108,7 @@ void thcl_apply_expr(THClState *state, const std::string &expr, ApplyCall &call)
 std::string thcl_rewrite_expr(const char *expr, int ntensors);
 std::string thcl_expr_source(const std::string &rewritten, int ntensors);
 std::string thcl_expr_tag(const std::string &rewritten, int ntensors);
+std::string thcl_apply_config_defines();
 
 // ------------------------------------------------------------- reductions ---
 enum ThclReduce : int { RED_SUM = 0, RED_PROD = 1, RED_MAX = 2, RED_MIN = 3 };

@@ -223,7 +223,9 @@ def _plan(lib, views, misalign=None):
 
 def test_planner_picks_the_kernel_family_for_each_layout(lib):
     dense = ((512, 512, 256), (131072, 256, 1), 0)
-    assert _plan(lib, [dense, dense]) == ("dense128", 2 ** 26 // 4 // 256)
+    assert _plan(lib, [dense, dense]) == ("dense128", 2 ** 26 // 4 // 64)         # one-wave blocks, 4 floats per lane
+    assert _plan(lib, [dense, dense, dense]) == ("dense128", 2 ** 26 // 2 // 64)  # three operands: 2 floats per lane
+    assert _plan(lib, [dense]) == ("dense128", 2 ** 26 // 4 // 256)
     assert _plan(lib, [dense, dense], [0, 4])[0] == "dense32"                       # one operand 4 bytes off
     assert _plan(lib, [((100,), (1,), 1), ((100,), (1,), 0)])[0] == "dense32"       # odd element offset
     tr = ((256, 512, 512), (1, 256, 131072), 0)
