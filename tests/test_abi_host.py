@@ -232,7 +232,11 @@ def test_planner_picks_the_kernel_family_for_each_layout(lib):
     assert _plan(lib, [tr, tr])[0] == "dense128"                                    # identically transposed: dense walk
     dst = ((256, 512, 512), (262144, 512, 1), 0)
     kind, grid = _plan(lib, [dst, tr])
-    assert kind == "tiled" and grid == 512 * (512 // 64) * (256 // 128)             # 64 x 128 tiles, 512 outer slices
+    assert kind == "tiled" and grid == 512 * (512 // 64) * (256 // 256)             # 64 x 256 tiles, 512 outer slices
+    sq = _plan(lib, [((8192, 8192), (8192, 1), 0), ((8192, 8192), (1, 8192), 0)])
+    assert sq == ("tiled", (8192 // 128) ** 2)                                      # plain 2-d transpose: 128 x 128 tiles
+    thin = _plan(lib, [((1024, 64, 1024), (65536, 1024, 1), 0), ((1024, 64, 1024), (65536, 1, 64), 0)])
+    assert thin == ("tiled", 1024 * (1024 // 256) * (64 // 64))                     # dim B of 64: 256 x 64 tiles waste nothing
     assert _plan(lib, [tr, dst])[0] == "tiled"                                      # scatter into the transposed view
     s2 = ((512, 512, 128), (131072, 256, 2), 0)
     assert _plan(lib, [s2, s2])[0] == "joint32"

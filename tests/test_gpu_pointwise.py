@@ -309,10 +309,13 @@ def test_host_roundtrip_of_strided_views(cl):
 
 
 # ------------------------------------------------- transposed operands (LDS tiles) ---
-@pytest.mark.parametrize("shape", [(130, 70), (64, 128), (200, 300), (3, 150, 90), (5, 17, 260), (2, 3, 70, 129)])
+@pytest.mark.parametrize("shape", [(130, 70), (64, 128), (200, 300), (3, 150, 90), (5, 17, 260), (2, 3, 70, 129),
+                                   (64, 300), (300, 64), (256, 1024), (2, 512, 1024), (3, 1024, 272)])
 def test_transposed_operand_meets_dense_one(cl, shape):
     """Operands whose unit-stride dims differ: the library stages the transposed
-    ones through LDS tiles; full tiles, ragged edges and outer dims."""
+    ones through LDS tiles; full tiles, ragged edges and outer dims, each of the
+    three tile shapes (thin dims pick 256 x 64 or 64 x 256) and the diagonal
+    tile order that power-of-two pitches switch on."""
     n = int(np.prod(shape))
     nd = len(shape)
     x, y, z = oracle.uniform(31, n), oracle.uniform(32, n), oracle.uniform(33, n)
