@@ -26,8 +26,9 @@ constexpr int kThreads = 256;
 constexpr int kWave = 64;
 
 // scratch block layout (bytes)
-constexpr size_t kTicketOff = 0;            // 1024 uint32 tickets
-constexpr size_t kPartialOff = 4096;        // partials
+constexpr size_t kTicketOff = 0;            // 4096 uint32 tickets: [0] whole-tensor reductions, [64..] column tiles
+constexpr size_t kPartialOff = 16384;       // partials
+constexpr unsigned kColTicket0 = 64, kColTickets = 4096 - 64;
 constexpr size_t kResultSlot = 256;         // tail reserved for scalar results
 
 // --------------------------------------------------------------- combiners ---
@@ -142,6 +143,28 @@ __device__ __forceinline__ float load_fresh(const float *p) {
   return __uint_as_float(__atomic_load_n((const unsigned *)p, __ATOMIC_RELAXED));
 }
 
+// Partials that other blocks of the same launch will read: written through to
+// device scope (no dirty line stays in this XCD's L2) and read back with
+// device-scope loads.
+__device__ __forceinline__ void store_shared(double *p, double v) {
+  __hip_atomic_store((unsigned long long *)p, (unsigned long long)__double_as_longlong(v), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_shared(float *p, float v) {
+  __hip_atomic_store((unsigned *)p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_shared(VI *p, VI v) {
+  const unsigned long long bits = (unsigned long long)__float_as_uint(v.v) | ((unsigned long long)(unsigned)v.i << 32);
+  __hip_atomic_store((unsigned long long *)p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ VI load_fresh(const VI *p) {
+  const unsigned long long bits = __atomic_load_n((const unsigned long long *)p, __ATOMIC_RELAXED);
+  VI r;
+  r.v = __uint_as_float((unsigned)bits);
+  r.i = (int)(unsigned)(bits >> 32);
+  return r;
+}
+
 // ------------------------------------------------------------- reduce all ---
 struct ReduceAllParams {
   const float *in;
@@ -253,11 +276,13 @@ struct ReduceDimParams {
   float *idx_f32;        // dense 1-based positions as fp32, or NULL
   long long *idx_i64;    // dense 1-based positions as int64, or NULL
   void *partials;        // [split][nslices] when the reduction length is split over blocks
+  unsigned *ticket;      // one arrival counter per column tile (split > 1), zero between launches
   thcl_u32 nslices;      // output elements
   thcl_u32 nunits;       // slices / VEC (column kernel)
   thcl_u32 R;            // reduction length
   thcl_u32 rstride;      // elements between consecutive reduced elements
   thcl_u32 split;        // blocks sharing one slice's reduction (column kernel)
+  thcl_u32 fused;        // split > 1: the last block of a tile folds its partials (else a second kernel does)
   thcl_u32 rows_per_split;
   ThclGenericOperand L;  // layout of the slice starts (the view without `dim`)
 };
@@ -269,6 +294,7 @@ struct Slot<KIND, false> {
   typedef typename Acc<KIND>::T T;
   static __device__ __forceinline__ T init() { return Acc<KIND>::init(); }
   static __device__ __forceinline__ T take(T cur, float x, int) { return Acc<KIND>::comb(cur, Acc<KIND>::lift(x)); }
+  static __device__ __forceinline__ T seal(T acc, int, bool) { return acc; }
   static __device__ __forceinline__ T comb(T a, T b) { return Acc<KIND>::comb(a, b); }
   static __device__ __forceinline__ T reduce(T v, int width) { return group_reduce<KIND, T>(v, width); }
   static __device__ __forceinline__ void store(const ReduceDimParams &P, thcl_u32 s, T v) { P.out[s] = Acc<KIND>::lower(v); }
@@ -277,11 +303,23 @@ template <int KIND>
 struct Slot<KIND, true> {
   typedef VI T;
   static __device__ __forceinline__ T init() { return vi_init<KIND>(); }
+  // For a thread that meets positions in increasing order: replace when
+  // !(x <= cur) (max) unless cur is already NaN.  Five instructions where the
+  // order-free rule takes ten; an element equal to the start value is never
+  // taken, which seal() repairs.
   static __device__ __forceinline__ T take(T cur, float x, int i) {
-    VI n;
-    n.v = x;
-    n.i = i;
-    return vi_comb<KIND>(cur, n);
+    const bool beats = (KIND == RED_MAX) ? !(x <= cur.v) : !(x >= cur.v);
+    const bool take = beats & (cur.v == cur.v);
+    VI r;
+    r.v = take ? x : cur.v;
+    r.i = take ? i : cur.i;
+    return r;
+  }
+  // After the thread's last element: if nothing was ever taken, every element
+  // equalled the start value and the first position met is the answer.
+  static __device__ __forceinline__ T seal(T acc, int first, bool any) {
+    if (any & (acc.i == 0x7fffffff)) acc.i = first;
+    return acc;
   }
   static __device__ __forceinline__ T comb(T a, T b) { return vi_comb<KIND>(a, b); }
   static __device__ __forceinline__ T reduce(T v, int width) { return group_reduce_vi<KIND>(v, width); }
@@ -338,6 +376,8 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
         }
         for (; i < P.R; i += LPR) acc = S::take(acc, row[i], (int)i);
       }
+      // the first position this thread met
+      acc = S::seal(acc, (int)(VEC == 4 ? sub * 4 : sub), (VEC == 4 ? (thcl_u32)sub < (P.R >> 2) : (thcl_u32)sub < P.R));
     }
     if (LPR <= kWave) {
       acc = S::reduce(acc, LPR);
@@ -392,7 +432,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
       }
       // this wave takes rows r_begin + wave, + WAVES, ...; FLY of them are loaded
       // before any is consumed, the address advances by a constant step
-      constexpr int FLY = 4;
+      constexpr int FLY = 8;
       thcl_u32 r = r_begin + wave;
       const float *ptr = P.in + off + (thcl_u64)r * P.rstride;
       const thcl_u64 step = (thcl_u64)WAVES * P.rstride;
@@ -429,6 +469,8 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
         }
         ptr += step;
       }
+#pragma unroll
+      for (int c = 0; c < VEC; c++) acc[c] = S::seal(acc[c], (int)(r_begin + wave), r_begin + wave < r_end);
     }
     __syncthreads();
 #pragma unroll
@@ -440,11 +482,46 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
         T r = lds[0][lane * VEC + c];
         for (int w = 1; w < WAVES; w++) r = S::comb(r, lds[w][lane * VEC + c]);
         const thcl_u32 s = u * VEC + c;
-        if (P.split > 1) ((T *)P.partials)[(thcl_u64)blockIdx.y * P.nslices + s] = r;
+        if (P.split > 1) store_shared((T *)P.partials + (thcl_u64)blockIdx.y * P.nslices + s, r);
         else S::store(P, s, r);
       }
     }
   }
+  if (P.split == 1 || !P.fused) return;
+  // Short splits (one tile per block column, gridDim.x == ntiles): the
+  // block that arrives last at its tile folds the tile's partials in split
+  // order.  Wave 0 wrote this block's partials; once its stores are
+  // acknowledged they are visible device-wide, so the ticket taken afterwards
+  // orders them before the last block's reads.
+  __shared__ unsigned s_last;
+  if (wave == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (lane == 0) {
+      const unsigned t = atomicAdd(P.ticket + blockIdx.x, 1u);
+      s_last = (t == P.split - 1) ? 1u : 0u;
+    }
+  }
+  __syncthreads();
+  if (!s_last) return;
+  const T *partials = (const T *)P.partials;
+  for (thcl_u32 j = threadIdx.x; j < kWave * VEC; j += kThreads) {
+    const thcl_u32 s = blockIdx.x * (kWave * VEC) + j;
+    if (s < P.nslices) {
+      T t = S::init();
+      thcl_u32 k = 0;
+      constexpr int B = 16;  // partials fetched together
+      for (; k + B <= P.split; k += B) {
+        T v[B];
+#pragma unroll
+        for (int b = 0; b < B; b++) v[b] = load_fresh(partials + (thcl_u64)(k + b) * P.nslices + s);
+#pragma unroll
+        for (int b = 0; b < B; b++) t = S::comb(t, v[b]);
+      }
+      for (; k < P.split; k++) t = S::comb(t, load_fresh(partials + (thcl_u64)k * P.nslices + s));
+      S::store(P, s, t);
+    }
+  }
+  if (threadIdx.x == 0) P.ticket[blockIdx.x] = 0u;
 }
 
 // Folds the [split][nslices] partials.  A block owns 16 adjacent slices; its 16
@@ -637,6 +714,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   size_t sbytes = 0;
   char *scratch = (char *)thcl_rt_scratch(rt, &sbytes);
   P.partials = scratch + kPartialOff;
+  P.ticket = (unsigned *)(scratch + kTicketOff) + kColTicket0;
   const long partial_cap = (long)((sbytes - kPartialOff - kResultSlot) / 8);  // 8-byte entries
   const int cus = thcl_rt_get_props(rt)->compute_units;
 
@@ -660,7 +738,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     const long tiles = (P.nunits + kWave - 1) / kWave;
     // enough blocks to fill the chip: split the reduced dim when slices are few
     long split = 1;
-    const long target = (long)cus * 8;
+    const long target = (long)cus * 4;
     if (tiles < target) {
       split = (target + tiles - 1) / tiles;
       const long max_by_rows = (R + 31) / 32;  // at least 32 rows per block
@@ -673,6 +751,9 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     split = (R + rps - 1) / rps;
     P.split = (thcl_u32)split;
     P.rows_per_split = (thcl_u32)rps;
+    // One block folding a tile's partials is quick while they are few; a long
+    // split (few, tall slices) is folded by a second, chip-wide kernel.
+    P.fused = (split > 1 && split <= 32 && tiles <= (long)kColTickets) ? 1u : 0u;
     grid.x = (unsigned)(tiles > (1l << 20) ? (1l << 20) : tiles);
     grid.y = (unsigned)split;
   }
@@ -681,7 +762,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   if (arg) launch_dim<K, true>(rows, lpr, vec, grid, stream, P);          \
   else launch_dim<K, false>(rows, lpr, vec, grid, stream, P);             \
   check_launch("reduce-dim");                                             \
-  if (!rows && P.split > 1) {                                             \
+  if (!rows && P.split > 1 && !P.fused) {                                 \
     unsigned fg = (unsigned)((nslices + kFinSlices - 1) / kFinSlices);    \
     if (arg) launch_finish<K, true>(fg, stream, P);                       \
     else launch_finish<K, false>(fg, stream, P);                          \

@@ -173,6 +173,24 @@ def test_positions_ties_and_nans(cl):
     assert p.dev.min(2)[1].long()[2, 0] == 2
 
 
+@pytest.mark.parametrize("shape", [(3, 70), (70, 3), (5, 4096), (4096, 8), (300, 260)])
+def test_positions_when_every_element_is_the_start_value(cl, shape):
+    """max over slices of -inf (min over +inf): nothing ever beats the start
+    value, the answer is still position 1; one finite or NaN element moves it."""
+    for kind, start in (("max", -np.inf), ("min", np.inf)):
+        x = np.full(shape, start, dtype=F)
+        x[shape[0] // 2, shape[1] // 2] = 1.0 if kind == "max" else -1.0
+        x[shape[0] - 1, 0] = np.nan
+        p = Pair.dense(cl, x)
+        for d in (0, 1):
+            wv, wi = oracle.reduce_dim(kind, p.view, d)
+            gv, gi = getattr(p.dev, kind)(d + 1)
+            assert_bit_equal(gv.float(), wv, f"{kind} values dim {d + 1}")
+            assert np.array_equal(gi.long(), wi), f"{kind} positions dim {d + 1}"
+            # untouched slices report position 1
+            assert (wi == 1).sum() >= min(shape[1 - d], 2) - 2
+
+
 def test_results_into_existing_strided_tensors(cl):
     x = oracle.uniform(19, 40 * 24).reshape(40, 24)
     X = cl.ClTensor(x)
