@@ -346,6 +346,82 @@ class ClTensor:
     def floor(self, src=None): return self._unary("floor", src)
     def ceil(self, src=None): return self._unary("ceil", src)
 
+    def log1p(self, src=None): return self._unary("log1p", src)
+    def cos(self, src=None): return self._unary("cos", src)
+    def acos(self, src=None): return self._unary("acos", src)
+    def cosh(self, src=None): return self._unary("cosh", src)
+    def sin(self, src=None): return self._unary("sin", src)
+    def asin(self, src=None): return self._unary("asin", src)
+    def sinh(self, src=None): return self._unary("sinh", src)
+    def tan(self, src=None): return self._unary("tan", src)
+    def atan(self, src=None): return self._unary("atan", src)
+    def round(self, src=None): return self._unary("round", src)
+    def sign(self, src=None): return self._unary("sign", src)
+
+    def pow(self, *args) -> "ClTensor":
+        """``x:pow(v)`` in place, ``res:pow(src, v)``, and ``res:pow(v, src)`` = v ^ src
+        (``src/TensorMath.lua:1025-1033``)."""
+        if len(args) == 1:
+            _call("THClTensor_pow", self._h, self._h, C.c_float(args[0]))
+        elif isinstance(args[0], ClTensor):
+            _call("THClTensor_pow", self._h, args[0]._h, C.c_float(args[1]))
+        else:
+            _call("THClTensor_tpow", self._h, C.c_float(args[0]), args[1]._h)
+        return self
+
+    def cpow(self, *args) -> "ClTensor":
+        return self._binary("cpow", args)
+
+    def clamp(self, *args) -> "ClTensor":
+        """``x:clamp(lo, hi)`` in place or ``res:clamp(src, lo, hi)``."""
+        src, lo, hi = (self,) + tuple(args) if len(args) == 2 else args
+        _call("THClTensor_clamp", self._h, src._h, C.c_float(lo), C.c_float(hi))
+        return self
+
+    def atan2(self, *args) -> "ClTensor":
+        """``x:atan2(y)`` = atan2(x, y) in place, or ``res:atan2(a, b)``."""
+        a, b = (self, args[0]) if len(args) == 1 else args
+        _call("THClTensor_atan2", self._h, a._h, b._h)
+        return self
+
+    def _cminmax(self, name: str, args) -> "ClTensor":
+        src, other = (self, args[0]) if len(args) == 1 else args
+        if isinstance(other, ClTensor):
+            _call(f"THClTensor_{name}", self._h, src._h, other._h)
+        else:
+            _call(f"THClTensor_{name}Value", self._h, src._h, C.c_float(other))
+        return self
+
+    def cmax(self, *args) -> "ClTensor":
+        return self._cminmax("cmax", args)
+
+    def cmin(self, *args) -> "ClTensor":
+        return self._cminmax("cmin", args)
+
+    def _compare(self, name: str, args) -> "ClTensor":
+        """``a:lt(v)`` / ``a:lt(b)`` give a new 0/1 tensor; ``res:lt(a, v)`` / ``res:lt(a, b)``
+        write into res (``src/TensorMath.lua:1052-1062``).  A 0-dim ClTensor on the right
+        is a point tensor: the comparison reads it on the device."""
+        res, src, other = (ClTensor(), self, args[0]) if len(args) == 1 else (self, args[0], args[1])
+        if isinstance(other, ClTensor) and other.nDimension() == 0:
+            _call(f"THClTensor_{name}PointTensor", res._h, src._h, other._h)
+        elif isinstance(other, ClTensor):
+            _call(f"THClTensor_{name}Tensor", res._h, src._h, other._h)
+        else:
+            _call(f"THClTensor_{name}Value", res._h, src._h, C.c_float(other))
+        return res
+
+    def lt(self, *args): return self._compare("lt", args)
+    def gt(self, *args): return self._compare("gt", args)
+    def le(self, *args): return self._compare("le", args)
+    def ge(self, *args): return self._compare("ge", args)
+    def eq(self, *args): return self._compare("eq", args)
+    def ne(self, *args): return self._compare("ne", args)
+
+    def maskedFill(self, mask: "ClTensor", value: float) -> "ClTensor":
+        _call("THClTensor_maskedFill", self._h, mask._h, C.c_float(value))
+        return self
+
     # ---- user expressions ---------------------------------------------------
     def apply_on_gpu(self, expr: str) -> "ClTensor":
         _call("THClTensor_apply", self._h, expr.encode())

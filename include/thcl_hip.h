@@ -283,6 +283,51 @@ void THClTensor_tanh(THClState *state, THClTensor *self, THClTensor *src);
 void THClTensor_sigmoid(THClState *state, THClTensor *self, THClTensor *src);
 void THClTensor_floor(THClState *state, THClTensor *self, THClTensor *src);
 void THClTensor_ceil(THClState *state, THClTensor *self, THClTensor *src);
+/* More of the operator catalogue; each is the reference's operator string run
+ * through the same apply engine (src/lib/THClTensorMath.h:21,53-84,112,138-144). */
+void THClTensor_log1p(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_cos(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_acos(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_cosh(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_sin(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_asin(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_sinh(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_tan(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_atan(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_round(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_sign(THClState *state, THClTensor *self, THClTensor *src);
+/* src ^ value (integer-valued exponents by repeated multiplication: src/lib/THClTensorMath2.cpp:22-61) */
+void THClTensor_pow(THClState *state, THClTensor *self, THClTensor *src, float value);
+/* value ^ src */
+void THClTensor_tpow(THClState *state, THClTensor *self, float value, THClTensor *src);
+void THClTensor_cpow(THClState *state, THClTensor *self, THClTensor *src1, THClTensor *src2);
+void THClTensor_clamp(THClState *state, THClTensor *self, THClTensor *src, float min_value, float max_value);
+void THClTensor_atan2(THClState *state, THClTensor *r_, THClTensor *tx, THClTensor *ty);
+void THClTensor_cmax(THClState *state, THClTensor *self, THClTensor *src1, THClTensor *src2);
+void THClTensor_cmin(THClState *state, THClTensor *self, THClTensor *src1, THClTensor *src2);
+void THClTensor_cmaxValue(THClState *state, THClTensor *self, THClTensor *src, float value);
+void THClTensor_cminValue(THClState *state, THClTensor *self, THClTensor *src, float value);
+/* comparisons write 1.0f / 0.0f; `self_` is resized to `src` */
+void THClTensor_ltValue(THClState *state, THClTensor *self_, THClTensor *src, float value);
+void THClTensor_gtValue(THClState *state, THClTensor *self_, THClTensor *src, float value);
+void THClTensor_leValue(THClState *state, THClTensor *self_, THClTensor *src, float value);
+void THClTensor_geValue(THClState *state, THClTensor *self_, THClTensor *src, float value);
+void THClTensor_eqValue(THClState *state, THClTensor *self_, THClTensor *src, float value);
+void THClTensor_neValue(THClState *state, THClTensor *self_, THClTensor *src, float value);
+void THClTensor_ltTensor(THClState *state, THClTensor *self_, THClTensor *src1, THClTensor *src2);
+void THClTensor_gtTensor(THClState *state, THClTensor *self_, THClTensor *src1, THClTensor *src2);
+void THClTensor_leTensor(THClState *state, THClTensor *self_, THClTensor *src1, THClTensor *src2);
+void THClTensor_geTensor(THClState *state, THClTensor *self_, THClTensor *src1, THClTensor *src2);
+void THClTensor_eqTensor(THClState *state, THClTensor *self_, THClTensor *src1, THClTensor *src2);
+void THClTensor_neTensor(THClState *state, THClTensor *self_, THClTensor *src1, THClTensor *src2);
+void THClTensor_ltPointTensor(THClState *state, THClTensor *self_, THClTensor *src, THClTensor *value);
+void THClTensor_gtPointTensor(THClState *state, THClTensor *self_, THClTensor *src, THClTensor *value);
+void THClTensor_lePointTensor(THClState *state, THClTensor *self_, THClTensor *src, THClTensor *value);
+void THClTensor_gePointTensor(THClState *state, THClTensor *self_, THClTensor *src, THClTensor *value);
+void THClTensor_eqPointTensor(THClState *state, THClTensor *self_, THClTensor *src, THClTensor *value);
+void THClTensor_nePointTensor(THClState *state, THClTensor *self_, THClTensor *src, THClTensor *value);
+/* tensor[i] = value where mask[i] != 0; mask is a ClTensor of 0 / 1 */
+void THClTensor_maskedFill(THClState *state, THClTensor *tensor, THClTensor *mask, float value);
 
 /* User expressions over x (read-write), y, z -- or *out, *in1, *in2 -- compiled
  * at run time (reference: src/lib/THClTensorMathPointwise.cpp:79-146; Lua names

@@ -1,0 +1,101 @@
+"""CPU restatement of the pointwise operator catalogue: TEST INFRASTRUCTURE.
+
+Each entry follows the operator string the reference compiles
+(src/lib/THClTensorMathPointwise.cpp:39-58,191-319, src/lib/THClTensorMath2.cpp:22-188,
+src/lib/THClTensorMathCompare.cpp:26-82, src/lib/THClTensorMathCompareT.cpp:28-57,
+src/lib/THClTensorMasked.cpp:29-38) evaluated in fp32 with numpy.  Exact
+operators (compare, clamp, sign, round, cmax/cmin, maskedFill, integer powers
+of small integers) are compared bit for bit; the transcendental ones within
+the tolerance the reference's own tests use (src/test/unit_tensor.lua:73-93).
+Pinned in tests/test_oracle.py by special values and identities.
+"""
+import numpy as np
+
+F = np.float32
+
+
+def _f(x):
+    return np.asarray(x, dtype=F)
+
+
+UNARY = {
+    "log1p": np.log1p, "cos": np.cos, "acos": np.arccos, "cosh": np.cosh, "sin": np.sin, "asin": np.arcsin,
+    "sinh": np.sinh, "tan": np.tan, "atan": np.arctan, "exp": np.exp, "log": np.log, "tanh": np.tanh,
+    "floor": np.floor, "ceil": np.ceil, "sqrt": np.sqrt, "abs": np.abs,
+}
+
+
+def unary(name, x):
+    x = _f(x)
+    if name == "round":          # C round(): halves away from zero (numpy's rounds them to even)
+        return np.trunc(x.astype(np.float64) + np.copysign(0.5, x.astype(np.float64))).astype(F)
+    if name == "sign":           # (x > 0) - (x < 0)
+        return ((x > 0).astype(np.int32) - (x < 0).astype(np.int32)).astype(F)
+    with np.errstate(all="ignore"):
+        return UNARY[name](x).astype(F)
+
+
+def pown(x, n: int):
+    """Repeated multiplication in fp32 (square and multiply), 1/x^|n| for negative n."""
+    x = _f(x)
+    r = np.ones_like(x)
+    b = x.copy()
+    e = abs(int(n))
+    with np.errstate(all="ignore"):
+        while e:
+            if e & 1:
+                r = (r * b).astype(F)
+            b = (b * b).astype(F)
+            e >>= 1
+        return (F(1.0) / r).astype(F) if n < 0 else r
+
+
+def pow_value(x, v: float):
+    """src ^ v: integer-valued v goes through pown (src/lib/THClTensorMath2.cpp:28-35)."""
+    if float(int(v)) == float(v):
+        return pown(x, int(v))
+    with np.errstate(all="ignore"):
+        return np.power(_f(x), F(v)).astype(F)
+
+
+def tpow(v: float, x):
+    with np.errstate(all="ignore"):
+        return np.power(F(v), _f(x)).astype(F)
+
+
+def cpow(a, b):
+    with np.errstate(all="ignore"):
+        return np.power(_f(a), _f(b)).astype(F)
+
+
+def clamp(x, lo, hi):
+    """fmax(fmin(x, hi), lo): NaN-ignoring min then max."""
+    return np.fmax(np.fmin(_f(x), F(hi)), F(lo))
+
+
+def atan2(a, b):
+    return np.arctan2(_f(a), _f(b)).astype(F)
+
+
+def cmax(a, b):
+    """OpenCL max(x, y): y if x < y else x."""
+    a, b = _f(a), np.broadcast_to(_f(b), np.shape(a))
+    return np.where(a < b, b, a).astype(F)
+
+
+def cmin(a, b):
+    """OpenCL min(x, y): y if y < x else x."""
+    a, b = _f(a), np.broadcast_to(_f(b), np.shape(a))
+    return np.where(b < a, b, a).astype(F)
+
+
+_REL = {"lt": np.less, "gt": np.greater, "le": np.less_equal, "ge": np.greater_equal, "eq": np.equal, "ne": np.not_equal}
+
+
+def compare(name, a, b):
+    with np.errstate(invalid="ignore"):
+        return _REL[name](_f(a), _f(b)).astype(F)
+
+
+def masked_fill(x, mask, value):
+    return np.where(_f(mask) != 0, F(value), _f(x)).astype(F)

@@ -265,3 +265,37 @@ def test_overlap_rule():
         if oracle.overlapping(sizes, strides) != brute:
             # the rule is conservative: it may report overlap for interleaved but disjoint views
             assert oracle.overlapping(sizes, strides) and not brute
+
+
+# ------------------------------------------------------ operator catalogue pins ---
+def test_catalogue_special_values_and_identities():
+    from oracle import catalogue as cat
+    halves = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 0.49999997, -0.49999997, 2.4, -2.6, 8388609.0], dtype=np.float32)
+    assert cat.unary("round", halves).tolist() == [1, 2, 3, -1, -2, -3, 0, -0.0, 2, -3, 8388609.0]
+    assert cat.unary("sign", [-3.5, -0.0, 0.0, 7.0]).tolist() == [-1, 0, 0, 1]
+    assert np.isnan(cat.unary("sign", [np.nan])[0]) == False and cat.unary("sign", [np.nan])[0] == 0   # both tests false
+    assert cat.pown([2.0, -3.0, 0.5], 3).tolist() == [8.0, -27.0, 0.125]
+    assert cat.pown([2.0, 4.0], -2).tolist() == [0.25, 0.0625]
+    assert cat.pown([5.0], 0).tolist() == [1.0]
+    assert cat.pow_value([2.0, 3.0], 2.0).tolist() == [4.0, 9.0]            # integer-valued exponent: exact
+    assert abs(cat.pow_value([2.0], 0.5)[0] - np.float32(np.sqrt(2.0))) <= np.spacing(np.float32(1.4142135))
+    assert cat.tpow(2.0, [0.0, 1.0, 10.0]).tolist() == [1.0, 2.0, 1024.0]
+    assert cat.cpow([2.0, 9.0], [3.0, 0.5]).tolist() == [8.0, 3.0]
+    assert cat.clamp([-2.0, 0.25, 9.0, np.nan], -1.0, 1.0).tolist() == [-1.0, 0.25, 1.0, 1.0]   # fmin(NaN, hi) = hi, then fmax(hi, lo) = hi
+    assert cat.cmax([1.0, 5.0, -0.0], [2.0, 4.0, 0.0]).tolist() == [2.0, 5.0, -0.0]
+    assert cat.cmin([1.0, 5.0], [2.0, 4.0]).tolist() == [1.0, 4.0]
+    assert cat.cmax([1.0, 5.0], 3.0).tolist() == [3.0, 5.0]
+    a, b = np.array([1.0, 2.0, 3.0, np.nan], dtype=np.float32), np.array([2.0, 2.0, 2.0, 2.0], dtype=np.float32)
+    assert cat.compare("lt", a, b).tolist() == [1, 0, 0, 0] and cat.compare("ge", a, b).tolist() == [0, 1, 1, 0]
+    assert cat.compare("eq", a, b).tolist() == [0, 1, 0, 0] and cat.compare("ne", a, b).tolist() == [1, 0, 1, 1]
+    assert cat.compare("le", a, 2.0).tolist() == [1, 1, 0, 0] and cat.compare("gt", a, 2.0).tolist() == [0, 0, 1, 0]
+    assert cat.masked_fill([1.0, 2.0, 3.0], [0.0, 1.0, -2.0], 9.0).tolist() == [1.0, 9.0, 9.0]
+    # identities that a swapped argument or a wrong function breaks
+    x = np.linspace(-0.9, 0.9, 101).astype(np.float32)
+    assert np.allclose(cat.unary("sin", x) ** 2 + cat.unary("cos", x) ** 2, 1.0, atol=1e-6)
+    assert np.allclose(cat.unary("cosh", x) ** 2 - cat.unary("sinh", x) ** 2, 1.0, atol=1e-5)
+    assert np.allclose(cat.unary("sin", cat.unary("asin", x)), x, atol=1e-6)
+    assert np.allclose(cat.unary("cos", cat.unary("acos", x)), x, atol=1e-6)
+    assert np.allclose(cat.unary("tan", cat.unary("atan", x)), x, atol=1e-6)
+    assert np.allclose(cat.unary("log1p", x), np.log(1.0 + x.astype(np.float64)), atol=1e-6)
+    assert cat.atan2([1.0, -1.0, 0.0], [0.0, 0.0, -1.0]).tolist() == [np.float32(np.pi / 2), np.float32(-np.pi / 2), np.float32(np.pi)]
