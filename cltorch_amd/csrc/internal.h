@@ -111,14 +111,22 @@ std::string thcl_expr_tag(const std::string &rewritten, int ntensors);
 std::string thcl_apply_config_defines();
 
 // ------------------------------------------------------------- reductions ---
-enum ThclReduce : int { RED_SUM = 0, RED_PROD = 1, RED_MAX = 2, RED_MIN = 3 };
+// The first four also run along a dimension with positions (max, min).  The
+// rest are sums / extrema of a modified element: x != 0, |x|, x^2, |x|^p (p in
+// the `exponent` argument), and the truth value (int)x != 0 the reference's
+// all / any reductions use (src/lib/THClTensorMath.cpp:444-458).
+enum ThclReduce : int {
+  RED_SUM = 0, RED_PROD = 1, RED_MAX = 2, RED_MIN = 3,
+  RED_SUM_NE0 = 4, RED_SUM_ABS = 5, RED_SUM_SQ = 6, RED_SUM_POW = 7, RED_ALL = 8, RED_ANY = 9
+};
 // whole tensor -> one float at device address `out`
-void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out);
+void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *src, long dim);
+void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent = 0.f);
 // along `dim`; `values` resized to size 1 along dim; idx outputs optional:
 // idx_f32 = fp32 device buffer of 1-based positions laid out like `values`,
 // idx_i64 = contiguous int64 device buffer.
 void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THClTensor *indices_f32,
-                     int64_t *idx_i64_dev, THClTensor *src, long dim);
+                     int64_t *idx_i64_dev, THClTensor *src, long dim, float exponent = 0.f);
 
 // ------------------------------------------------------------------ gemm ---
 // column-major C[m x n] = alpha * op(A) * op(B) + beta * C on device pointers

@@ -485,7 +485,7 @@ void THLongTensor_copyCl(THClState *state, THLongTensor *self, THClTensor *src) 
 }
 
 // -------------------------------------------------------------- reductions ---
-static float reduce_all_to_host(THClState *state, ThclReduce kind, THClTensor *self) {
+static float reduce_all_to_host(THClState *state, ThclReduce kind, THClTensor *self, float exponent = 0.f) {
   // result lands in the device scratch block, then one word comes back: the
   // only synchronising step (src/lib/THClTensorMath.cpp:346-368)
   THCL_CHECK(self->storage != nullptr || self->nDimension <= 0, "tensor has no storage");
@@ -494,7 +494,7 @@ static float reduce_all_to_host(THClState *state, ThclReduce kind, THClTensor *s
   size_t sb = 0;
   char *scratch = (char *)thcl_rt_scratch(rt, &sb);
   float *dres = (float *)(scratch + sb - 256);  // last 256 bytes of the block are the result slot
-  thcl_reduce_all(state, kind, self, dres);
+  thcl_reduce_all(state, kind, self, dres, exponent);
   float *hw = thcl_rt_host_word(rt);
   THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, dres, sizeof(float)) == 0, "%s", thcl_rt_error());
   return hw[0];
@@ -622,6 +622,62 @@ void THClTensor_maxLong(THClState *state, THClTensor *values, THLongTensor *indi
 void THClTensor_minLong(THClState *state, THClTensor *values, THLongTensor *indices, THClTensor *src, long dim) {
   THCL_GUARD_BEGIN
   arg_reduce_long(state, RED_MIN, values, indices, src, dim);
+  THCL_GUARD_END()
+}
+
+// ---- mean, norms, all / any (src/lib/THClTensorMath2.cpp:190-203,336-417,
+//      src/lib/THClTensorMath.cpp:444-528)
+float THClTensor_meanall(THClState *state, THClTensor *self) {
+  THCL_GUARD_BEGIN
+  THCL_ARGCHECK(self->nDimension > 0, 1, "empty Tensor");
+  return reduce_all_to_host(state, RED_SUM, self) / (float)THClTensor_nElement(state, self);
+  THCL_GUARD_END(0.f)
+}
+void THClTensor_mean(THClState *state, THClTensor *self, THClTensor *src, long dim) {
+  THCL_GUARD_BEGIN
+  THCL_ARGCHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
+  const long len = src->size[dim];
+  thcl_reduce_dim(state, RED_SUM, self, nullptr, nullptr, src, dim);
+  THClTensor_div(state, self, self, (float)len);
+  THCL_GUARD_END()
+}
+static ThclReduce norm_kind(float value) {
+  if (value == 0.0f) return RED_SUM_NE0;   // number of non-zero elements
+  if (value == 1.0f) return RED_SUM_ABS;
+  if (value == 2.0f) return RED_SUM_SQ;
+  return RED_SUM_POW;
+}
+float THClTensor_normall(THClState *state, THClTensor *self, float value) {
+  THCL_GUARD_BEGIN
+  const float sum = reduce_all_to_host(state, norm_kind(value), self, value);
+  if (value == 0.0f) return sum;
+  return (float)std::pow((double)sum, 1.0 / (double)value);
+  THCL_GUARD_END(0.f)
+}
+void THClTensor_norm(THClState *state, THClTensor *self, THClTensor *src, float value, long dimension) {
+  THCL_GUARD_BEGIN
+  thcl_reduce_dim(state, norm_kind(value), self, nullptr, nullptr, src, dimension, value);
+  if (value != 0.0f) THClTensor_pow(state, self, self, 1.0f / value);
+  THCL_GUARD_END()
+}
+int THClTensor_logicalall(THClState *state, THClTensor *self) {
+  THCL_GUARD_BEGIN
+  return (int)reduce_all_to_host(state, RED_ALL, self);
+  THCL_GUARD_END(0)
+}
+int THClTensor_logicalany(THClState *state, THClTensor *self) {
+  THCL_GUARD_BEGIN
+  return (int)reduce_all_to_host(state, RED_ANY, self);
+  THCL_GUARD_END(0)
+}
+void THClTensor_logicalall_gpu(THClState *state, THClTensor *self, THClTensor *src) {
+  THCL_GUARD_BEGIN
+  reduce_all_to_point(state, RED_ALL, self, src);
+  THCL_GUARD_END()
+}
+void THClTensor_logicalany_gpu(THClState *state, THClTensor *self, THClTensor *src) {
+  THCL_GUARD_BEGIN
+  reduce_all_to_point(state, RED_ANY, self, src);
   THCL_GUARD_END()
 }
 

@@ -39,7 +39,7 @@ template <>
 struct Acc<RED_SUM> {
   typedef double T;
   static __device__ __forceinline__ T init() { return 0.0; }
-  static __device__ __forceinline__ T lift(float x) { return (double)x; }
+  static __device__ __forceinline__ T lift(float x, float) { return (double)x; }
   static __device__ __forceinline__ T comb(T a, T b) { return a + b; }
   static __device__ __forceinline__ float lower(T a) { return (float)a; }
 };
@@ -47,7 +47,7 @@ template <>
 struct Acc<RED_PROD> {
   typedef double T;
   static __device__ __forceinline__ T init() { return 1.0; }
-  static __device__ __forceinline__ T lift(float x) { return (double)x; }
+  static __device__ __forceinline__ T lift(float x, float) { return (double)x; }
   static __device__ __forceinline__ T comb(T a, T b) { return a * b; }
   static __device__ __forceinline__ float lower(T a) { return (float)a; }
 };
@@ -55,7 +55,7 @@ template <>
 struct Acc<RED_MAX> {
   typedef float T;
   static __device__ __forceinline__ T init() { return -INFINITY; }
-  static __device__ __forceinline__ T lift(float x) { return x; }
+  static __device__ __forceinline__ T lift(float x, float) { return x; }
   // NaN on either side gives NaN
   static __device__ __forceinline__ T comb(T a, T b) { return ((b > a) | (b != b)) ? b : a; }
   static __device__ __forceinline__ float lower(T a) { return a; }
@@ -64,8 +64,49 @@ template <>
 struct Acc<RED_MIN> {
   typedef float T;
   static __device__ __forceinline__ T init() { return INFINITY; }
-  static __device__ __forceinline__ T lift(float x) { return x; }
+  static __device__ __forceinline__ T lift(float x, float) { return x; }
   static __device__ __forceinline__ T comb(T a, T b) { return ((b < a) | (b != b)) ? b : a; }
+  static __device__ __forceinline__ float lower(T a) { return a; }
+};
+
+// Sums of a modified element (fp64 like every sum), and the all / any truth
+// reductions as min / max over 0 / 1.
+struct AccSum {
+  typedef double T;
+  static __device__ __forceinline__ T init() { return 0.0; }
+  static __device__ __forceinline__ T comb(T a, T b) { return a + b; }
+  static __device__ __forceinline__ float lower(T a) { return (float)a; }
+};
+template <>
+struct Acc<RED_SUM_NE0> : AccSum {
+  static __device__ __forceinline__ T lift(float x, float) { return x != 0.0f ? 1.0 : 0.0; }
+};
+template <>
+struct Acc<RED_SUM_ABS> : AccSum {
+  static __device__ __forceinline__ T lift(float x, float) { return (double)fabsf(x); }
+};
+template <>
+struct Acc<RED_SUM_SQ> : AccSum {
+  static __device__ __forceinline__ T lift(float x, float) { return (double)x * (double)x; }
+};
+template <>
+struct Acc<RED_SUM_POW> : AccSum {
+  static __device__ __forceinline__ T lift(float x, float e) { return pow(fabs((double)x), (double)e); }
+};
+template <>
+struct Acc<RED_ALL> {
+  typedef float T;
+  static __device__ __forceinline__ T init() { return 1.0f; }
+  static __device__ __forceinline__ T lift(float x, float) { return (int)x != 0 ? 1.0f : 0.0f; }
+  static __device__ __forceinline__ T comb(T a, T b) { return fminf(a, b); }
+  static __device__ __forceinline__ float lower(T a) { return a; }
+};
+template <>
+struct Acc<RED_ANY> {
+  typedef float T;
+  static __device__ __forceinline__ T init() { return 0.0f; }
+  static __device__ __forceinline__ T lift(float x, float) { return (int)x != 0 ? 1.0f : 0.0f; }
+  static __device__ __forceinline__ T comb(T a, T b) { return fmaxf(a, b); }
   static __device__ __forceinline__ float lower(T a) { return a; }
 };
 
@@ -172,6 +213,7 @@ struct ReduceAllParams {
   void *partials;
   unsigned *ticket;
   float *out;
+  float exponent;        // p of the |x|^p sum
   ThclGenericOperand L;  // strided input only
 };
 
@@ -243,15 +285,15 @@ __global__ __launch_bounds__(kThreads) void reduce_all_dense(ReduceAllParams P) 
       const thcl_u64 i = base + (thcl_u64)k * kThreads;
       if (i < n4) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) acc[k] = Acc<KIND>::comb(acc[k], Acc<KIND>::lift(v[k][c]));
+        for (int c = 0; c < 4; c++) acc[k] = Acc<KIND>::comb(acc[k], Acc<KIND>::lift(v[k][c], P.exponent));
       }
     }
   }
   if (blockIdx.x == 0) {
     const thcl_u64 tail0 = head + (n4 << 2);
-    for (thcl_u64 i = threadIdx.x; i < head; i += kThreads) acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i]));
+    for (thcl_u64 i = threadIdx.x; i < head; i += kThreads) acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i], P.exponent));
     for (thcl_u64 i = tail0 + threadIdx.x; i < P.n; i += kThreads)
-      acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i]));
+      acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i], P.exponent));
   }
   T v = Acc<KIND>::comb(Acc<KIND>::comb(acc[0], acc[1]), Acc<KIND>::comb(acc[2], acc[3]));
   v = block_reduce<KIND, T>(v, lds);
@@ -264,7 +306,7 @@ __global__ __launch_bounds__(kThreads) void reduce_all_strided(ReduceAllParams P
   __shared__ T lds[kThreads / kWave];
   T acc = Acc<KIND>::init();
   for (thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x; i < P.n; i += (thcl_u64)gridDim.x * kThreads)
-    acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(P.in[thcl_generic_offset((thcl_u32)i, P.L)]));
+    acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(P.in[thcl_generic_offset((thcl_u32)i, P.L)], P.exponent));
   acc = block_reduce<KIND, T>(acc, lds);
   finish_all<KIND>(acc, P, lds);
 }
@@ -284,6 +326,7 @@ struct ReduceDimParams {
   thcl_u32 split;        // blocks sharing one slice's reduction (column kernel)
   thcl_u32 fused;        // split > 1: the last block of a tile folds its partials (else a second kernel does)
   thcl_u32 rows_per_split;
+  float exponent;        // p of the |x|^p sum
   ThclGenericOperand L;  // layout of the slice starts (the view without `dim`)
 };
 
@@ -293,7 +336,7 @@ template <int KIND>
 struct Slot<KIND, false> {
   typedef typename Acc<KIND>::T T;
   static __device__ __forceinline__ T init() { return Acc<KIND>::init(); }
-  static __device__ __forceinline__ T take(T cur, float x, int) { return Acc<KIND>::comb(cur, Acc<KIND>::lift(x)); }
+  static __device__ __forceinline__ T take(T cur, float x, int, float e) { return Acc<KIND>::comb(cur, Acc<KIND>::lift(x, e)); }
   static __device__ __forceinline__ T seal(T acc, int, bool) { return acc; }
   static __device__ __forceinline__ T comb(T a, T b) { return Acc<KIND>::comb(a, b); }
   static __device__ __forceinline__ T reduce(T v, int width) { return group_reduce<KIND, T>(v, width); }
@@ -307,7 +350,7 @@ struct Slot<KIND, true> {
   // !(x <= cur) (max) unless cur is already NaN.  Five instructions where the
   // order-free rule takes ten; an element equal to the start value is never
   // taken, which seal() repairs.
-  static __device__ __forceinline__ T take(T cur, float x, int i) {
+  static __device__ __forceinline__ T take(T cur, float x, int i, float) {
     const bool beats = (KIND == RED_MAX) ? !(x <= cur.v) : !(x >= cur.v);
     const bool take = beats & (cur.v == cur.v);
     VI r;
@@ -357,12 +400,12 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
 #pragma unroll
           for (int f = 0; f < FLY; f++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) acc = S::take(acc, v[f][c], (int)((i + f * LPR) * 4 + c));
+            for (int c = 0; c < 4; c++) acc = S::take(acc, v[f][c], (int)((i + f * LPR) * 4 + c), P.exponent);
         }
         for (; i < r4; i += LPR) {
           const thcl_f4 v = __builtin_nontemporal_load(row4 + i);
 #pragma unroll
-          for (int c = 0; c < 4; c++) acc = S::take(acc, v[c], (int)(i * 4 + c));
+          for (int c = 0; c < 4; c++) acc = S::take(acc, v[c], (int)(i * 4 + c), P.exponent);
         }
       } else {
         constexpr int FLY = 4;
@@ -372,9 +415,9 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
 #pragma unroll
           for (int f = 0; f < FLY; f++) v[f] = row[i + f * LPR];
 #pragma unroll
-          for (int f = 0; f < FLY; f++) acc = S::take(acc, v[f], (int)(i + f * LPR));
+          for (int f = 0; f < FLY; f++) acc = S::take(acc, v[f], (int)(i + f * LPR), P.exponent);
         }
-        for (; i < P.R; i += LPR) acc = S::take(acc, row[i], (int)i);
+        for (; i < P.R; i += LPR) acc = S::take(acc, row[i], (int)i, P.exponent);
       }
       // the first position this thread met
       acc = S::seal(acc, (int)(VEC == 4 ? sub * 4 : sub), (VEC == 4 ? (thcl_u32)sub < (P.R >> 2) : (thcl_u32)sub < P.R));
@@ -447,7 +490,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
 #pragma unroll
           for (int f = 0; f < FLY; f++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v[f][c], (int)(r + f * WAVES));
+            for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v[f][c], (int)(r + f * WAVES), P.exponent);
         } else {
           float v[FLY];
 #pragma unroll
@@ -456,16 +499,16 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
             ptr += step;
           }
 #pragma unroll
-          for (int f = 0; f < FLY; f++) acc[0] = S::take(acc[0], v[f], (int)(r + f * WAVES));
+          for (int f = 0; f < FLY; f++) acc[0] = S::take(acc[0], v[f], (int)(r + f * WAVES), P.exponent);
         }
       }
       for (; r < r_end; r += WAVES) {
         if (VEC == 4) {
           const thcl_f4 v0 = *(const thcl_f4 *)ptr;
 #pragma unroll
-          for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v0[c], (int)r);
+          for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v0[c], (int)r, P.exponent);
         } else {
-          acc[0] = S::take(acc[0], *ptr, (int)r);
+          acc[0] = S::take(acc[0], *ptr, (int)r, P.exponent);
         }
         ptr += step;
       }
@@ -564,10 +607,11 @@ void fill_operand(ThclGenericOperand &o, const Layout &L) {
 
 float init_value(ThclReduce kind) {
   switch (kind) {
-    case RED_SUM: return 0.f;
     case RED_PROD: return 1.f;
+    case RED_ALL: return 1.f;
     case RED_MAX: return -INFINITY;
-    default: return INFINITY;
+    case RED_MIN: return INFINITY;
+    default: return 0.f;  // every sum, and any
   }
 }
 
@@ -606,7 +650,7 @@ bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 }  // namespace
 
 // ----------------------------------------------------------------- reduce all
-void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out) {
+void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent) {
   const long n = THClTensor_nElement(state, src);
   THCL_CHECK(src->nDimension <= THCL_MAX_DIMS, THCL_DIM_WARNING);
   int device = THClTensor_getDevice(state, src);
@@ -627,6 +671,7 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
   P.partials = scratch + kPartialOff;
   P.ticket = (unsigned *)(scratch + kTicketOff);
   P.out = out;
+  P.exponent = exponent;
   const bool dense = THClTensor_isContiguous(state, src);
   const int cus = thcl_rt_get_props(rt)->compute_units;
   long want;
@@ -646,6 +691,12 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
     case RED_PROD: launch_all<RED_PROD>(dense, grid, stream, P); break;
     case RED_MAX: launch_all<RED_MAX>(dense, grid, stream, P); break;
     case RED_MIN: launch_all<RED_MIN>(dense, grid, stream, P); break;
+    case RED_SUM_NE0: launch_all<RED_SUM_NE0>(dense, grid, stream, P); break;
+    case RED_SUM_ABS: launch_all<RED_SUM_ABS>(dense, grid, stream, P); break;
+    case RED_SUM_SQ: launch_all<RED_SUM_SQ>(dense, grid, stream, P); break;
+    case RED_SUM_POW: launch_all<RED_SUM_POW>(dense, grid, stream, P); break;
+    case RED_ALL: launch_all<RED_ALL>(dense, grid, stream, P); break;
+    case RED_ANY: launch_all<RED_ANY>(dense, grid, stream, P); break;
   }
   check_launch("reduce-all");
   thcl_after_launch(state, rt);
@@ -653,7 +704,7 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
 
 // ------------------------------------------------------------ reduce along dim
 void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THClTensor *indices_f32,
-                     int64_t *idx_i64_dev, THClTensor *src, long dim) {
+                     int64_t *idx_i64_dev, THClTensor *src, long dim, float exponent) {
   thcl_check_same_device(state, 3, values, indices_f32, src);
   THCL_CHECK(src->nDimension <= THCL_MAX_DIMS, THCL_DIM_WARNING);
   if (src->nDimension <= 0) return;  // nothing to reduce (src/lib/THClReduce.cpp:234-237)
@@ -708,6 +759,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   P.rstride = (thcl_u32)src->stride[dim];
   P.split = 1;
   P.rows_per_split = P.R;
+  P.exponent = exponent;
   Layout L = thcl_collapse(src, (int)dim);
   fill_operand(P.L, L);
 
@@ -768,12 +820,26 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     else launch_finish<K, false>(fg, stream, P);                          \
     check_launch("reduce-dim finish");                                    \
   }
+#define DISPATCH_VALUES(K)                                                \
+  launch_dim<K, false>(rows, lpr, vec, grid, stream, P);                  \
+  check_launch("reduce-dim");                                             \
+  if (!rows && P.split > 1 && !P.fused) {                                 \
+    unsigned fg = (unsigned)((nslices + kFinSlices - 1) / kFinSlices);    \
+    launch_finish<K, false>(fg, stream, P);                               \
+    check_launch("reduce-dim finish");                                    \
+  }
   switch (kind) {
     case RED_SUM: DISPATCH(RED_SUM) break;
     case RED_PROD: DISPATCH(RED_PROD) break;
     case RED_MAX: DISPATCH(RED_MAX) break;
     case RED_MIN: DISPATCH(RED_MIN) break;
+    case RED_SUM_NE0: DISPATCH_VALUES(RED_SUM_NE0) break;
+    case RED_SUM_ABS: DISPATCH_VALUES(RED_SUM_ABS) break;
+    case RED_SUM_SQ: DISPATCH_VALUES(RED_SUM_SQ) break;
+    case RED_SUM_POW: DISPATCH_VALUES(RED_SUM_POW) break;
+    default: thcl_throw("internal: reduction kind %d does not run along a dimension", (int)kind);
   }
+#undef DISPATCH_VALUES
 #undef DISPATCH
   thcl_after_launch(state, rt);
   if (vdense != values) THClTensor_freeCopyTo(state, vdense, values);

@@ -1,0 +1,276 @@
+// Inclusive scans along one dimension: cumsum, cumprod.
+//
+// What it replaces (reference): THClTensor_scanDim and its two kernels
+// (src/lib/THClTensorMathScan.cpp:27-156, THClTensorMathScan.cl), which walk
+// every row with one thread (outer dims) or 16 threads (innermost dim).
+//
+// The tensor is taken as dense [O][R][I] (outer, scanned, inner).  Numerics
+// follow Torch7's CPU path: the running value is fp64 and every output is its
+// rounding to fp32.  Two kernels:
+//   * scan_seq: one thread per (o, i) walks r; adjacent threads are adjacent in
+//     i, so accesses coalesce whenever I is not tiny.  Also serves short
+//     innermost scans.
+//   * scan_row: I == 1 and long rows; a block walks the row 1024 elements at a
+//     time with a block-wide fp64 prefix in each step.
+// When O * I alone cannot fill the chip, R is cut into S segments and the scan
+// becomes three passes: segment totals, an exclusive scan of the totals, then
+// the scan proper with each segment's carry-in.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "apply_device.h"
+#include "internal.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWave = 64;
+
+struct ScanParams {
+  const float *in;
+  float *out;
+  double *totals;  // [O][S][I]: segment totals, turned into carries in place
+  thcl_u64 O, R, I;
+  thcl_u64 S, seg;  // segments per scanned line and their length
+};
+
+template <bool PROD>
+struct Op {
+  static __device__ __forceinline__ double identity() { return PROD ? 1.0 : 0.0; }
+  static __device__ __forceinline__ double comb(double a, double b) { return PROD ? a * b : a + b; }
+};
+
+// PHASE 0: segment totals only.  PHASE 1: the scan, seeded with the carry when S > 1.
+template <bool PROD, int PHASE>
+__global__ __launch_bounds__(kThreads) void scan_seq(ScanParams P) {
+  const thcl_u64 t = (thcl_u64)blockIdx.x * kThreads + threadIdx.x;
+  if (t >= P.O * P.S * P.I) return;
+  const thcl_u64 i = t % P.I, s = (t / P.I) % P.S, o = t / (P.I * P.S);
+  const thcl_u64 r0 = s * P.seg;
+  thcl_u64 r1 = r0 + P.seg;
+  if (r1 > P.R) r1 = P.R;
+  const thcl_u64 first = (o * P.R + r0) * P.I + i;
+  const float *src = P.in + first;
+  float *dst = P.out + first;
+  double acc = Op<PROD>::identity();
+  if (PHASE == 1 && P.S > 1) acc = P.totals[t];
+  constexpr int FLY = 8;  // independent loads in flight per thread
+  thcl_u64 r = r0;
+  for (; r + FLY <= r1; r += FLY) {
+    float v[FLY];
+#pragma unroll
+    for (int k = 0; k < FLY; k++) v[k] = __builtin_nontemporal_load(src + (thcl_u64)k * P.I);
+    src += (thcl_u64)FLY * P.I;
+#pragma unroll
+    for (int k = 0; k < FLY; k++) {
+      acc = Op<PROD>::comb(acc, (double)v[k]);
+      if (PHASE == 1) __builtin_nontemporal_store((float)acc, dst + (thcl_u64)k * P.I);
+    }
+    if (PHASE == 1) dst += (thcl_u64)FLY * P.I;
+  }
+  for (; r < r1; r++) {
+    acc = Op<PROD>::comb(acc, (double)*src);
+    src += P.I;
+    if (PHASE == 1) {
+      *dst = (float)acc;
+      dst += P.I;
+    }
+  }
+  if (PHASE == 0) P.totals[t] = acc;
+}
+
+// totals[o][s][i] -> combination of totals[o][0..s-1][i] (exclusive), one thread per (o, i)
+template <bool PROD>
+__global__ __launch_bounds__(kThreads) void scan_carries(ScanParams P) {
+  const thcl_u64 t = (thcl_u64)blockIdx.x * kThreads + threadIdx.x;
+  if (t >= P.O * P.I) return;
+  const thcl_u64 i = t % P.I, o = t / P.I;
+  double *p = P.totals + o * P.S * P.I + i;
+  double acc = Op<PROD>::identity();
+  for (thcl_u64 s = 0; s < P.S; s++) {
+    const double v = *p;
+    *p = acc;
+    acc = Op<PROD>::comb(acc, v);
+    p += P.I;
+  }
+}
+
+template <bool PROD>
+__device__ __forceinline__ double wave_inclusive(double v) {
+  const int lane = threadIdx.x % kWave;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const double up = __shfl_up(v, d, kWave);
+    if (lane >= d) v = Op<PROD>::comb(up, v);
+  }
+  return v;
+}
+
+// I == 1: block (o, s) walks its segment of row o, 4 consecutive elements per thread per step.
+template <bool PROD, int PHASE, bool VEC>
+__global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
+  constexpr int WAVES = kThreads / kWave, PER = 4, STEP = kThreads * PER;
+  __shared__ double wave_tot[WAVES];
+  const thcl_u64 o = blockIdx.x / P.S, s = blockIdx.x % P.S;
+  const thcl_u64 r0 = s * P.seg;
+  thcl_u64 r1 = r0 + P.seg;
+  if (r1 > P.R) r1 = P.R;
+  const float *row = P.in + o * P.R;
+  float *orow = P.out + o * P.R;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  double carry = Op<PROD>::identity();
+  if (PHASE == 1 && P.S > 1) carry = P.totals[blockIdx.x];
+  for (thcl_u64 base = r0; base < r1; base += STEP) {
+    const thcl_u64 j = base + (thcl_u64)threadIdx.x * PER;
+    float x[PER];
+    if (VEC && j + PER <= r1) {
+      const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
+#pragma unroll
+      for (int c = 0; c < PER; c++) x[c] = v[c];
+    } else {
+#pragma unroll
+      for (int c = 0; c < PER; c++) x[c] = (j + c < r1) ? row[j + c] : (PROD ? 1.0f : 0.0f);
+    }
+    double a[PER];
+    a[0] = (double)x[0];
+#pragma unroll
+    for (int c = 1; c < PER; c++) a[c] = Op<PROD>::comb(a[c - 1], (double)x[c]);
+    const double incl = wave_inclusive<PROD>(a[PER - 1]);
+    __syncthreads();  // wave_tot of the previous step has been read
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    double before = carry;  // everything ahead of this thread's first element
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) {
+      if (w < wave) before = Op<PROD>::comb(before, wave_tot[w]);
+      carry = Op<PROD>::comb(carry, wave_tot[w]);
+    }
+    if (PHASE == 1) {
+      // lanes ahead in this wave: the exclusive prefix is the neighbour's inclusive one
+      const double prev = __shfl_up(incl, 1, kWave);
+      if (lane > 0) before = Op<PROD>::comb(before, prev);
+      if (VEC && j + PER <= r1) {
+        thcl_f4 v;
+#pragma unroll
+        for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[c]);
+        __builtin_nontemporal_store(v, (thcl_f4 *)(orow + j));
+      } else {
+#pragma unroll
+        for (int c = 0; c < PER; c++)
+          if (j + c < r1) orow[j + c] = (float)Op<PROD>::comb(before, a[c]);
+      }
+    }
+  }
+  if (PHASE == 0 && threadIdx.x == 0) P.totals[blockIdx.x] = carry;
+}
+
+void check(const char *what) {
+  hipError_t e = hipGetLastError();
+  THCL_CHECK(e == hipSuccess, "%s launch failed: %s", what, hipGetErrorString(e));
+}
+
+template <bool PROD>
+void run_scan(hipStream_t stream, ScanParams &P, bool rows, bool vec) {
+  if (rows) {
+    const dim3 grid((unsigned)(P.O * P.S)), block(kThreads);
+    if (P.S > 1) {
+      if (vec) hipLaunchKernelGGL((scan_row<PROD, 0, true>), grid, block, 0, stream, P);
+      else hipLaunchKernelGGL((scan_row<PROD, 0, false>), grid, block, 0, stream, P);
+      check("scan totals");
+      hipLaunchKernelGGL((scan_carries<PROD>), dim3((unsigned)((P.O + kThreads - 1) / kThreads)), block, 0, stream, P);
+      check("scan carries");
+    }
+    if (vec) hipLaunchKernelGGL((scan_row<PROD, 1, true>), grid, block, 0, stream, P);
+    else hipLaunchKernelGGL((scan_row<PROD, 1, false>), grid, block, 0, stream, P);
+    check("scan");
+  } else {
+    const thcl_u64 threads = P.O * P.S * P.I;
+    const dim3 grid((unsigned)((threads + kThreads - 1) / kThreads)), block(kThreads);
+    if (P.S > 1) {
+      hipLaunchKernelGGL((scan_seq<PROD, 0>), grid, block, 0, stream, P);
+      check("scan totals");
+      hipLaunchKernelGGL((scan_carries<PROD>), dim3((unsigned)((P.O * P.I + kThreads - 1) / kThreads)), block, 0, stream,
+                         P);
+      check("scan carries");
+    }
+    hipLaunchKernelGGL((scan_seq<PROD, 1>), grid, block, 0, stream, P);
+    check("scan");
+  }
+}
+}  // namespace
+
+// self = inclusive scan of src along `dim` (0-based).  Operands that are not
+// dense go through dense stand-ins, as in the reference
+// (src/lib/THClTensorMathScan.cpp:127-142).
+void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *src, long dim) {
+  thcl_check_same_device(state, 2, self, src);
+  THCL_ARGCHECK(src->nDimension > 0, 2, "cannot scan an empty tensor");
+  THCL_ARGCHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
+  THClTensor *srcc = THClTensor_newContiguous(state, src);  // before resizing self: they may be the same tensor
+  THClTensor_resizeAs(state, self, src);
+  THClTensor *selfc = self;
+  if (!THClTensor_isContiguous(state, self)) {
+    selfc = THClTensor_newv2(state, THClTensor_getDevice(state, self));
+    THClTensor_resizeAs(state, selfc, self);
+  }
+  thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, src));
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+
+  ScanParams P;
+  memset(&P, 0, sizeof(P));
+  P.in = thcl_dptr(srcc);
+  P.out = thcl_dptr(selfc);
+  P.O = P.I = 1;
+  for (int d = 0; d < dim; d++) P.O *= (thcl_u64)src->size[d];
+  for (int d = (int)dim + 1; d < src->nDimension; d++) P.I *= (thcl_u64)src->size[d];
+  P.R = (thcl_u64)src->size[dim];
+  const thcl_u64 total = P.O * P.R * P.I;
+  if (total > 0) {
+    const long cus = thcl_rt_get_props(rt)->compute_units;
+    const bool rows = (P.I == 1 && P.R >= 1024);
+    // cut R into segments until the launch fills the chip; a segment keeps
+    // enough elements to amortise the extra pass
+    thcl_u64 S = 1;
+    if (rows) {
+      const thcl_u64 want = (thcl_u64)cus * 8;  // blocks
+      if (P.O < want) S = (want + P.O - 1) / P.O;
+      const thcl_u64 most = P.R / 4096;
+      if (S > most) S = most;
+    } else {
+      const thcl_u64 want = (thcl_u64)cus * 512;  // threads
+      if (P.O * P.I < want) S = (want + P.O * P.I - 1) / (P.O * P.I);
+      const thcl_u64 most = P.R / 32;
+      if (S > most) S = most;
+    }
+    if (S < 1) S = 1;
+    thcl_u64 seg = (P.R + S - 1) / S;
+    if (rows) seg = (seg + 1023) / 1024 * 1024;  // whole steps, so vector accesses stay aligned
+    S = (P.R + seg - 1) / seg;
+    P.S = S;
+    P.seg = seg;
+    THCL_CHECK(P.O * P.S < (1ull << 31) && (P.O * P.S * P.I + kThreads - 1) / kThreads < (1ull << 31), THCL_DIM_WARNING);
+    if (S > 1) P.totals = (double *)thcl_rt_workspace(rt, (size_t)(P.O * P.S * P.I) * sizeof(double));
+    THCL_CHECK(S == 1 || P.totals != nullptr, "%s", thcl_rt_error());
+    const bool vec = rows && (P.R % 4 == 0) && ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
+    if (prod) run_scan<true>(stream, P, rows, vec);
+    else run_scan<false>(stream, P, rows, vec);
+    thcl_after_launch(state, rt);
+  }
+  THClTensor_free(state, srcc);
+  if (selfc != self) THClTensor_freeCopyTo(state, selfc, self);
+}
+
+extern "C" {
+// (src/lib/THClTensorMathScan.cpp:144-156)
+void THClTensor_cumsum(THClState *state, THClTensor *self, THClTensor *src, long dim) {
+  THCL_GUARD_BEGIN
+  thcl_scan_dim(state, false, self, src, dim);
+  THCL_GUARD_END()
+}
+void THClTensor_cumprod(THClState *state, THClTensor *self, THClTensor *src, long dim) {
+  THCL_GUARD_BEGIN
+  thcl_scan_dim(state, true, self, src, dim);
+  THCL_GUARD_END()
+}
+}

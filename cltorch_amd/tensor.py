@@ -462,6 +462,51 @@ class ClTensor:
             return res
         return self._reduce("prod", args)
 
+    def _scan(self, name: str, args):
+        """``a:cumsum()`` / ``a:cumsum(dim)`` -> new tensor (dim defaults to 1); ``res:cumsum(a, dim)``
+        (``src/TensorMath.lua:955-961``)."""
+        if len(args) >= 1 and isinstance(args[0], ClTensor):
+            res, src, dim = self, args[0], (args[1] if len(args) > 1 else 1)
+        else:
+            res, src, dim = ClTensor(), self, (args[0] if args else 1)
+        _call(f"THClTensor_{name}", res._h, src._h, C.c_long(dim - 1))
+        return res
+
+    def cumsum(self, *args):
+        return self._scan("cumsum", args)
+
+    def cumprod(self, *args):
+        return self._scan("cumprod", args)
+
+    def mean(self, *args):
+        """``a:mean()`` -> number, ``a:mean(dim)`` -> new tensor (``src/TensorMath.lua:1104-1111``)."""
+        if len(args) == 0:
+            return float(_call("THClTensor_meanall", self._h))
+        res = ClTensor()
+        _call("THClTensor_mean", res._h, self._h, C.c_long(args[0] - 1))
+        return res
+
+    def norm(self, *args):
+        """``a:norm()``, ``a:norm(p)`` -> number; ``a:norm(p, dim)`` -> new tensor."""
+        if len(args) <= 1:
+            return float(_call("THClTensor_normall", self._h, C.c_float(args[0] if args else 2.0)))
+        res = ClTensor()
+        _call("THClTensor_norm", res._h, self._h, C.c_float(args[0]), C.c_long(args[1] - 1))
+        return res
+
+    def _logical(self, name: str, args):
+        if len(args) == 0:
+            return bool(_call(f"THClTensor_logical{name}", self._h))
+        _call(f"THClTensor_logical{name}_gpu", self._h, args[0]._h)
+        return self
+
+    def all(self, *args):
+        """``a:all()`` -> boolean; ``res:all(a)`` leaves 1 / 0 in the point tensor res."""
+        return self._logical("all", args)
+
+    def any(self, *args):
+        return self._logical("any", args)
+
     def _minmax(self, name: str, args):
         if len(args) == 1 and not isinstance(args[0], ClTensor):
             values, indices = ClTensor(), ClTensor()

@@ -362,6 +362,25 @@ void THClTensor_min(THClState *state, THClTensor *values, THClTensor *indices, T
 void THClTensor_maxLong(THClState *state, THClTensor *values, THLongTensor *indices, THClTensor *src, long dim);
 void THClTensor_minLong(THClState *state, THClTensor *values, THLongTensor *indices, THClTensor *src, long dim);
 
+/* mean = sum / count; norms: value 0 counts non-zero elements, otherwise
+ * (sum |x|^value)^(1/value), accumulated in fp64 like every sum here; all / any
+ * take (int)x != 0 as an element's truth value
+ * (reference: src/lib/THClTensorMath.h:86-96,125-126,138-139) */
+float THClTensor_meanall(THClState *state, THClTensor *self);
+void THClTensor_mean(THClState *state, THClTensor *self, THClTensor *src, long dim);
+float THClTensor_normall(THClState *state, THClTensor *self, float value);
+void THClTensor_norm(THClState *state, THClTensor *self, THClTensor *src, float value, long dimension);
+int THClTensor_logicalall(THClState *state, THClTensor *self);
+int THClTensor_logicalany(THClState *state, THClTensor *self);
+void THClTensor_logicalall_gpu(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_logicalany_gpu(THClState *state, THClTensor *self, THClTensor *src);
+
+/* inclusive running sum / product along `dim` (0-based); the running value is
+ * fp64, each output its rounding to fp32
+ * (reference: src/lib/THClTensorMath.h:36-37, src/lib/THClTensorMathScan.cpp:127-156) */
+void THClTensor_cumsum(THClState *state, THClTensor *self, THClTensor *src, long dim);
+void THClTensor_cumprod(THClState *state, THClTensor *self, THClTensor *src, long dim);
+
 /* ------------------------------------------------------------------------- */
 /* Dense contraction (reference: src/lib/THClTensorMath.h:47, THClBlas.h:42)  */
 /* ------------------------------------------------------------------------- */

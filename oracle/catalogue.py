@@ -99,3 +99,28 @@ def compare(name, a, b):
 
 def masked_fill(x, mask, value):
     return np.where(_f(mask) != 0, F(value), _f(x)).astype(F)
+
+
+# ------------------------------------------------------------- reductions / scans ---
+def cumulate(x, axis: int, prod: bool = False):
+    """Torch7's CPU cumsum / cumprod: a sequential fp64 running value, every
+    output its rounding to fp32 (numpy's cumsum / cumprod on float64 run sequentially)."""
+    x64 = np.asarray(x, dtype=np.float64)
+    with np.errstate(all="ignore"):
+        return (np.cumprod(x64, axis=axis) if prod else np.cumsum(x64, axis=axis)).astype(F)
+
+
+def norm(x, p: float, axis=None):
+    """p == 0 counts non-zero elements; otherwise (sum |x|^p)^(1/p) with fp64
+    accumulation (TH's accreal), rounded to fp32 once per output."""
+    x64 = np.abs(np.asarray(x, dtype=np.float64))
+    keep = axis is not None
+    if p == 0:
+        return (x64 != 0).sum(axis=axis, keepdims=keep).astype(F)
+    return np.power(np.power(x64, p).sum(axis=axis, keepdims=keep), 1.0 / p).astype(F)
+
+
+def truth(x):
+    """Element truth value of the reference's all / any reductions: (int)x != 0,
+    i.e. truncation toward zero (src/lib/THClTensorMath.cpp:444-458)."""
+    return np.trunc(_f(x)) != 0

@@ -1,0 +1,122 @@
+"""cumsum / cumprod, mean, norms and all / any through the C ABI against
+oracle/catalogue.py (Torch7 CPU semantics: fp64 running values).  Scans: the
+device combines fp64 partial results in a different order than the sequential
+oracle, so an output may land on the neighbouring fp32 value when the fp64
+result sits within 1e-16 of a rounding boundary: the bar is <= 1 ulp everywhere
+and bit-equality for at least 99.99 % of the elements."""
+import numpy as np
+import pytest
+
+import oracle
+from oracle import catalogue as cat
+from gpu_util import Pair, assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+def _scan_close(got, want, what):
+    assert got.shape == want.shape, what
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.mean() >= 0.9999, f"{what}: only {same.mean():.6f} bit-equal"
+    bad = ~same
+    if bad.any():
+        assert np.all(np.abs(got[bad] - want[bad]) <= np.spacing(np.abs(want[bad]))), f"{what}: more than 1 ulp"
+
+
+SHAPES = [(1,), (5,), (1023,), (1024,), (4099,), (300000,), (7, 5), (3, 2000), (2000, 3), (64, 4096), (33, 70, 9),
+          (4, 300, 128), (2, 3, 4, 5), (1, 50000), (50000, 1), (6, 1 << 16)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_cumsum_every_dim(cl, shape):
+    x = oracle.uniform(61, int(np.prod(shape))).reshape(shape)
+    X = cl.ClTensor(x)
+    for d in range(len(shape)):
+        _scan_close(X.cumsum(d + 1).float(), cat.cumulate(x, d), f"cumsum {shape} dim {d + 1}")
+
+
+@pytest.mark.parametrize("shape", [(37,), (5000,), (40, 300), (300, 40), (9, 33, 17)])
+def test_cumprod_every_dim(cl, shape):
+    x = oracle.uniform(62, int(np.prod(shape)), 0.9, 1.1)
+    x[::7] *= -1
+    x = x.reshape(shape)
+    X = cl.ClTensor(x)
+    for d in range(len(shape)):
+        _scan_close(X.cumprod(d + 1).float(), cat.cumulate(x, d, prod=True), f"cumprod {shape} dim {d + 1}")
+
+
+def test_scan_closed_forms_views_and_in_place(cl):
+    n = 1 << 22                                             # long row: segments + carries
+    ones = cl.ClTensor(n)
+    ones.fill(1.0)
+    got = ones.cumsum().float()
+    assert np.array_equal(got, np.arange(1, n + 1, dtype=np.float64).astype(F))   # exact: fp64 running value
+    big = cl.ClTensor(np.array([16777216.0, 1.0, 1.0, 1.0], dtype=F))
+    assert big.cumsum().float().tolist() == [16777216.0, 16777216.0, 16777218.0, 16777220.0]
+    twos = cl.ClTensor(30)
+    twos.fill(2.0)
+    assert np.array_equal(twos.cumprod().float(), (2.0 ** np.arange(1, 31)).astype(F))
+    # strided source and destination
+    x = oracle.uniform(63, 60 * 50).reshape(60, 50)
+    p = Pair.dense(cl, x).transpose(0, 1)
+    for d in (0, 1):
+        _scan_close(p.dev.cumsum(d + 1).float(), cat.cumulate(p.view.gather(), d), f"transposed source dim {d + 1}")
+    dst = Pair.dense(cl, np.zeros((50, 60), dtype=F)).transpose(0, 1)      # 60 x 50 view of a 50 x 60 storage
+    dst.dev.cumsum(Pair.dense(cl, x).dev, 1)
+    _scan_close(dst.dev.float(), cat.cumulate(x, 0), "strided destination")
+    same = cl.ClTensor(x)
+    same.cumsum(same, 2)                                   # result and source are one tensor
+    _scan_close(same.float(), cat.cumulate(x, 1), "in place")
+    with pytest.raises(cl.ClError):
+        cl.ClTensor(x).cumsum(3)
+
+
+def test_mean_and_norms(cl):
+    x = oracle.normal(64, 300 * 700).reshape(300, 700)
+    x[5, :40] = 0.0
+    X = cl.ClTensor(x)
+    x64 = x.astype(np.float64)
+    assert abs(X.mean() - x64.mean()) <= 1e-5 * abs(x64.mean()) + 1e-7
+    for d in (0, 1):
+        got = X.mean(d + 1).float()
+        want = (x64.sum(axis=d, keepdims=True).astype(F) / F(x.shape[d])).astype(F)   # fp32 sum, then one division
+        assert_bit_equal(got, want, f"mean dim {d + 1}")
+    for p in (0.0, 1.0, 2.0, 3.0, 0.5, 2.5):
+        want = float(cat.norm(x, p))
+        assert abs(X.norm(p) - want) <= 1e-5 * want, (p, X.norm(p), want)
+        for d in (0, 1):
+            got = X.norm(p, d + 1).float()
+            wd = cat.norm(x, p, axis=d)
+            assert got.shape == wd.shape
+            assert np.all(np.abs(got - wd) <= 1e-5 * np.abs(wd) + 1e-30), (p, d)
+    assert X.norm() == X.norm(2.0)                          # default exponent
+    assert X.norm(0.0) == float((x != 0).sum())             # exact count
+    t = Pair.dense(cl, x).transpose(0, 1).narrow(0, 3, 500)
+    want = float(cat.norm(t.view.gather(), 2.0))
+    assert abs(t.dev.norm(2.0) - want) <= 1e-5 * want
+    with pytest.raises(cl.ClError):
+        cl.ClTensor().mean()
+
+
+def test_all_any(cl):
+    n = 1 << 20
+    x = oracle.uniform(65, n, 1.0, 5.0)
+    X = cl.ClTensor(x)
+    assert X.all() is True and X.any() is True
+    x2 = x.copy()
+    x2[n - 7] = 0.5                                         # (int)0.5 == 0: false for the reference's all
+    assert cl.ClTensor(x2).all() is False and bool(cat.truth(x2).all()) is False
+    z = np.zeros(n, dtype=F)
+    assert cl.ClTensor(z).any() is False and cl.ClTensor(z).all() is False
+    z[12345] = -3.0
+    assert cl.ClTensor(z).any() is True
+    z[12345] = 0.99
+    assert cl.ClTensor(z).any() is False and bool(cat.truth(z).any()) is False
+    pt = cl.ClTensor()
+    pt.all(X)
+    assert pt.nDimension() == 0 and pt.s() == 1.0
+    pt.any(cl.ClTensor(np.zeros(100, dtype=F)))
+    assert pt.s() == 0.0
+    s = Pair.dense(cl, x2.reshape(1024, 1024)).transpose(0, 1).narrow(1, 0, 1000)   # drops row 1023 with the 0.5
+    assert s.dev.all() is bool(cat.truth(s.view.gather()).all())

@@ -299,3 +299,31 @@ def test_catalogue_special_values_and_identities():
     assert np.allclose(cat.unary("tan", cat.unary("atan", x)), x, atol=1e-6)
     assert np.allclose(cat.unary("log1p", x), np.log(1.0 + x.astype(np.float64)), atol=1e-6)
     assert cat.atan2([1.0, -1.0, 0.0], [0.0, 0.0, -1.0]).tolist() == [np.float32(np.pi / 2), np.float32(-np.pi / 2), np.float32(np.pi)]
+
+
+def test_scan_norm_truth_closed_forms():
+    from oracle import catalogue as cat
+    n = 3000
+    assert np.array_equal(cat.cumulate(np.ones(n, dtype=np.float32), 0), np.arange(1, n + 1, dtype=np.float32))
+    k = np.arange(1, n + 1, dtype=np.float64)
+    assert np.array_equal(cat.cumulate(np.arange(1, n + 1, dtype=np.float32), 0), (k * (k + 1) / 2).astype(np.float32))
+    assert np.array_equal(cat.cumulate(np.full(30, 2.0, dtype=np.float32), 0, prod=True), (2.0 ** np.arange(1, 31)).astype(np.float32))
+    # a python loop with an fp64 running value on a small 2-d case, both axes
+    x = oracle.uniform(3, 6 * 7).reshape(6, 7)
+    for axis in (0, 1):
+        want = np.empty_like(x)
+        for line in range(x.shape[1 - axis]):
+            acc = 0.0
+            for r in range(x.shape[axis]):
+                idx = (r, line) if axis == 0 else (line, r)
+                acc += float(x[idx])
+                want[idx] = np.float32(acc)
+        assert np.array_equal(cat.cumulate(x, axis), want)
+    # fp64 running value matters: 2^24 + 1 + 1 ... stays exact in fp64, then rounds
+    big = np.array([16777216.0, 1.0, 1.0, 1.0], dtype=np.float32)
+    assert cat.cumulate(big, 0).tolist() == [16777216.0, 16777216.0, 16777218.0, 16777220.0]
+    v = np.array([[3.0, -4.0, 0.0], [0.0, 0.0, -2.0]], dtype=np.float32)
+    assert cat.norm(v, 2) == 29.0 ** 0.5 or abs(cat.norm(v, 2) - np.float32(29.0 ** 0.5)) < 1e-6
+    assert cat.norm(v, 1) == 9.0 and cat.norm(v, 0) == 3.0
+    assert cat.norm(v, 2, axis=1).ravel().tolist() == [5.0, 2.0] and cat.norm(v, 0, axis=0).ravel().tolist() == [1.0, 1.0, 1.0]
+    assert cat.truth([0.0, 0.5, -0.99, 1.0, -1.0, 2.5]).tolist() == [False, False, False, True, True, True]
