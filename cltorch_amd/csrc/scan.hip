@@ -6,12 +6,13 @@
 //
 // The tensor is taken as dense [O][R][I] (outer, scanned, inner).  Numerics
 // follow Torch7's CPU path: the running value is fp64 and every output is its
-// rounding to fp32.  Two kernels:
+// rounding to fp32.  Three kernels:
 //   * scan_seq: one thread per (o, i) walks r; adjacent threads are adjacent in
-//     i, so accesses coalesce whenever I is not tiny.  Also serves short
-//     innermost scans.
+//     i, so accesses coalesce whenever I is not tiny.
 //   * scan_row: I == 1 and long rows; a block walks the row 1024 elements at a
 //     time with a block-wide fp64 prefix in each step.
+//   * scan_short_rows: I == 1 and many short rows; 1 to 64 lanes share a row
+//     and adjacent lane groups take adjacent rows.
 // When O * I alone cannot fill the chip, R is cut into S segments and the scan
 // becomes three passes: segment totals, an exclusive scan of the totals, then
 // the scan proper with each segment's carry-in.
@@ -165,6 +166,85 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
   if (PHASE == 0 && threadIdx.x == 0) P.totals[blockIdx.x] = carry;
 }
 
+// I == 1 and short rows: G lanes (a power of two <= 64) share a row, 4
+// consecutive elements per lane per step; a block holds 256 / G rows.  No LDS:
+// the prefix over a row's lanes is a shuffle scan of width G.
+template <bool PROD, int G, bool VEC>
+__global__ __launch_bounds__(kThreads) void scan_short_rows(ScanParams P) {
+  constexpr int PER = 4, ROWS = kThreads / G;
+  const int sub = threadIdx.x % G;
+  const thcl_u64 o = (thcl_u64)blockIdx.x * ROWS + threadIdx.x / G;
+  const bool live = o < P.O;   // dead groups still take part in the shuffles of their wave
+  const float *row = P.in + (live ? o : 0) * P.R;
+  float *orow = P.out + (live ? o : 0) * P.R;
+  double carry = Op<PROD>::identity();
+  for (thcl_u64 base = 0; base < P.R; base += G * PER) {
+    const thcl_u64 j = base + (thcl_u64)sub * PER;
+    float x[PER];
+    if (VEC && live && j + PER <= P.R) {
+      const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
+#pragma unroll
+      for (int c = 0; c < PER; c++) x[c] = v[c];
+    } else {
+#pragma unroll
+      for (int c = 0; c < PER; c++) x[c] = (live && j + c < P.R) ? row[j + c] : (PROD ? 1.0f : 0.0f);
+    }
+    double a[PER];
+    a[0] = (double)x[0];
+#pragma unroll
+    for (int c = 1; c < PER; c++) a[c] = Op<PROD>::comb(a[c - 1], (double)x[c]);
+    double incl = a[PER - 1];
+#pragma unroll
+    for (int d = 1; d < G; d <<= 1) {
+      const double up = __shfl_up(incl, d, G);
+      if (sub >= d) incl = Op<PROD>::comb(up, incl);
+    }
+    double before = carry;
+    if (G > 1) {
+      const double prev = __shfl_up(incl, 1, G);
+      if (sub > 0) before = Op<PROD>::comb(before, prev);
+      carry = Op<PROD>::comb(carry, __shfl(incl, G - 1, G));
+    } else {
+      carry = Op<PROD>::comb(carry, incl);
+    }
+    if (live) {
+      if (VEC && j + PER <= P.R) {
+        thcl_f4 v;
+#pragma unroll
+        for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[c]);
+        __builtin_nontemporal_store(v, (thcl_f4 *)(orow + j));
+      } else {
+#pragma unroll
+        for (int c = 0; c < PER; c++)
+          if (j + c < P.R) orow[j + c] = (float)Op<PROD>::comb(before, a[c]);
+      }
+    }
+  }
+}
+
+template <bool PROD, int G>
+void launch_short(hipStream_t stream, const ScanParams &P, bool vec) {
+  const dim3 grid((unsigned)((P.O + kThreads / G - 1) / (kThreads / G))), block(kThreads);
+  if (vec) hipLaunchKernelGGL((scan_short_rows<PROD, G, true>), grid, block, 0, stream, P);
+  else hipLaunchKernelGGL((scan_short_rows<PROD, G, false>), grid, block, 0, stream, P);
+}
+
+template <bool PROD>
+void run_short(hipStream_t stream, const ScanParams &P, bool vec) {
+  // lanes per row: enough to cover the row in one step, at most a wave
+  int g = 1;
+  while (g < kWave && (thcl_u64)g * 4 < P.R) g <<= 1;
+  switch (g) {
+    case 1: launch_short<PROD, 1>(stream, P, vec); break;
+    case 2: launch_short<PROD, 2>(stream, P, vec); break;
+    case 4: launch_short<PROD, 4>(stream, P, vec); break;
+    case 8: launch_short<PROD, 8>(stream, P, vec); break;
+    case 16: launch_short<PROD, 16>(stream, P, vec); break;
+    case 32: launch_short<PROD, 32>(stream, P, vec); break;
+    default: launch_short<PROD, 64>(stream, P, vec); break;
+  }
+}
+
 void check(const char *what) {
   hipError_t e = hipGetLastError();
   THCL_CHECK(e == hipSuccess, "%s launch failed: %s", what, hipGetErrorString(e));
@@ -228,11 +308,16 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
   const thcl_u64 total = P.O * P.R * P.I;
   if (total > 0) {
     const long cus = thcl_rt_get_props(rt)->compute_units;
-    const bool rows = (P.I == 1 && P.R >= 1024);
+    // innermost scans: long rows (or few of them) take a block per row segment,
+    // many short rows take a lane group per row
+    const bool shortrows = P.I == 1 && P.R > 1 && (P.R < 1024 || (P.R < 8192 && P.O >= (thcl_u64)cus * 16));
+    const bool rows = (P.I == 1 && P.R >= 1024) && !shortrows;
     // cut R into segments until the launch fills the chip; a segment keeps
     // enough elements to amortise the extra pass
     thcl_u64 S = 1;
-    if (rows) {
+    if (shortrows) {
+      S = 1;
+    } else if (rows) {
       const thcl_u64 want = (thcl_u64)cus * 8;  // blocks
       if (P.O < want) S = (want + P.O - 1) / P.O;
       const thcl_u64 most = P.R / 4096;
@@ -252,9 +337,17 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     THCL_CHECK(P.O * P.S < (1ull << 31) && (P.O * P.S * P.I + kThreads - 1) / kThreads < (1ull << 31), THCL_DIM_WARNING);
     if (S > 1) P.totals = (double *)thcl_rt_workspace(rt, (size_t)(P.O * P.S * P.I) * sizeof(double));
     THCL_CHECK(S == 1 || P.totals != nullptr, "%s", thcl_rt_error());
-    const bool vec = rows && (P.R % 4 == 0) && ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
-    if (prod) run_scan<true>(stream, P, rows, vec);
-    else run_scan<false>(stream, P, rows, vec);
+    const bool vec = (rows || shortrows) && (P.R % 4 == 0) && ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
+    if (shortrows) {
+      THCL_CHECK(P.O < (1ull << 31), THCL_DIM_WARNING);
+      if (prod) run_short<true>(stream, P, vec);
+      else run_short<false>(stream, P, vec);
+      check("scan");
+    } else if (prod) {
+      run_scan<true>(stream, P, rows, vec);
+    } else {
+      run_scan<false>(stream, P, rows, vec);
+    }
     thcl_after_launch(state, rt);
   }
   THClTensor_free(state, srcc);

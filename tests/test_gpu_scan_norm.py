@@ -25,7 +25,8 @@ def _scan_close(got, want, what):
 
 
 SHAPES = [(1,), (5,), (1023,), (1024,), (4099,), (300000,), (7, 5), (3, 2000), (2000, 3), (64, 4096), (33, 70, 9),
-          (4, 300, 128), (2, 3, 4, 5), (1, 50000), (50000, 1), (6, 1 << 16)]
+          (4, 300, 128), (2, 3, 4, 5), (1, 50000), (50000, 1), (6, 1 << 16),
+          (5000, 2), (5000, 3), (3000, 16), (3000, 18), (700, 100), (700, 256), (300, 1000), (20000, 2048), (9, 7, 130)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
