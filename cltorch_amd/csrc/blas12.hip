@@ -1,0 +1,424 @@
+// Level-1 / level-2 contractions: dot, matrix-vector (addmv), rank-1 update (addr).
+//
+// What it replaces (reference): THClTensor_dot / addmv / addr
+// (src/lib/THClTensorMathBlas.cpp:17-105,216-277) and the clBLAS calls behind
+// THClBlas_dot / gemv / ger (src/lib/THClBlas.cpp:149-347).
+//
+// All three are bound by HBM: gemv reads the matrix once (4 bytes per 2
+// flops), so the kernels are streaming reductions, with fp64 accumulators
+// like the other sums of this library.  The rank-1 update is a pointwise
+// operator over the matrix with the vectors as stride-0 views, and runs on the
+// apply engine.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "apply_device.h"
+#include "internal.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWave = 64;
+
+// Column-major A (m x n, leading dimension lda), BLAS meaning of the rest.
+struct GemvParams {
+  const float *a;
+  const float *x;
+  float *y;
+  double *partials;  // [split][outputs] when the contraction is split over blocks
+  thcl_u32 m, n;
+  thcl_u64 lda;
+  long incx, incy;
+  float alpha, beta;
+  thcl_u32 split, per_split;
+};
+
+__device__ __forceinline__ void store_result(const GemvParams &P, thcl_u32 i, double acc) {
+  float *yp = P.y + (long)i * P.incy;
+  const float scaled = (float)((double)P.alpha * acc);
+  *yp = (P.beta == 0.f) ? scaled : P.beta * *yp + scaled;  // beta == 0: y is not read (BLAS rule)
+}
+
+// trans = 't': y[j] = alpha * dot(A[:, j], x) + beta * y[j].  Column j is m
+// contiguous floats; LPR lanes walk it (8, 64 or a whole block).
+template <int LPR, bool VEC>
+__global__ __launch_bounds__(kThreads) void gemv_t(GemvParams P) {
+  constexpr int COLS = kThreads / LPR;
+  __shared__ double lds[kThreads / kWave];
+  const int sub = threadIdx.x % LPR;
+  const thcl_u32 j = blockIdx.x * COLS + threadIdx.x / LPR;
+  double acc = 0.0;
+  if (j < P.n) {
+    const float *col = P.a + (thcl_u64)j * P.lda;
+    if (VEC) {  // m % 4 == 0, 16-byte aligned columns, incx == 1
+      const thcl_f4 *c4 = (const thcl_f4 *)col, *x4 = (const thcl_f4 *)P.x;
+      const thcl_u32 m4 = P.m >> 2;
+      constexpr int FLY = 4;
+      thcl_u32 i = sub;
+      for (; i + (FLY - 1) * LPR < m4; i += FLY * LPR) {
+        thcl_f4 v[FLY], w[FLY];
+#pragma unroll
+        for (int f = 0; f < FLY; f++) {
+          v[f] = __builtin_nontemporal_load(c4 + i + f * LPR);
+          w[f] = x4[i + f * LPR];
+        }
+#pragma unroll
+        for (int f = 0; f < FLY; f++)
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc += (double)v[f][c] * (double)w[f][c];
+      }
+      for (; i < m4; i += LPR) {
+        const thcl_f4 v = c4[i], w = x4[i];
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc += (double)v[c] * (double)w[c];
+      }
+    } else {
+      for (thcl_u32 i = sub; i < P.m; i += LPR) acc += (double)col[i] * (double)P.x[(long)i * P.incx];
+    }
+  }
+  // fold the LPR lanes of a column
+#pragma unroll
+  for (int d = (LPR < kWave ? LPR : kWave) >> 1; d > 0; d >>= 1) acc += __shfl_xor(acc, d, kWave);
+  if (LPR <= kWave) {
+    if (sub == 0 && j < P.n) store_result(P, j, acc);
+  } else {
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) lds[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0 && j < P.n) {
+      double r = lds[0];
+      for (int w = 1; w < kThreads / kWave; w++) r += lds[w];
+      store_result(P, j, r);
+    }
+  }
+}
+
+// trans = 'n': y[i] = alpha * sum_j A[i + j*lda] * x[j] + beta * y[i].  Lanes lie
+// along i (VEC rows each), the 4 waves of a block interleave over j and meet in
+// LDS; blockIdx.y splits long contractions, leaving partials for gemv_n_finish.
+template <int VEC>
+__global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
+  constexpr int WAVES = kThreads / kWave;
+  __shared__ double lds[WAVES][kWave * VEC];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const thcl_u32 units = (P.m + VEC - 1) / VEC;
+  const thcl_u32 u = blockIdx.x * kWave + lane;
+  const thcl_u32 j0 = blockIdx.y * P.per_split;
+  thcl_u32 j1 = j0 + P.per_split;
+  if (j1 > P.n) j1 = P.n;
+  double acc[VEC];
+#pragma unroll
+  for (int c = 0; c < VEC; c++) acc[c] = 0.0;
+  if (u < units) {
+    constexpr int FLY = 4;
+    thcl_u32 j = j0 + wave;
+    const float *ptr = P.a + (thcl_u64)j * P.lda + (thcl_u64)u * VEC;
+    const thcl_u64 step = (thcl_u64)WAVES * P.lda;
+    for (; j + (FLY - 1) * WAVES < j1; j += FLY * WAVES) {
+      float xs[FLY];
+      if (VEC == 4) {
+        thcl_f4 v[FLY];
+#pragma unroll
+        for (int f = 0; f < FLY; f++) {
+          v[f] = __builtin_nontemporal_load((const thcl_f4 *)ptr);
+          xs[f] = P.x[(long)(j + f * WAVES) * P.incx];
+          ptr += step;
+        }
+#pragma unroll
+        for (int f = 0; f < FLY; f++)
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc[c] += (double)v[f][c] * (double)xs[f];
+      } else {
+        float v[FLY];
+#pragma unroll
+        for (int f = 0; f < FLY; f++) {
+          v[f] = *ptr;
+          xs[f] = P.x[(long)(j + f * WAVES) * P.incx];
+          ptr += step;
+        }
+#pragma unroll
+        for (int f = 0; f < FLY; f++) acc[0] += (double)v[f] * (double)xs[f];
+      }
+    }
+    for (; j < j1; j += WAVES) {
+      const double xj = (double)P.x[(long)j * P.incx];
+      if (VEC == 4) {
+        const thcl_f4 v = *(const thcl_f4 *)ptr;
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[c] += (double)v[c] * xj;
+      } else {
+        acc[0] += (double)*ptr * xj;
+      }
+      ptr += step;
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < VEC; c++) lds[wave][lane * VEC + c] = acc[c];
+  __syncthreads();
+  if (wave == 0 && u < units) {
+#pragma unroll
+    for (int c = 0; c < VEC; c++) {
+      double r = lds[0][lane * VEC + c];
+      for (int w = 1; w < WAVES; w++) r += lds[w][lane * VEC + c];
+      const thcl_u32 i = u * VEC + c;
+      if (i < P.m) {
+        if (P.split > 1) P.partials[(thcl_u64)blockIdx.y * P.m + i] = r;
+        else store_result(P, i, r);
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void gemv_n_finish(GemvParams P) {
+  const thcl_u32 i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= P.m) return;
+  double r = 0.0;
+  for (thcl_u32 k = 0; k < P.split; k++) r += P.partials[(thcl_u64)k * P.m + i];
+  store_result(P, i, r);
+}
+
+void check(const char *what) {
+  hipError_t e = hipGetLastError();
+  THCL_CHECK(e == hipSuccess, "%s launch failed: %s", what, hipGetErrorString(e));
+}
+bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+
+// 1-d vector as an (rows x cols) view that repeats it along the other dim
+THClTensor *expanded(THClState *state, THClTensor *vec, long rows, long cols, bool along_rows) {
+  long sz[2] = {rows, cols};
+  long st[2] = {along_rows ? vec->stride[0] : 0, along_rows ? 0 : vec->stride[0]};
+  THLongStorage sizes, strides;
+  memset(&sizes, 0, sizeof(sizes));
+  memset(&strides, 0, sizeof(strides));
+  sizes.data = sz;
+  sizes.size = 2;
+  strides.data = st;
+  strides.size = 2;
+  return THClTensor_newWithStorage(state, vec->storage->device, vec->storage, vec->storageOffset, &sizes, &strides);
+}
+}  // namespace
+
+extern "C" {
+
+// y = alpha * op(A) * x + beta * y on column-major A (m x n, lda); BLAS argument
+// meaning, operands given as tensors whose storage + offset mark the first element
+// (src/lib/THClBlas.h:26-30, src/lib/THClBlas.cpp:199-262)
+void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, THClTensor *a, long lda, THClTensor *x,
+                   long incx, float beta, THClTensor *y, long incy) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, a, x, y);
+  THCL_CHECK(a->storage && x->storage && y->storage, "gemv operands need device storage");
+  const bool t = (trans == 't' || trans == 'T');
+  THCL_ARGCHECK(t || trans == 'n' || trans == 'N', 2, "trans must be 'n' or 't'");
+  THCL_ARGCHECK(m >= 0 && n >= 0 && m < (1l << 31) && n < (1l << 31), 3, THCL_DIM_WARNING);
+  if (n == 1) lda = m;  // a single column: any leading dimension does (src/lib/THClBlas.cpp:201-202)
+  THCL_ARGCHECK(lda >= (m > 1 ? m : 1), 7, "lda must be at least m");
+  const long outputs = t ? n : m;
+  if (outputs == 0) return;
+  thcl_rt *rt = thcl_ctx(state, y->storage->device);
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  GemvParams P;
+  memset(&P, 0, sizeof(P));
+  P.a = thcl_dptr(a);
+  P.x = thcl_dptr(x);
+  P.y = thcl_dptr(y);
+  P.m = (thcl_u32)m;
+  P.n = (thcl_u32)n;
+  P.lda = (thcl_u64)lda;
+  P.incx = incx;
+  P.incy = incy;
+  P.alpha = alpha;
+  P.beta = beta;
+  P.split = 1;
+  P.per_split = (thcl_u32)n;
+  const bool rows_aligned = aligned16(P.a) && (lda % 4 == 0) && (m % 4 == 0);
+  if (t) {
+    const bool vec = rows_aligned && incx == 1 && aligned16(P.x);
+#define GEMV_T(L)                                                                                        \
+  {                                                                                                      \
+    const dim3 grid((unsigned)((n + (kThreads / L) - 1) / (kThreads / L)));                              \
+    if (vec) hipLaunchKernelGGL((gemv_t<L, true>), grid, dim3(kThreads), 0, stream, P);                  \
+    else hipLaunchKernelGGL((gemv_t<L, false>), grid, dim3(kThreads), 0, stream, P);                     \
+  }
+    if (m >= 2048) GEMV_T(256) else if (m >= 128) GEMV_T(64) else GEMV_T(8)
+#undef GEMV_T
+    check("gemv");
+  } else {
+    const int vecw = rows_aligned ? 4 : 1;
+    const long units = (m + vecw - 1) / vecw;
+    const long tiles = (units + kWave - 1) / kWave;
+    const long target = (long)thcl_rt_get_props(rt)->compute_units * 4;
+    long split = 1;
+    if (tiles < target) {
+      split = (target + tiles - 1) / tiles;
+      const long most = (n + 31) / 32;  // at least 32 columns per block
+      if (split > most) split = most;
+      if (split > 256) split = 256;
+      if (split < 1) split = 1;
+    }
+    long per = (n + split - 1) / split;
+    if (per < 1) per = 1;
+    split = n > 0 ? (n + per - 1) / per : 1;
+    P.split = (thcl_u32)split;
+    P.per_split = (thcl_u32)per;
+    if (split > 1) {
+      P.partials = (double *)thcl_rt_workspace(rt, (size_t)split * (size_t)m * sizeof(double));
+      THCL_CHECK(P.partials != nullptr, "%s", thcl_rt_error());
+    }
+    const dim3 grid((unsigned)tiles, (unsigned)split);
+    if (vecw == 4) hipLaunchKernelGGL((gemv_n<4>), grid, dim3(kThreads), 0, stream, P);
+    else hipLaunchKernelGGL((gemv_n<1>), grid, dim3(kThreads), 0, stream, P);
+    check("gemv");
+    if (split > 1) {
+      hipLaunchKernelGGL(gemv_n_finish, dim3((unsigned)((m + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P);
+      check("gemv finish");
+    }
+  }
+  thcl_after_launch(state, rt);
+  THCL_GUARD_END()
+}
+
+// A += alpha * x * y^T on column-major A (m x n, lda)
+// (src/lib/THClBlas.h:32-35, src/lib/THClBlas.cpp:264-347)
+void THClBlas_ger(THClState *state, long m, long n, float alpha, THClTensor *x, long incx, THClTensor *y, long incy,
+                  THClTensor *a, long lda) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, a, x, y);
+  THCL_CHECK(a->storage && x->storage && y->storage, "ger operands need device storage");
+  if (n == 1) lda = m;
+  if (m == 0 || n == 0) return;
+  // views over the three storages: A as (n x m) with strides (lda, 1); x along the unit dim, y along the other
+  long asz[2] = {n, m}, ast[2] = {lda, 1}, xst[2] = {0, incx}, yst[2] = {incy, 0};
+  THLongStorage sizes, sa, sx, sy;
+  memset(&sizes, 0, sizeof(sizes));
+  sa = sx = sy = sizes;
+  sizes.data = asz;
+  sa.data = ast;
+  sx.data = xst;
+  sy.data = yst;
+  sizes.size = sa.size = sx.size = sy.size = 2;
+  const int dev = a->storage->device;
+  THClTensor *av = THClTensor_newWithStorage(state, dev, a->storage, a->storageOffset, &sizes, &sa);
+  THClTensor *xv = THClTensor_newWithStorage(state, dev, x->storage, x->storageOffset, &sizes, &sx);
+  THClTensor *yv = THClTensor_newWithStorage(state, dev, y->storage, y->storageOffset, &sizes, &sy);
+  ApplyCall c;
+  c.n = 3;
+  c.t[0] = av;
+  c.t[1] = xv;
+  c.t[2] = yv;
+  c.val[0] = alpha;
+  try {
+    thcl_apply_expr(state, "*out += val1 * *in1 * *in2", c);
+  } catch (...) {
+    THClTensor_free(state, av);
+    THClTensor_free(state, xv);
+    THClTensor_free(state, yv);
+    throw;
+  }
+  THClTensor_free(state, av);
+  THClTensor_free(state, xv);
+  THClTensor_free(state, yv);
+  THCL_GUARD_END()
+}
+
+// (src/lib/THClTensorMathBlas.cpp:17-41); products and the running sum are fp64
+float THClTensor_dot(THClState *state, THClTensor *self, THClTensor *src) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 2, self, src);
+  const long n = THClTensor_nElement(state, self);
+  THCL_ARGCHECK(n == THClTensor_nElement(state, src), 2, "sizes do not match");
+  if (n == 0) return 0.f;
+  THClTensor *a = THClTensor_newContiguous(state, self);
+  THClTensor *b = THClTensor_newContiguous(state, src);
+  thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, self));
+  size_t sb = 0;
+  char *scratch = (char *)thcl_rt_scratch(rt, &sb);
+  float *dres = (float *)(scratch + sb - 256);
+  float result = 0.f;
+  try {
+    thcl_dot_dense(state, rt, thcl_dptr(a), thcl_dptr(b), n, dres);
+    float *hw = thcl_rt_host_word(rt);
+    THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, dres, sizeof(float)) == 0, "%s", thcl_rt_error());
+    result = hw[0];
+  } catch (...) {
+    THClTensor_free(state, a);
+    THClTensor_free(state, b);
+    throw;
+  }
+  THClTensor_free(state, a);
+  THClTensor_free(state, b);
+  return result;
+  THCL_GUARD_END(0.f)
+}
+
+// r_ = beta * t + alpha * mat * vec  (src/lib/THClTensorMathBlas.cpp:43-105)
+void THClTensor_addmv(THClState *state, THClTensor *r_, float beta, THClTensor *t, float alpha, THClTensor *mat,
+                      THClTensor *vec) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 4, r_, t, mat, vec);
+  THCL_CHECK(mat->nDimension == 2 && vec->nDimension == 1, "matrix and vector expected");
+  THCL_CHECK(mat->size[1] == vec->size[0], "size mismatch");
+  THCL_CHECK(t->nDimension == 1 && t->size[0] == mat->size[0], "size mismatch");
+  if (r_ != t) {
+    THClTensor_resizeAs(state, r_, t);
+    THClTensor_copy(state, r_, t);
+  }
+  if (mat->stride[0] == 1 && mat->stride[1] >= (mat->size[0] > 1 ? mat->size[0] : 1)) {
+    THClBlas_gemv(state, 'n', mat->size[0], mat->size[1], alpha, mat, mat->stride[1], vec, vec->stride[0], beta, r_,
+                  r_->stride[0]);
+  } else if (mat->stride[1] == 1 && mat->stride[0] >= (mat->size[1] > 1 ? mat->size[1] : 1)) {
+    THClBlas_gemv(state, 't', mat->size[1], mat->size[0], alpha, mat, mat->stride[0], vec, vec->stride[0], beta, r_,
+                  r_->stride[0]);
+  } else {
+    THClTensor *cmat = THClTensor_newContiguous(state, mat);
+    try {
+      THClBlas_gemv(state, 't', mat->size[1], mat->size[0], alpha, cmat, cmat->stride[0], vec, vec->stride[0], beta, r_,
+                    r_->stride[0]);
+    } catch (...) {
+      THClTensor_free(state, cmat);
+      throw;
+    }
+    THClTensor_free(state, cmat);
+  }
+  THCL_GUARD_END()
+}
+
+// r_ = beta * t + alpha * vec1 (x) vec2  (src/lib/THClTensorMathBlas.cpp:216-277).
+// One pointwise pass over r_ with the vectors as stride-0 views; the reference
+// scales r_ in one launch and calls ger in a second.
+void THClTensor_addr(THClState *state, THClTensor *r_, float beta, THClTensor *t, float alpha, THClTensor *vec1,
+                     THClTensor *vec2) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 4, r_, t, vec1, vec2);
+  THCL_CHECK(vec1->nDimension == 1 && vec2->nDimension == 1, "vector and vector expected");
+  THCL_CHECK(t->nDimension == 2, "size mismatch");
+  THCL_CHECK(t->size[0] == vec1->size[0] && t->size[1] == vec2->size[0], "size mismatch");
+  if (r_ != t) {
+    THClTensor_resizeAs(state, r_, t);
+    THClTensor_copy(state, r_, t);
+  }
+  if (r_->size[0] == 0 || r_->size[1] == 0) return;
+  THClTensor *v1 = expanded(state, vec1, r_->size[0], r_->size[1], true);
+  THClTensor *v2 = expanded(state, vec2, r_->size[0], r_->size[1], false);
+  ApplyCall c;
+  c.n = 3;
+  c.t[0] = r_;
+  c.t[1] = v1;
+  c.t[2] = v2;
+  c.val[0] = beta;
+  c.val[1] = alpha;
+  try {
+    if (beta == 1.f) thcl_apply_expr(state, "*out += val2 * *in1 * *in2", c);
+    else thcl_apply_expr(state, "*out = val1 * *out + val2 * *in1 * *in2", c);
+  } catch (...) {
+    THClTensor_free(state, v1);
+    THClTensor_free(state, v2);
+    throw;
+  }
+  THClTensor_free(state, v1);
+  THClTensor_free(state, v2);
+  THCL_GUARD_END()
+}
+
+}  // extern "C"

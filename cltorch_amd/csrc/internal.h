@@ -120,6 +120,7 @@ enum ThclReduce : int {
   RED_SUM_NE0 = 4, RED_SUM_ABS = 5, RED_SUM_SQ = 6, RED_SUM_POW = 7, RED_ALL = 8, RED_ANY = 9
 };
 // whole tensor -> one float at device address `out`
+void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out);
 void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *src, long dim);
 void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent = 0.f);
 // along `dim`; `values` resized to size 1 along dim; idx outputs optional:

@@ -311,6 +311,45 @@ __global__ __launch_bounds__(kThreads) void reduce_all_strided(ReduceAllParams P
   finish_all<KIND>(acc, P, lds);
 }
 
+// sum of a[i] * b[i] over two dense arrays: products and the running sum in fp64
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void dot_dense(ReduceAllParams P, const float *other) {
+  __shared__ double lds[kThreads / kWave];
+  constexpr int U = 4;
+  double acc[U] = {0.0, 0.0, 0.0, 0.0};
+  if (VEC) {
+    const thcl_u64 n4 = P.n >> 2, tile = (thcl_u64)kThreads * U;
+    const thcl_f4 *a4 = (const thcl_f4 *)P.in, *b4 = (const thcl_f4 *)other;
+    for (thcl_u64 base = (thcl_u64)blockIdx.x * tile + threadIdx.x; base < n4; base += (thcl_u64)gridDim.x * tile) {
+      thcl_f4 x[U], y[U];
+#pragma unroll
+      for (int k = 0; k < U; k++) {
+        const thcl_u64 i = base + (thcl_u64)k * kThreads;
+        if (i < n4) {
+          x[k] = __builtin_nontemporal_load(a4 + i);
+          y[k] = __builtin_nontemporal_load(b4 + i);
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < U; k++) {
+        const thcl_u64 i = base + (thcl_u64)k * kThreads;
+        if (i < n4) {
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc[k] += (double)x[k][c] * (double)y[k][c];
+        }
+      }
+    }
+    if (blockIdx.x == 0)
+      for (thcl_u64 i = (n4 << 2) + threadIdx.x; i < P.n; i += kThreads) acc[0] += (double)P.in[i] * (double)other[i];
+  } else {
+    for (thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x; i < P.n; i += (thcl_u64)gridDim.x * kThreads)
+      acc[0] += (double)P.in[i] * (double)other[i];
+  }
+  double v = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+  v = block_reduce<RED_SUM, double>(v, lds);
+  finish_all<RED_SUM>(v, P, lds);
+}
+
 // ------------------------------------------------------- reduce along dim ---
 struct ReduceDimParams {
   const float *in;       // first element of the view
@@ -699,6 +738,35 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
     case RED_ANY: launch_all<RED_ANY>(dense, grid, stream, P); break;
   }
   check_launch("reduce-all");
+  thcl_after_launch(state, rt);
+}
+
+// out[0] = sum a[i] * b[i], both dense with n elements
+void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out) {
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  if (n == 0) {
+    thcl_fill_contig(rt, out, 0.f, 1);
+    thcl_after_launch(state, rt);
+    return;
+  }
+  size_t sbytes = 0;
+  char *scratch = (char *)thcl_rt_scratch(rt, &sbytes);
+  ReduceAllParams P;
+  memset(&P, 0, sizeof(P));
+  P.in = a;
+  P.n = (thcl_u64)n;
+  P.partials = scratch + kPartialOff;
+  P.ticket = (unsigned *)(scratch + kTicketOff);
+  P.out = out;
+  const bool vec = aligned16(a) && aligned16(b);
+  const long want = vec ? (n / 4 + kThreads * 4 - 1) / (kThreads * 4) : (n + kThreads - 1) / kThreads;
+  long cap = (long)thcl_rt_get_props(rt)->compute_units * 2;
+  const long max_partials = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
+  if (cap > max_partials) cap = max_partials;
+  const unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));
+  if (vec) hipLaunchKernelGGL(dot_dense<true>, dim3(grid), dim3(kThreads), 0, stream, P, b);
+  else hipLaunchKernelGGL(dot_dense<false>, dim3(grid), dim3(kThreads), 0, stream, P, b);
+  check_launch("dot");
   thcl_after_launch(state, rt);
 }
 

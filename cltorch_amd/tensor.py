@@ -571,6 +571,31 @@ class ClTensor:
         _call("THClTensor_addmm", self._h, C.c_float(beta), t._h, C.c_float(alpha), m1._h, m2._h)
         return self
 
+    def dot(self, other: "ClTensor") -> float:
+        """``a:dot(b)`` (``src/TensorMath.lua:932-936``)."""
+        return float(_call("THClTensor_dot", self._h, other._h))
+
+    def _addblas(self, cfn: str, args) -> "ClTensor":
+        """``r:addmv([beta,] [t,] [alpha,] mat, vec)`` and ``r:addr([beta,] [t,] [alpha,] v1, v2)``
+        (``src/TensorMath.lua:896-929``)."""
+        nums = [a for a in args if not isinstance(a, ClTensor)]
+        tens = [a for a in args if isinstance(a, ClTensor)]
+        if len(tens) == 2:
+            t, a, b = self, tens[0], tens[1]
+        elif len(tens) == 3:
+            t, a, b = tens
+        else:
+            raise ClError(f"invalid arguments to {cfn}")
+        beta, alpha = (1.0, 1.0) if not nums else ((1.0, nums[0]) if len(nums) == 1 else (nums[0], nums[1]))
+        _call(f"THClTensor_{cfn}", self._h, C.c_float(beta), t._h, C.c_float(alpha), a._h, b._h)
+        return self
+
+    def addmv(self, *args) -> "ClTensor":
+        return self._addblas("addmv", args)
+
+    def addr(self, *args) -> "ClTensor":
+        return self._addblas("addr", args)
+
     def __repr__(self):
         return f"ClTensor(size={self.size()}, stride={self.stride()})"
 
@@ -579,4 +604,18 @@ def mm(a: ClTensor, b: ClTensor) -> ClTensor:
     """``torch.mm(a, b)``: zeroed result, then addmm with beta 0 (``src/TensorMath.lua:867-893``)."""
     r = ClTensor(a.size(1), b.size(2)).zero()
     _call("THClTensor_addmm", r._h, C.c_float(0.0), r._h, C.c_float(1.0), a._h, b._h)
+    return r
+
+
+def mv(mat: ClTensor, vec: ClTensor) -> ClTensor:
+    """``torch.mv(mat, vec)``: zeroed result, then addmv (``src/TensorMath.lua:800-825``)."""
+    r = ClTensor(mat.size(1)).zero()
+    _call("THClTensor_addmv", r._h, C.c_float(1.0), r._h, C.c_float(1.0), mat._h, vec._h)
+    return r
+
+
+def ger(v1: ClTensor, v2: ClTensor) -> ClTensor:
+    """``torch.ger(v1, v2)``: zeroed result, then addr (``src/TensorMath.lua:869-894``)."""
+    r = ClTensor(v1.size(1), v2.size(1)).zero()
+    _call("THClTensor_addr", r._h, C.c_float(1.0), r._h, C.c_float(1.0), v1._h, v2._h)
     return r

@@ -390,6 +390,19 @@ void THClTensor_addmm(THClState *state, THClTensor *self, float beta, THClTensor
 void THClBlas_gemm(THClState *state, char transa, char transb, long m, long n, long k, float alpha,
                    THClTensor *a, long lda, THClTensor *b, long ldb, float beta, THClTensor *c, long ldc);
 
+/* Level 1 / level 2 (reference: src/lib/THClTensorMath.h:28,46,48, THClBlas.h:21-35).
+ * Sums run in fp64 and round to fp32 once.  The THClBlas_* forms take the
+ * tensors whose storage + offset mark each operand's first element. */
+float THClTensor_dot(THClState *state, THClTensor *self, THClTensor *src);
+void THClTensor_addmv(THClState *state, THClTensor *self, float beta, THClTensor *t, float alpha, THClTensor *mat,
+                      THClTensor *vec);
+void THClTensor_addr(THClState *state, THClTensor *self, float beta, THClTensor *t, float alpha, THClTensor *vec1,
+                     THClTensor *vec2);
+void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, THClTensor *a, long lda, THClTensor *x,
+                   long incx, float beta, THClTensor *y, long incy);
+void THClBlas_ger(THClState *state, long m, long n, float alpha, THClTensor *x, long incx, THClTensor *y, long incy,
+                  THClTensor *a, long lda);
+
 #ifdef __cplusplus
 }
 #endif

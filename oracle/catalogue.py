@@ -124,3 +124,20 @@ def truth(x):
     """Element truth value of the reference's all / any reductions: (int)x != 0,
     i.e. truncation toward zero (src/lib/THClTensorMath.cpp:444-458)."""
     return np.trunc(_f(x)) != 0
+
+
+# --------------------------------------------------------------- level 1 / 2 ---
+def dot(a, b):
+    """fp64 products and running sum, one rounding (the reference tests compare
+    its clBLAS result with Torch7's CPU dot within 1e-4: src/test/unit_tensor.lua:413-461)."""
+    return F(np.dot(np.asarray(a, dtype=np.float64).ravel(), np.asarray(b, dtype=np.float64).ravel()))
+
+
+def addmv(beta, t, alpha, mat, vec):
+    """beta * t + alpha * mat @ vec in fp64 (src/lib/THClTensorMathBlas.cpp:43-105)."""
+    return beta * np.asarray(t, dtype=np.float64) + alpha * (np.asarray(mat, dtype=np.float64) @ np.asarray(vec, dtype=np.float64))
+
+
+def addr(beta, t, alpha, v1, v2):
+    """beta * t + alpha * outer(v1, v2) in fp64 (src/lib/THClTensorMathBlas.cpp:216-277)."""
+    return beta * np.asarray(t, dtype=np.float64) + alpha * np.outer(np.asarray(v1, dtype=np.float64), np.asarray(v2, dtype=np.float64))

@@ -1,0 +1,137 @@
+"""dot, addmv, addr (and the THClBlas-level gemv / ger they sit on) through the
+C ABI against fp64 numpy (oracle/catalogue.py).  Tolerance 1e-5 relative to the
+result's scale for the sums (fp64 accumulation on the device), bit-exact for
+the small-integer cases of the reference's own tests."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import catalogue as cat
+from gpu_util import Pair
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+def _close(got, want, tol=1e-5):
+    want = np.asarray(want, dtype=np.float64)
+    scale = max(float(np.sqrt(np.mean(want ** 2))), 1e-30)
+    assert got.shape == want.shape
+    assert np.max(np.abs(got.astype(np.float64) - want)) / scale < tol
+
+
+def test_reference_integer_matrices(cl):
+    A = cl.ClTensor(np.array([[1, 2, -1], [3, 4, 0]], dtype=F))
+    B = np.array([[0, 1], [1, 2], [4, 5]], dtype=F)
+    assert cl.mv(A, cl.ClTensor(B[:, 0].copy())).float().tolist() == [-2.0, 4.0]
+    assert cl.mv(A, cl.ClTensor(B[:, 1].copy())).float().tolist() == [0.0, 11.0]
+    assert cl.ClTensor(np.array([1, 2, 3], dtype=F)).dot(cl.ClTensor(np.array([4, -5, 6], dtype=F))) == 12.0
+    assert cl.ger(cl.ClTensor(np.array([1, 2], dtype=F)), cl.ClTensor(np.array([3, 4, 5], dtype=F))).float().tolist() == \
+        [[3, 4, 5], [6, 8, 10]]
+
+
+@pytest.mark.parametrize("n", [1, 3, 64, 1023, 4099, 1 << 20, (1 << 22) + 5])
+def test_dot_lengths_and_views(cl, n):
+    a, b = oracle.uniform(71, n), oracle.uniform(72, n)
+    got = cl.ClTensor(a).dot(cl.ClTensor(b))
+    want = float(cat.dot(a, b))
+    assert abs(got - want) <= 1e-5 * max(abs(want), np.sqrt(n) * 1e-2)
+    if n >= 64:
+        pa = Pair(cl, a, 1, (n // 2,), (2,))                 # stride-2 view with an odd offset
+        pb = Pair(cl, b, 0, (n // 2,), (1,))
+        want = float(cat.dot(pa.view.gather(), pb.view.gather()))
+        assert abs(pa.dev.dot(pb.dev) - want) <= 1e-5 * max(abs(want), np.sqrt(n) * 1e-2)
+    with pytest.raises(cl.ClError):
+        cl.ClTensor(a).dot(cl.ClTensor(n + 1))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (2, 3), (7, 130), (130, 7), (64, 64), (300, 1000), (1000, 300), (4096, 33),
+                                       (33, 4096), (5, 70000), (70000, 5), (2048, 2048)])
+def test_addmv_layouts(cl, rows, cols):
+    m = oracle.normal(73, rows * cols).reshape(rows, cols)
+    v, t = oracle.normal(74, cols), oracle.normal(75, rows)
+    M, V, T = cl.ClTensor(m), cl.ClTensor(v), cl.ClTensor(t)
+    r = cl.ClTensor().addmv(0.5, T, 2.0, M, V)               # row-major matrix: the 't' kernel
+    _close(r.float(), cat.addmv(0.5, t, 2.0, m, v))
+    Mt = cl.ClTensor(np.ascontiguousarray(m.T)).t()          # same matrix stored column-major: the 'n' kernel
+    assert Mt.size() == (rows, cols) and Mt.stride()[0] == 1
+    r2 = cl.ClTensor().addmv(0.5, T, 2.0, Mt, V)
+    _close(r2.float(), cat.addmv(0.5, t, 2.0, m, v))
+    T2 = cl.ClTensor(t)
+    T2.addmv(M, V)                                           # in place, beta = alpha = 1
+    _close(T2.float(), cat.addmv(1.0, t, 1.0, m, v))
+    _close(cl.mv(M, V).float(), cat.addmv(0.0, np.zeros(rows), 1.0, m, v))
+    if rows >= 4 and cols >= 4:                              # neither stride is 1: dense copy, then 't'
+        big = Pair.dense(cl, oracle.normal(76, rows * cols * 4).reshape(rows * 2, cols * 2))
+        sub = big.step(0, 2).step(1, 2)
+        r3 = cl.ClTensor().addmv(1.0, T, 1.0, sub.dev, V)
+        _close(r3.float(), cat.addmv(1.0, t, 1.0, sub.view.gather(), v))
+        # strided vector and result
+        vv = Pair(cl, oracle.normal(77, cols * 3), 1, (cols,), (3,))
+        rr = Pair(cl, np.zeros(rows * 2, dtype=F), 0, (rows,), (2,))
+        rr.dev.addmv(0.0, rr.dev, 1.0, M, vv.dev)
+        _close(rr.dev.float(), cat.addmv(0.0, np.zeros(rows), 1.0, m, vv.view.gather()))
+
+
+def test_addmv_beta_zero_ignores_old_contents_and_checks_shapes(cl):
+    m = oracle.normal(78, 40 * 30).reshape(40, 30)
+    v = oracle.normal(79, 30)
+    t = np.full(40, np.nan, dtype=F)                          # BLAS: beta == 0 means y is not read
+    r = cl.ClTensor().addmv(0.0, cl.ClTensor(t), 1.0, cl.ClTensor(m), cl.ClTensor(v))
+    _close(r.float(), cat.addmv(0.0, np.zeros(40), 1.0, m, v))
+    with pytest.raises(cl.ClError):
+        cl.ClTensor().addmv(cl.ClTensor(t), cl.ClTensor(m), cl.ClTensor(31))
+    with pytest.raises(cl.ClError):
+        cl.ClTensor().addmv(cl.ClTensor(39), cl.ClTensor(m), cl.ClTensor(v))
+    with pytest.raises(cl.ClError):
+        cl.ClTensor().addmv(cl.ClTensor(t), cl.ClTensor(v), cl.ClTensor(v))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (2, 3), (130, 70), (64, 256), (1000, 1000), (5, 50000), (50000, 5)])
+def test_addr_layouts(cl, rows, cols):
+    t = oracle.normal(80, rows * cols).reshape(rows, cols)
+    a, b = oracle.normal(81, rows), oracle.normal(82, cols)
+    T, A, B = cl.ClTensor(t), cl.ClTensor(a), cl.ClTensor(b)
+    r = cl.ClTensor().addr(0.5, T, 2.0, A, B)
+    _close(r.float(), cat.addr(0.5, t, 2.0, a, b))
+    T2 = cl.ClTensor(t)
+    T2.addr(A, B)                                            # in place, beta = alpha = 1
+    _close(T2.float(), cat.addr(1.0, t, 1.0, a, b))
+    _close(cl.ger(A, B).float(), cat.addr(0.0, np.zeros((rows, cols)), 1.0, a, b))
+    Tt = Pair.dense(cl, np.ascontiguousarray(t.T)).transpose(0, 1)    # column-major result
+    Tt.dev.addr(1.0, 3.0, A, B)
+    _close(Tt.dev.float(), cat.addr(1.0, t, 3.0, a, b))
+    if rows >= 2:
+        aa = Pair(cl, oracle.normal(83, rows * 2 + 1), 1, (rows,), (2,))   # strided vector
+        T3 = cl.ClTensor(t)
+        T3.addr(1.0, 1.0, aa.dev, B)
+        _close(T3.float(), cat.addr(1.0, t, 1.0, aa.view.gather(), b))
+    with pytest.raises(cl.ClError):
+        cl.ClTensor().addr(T, A, cl.ClTensor(cols + 1))
+
+
+def test_blas_level_entry_points(cl):
+    """THClBlas_gemv / ger with explicit leading dimensions, as the reference's
+    tensor-level code calls them (src/lib/THClTensorMathBlas.cpp:62-104,241-276)."""
+    from cltorch_amd.tensor import _call
+    m, n, lda = 37, 29, 48
+    store = oracle.normal(84, lda * n)
+    a = cl.ClTensor(store)
+    x, y = oracle.normal(85, n), oracle.normal(86, m)
+    X, Y = cl.ClTensor(x), cl.ClTensor(y)
+    _call("THClBlas_gemv", C.c_char(b"n"), C.c_long(m), C.c_long(n), C.c_float(1.5), a._h, C.c_long(lda), X._h, C.c_long(1),
+                      C.c_float(0.25), Y._h, C.c_long(1))
+    A = store.reshape(n, lda)[:, :m].T.astype(np.float64)     # column-major m x n
+    _close(Y.float(), 0.25 * y + 1.5 * (A @ x))
+    xt, yt = oracle.normal(87, m), oracle.normal(88, n)
+    XT, YT = cl.ClTensor(xt), cl.ClTensor(yt)
+    _call("THClBlas_gemv", C.c_char(b"t"), C.c_long(m), C.c_long(n), C.c_float(1.0), a._h, C.c_long(lda), XT._h, C.c_long(1),
+                      C.c_float(1.0), YT._h, C.c_long(1))
+    _close(YT.float(), yt + A.T @ xt)
+    _call("THClBlas_ger", C.c_long(m), C.c_long(n), C.c_float(2.0), XT._h, C.c_long(1), X._h, C.c_long(1), a._h, C.c_long(lda))
+    want = store.reshape(n, lda).astype(np.float64).copy()
+    want[:, :m] += 2.0 * np.outer(x, xt)
+    _close(a.float().reshape(n, lda), want)                  # padding rows beyond m untouched
+    assert np.array_equal(a.float().reshape(n, lda)[:, m:], store.reshape(n, lda)[:, m:])

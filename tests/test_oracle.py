@@ -327,3 +327,15 @@ def test_scan_norm_truth_closed_forms():
     assert cat.norm(v, 1) == 9.0 and cat.norm(v, 0) == 3.0
     assert cat.norm(v, 2, axis=1).ravel().tolist() == [5.0, 2.0] and cat.norm(v, 0, axis=0).ravel().tolist() == [1.0, 1.0, 1.0]
     assert cat.truth([0.0, 0.5, -0.99, 1.0, -1.0, 2.5]).tolist() == [False, False, False, True, True, True]
+
+
+def test_level12_small_integer_cases(golden):
+    from oracle import catalogue as cat
+    # the reference's own test matrices (src/test/unit_tensor.lua:413-438): {{1,2,-1},{3,4,0}} . {{0,1},{1,2},{4,5}}
+    A = np.array([[1, 2, -1], [3, 4, 0]], dtype=np.float32)
+    B = np.array([[0, 1], [1, 2], [4, 5]], dtype=np.float32)
+    assert cat.addmv(0.0, np.zeros(2), 1.0, A, B[:, 0]).tolist() == [-2.0, 4.0]      # first column of {{-2,0},{4,11}}
+    assert cat.addmv(2.0, np.array([1.0, 1.0]), 1.0, A, B[:, 1]).tolist() == [2.0, 13.0]
+    assert cat.dot([1, 2, 3], [4, -5, 6]) == 12.0
+    assert cat.addr(1.0, np.ones((2, 3)), 2.0, [1, 2], [3, 4, 5]).tolist() == [[7, 9, 11], [13, 17, 21]]
+    assert cat.addr(0.5, np.full((2, 2), 4.0), 1.0, [1, -1], [2, 3]).tolist() == [[4, 5], [0, -1]]
