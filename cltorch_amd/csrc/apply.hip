@@ -110,7 +110,7 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
     int B = -1;
     if (J.strides[0][A] == 1 && J.sizes[A] >= 16) {
       for (int i = 1; i < n && B < 0; i++) {
-        if (J.strides[i][A] == 1) continue;
+        if (J.strides[i][A] == 1 || J.strides[i][A] == 0) continue;  // dense, or one value repeated along A
         for (int d = A - 1; d >= 0; d--)
           if (J.strides[i][d] == 1 && J.sizes[d] >= 16) {
             B = d;
@@ -182,6 +182,8 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
     const int last = J.dims - 1;
     bool vec = (J.sizes[last] % 4 == 0);
     for (int i = 0; i < n && vec; i++) {
+      // inputs may repeat one value along the innermost dim (stride 0: an expanded vector)
+      if (i > 0 && J.strides[i][last] == 0) continue;
       vec = vec && J.strides[i][last] == 1 && aligned16(p[i]);
       for (int d = 0; d < last; d++) vec = vec && (J.strides[i][d] % 4 == 0);
     }

@@ -121,6 +121,21 @@ __device__ __forceinline__ void thcl_st(V v, V *p) {
   __builtin_nontemporal_store(v, p);
 }
 
+// A unit of an input: 4 adjacent floats, or one float repeated (stride-0 innermost dim).
+template <class V>
+__device__ __forceinline__ V thcl_ld_unit(const float *p, bool same) {
+  if (same) {
+    const float x = *p;
+    V v;
+    v[0] = x;
+    v[1] = x;
+    v[2] = x;
+    v[3] = x;
+    return v;
+  }
+  return thcl_ld((const V *)p);
+}
+
 // ------------------------------------------------------------ contiguous ---
 // All operands dense and 16-byte aligned.  A tile is THREADS*UNROLL float4
 // units; lane l of a block touches units l, l+THREADS, ... so every wave reads
@@ -260,13 +275,15 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
       off[k][2] = o2 + (thcl_u64)r0 * P.stride[2][0];
     }
     if (VEC == 4) {
+      // an input whose innermost stride is 0 repeats one value along the unit
+      const bool same1 = NT > 1 && P.stride[1][P.dims - 1] == 0, same2 = NT > 2 && P.stride[2][P.dims - 1] == 0;
       thcl_f4 o[U], a[U], b[U];
 #pragma unroll
       for (int k = 0; k < U; k++) {
         if (base + k * THCL_APPLY_THREADS < P.nunits) {
           o[k] = thcl_ld((const thcl_f4 *)(P.p[0] + off[k][0]));
-          if (NT > 1) a[k] = thcl_ld((const thcl_f4 *)(P.p[1] + off[k][1]));
-          if (NT > 2) b[k] = thcl_ld((const thcl_f4 *)(P.p[2] + off[k][2]));
+          if (NT > 1) a[k] = thcl_ld_unit<thcl_f4>(P.p[1] + off[k][1], same1);
+          if (NT > 2) b[k] = thcl_ld_unit<thcl_f4>(P.p[2] + off[k][2], same2);
         }
       }
 #pragma unroll

@@ -235,6 +235,9 @@ def test_planner_picks_the_kernel_family_for_each_layout(lib):
     assert kind == "tiled" and grid == 512 * (512 // 64) * (256 // 256)             # 64 x 256 tiles, 512 outer slices
     sq = _plan(lib, [((8192, 8192), (8192, 1), 0), ((8192, 8192), (1, 8192), 0)])
     assert sq == ("tiled", (8192 // 128) ** 2)                                      # plain 2-d transpose: 128 x 128 tiles
+    # a rank-1 update: vectors expanded with stride 0 ride the vector kernel, not the transposing tiles
+    outer = _plan(lib, [((4096, 4096), (4096, 1), 0), ((4096, 4096), (1, 0), 0), ((4096, 4096), (0, 1), 0)])
+    assert outer[0] == "joint128"
     thin = _plan(lib, [((1024, 64, 1024), (65536, 1024, 1), 0), ((1024, 64, 1024), (65536, 1, 64), 0)])
     assert thin == ("tiled", 1024 * (1024 // 256) * (64 // 64))                     # dim B of 64: 256 x 64 tiles waste nothing
     assert _plan(lib, [tr, dst])[0] == "tiled"                                      # scatter into the transposed view
