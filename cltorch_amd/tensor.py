@@ -619,3 +619,70 @@ def ger(v1: ClTensor, v2: ClTensor) -> ClTensor:
     r = ClTensor(v1.size(1), v2.size(1)).zero()
     _call("THClTensor_addr", r._h, C.c_float(1.0), r._h, C.c_float(1.0), v1._h, v2._h)
     return r
+
+
+class ClKernel:
+    """``torch.ClKernel({input={...}, output={...}, inout={...}, src=..., funcs=..., name=...})``
+    and ``k:run(params [, {numWorkgroups=, workgroupSize=}])`` (``src/UserKernel.cpp:217-383``).
+    Argument types are ``'int'``, ``'float'`` and ``'ClTensor'`` / ``'torch.ClTensor'``."""
+
+    _TYPES = {"int": 0, "float": 1, "ClTensor": 2, "torch.ClTensor": 2}
+
+    def __init__(self, spec: dict):
+        if not isinstance(spec, dict):
+            raise ClError("First parameter to torch.ClKernel should be a table")
+        unknown = set(spec) - {"input", "output", "inout", "src", "funcs", "name"}
+        if unknown:
+            raise ClError(f"Parameter {sorted(unknown)[0]} not recognized")
+        self._args = []
+        for direction, key in ((0, "input"), (1, "output"), (2, "inout")):
+            for name, typename in (spec.get(key) or {}).items():
+                if typename not in self._TYPES:
+                    raise ClError(f"Unrecognized typename {typename}")
+                self._args.append((name, self._TYPES[typename], direction))
+        n = len(self._args)
+        names = (C.c_char_p * max(n, 1))(*[a[0].encode() for a in self._args])
+        types = (C.c_int * max(n, 1))(*[a[1] for a in self._args])
+        dirs = (C.c_int * max(n, 1))(*[a[2] for a in self._args])
+        name = spec.get("name")
+        funcs = spec.get("funcs")
+        self._lib = state().lib
+        self._h = _call("THClKernel_new", name.encode() if name else None, (spec.get("src") or "").encode(),
+                        funcs.encode() if funcs else None, C.c_int(n), names, types, dirs)
+        if not self._h:
+            raise ClError("kernel construction failed")
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                self._lib.THClKernel_free(None, self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    def getRenderedKernel(self) -> str:
+        return self._lib.THClKernel_getRenderedKernel(self._h).decode()
+
+    def run(self, params: dict, options: Optional[dict] = None) -> None:
+        options = options or {}
+        unknown = set(options) - {"numWorkgroups", "workgroupSize"}
+        if unknown:
+            raise ClError(f"option {sorted(unknown)[0]} not recognized")
+        n = len(self._args)
+        ints, floats = (C.c_int * max(n, 1))(), (C.c_float * max(n, 1))()
+        tensors = (C.c_void_p * max(n, 1))()
+        for i, (name, typ, _) in enumerate(self._args):
+            if name not in params:
+                raise ClError(f"missing value for parameter {name}")
+            v = params[name]
+            if typ == 2:
+                if not isinstance(v, ClTensor):
+                    raise ClError(f"parameter {name} must be a ClTensor")
+                tensors[i] = v._h
+            elif typ == 0:
+                ints[i] = int(v)
+            else:
+                floats[i] = float(v)
+        _call("THClKernel_run", self._h, ints, floats, tensors, C.c_long(int(options.get("numWorkgroups", 0))),
+              C.c_long(int(options.get("workgroupSize", 0))))
+

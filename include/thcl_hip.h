@@ -403,6 +403,33 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
 void THClBlas_ger(THClState *state, long m, long n, float alpha, THClTensor *x, long incx, THClTensor *y, long incy,
                   THClTensor *a, long lda);
 
+/* ------------------------------------------------------------------------- */
+/* User kernels compiled at run time: the C side of torch.ClKernel.  The      */
+/* reference offers this to Lua only (src/UserKernel.cpp:217-383); these       */
+/* entry points carry what its constructor and run() read from Lua tables.    */
+/* ------------------------------------------------------------------------- */
+typedef struct THClKernel THClKernel;
+enum { THCL_KARG_INT = 0, THCL_KARG_FLOAT = 1, THCL_KARG_TENSOR = 2 };
+enum { THCL_KDIR_INPUT = 0, THCL_KDIR_OUTPUT = 1, THCL_KDIR_INOUT = 2 };
+/* `src` is the kernel body in OpenCL C as the reference's users write it
+ * (get_global_id(0), NAME_data[..], NAME_info->offset, barrier(...)); `funcs`
+ * optional helper functions placed ahead of the kernel; `name` NULL for
+ * "user_kernel".  A tensor argument NAME appears in the body as
+ * `struct THClTensorInfoCl *NAME_info` and `float *NAME_data` (first element of
+ * the storage).  Returns NULL after reporting an error. */
+THClKernel *THClKernel_new(THClState *state, const char *name, const char *src, const char *funcs, int nargs,
+                           const char *const *arg_names, const int *arg_types, const int *arg_dirs);
+void THClKernel_free(THClState *state, THClKernel *kernel);
+const char *THClKernel_getRenderedKernel(THClKernel *kernel);
+int THClKernel_numArgs(THClKernel *kernel);
+/* Values by argument position (entries of the other two arrays are ignored
+ * for that position).  numWorkgroups / workgroupSize <= 0 select the
+ * reference's defaults: groups of 64 covering the first output or inout
+ * tensor's elements.  Compilation happens on a kernel's first run per device. */
+void THClKernel_run(THClState *state, THClKernel *kernel, const int *ints, const float *floats,
+                    THClTensor *const *tensors, long numWorkgroups, long workgroupSize);
+int THClKernel_compileCheck(THClKernel *kernel, const char *arch, size_t *code_bytes);
+
 #ifdef __cplusplus
 }
 #endif

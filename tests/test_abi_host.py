@@ -251,3 +251,25 @@ def test_planner_picks_the_kernel_family_for_each_layout(lib):
     assert _plan(lib, [((3, 4), (4, 1), 0)])[0] == "dense128"
     # tiny transposed operands are not worth a tile
     assert _plan(lib, [((8, 8), (8, 1), 0), ((8, 8), (1, 8), 0)])[0] == "joint32"
+
+
+def test_user_kernel_renders_and_compiles_for_gfx950(lib):
+    """The reference's README kernel (README.md:135-160) through THClKernel_new, compiled offline."""
+    lib.THClKernel_new.restype = C.c_void_p
+    lib.THClKernel_new.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_char_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.THClKernel_getRenderedKernel.restype = C.c_char_p
+    lib.THClKernel_getRenderedKernel.argtypes = [C.c_void_p]
+    lib.THClKernel_compileCheck.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_size_t)]
+    lib.THClKernel_free.argtypes = [C.c_void_p, C.c_void_p]
+    names = (C.c_char_p * 3)(b"input", b"nElements", b"output")
+    types, dirs = (C.c_int * 3)(2, 0, 2), (C.c_int * 3)(0, 0, 1)
+    src = b"int linearId = get_global_id(0); if(linearId < nElements) { output_data[linearId] = input_data[linearId] + 3.0f; }"
+    k = lib.THClKernel_new(None, None, src, None, 3, names, types, dirs)
+    assert k
+    text = lib.THClKernel_getRenderedKernel(k).decode()
+    assert "void user_kernel(" in text and "const float *input_data" in text and "int nElements" in text
+    size = C.c_size_t(0)
+    assert lib.THClKernel_compileCheck(k, b"gfx950", C.byref(size)) == 0, lib.thcl_rt_error().decode()
+    assert size.value > 1000
+    lib.THClKernel_free(None, k)
+
