@@ -1,0 +1,587 @@
+// Indexed movement: indexSelect / indexCopy / indexFill along a dimension,
+// gather / scatter / scatterFill, maskedSelect / maskedCopy.
+//
+// What it replaces (reference): src/lib/THClTensorIndex.cpp:16-330 (one thread
+// per slice position looping over the whole index vector), src/lib/THClGather.cpp,
+// src/lib/THClScatter.cpp (one thread per index element, per-element div/mod
+// over every dim) and src/lib/THClTensorMasked.cpp:126-246 (maskedSelect through
+// boost::compute, maskedCopy left unimplemented).
+//
+// Indices are 1-based floats held in a ClTensor, the reference's convention.
+// The indexed tensor is taken as dense [O][N][I] around the dimension; one
+// thread moves one unit (4 adjacent floats along I where alignment allows), so
+// accesses coalesce along I and the index vector is read from cache.  An index
+// outside 1..N moves nothing (the reference reads or writes out of bounds).
+// All of it is bound by HBM.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "apply_device.h"
+#include "internal.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct IndexParams {
+  float *a;            // the tensor indexed along its dim: [O][N][I]
+  float *b;            // the other one: [O][M][I]
+  const float *index;  // [M] (select / copy / fill) or [O][M][I] (gather / scatter)
+  int *winner;         // indexCopy: for every target slice, the last position of the index vector naming it
+  ThclDivisor units_i, m;  // units along I, entries along the dim
+  thcl_u32 total;      // units in [O][M][I]
+  thcl_u32 N, M, I;
+  float value;
+};
+
+enum Mode { SELECT = 0, COPY = 1, FILL = 2, GATHER = 3, SCATTER = 4, SCATTER_FILL = 5 };
+
+// For duplicate targets the sequential CPU loop leaves the last source slice;
+// winner[j] = max position i with index[i] == j + 1 reproduces that in parallel.
+__global__ __launch_bounds__(kThreads) void index_winner(IndexParams P) {
+  const thcl_u32 i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= P.M) return;
+  const long j = (long)P.index[i] - 1;
+  if (j >= 0 && j < (long)P.N) atomicMax(P.winner + j, (int)i);
+}
+
+template <int MODE, int VEC>
+__global__ __launch_bounds__(kThreads) void index_move(IndexParams P) {
+  typedef typename ThclVec<VEC == 4 ? 4 : 2>::T V4;  // only used when VEC == 4
+  const thcl_u32 e = blockIdx.x * kThreads + threadIdx.x;
+  if (e >= P.total) return;
+  // e -> (o, i, unit along I)
+  const thcl_u32 q = thcl_div(e, P.units_i);
+  const thcl_u32 ku = e - q * P.units_i.d;
+  const thcl_u32 o = thcl_div(q, P.m);
+  const thcl_u32 i = q - o * P.m.d;
+  const thcl_u64 k = (thcl_u64)ku * VEC;
+  const thcl_u64 boff = ((thcl_u64)o * P.M + i) * P.I + k;  // position in [O][M][I]
+  if (MODE == GATHER || MODE == SCATTER || MODE == SCATTER_FILL) {
+    // one index per element
+#pragma unroll
+    for (int c = 0; c < VEC; c++) {
+      const long j = (long)P.index[boff + c] - 1;
+      if (j < 0 || j >= (long)P.N) continue;
+      const thcl_u64 aoff = ((thcl_u64)o * P.N + (thcl_u64)j) * P.I + k + c;
+      if (MODE == GATHER) P.b[boff + c] = P.a[aoff];
+      else if (MODE == SCATTER) P.a[aoff] = P.b[boff + c];
+      else P.a[aoff] = P.value;
+    }
+    return;
+  }
+  const long j = (long)P.index[i] - 1;
+  if (j < 0 || j >= (long)P.N) return;
+  if (MODE == COPY && P.winner[j] != (int)i) return;
+  const thcl_u64 aoff = ((thcl_u64)o * P.N + (thcl_u64)j) * P.I + k;
+  if (VEC == 4) {
+    if (MODE == SELECT) __builtin_nontemporal_store(*(const V4 *)(P.a + aoff), (V4 *)(P.b + boff));
+    else if (MODE == COPY) *(V4 *)(P.a + aoff) = __builtin_nontemporal_load((const V4 *)(P.b + boff));
+    else {
+      V4 v;
+      v[0] = v[1] = v[2] = v[3] = P.value;
+      *(V4 *)(P.a + aoff) = v;
+    }
+  } else {
+    if (MODE == SELECT) P.b[boff] = P.a[aoff];
+    else if (MODE == COPY) P.a[aoff] = P.b[boff];
+    else P.a[aoff] = P.value;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void fill_int(int *p, int v, thcl_u32 n) {
+  const thcl_u32 i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// ---------------------------------------------------------------- masked ---
+// Stream compaction in three passes over blocks of kChunk elements: count the
+// selected elements of every block, turn the counts into offsets (one block,
+// the list is short), then every block re-derives its elements' ranks and moves them.
+constexpr int kPer = 16, kChunk = kThreads * kPer;
+
+struct MaskParams {
+  const float *mask;
+  const float *src;   // select: [n] values; copy: the packed source
+  float *dst;         // select: packed output; copy: [n] destination
+  unsigned *counts;   // per block, then exclusive offsets; counts[nblocks] = total
+  thcl_u64 n;
+  thcl_u32 nblocks;
+  thcl_u64 src_len;   // copy: elements available in src
+};
+
+__device__ __forceinline__ unsigned block_exclusive(unsigned v, unsigned *lds, unsigned *total) {
+  // exclusive prefix of v over the block's threads
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  unsigned incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const unsigned up = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += up;
+  }
+  __syncthreads();
+  if (lane == 63) lds[wave] = incl;
+  __syncthreads();
+  unsigned before = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < kThreads / 64; w++) {
+    if (w < wave) before += lds[w];
+    all += lds[w];
+  }
+  *total = all;
+  return before + incl - v;
+}
+
+__global__ __launch_bounds__(kThreads) void mask_count(MaskParams P) {
+  __shared__ unsigned lds[kThreads / 64];
+  const thcl_u64 base = (thcl_u64)blockIdx.x * kChunk;
+  unsigned c = 0;
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    const thcl_u64 i = base + (thcl_u64)k * kThreads + threadIdx.x;
+    if (i < P.n) c += (__builtin_nontemporal_load(P.mask + i) != 0.0f) ? 1u : 0u;
+  }
+  unsigned total;
+  (void)block_exclusive(c, lds, &total);
+  if (threadIdx.x == 0) P.counts[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(1024) void mask_offsets(MaskParams P) {
+  __shared__ unsigned lds[1024 / 64];
+  __shared__ unsigned carry_s;
+  if (threadIdx.x == 0) carry_s = 0;
+  __syncthreads();
+  for (thcl_u32 base = 0; base < P.nblocks; base += 1024) {
+    const thcl_u32 i = base + threadIdx.x;
+    const unsigned v = i < P.nblocks ? P.counts[i] : 0u;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    unsigned incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const unsigned up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) lds[wave] = incl;
+    __syncthreads();
+    unsigned before = carry_s, all = 0;
+    for (int w = 0; w < 1024 / 64; w++) {
+      if (w < wave) before += lds[w];
+      all += lds[w];
+    }
+    if (i < P.nblocks) P.counts[i] = before + incl - v;
+    __syncthreads();
+    if (threadIdx.x == 0) carry_s += all;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) P.counts[P.nblocks] = carry_s;
+}
+
+// COPY false: dst[rank] = src[i] for selected i.  COPY true: dst[i] = src[rank].
+template <bool COPY>
+__global__ __launch_bounds__(kThreads) void mask_move(MaskParams P) {
+  __shared__ unsigned lds[kThreads / 64];
+  // a thread owns kPer consecutive elements so ranks follow element order
+  const thcl_u64 first = (thcl_u64)blockIdx.x * kChunk + (thcl_u64)threadIdx.x * kPer;
+  float m[kPer];
+  unsigned c = 0;
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    m[k] = (first + k < P.n) ? P.mask[first + k] : 0.0f;
+    c += (m[k] != 0.0f) ? 1u : 0u;
+  }
+  unsigned total;
+  unsigned rank = P.counts[blockIdx.x] + block_exclusive(c, lds, &total);
+#pragma unroll
+  for (int k = 0; k < kPer; k++) {
+    if (m[k] != 0.0f) {
+      if (COPY) {
+        if (rank < P.src_len) P.dst[first + k] = P.src[rank];
+      } else {
+        P.dst[rank] = P.src[first + k];
+      }
+      rank++;
+    }
+  }
+}
+
+void check(const char *what) {
+  hipError_t e = hipGetLastError();
+  THCL_CHECK(e == hipSuccess, "%s launch failed: %s", what, hipGetErrorString(e));
+}
+bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+
+struct Dense {  // a dense stand-in for a tensor that kernels write or read
+  THClState *state;
+  THClTensor *orig, *t;
+  bool write_back;
+  Dense(THClState *s, THClTensor *x, bool load, bool store) : state(s), orig(x), t(x), write_back(false) {
+    if (!THClTensor_isContiguous(s, x)) {
+      if (load) {
+        t = THClTensor_newContiguous(s, x);
+      } else {
+        t = THClTensor_newv2(s, THClTensor_getDevice(s, x));
+        THClTensor_resizeAs(s, t, x);
+      }
+      write_back = store;
+    }
+  }
+  void finish() {
+    if (t != orig) {
+      if (write_back) THClTensor_freeCopyTo(state, t, orig);
+      else THClTensor_free(state, t);
+      t = orig;
+    }
+  }
+  ~Dense() {
+    if (t != orig) THClTensor_free(state, t);  // error path: drop the stand-in
+  }
+};
+
+template <int MODE>
+void launch_move(hipStream_t stream, IndexParams &P, bool vec_ok) {
+  const bool vec = vec_ok && MODE != GATHER && MODE != SCATTER && MODE != SCATTER_FILL && (P.I % 4 == 0) &&
+                   aligned16(P.a) && (MODE == FILL || aligned16(P.b));
+  const thcl_u64 units_i = vec ? P.I / 4 : P.I;
+  const thcl_u64 total = (thcl_u64)units_i * P.M * (P.total /* O */);
+  THCL_CHECK(total < (1ull << 31), THCL_DIM_WARNING);
+  P.units_i = thcl_make_divisor((long)units_i);
+  P.m = thcl_make_divisor((long)P.M);
+  P.total = (thcl_u32)total;
+  if (total == 0) return;
+  const dim3 grid((unsigned)((total + kThreads - 1) / kThreads)), block(kThreads);
+  if (vec) hipLaunchKernelGGL((index_move<MODE, 4>), grid, block, 0, stream, P);
+  else hipLaunchKernelGGL((index_move<MODE, 1>), grid, block, 0, stream, P);
+  check("index kernel");
+}
+
+// sizes of `t` around `dim`
+void split_dims(THClTensor *t, int dim, long &O, long &N, long &I) {
+  O = I = 1;
+  for (int d = 0; d < dim; d++) O *= t->size[d];
+  for (int d = dim + 1; d < t->nDimension; d++) I *= t->size[d];
+  N = t->size[dim];
+}
+
+void index_checks(THClState *state, THClTensor *indices, THClTensor *t, int dim) {
+  THCL_ARGCHECK(indices->nDimension == 1, 3, "expecting vector of indices");
+  THCL_ARGCHECK(t->nDimension > 0, 2, "Source tensor is empty");
+  THCL_ARGCHECK(dim >= 0 && dim < t->nDimension, 4, "Indexing dim is out of bounds");
+  (void)state;
+}
+}  // namespace
+
+extern "C" {
+
+// res = src with its `dim` replaced by the slices index names (src/lib/THClTensorIndex.cpp:186-256)
+void THClTensor_indexSelect(THClState *state, THClTensor *res_, THClTensor *src, int dim, THClTensor *indices) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, res_, src, indices);
+  index_checks(state, indices, src, dim);
+  THCL_CHECK(res_ != src, "result and source must be different tensors");
+  const long M = indices->size[0];
+  long osz[THCL_MAX_DIMS];
+  for (int d = 0; d < src->nDimension; d++) osz[d] = (d == dim) ? M : src->size[d];
+  THLongStorage shape;
+  memset(&shape, 0, sizeof(shape));
+  shape.data = osz;
+  shape.size = src->nDimension;
+  THClTensor_resize(state, res_, &shape, nullptr);
+  Dense s(state, src, true, false), r(state, res_, false, true), ix(state, indices, true, false);
+  long O, N, I;
+  split_dims(src, dim, O, N, I);
+  THCL_CHECK(N < (1l << 31) && M < (1l << 31) && I < (1l << 31) && O < (1l << 31), THCL_DIM_WARNING);
+  thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, src));
+  IndexParams P;
+  memset(&P, 0, sizeof(P));
+  P.a = thcl_dptr(s.t);
+  P.b = thcl_dptr(r.t);
+  P.index = thcl_dptr(ix.t);
+  P.N = (thcl_u32)N;
+  P.M = (thcl_u32)M;
+  P.I = (thcl_u32)I;
+  P.total = (thcl_u32)O;
+  if (O * M * I > 0) launch_move<SELECT>((hipStream_t)thcl_rt_stream(rt), P, true);
+  thcl_after_launch(state, rt);
+  s.finish();
+  ix.finish();
+  r.finish();
+  THCL_GUARD_END()
+}
+
+// res[.., index[i], ..] = src[.., i, ..]; for a repeated target the last i wins, as in
+// the sequential CPU loop (src/lib/THClTensorIndex.cpp:32-88)
+void THClTensor_indexCopy(THClState *state, THClTensor *res_, int dim, THClTensor *indices, THClTensor *src) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, res_, src, indices);
+  index_checks(state, indices, src, dim);
+  THCL_ARGCHECK(dim < res_->nDimension, 4, "Indexing dim is out of bounds");
+  THCL_ARGCHECK(indices->size[0] == src->size[dim], 4, "length of src.size[dim] is not equal to length of indices");
+  THCL_ARGCHECK(res_->nDimension == src->nDimension, 2, "result and source differ in dimensions");
+  for (int d = 0; d < src->nDimension; d++)
+    if (d != dim) THCL_ARGCHECK(res_->size[d] == src->size[d], 2, "result and source sizes differ outside the indexed dim");
+  THCL_CHECK(res_ != src, "result and source must be different tensors");
+  Dense s(state, src, true, false), r(state, res_, true, true), ix(state, indices, true, false);
+  long O, N, I, M = indices->size[0];
+  split_dims(res_, dim, O, N, I);
+  THCL_CHECK(N < (1l << 31) && M < (1l << 31) && I < (1l << 31) && O < (1l << 31), THCL_DIM_WARNING);
+  thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, res_));
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  IndexParams P;
+  memset(&P, 0, sizeof(P));
+  P.a = thcl_dptr(r.t);
+  P.b = thcl_dptr(s.t);
+  P.index = thcl_dptr(ix.t);
+  P.N = (thcl_u32)N;
+  P.M = (thcl_u32)M;
+  P.I = (thcl_u32)I;
+  P.total = (thcl_u32)O;
+  if (O * M * I > 0 && N > 0) {
+    P.winner = (int *)thcl_rt_workspace(rt, (size_t)N * sizeof(int));
+    THCL_CHECK(P.winner != nullptr, "%s", thcl_rt_error());
+    hipLaunchKernelGGL(fill_int, dim3((unsigned)((N + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P.winner, -1,
+                       (thcl_u32)N);
+    hipLaunchKernelGGL(index_winner, dim3((unsigned)((M + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P);
+    check("index winners");
+    launch_move<COPY>(stream, P, true);
+  }
+  thcl_after_launch(state, rt);
+  s.finish();
+  ix.finish();
+  r.finish();
+  THCL_GUARD_END()
+}
+
+// (src/lib/THClTensorIndex.cpp:104-168)
+void THClTensor_indexFill(THClState *state, THClTensor *res_, int dim, THClTensor *indices, float val) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 2, res_, indices);
+  THCL_ARGCHECK(indices->nDimension == 1, 3, "Index is supposed to be a vector");
+  THCL_ARGCHECK(res_->nDimension > 0, 2, "Source tensor is empty");
+  THCL_ARGCHECK(dim >= 0 && dim < res_->nDimension, 4, "Indexing dim is out of bounds");
+  Dense r(state, res_, true, true), ix(state, indices, true, false);
+  long O, N, I, M = indices->size[0];
+  split_dims(res_, dim, O, N, I);
+  THCL_CHECK(N < (1l << 31) && M < (1l << 31) && I < (1l << 31) && O < (1l << 31), THCL_DIM_WARNING);
+  thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, res_));
+  IndexParams P;
+  memset(&P, 0, sizeof(P));
+  P.a = thcl_dptr(r.t);
+  P.index = thcl_dptr(ix.t);
+  P.N = (thcl_u32)N;
+  P.M = (thcl_u32)M;
+  P.I = (thcl_u32)I;
+  P.total = (thcl_u32)O;
+  P.value = val;
+  if (O * M * I > 0) launch_move<FILL>((hipStream_t)thcl_rt_stream(rt), P, true);
+  thcl_after_launch(state, rt);
+  ix.finish();
+  r.finish();
+  THCL_GUARD_END()
+}
+
+// host index vectors: uploaded as floats, like the reference (src/lib/THClTensorIndex.cpp:16-30,90-102,170-184)
+static THClTensor *upload_indices(THClState *state, int device, THLongTensor *indices) {
+  THCL_ARGCHECK(indices->nDimension == 1, 3, "expecting vector of indices");
+  THClTensor *t = THClTensor_newWithSize1d(state, device, indices->size[0]);
+  THClTensor_copyLong(state, t, indices);
+  return t;
+}
+void THClTensor_indexSelect_long(THClState *state, THClTensor *res_, THClTensor *src, int dim, THLongTensor *indices) {
+  THCL_GUARD_BEGIN
+  THClTensor *ix = upload_indices(state, THClTensor_getDevice(state, src), indices);
+  THClTensor_indexSelect(state, res_, src, dim, ix);
+  THClTensor_free(state, ix);
+  THCL_GUARD_END()
+}
+void THClTensor_indexCopy_long(THClState *state, THClTensor *res_, int dim, THLongTensor *indices, THClTensor *src) {
+  THCL_GUARD_BEGIN
+  THClTensor *ix = upload_indices(state, THClTensor_getDevice(state, src), indices);
+  THClTensor_indexCopy(state, res_, dim, ix, src);
+  THClTensor_free(state, ix);
+  THCL_GUARD_END()
+}
+void THClTensor_indexFill_long(THClState *state, THClTensor *res_, int dim, THLongTensor *indices, float val) {
+  THCL_GUARD_BEGIN
+  THClTensor *ix = upload_indices(state, THClTensor_getDevice(state, res_), indices);
+  THClTensor_indexFill(state, res_, dim, ix, val);
+  THClTensor_free(state, ix);
+  THCL_GUARD_END()
+}
+
+// ------------------------------------------------------- gather / scatter ---
+static void gather_scatter_checks(THClState *state, THClTensor *full, THClTensor *index, THClTensor *other, long dim) {
+  const int nd = index->nDimension;
+  THCL_ARGCHECK(nd >= 1, 2, "index tensor is empty");
+  THCL_ARGCHECK(full->nDimension == nd, 2, "All tensors should have same number of dims");
+  THCL_ARGCHECK(other == nullptr || other->nDimension == nd, 4, "All tensors should have same number of dims");
+  THCL_ARGCHECK(dim >= 0 && dim < nd, 4, "dim out of bounds");
+  for (int d = 0; d < nd; d++) {
+    if (d != dim)
+      THCL_CHECK(full->size[d] == index->size[d],
+                 "index tensor must have same dimensions as source tensor, but dimension %d doesnt match", d);
+    if (other) THCL_CHECK(other->size[d] == index->size[d], "index and value tensors differ in dimension %d", d);
+  }
+  (void)state;
+}
+
+static void run_gather_scatter(THClState *state, int mode, THClTensor *full, THClTensor *index, THClTensor *other,
+                               long dim, float value) {
+  long O, N, I;
+  split_dims(full, (int)dim, O, N, I);
+  const long M = index->size[dim];
+  THCL_CHECK(N < (1l << 31) && M < (1l << 31) && I < (1l << 31) && O < (1l << 31), THCL_DIM_WARNING);
+  thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, full));
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  IndexParams P;
+  memset(&P, 0, sizeof(P));
+  P.a = thcl_dptr(full);
+  P.b = other ? thcl_dptr(other) : nullptr;
+  P.index = thcl_dptr(index);
+  P.N = (thcl_u32)N;
+  P.M = (thcl_u32)M;
+  P.I = (thcl_u32)I;
+  P.total = (thcl_u32)O;
+  P.value = value;
+  if (O * M * I > 0) {
+    if (mode == GATHER) launch_move<GATHER>(stream, P, false);
+    else if (mode == SCATTER) launch_move<SCATTER>(stream, P, false);
+    else launch_move<SCATTER_FILL>(stream, P, false);
+  }
+  thcl_after_launch(state, rt);
+}
+
+// self[i][j][k] = src[index[i][j][k]][j][k] for dim 0, likewise for the others
+// (src/lib/THClGather.cpp:17-78); self takes the index tensor's shape
+void THClTensor_gather(THClState *state, THClTensor *self, THClTensor *src, long dim, THClTensor *index) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, self, src, index);
+  gather_scatter_checks(state, src, index, nullptr, dim);
+  THCL_CHECK(self != src && self != index, "result cannot alias the source or the index");
+  THClTensor_resizeAs(state, self, index);
+  Dense s(state, src, true, false), r(state, self, false, true), ix(state, index, true, false);
+  run_gather_scatter(state, GATHER, s.t, ix.t, r.t, dim, 0.f);
+  s.finish();
+  ix.finish();
+  r.finish();
+  THCL_GUARD_END()
+}
+// self[index[i][j][k]][j][k] = src[i][j][k]; targets named twice keep either writer
+// (src/lib/THClScatter.cpp:15-80)
+void THClTensor_scatter(THClState *state, THClTensor *self, long dim, THClTensor *index, THClTensor *src) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, self, src, index);
+  gather_scatter_checks(state, self, index, src, dim);
+  THCL_ARGCHECK(self != index, 1, "self cannot alias index");
+  THCL_ARGCHECK(self != src, 1, "self cannot alias src");
+  Dense s(state, src, true, false), r(state, self, true, true), ix(state, index, true, false);
+  run_gather_scatter(state, SCATTER, r.t, ix.t, s.t, dim, 0.f);
+  s.finish();
+  ix.finish();
+  r.finish();
+  THCL_GUARD_END()
+}
+void THClTensor_scatterFill(THClState *state, THClTensor *self, long dim, THClTensor *index, float val) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 2, self, index);
+  gather_scatter_checks(state, self, index, nullptr, dim);
+  THCL_ARGCHECK(self != index, 1, "self cannot alias index");
+  Dense r(state, self, true, true), ix(state, index, true, false);
+  run_gather_scatter(state, SCATTER_FILL, r.t, ix.t, nullptr, dim, val);
+  ix.finish();
+  r.finish();
+  THCL_GUARD_END()
+}
+
+// ------------------------------------------------------------- masked ---
+static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long n) {
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  const long nb = (n + kChunk - 1) / kChunk;
+  THCL_CHECK(nb < (1l << 31) - 1, THCL_DIM_WARNING);
+  P.n = (thcl_u64)n;
+  P.nblocks = (thcl_u32)nb;
+  P.counts = (unsigned *)thcl_rt_workspace(rt, (size_t)(nb + 1) * sizeof(unsigned));
+  THCL_CHECK(P.counts != nullptr, "%s", thcl_rt_error());
+  hipLaunchKernelGGL(mask_count, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
+  check("mask count");
+  hipLaunchKernelGGL(mask_offsets, dim3(1), dim3(1024), 0, stream, P);
+  check("mask offsets");
+  (void)state;
+  return P.counts;
+}
+
+static long read_total(thcl_rt *rt, const unsigned *counts, thcl_u32 nblocks) {
+  float *hw = thcl_rt_host_word(rt);  // a pinned 4-byte word: carries the count's bits
+  THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, counts + nblocks, sizeof(unsigned)) == 0, "%s", thcl_rt_error());
+  unsigned total;
+  memcpy(&total, hw, sizeof(total));
+  return (long)total;
+}
+
+// tensor = the elements of src whose mask entry is non-zero, in order, as a vector
+// (src/lib/THClTensorMasked.cpp:193-246)
+void THClTensor_maskedSelect(THClState *state, THClTensor *tensor, THClTensor *src, THClTensor *mask) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, tensor, src, mask);
+  const long n = THClTensor_nElement(state, mask);
+  THCL_ARGCHECK(n == THClTensor_nElement(state, src), 2, "sizes do not match");
+  THCL_CHECK(tensor != src && tensor != mask, "result cannot alias the source or the mask");
+  const int device = THClTensor_getDevice(state, src);
+  if (tensor->nDimension < 0 && !tensor->storage) tensor->device = device;
+  if (n == 0) {
+    THClTensor_resize1d(state, tensor, 0);
+    return;
+  }
+  Dense s(state, src, true, false), m(state, mask, true, false);
+  thcl_rt *rt = thcl_ctx(state, device);
+  MaskParams P;
+  memset(&P, 0, sizeof(P));
+  P.mask = thcl_dptr(m.t);
+  P.src = thcl_dptr(s.t);
+  mask_prefix(state, rt, P, n);
+  const long total = read_total(rt, P.counts, P.nblocks);  // the one synchronising step: the result's size
+  THClTensor_resize1d(state, tensor, total);
+  if (total > 0) {
+    Dense r(state, tensor, false, true);
+    P.dst = thcl_dptr(r.t);
+    hipLaunchKernelGGL((mask_move<false>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
+    check("masked select");
+    thcl_after_launch(state, rt);
+    r.finish();
+  }
+  s.finish();
+  m.finish();
+  THCL_GUARD_END()
+}
+
+// tensor[i] = next element of src, for every i whose mask entry is non-zero
+// (declared at src/lib/THClTensorMath.h:113; the reference's body stops at
+// THError("Not implemented"), src/lib/THClTensorMasked.cpp:126-191)
+void THClTensor_maskedCopy(THClState *state, THClTensor *tensor, THClTensor *mask, THClTensor *src) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 3, tensor, src, mask);
+  const long n = THClTensor_nElement(state, mask);
+  THCL_ARGCHECK(n == THClTensor_nElement(state, tensor), 2, "mask and tensor must have the same number of elements");
+  THCL_CHECK(tensor != src && tensor != mask, "tensor cannot alias the source or the mask");
+  if (n == 0) return;
+  Dense s(state, src, true, false), m(state, mask, true, false), r(state, tensor, true, true);
+  thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, tensor));
+  MaskParams P;
+  memset(&P, 0, sizeof(P));
+  P.mask = thcl_dptr(m.t);
+  P.src = thcl_dptr(s.t);
+  P.dst = thcl_dptr(r.t);
+  P.src_len = (thcl_u64)THClTensor_nElement(state, src);
+  mask_prefix(state, rt, P, n);
+  hipLaunchKernelGGL((mask_move<true>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
+  check("masked copy");
+  const long total = read_total(rt, P.counts, P.nblocks);
+  thcl_after_launch(state, rt);
+  s.finish();
+  m.finish();
+  r.finish();
+  THCL_ARGCHECK(total <= (long)P.src_len, 2, "source nElements must be == mask `1` elements");
+  THCL_GUARD_END()
+}
+
+}  // extern "C"

@@ -87,6 +87,28 @@ def _long_storage(values: Sequence[int]):
     return s
 
 
+class _LongStorageStruct(C.Structure):
+    _fields_ = [("data", C.POINTER(C.c_long)), ("size", C.c_long)]
+
+
+class _LongTensorStruct(C.Structure):  # THLongTensor: size*, stride*, int nDimension, storage*
+    _fields_ = [("size", C.c_void_p), ("stride", C.c_void_p), ("nDimension", C.c_int),
+                ("storage", C.POINTER(_LongStorageStruct))]
+
+
+def _long_vector(values):
+    """A host ``torch.LongTensor`` vector holding ``values``; the caller frees it."""
+    lib = state().lib
+    vals = np.asarray(values, dtype=np.int64).reshape(-1)
+    sz = _long_storage([vals.size])
+    lt = lib.THLongTensor_newWithSize(sz, None)
+    lib.THLongStorage_free(sz)
+    if vals.size:
+        t = C.cast(lt, C.POINTER(_LongTensorStruct)).contents
+        np.ctypeslib.as_array(t.storage.contents.data, shape=(vals.size,))[:] = vals
+    return lt
+
+
 class ClTensor:
     """``torch.ClTensor``: a strided fp32 view of device storage."""
 
@@ -537,14 +559,7 @@ class ClTensor:
         values = ClTensor()
         try:
             _call(f"THClTensor_{cfn}", values._h, lt, self._h, C.c_long(dim - 1))
-            # THLongTensor: size*, stride*, int nDimension, storage* -> storage->data
-            class _LS(C.Structure):
-                _fields_ = [("data", C.POINTER(C.c_long)), ("size", C.c_long)]
-
-            class _LT(C.Structure):
-                _fields_ = [("size", C.c_void_p), ("stride", C.c_void_p), ("nDimension", C.c_int),
-                            ("storage", C.POINTER(_LS))]
-            t = C.cast(lt, C.POINTER(_LT)).contents
+            t = C.cast(lt, C.POINTER(_LongTensorStruct)).contents
             n = int(np.prod(shape))
             idx.reshape(-1)[:] = np.ctypeslib.as_array(t.storage.contents.data, shape=(n,))
         finally:
@@ -569,6 +584,56 @@ class ClTensor:
         else:
             beta, alpha = nums[0], nums[1]
         _call("THClTensor_addmm", self._h, C.c_float(beta), t._h, C.c_float(alpha), m1._h, m2._h)
+        return self
+
+    # ---- indexed movement (dims and indices 1-based, as in Lua) ---------------------
+    def _with_index(self, cfn: str, index, call):
+        """Runs ``call(name, handle)`` with a device index tensor, or a host LongTensor
+        built from a list / integer array (the ``_long`` entry points)."""
+        if isinstance(index, ClTensor):
+            return call(f"THClTensor_{cfn}", index._h)
+        lt = _long_vector(index)
+        try:
+            return call(f"THClTensor_{cfn}_long", lt)
+        finally:
+            self._lib.THLongTensor_free(lt)
+
+    def index(self, *args) -> "ClTensor":
+        """``a:index(dim, idx)`` -> new tensor; ``res:index(a, dim, idx)``."""
+        res, src, dim, idx = (ClTensor(), self) + tuple(args) if len(args) == 2 else (self,) + tuple(args)
+        self._with_index("indexSelect", idx, lambda fn, h: _call(fn, res._h, src._h, C.c_int(dim - 1), h))
+        return res
+
+    def indexCopy(self, dim: int, idx, src: "ClTensor") -> "ClTensor":
+        self._with_index("indexCopy", idx, lambda fn, h: _call(fn, self._h, C.c_int(dim - 1), h, src._h))
+        return self
+
+    def indexFill(self, dim: int, idx, value: float) -> "ClTensor":
+        self._with_index("indexFill", idx, lambda fn, h: _call(fn, self._h, C.c_int(dim - 1), h, C.c_float(value)))
+        return self
+
+    def gather(self, *args) -> "ClTensor":
+        """``a:gather(dim, index)`` -> new tensor; ``res:gather(a, dim, index)``."""
+        res, src, dim, idx = (ClTensor(), self) + tuple(args) if len(args) == 2 else (self,) + tuple(args)
+        _call("THClTensor_gather", res._h, src._h, C.c_long(dim - 1), idx._h)
+        return res
+
+    def scatter(self, dim: int, index: "ClTensor", src) -> "ClTensor":
+        """``a:scatter(dim, index, src)`` with a tensor or a number."""
+        if isinstance(src, ClTensor):
+            _call("THClTensor_scatter", self._h, C.c_long(dim - 1), index._h, src._h)
+        else:
+            _call("THClTensor_scatterFill", self._h, C.c_long(dim - 1), index._h, C.c_float(src))
+        return self
+
+    def maskedSelect(self, *args) -> "ClTensor":
+        """``a:maskedSelect(mask)`` -> new vector; ``res:maskedSelect(a, mask)``."""
+        res, src, mask = (ClTensor(), self, args[0]) if len(args) == 1 else (self, args[0], args[1])
+        _call("THClTensor_maskedSelect", res._h, src._h, mask._h)
+        return res
+
+    def maskedCopy(self, mask: "ClTensor", src: "ClTensor") -> "ClTensor":
+        _call("THClTensor_maskedCopy", self._h, mask._h, src._h)
         return self
 
     def dot(self, other: "ClTensor") -> float:

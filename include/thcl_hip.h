@@ -404,6 +404,24 @@ void THClBlas_ger(THClState *state, long m, long n, float alpha, THClTensor *x, 
                   THClTensor *a, long lda);
 
 /* ------------------------------------------------------------------------- */
+/* Indexed movement (reference: src/lib/THClTensorMath.h:101-116,130-132).     */
+/* Index tensors hold 1-based positions as floats; `dim` is 0-based.  An       */
+/* index outside the dimension moves nothing.                                  */
+/* ------------------------------------------------------------------------- */
+void THClTensor_indexSelect(THClState *state, THClTensor *tensor, THClTensor *src, int dim, THClTensor *index);
+void THClTensor_indexCopy(THClState *state, THClTensor *res_, int dim, THClTensor *indices, THClTensor *src);
+void THClTensor_indexFill(THClState *state, THClTensor *tensor, int dim, THClTensor *index, float val);
+void THClTensor_indexSelect_long(THClState *state, THClTensor *tensor, THClTensor *src, int dim, THLongTensor *index);
+void THClTensor_indexCopy_long(THClState *state, THClTensor *res_, int dim, THLongTensor *indices, THClTensor *src);
+void THClTensor_indexFill_long(THClState *state, THClTensor *tensor, int dim, THLongTensor *index, float val);
+void THClTensor_gather(THClState *state, THClTensor *self, THClTensor *src, long dim, THClTensor *index);
+void THClTensor_scatter(THClState *state, THClTensor *self, long dim, THClTensor *index, THClTensor *src);
+void THClTensor_scatterFill(THClState *state, THClTensor *self, long dim, THClTensor *index, float val);
+/* mask: a ClTensor of 0 / non-0 with as many elements as the tensor it selects from */
+void THClTensor_maskedSelect(THClState *state, THClTensor *tensor, THClTensor *src, THClTensor *mask);
+void THClTensor_maskedCopy(THClState *state, THClTensor *tensor, THClTensor *mask, THClTensor *src);
+
+/* ------------------------------------------------------------------------- */
 /* User kernels compiled at run time: the C side of torch.ClKernel.  The      */
 /* reference offers this to Lua only (src/UserKernel.cpp:217-383); these       */
 /* entry points carry what its constructor and run() read from Lua tables.    */

@@ -141,3 +141,57 @@ def addmv(beta, t, alpha, mat, vec):
 def addr(beta, t, alpha, v1, v2):
     """beta * t + alpha * outer(v1, v2) in fp64 (src/lib/THClTensorMathBlas.cpp:216-277)."""
     return beta * np.asarray(t, dtype=np.float64) + alpha * np.outer(np.asarray(v1, dtype=np.float64), np.asarray(v2, dtype=np.float64))
+
+
+# ------------------------------------------------------------ indexed movement ---
+# Torch7 CPU semantics (TH's sequential loops) behind the entry points of
+# src/lib/THClTensorIndex.cpp, THClGather.cpp, THClScatter.cpp, THClTensorMasked.cpp.
+# Indices are 1-based.
+def index_select(src, dim, idx):
+    return np.take(_f(src), np.asarray(idx, dtype=np.int64) - 1, axis=dim)
+
+
+def index_copy(res, dim, idx, src):
+    """res[.., idx[i], ..] = src[.., i, ..] in order of i: a repeated target keeps the last."""
+    res = _f(res).copy()
+    src = _f(src)
+    for i, j in enumerate(np.asarray(idx, dtype=np.int64) - 1):
+        sl = [slice(None)] * res.ndim
+        sl[dim] = int(j)
+        ss = [slice(None)] * res.ndim
+        ss[dim] = i
+        res[tuple(sl)] = src[tuple(ss)]
+    return res
+
+
+def index_fill(res, dim, idx, value):
+    res = _f(res).copy()
+    for j in np.asarray(idx, dtype=np.int64) - 1:
+        sl = [slice(None)] * res.ndim
+        sl[dim] = int(j)
+        res[tuple(sl)] = F(value)
+    return res
+
+
+def gather(src, dim, index):
+    return np.take_along_axis(_f(src), np.asarray(index, dtype=np.int64) - 1, axis=dim)
+
+
+def scatter(res, dim, index, src):
+    """res[index[i][j][k]][j][k] = src[i][j][k] (dim 0); src may be a number."""
+    res = _f(res).copy()
+    index = np.asarray(index, dtype=np.int64) - 1
+    vals = np.broadcast_to(_f(src), index.shape)
+    np.put_along_axis(res, index, vals, axis=dim)
+    return res
+
+
+def masked_select(src, mask):
+    return _f(src).reshape(-1)[_f(mask).reshape(-1) != 0]
+
+
+def masked_copy(res, mask, src):
+    res = _f(res).copy()
+    sel = _f(mask).reshape(res.shape) != 0
+    res[sel] = _f(src).reshape(-1)[:int(sel.sum())]
+    return res

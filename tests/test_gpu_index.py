@@ -1,0 +1,156 @@
+"""indexSelect / indexCopy / indexFill, gather / scatter, maskedSelect /
+maskedCopy through the C ABI against oracle/catalogue.py.  Pure data movement:
+every comparison is bit for bit."""
+import numpy as np
+import pytest
+
+import oracle
+from oracle import catalogue as cat
+from gpu_util import Pair, assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+def _rng(seed):
+    return np.random.RandomState(seed)
+
+
+@pytest.mark.parametrize("shape,dim", [((7,), 0), ((50, 64), 0), ((50, 64), 1), ((33, 17), 0), ((33, 17), 1),
+                                       ((6, 40, 12), 1), ((5, 9, 260), 0), ((5, 9, 260), 2), ((3000, 128), 0),
+                                       ((2, 3, 4, 5), 2)])
+def test_index_select_copy_fill(cl, shape, dim):
+    n = int(np.prod(shape))
+    x = oracle.uniform(101, n).reshape(shape)
+    X = cl.ClTensor(x)
+    r = _rng(dim + n)
+    m = max(1, shape[dim] // 2 + 3)
+    idx = r.randint(1, shape[dim] + 1, size=m)                      # repeats allowed
+    # select: device float indices, host long indices
+    want = cat.index_select(x, dim, idx)
+    assert_bit_equal(X.index(dim + 1, cl.ClTensor(idx.astype(F))).float(), want, "indexSelect")
+    assert_bit_equal(X.index(dim + 1, idx.tolist()).float(), want, "indexSelect_long")
+    # copy: repeated targets keep the last source slice
+    srcshape = list(shape)
+    srcshape[dim] = m
+    src = oracle.uniform(102, int(np.prod(srcshape))).reshape(srcshape)
+    R = cl.ClTensor(x)
+    R.indexCopy(dim + 1, cl.ClTensor(idx.astype(F)), cl.ClTensor(src))
+    assert_bit_equal(R.float(), cat.index_copy(x, dim, idx, src), "indexCopy")
+    R2 = cl.ClTensor(x)
+    R2.indexCopy(dim + 1, idx, cl.ClTensor(src))
+    assert_bit_equal(R2.float(), cat.index_copy(x, dim, idx, src), "indexCopy_long")
+    # fill
+    R3 = cl.ClTensor(x)
+    R3.indexFill(dim + 1, cl.ClTensor(idx.astype(F)), -7.0)
+    assert_bit_equal(R3.float(), cat.index_fill(x, dim, idx, -7.0), "indexFill")
+    R4 = cl.ClTensor(x)
+    R4.indexFill(dim + 1, idx[:1], 3.0)
+    assert_bit_equal(R4.float(), cat.index_fill(x, dim, idx[:1], 3.0), "indexFill_long")
+
+
+def test_index_ops_on_views_and_bad_arguments(cl):
+    x = oracle.uniform(103, 40 * 30).reshape(40, 30)
+    p = Pair.dense(cl, x).transpose(0, 1)                            # 30 x 40, strides (1, 30)
+    idx = np.array([5, 1, 30, 5, 2])
+    got = p.dev.index(1, cl.ClTensor(idx.astype(F)))
+    assert_bit_equal(got.float(), cat.index_select(p.view.gather(), 0, idx), "select from a transposed view")
+    dst = Pair.dense(cl, np.zeros((40, 30), dtype=F)).transpose(0, 1)
+    src = oracle.uniform(104, 5 * 40).reshape(5, 40)
+    dst.dev.indexCopy(1, cl.ClTensor(idx.astype(F)), cl.ClTensor(src))
+    assert_bit_equal(dst.dev.float(), cat.index_copy(np.zeros((30, 40), dtype=F), 0, idx, src), "copy into a transposed view")
+    dst.dev.indexFill(2, [1, 40], 9.0)
+    assert np.all(dst.dev.float()[:, [0, 39]] == 9.0)
+    # an index outside the dimension moves nothing
+    Y = cl.ClTensor(x)
+    out = Y.index(1, cl.ClTensor(np.array([1, 41, 0, 40], dtype=F))).float()
+    assert_bit_equal(out[[0, 3]], x[[0, 39]], "valid rows")
+    Y.indexFill(1, cl.ClTensor(np.array([0, 41, -3], dtype=F)), 5.0)
+    assert_bit_equal(Y.float(), x, "out-of-range fill is a no-op")
+    with pytest.raises(cl.ClError):
+        Y.index(3, [1])
+    with pytest.raises(cl.ClError):
+        Y.index(1, cl.ClTensor(np.ones((2, 2), dtype=F)))
+    with pytest.raises(cl.ClError):
+        Y.indexCopy(1, [1, 2, 3], cl.ClTensor(2, 30))
+
+
+@pytest.mark.parametrize("shape,dim", [((6, 5), 0), ((6, 5), 1), ((40, 300), 0), ((40, 300), 1), ((7, 30, 20), 1),
+                                       ((3, 4, 5, 6), 3), ((2000, 64), 0)])
+def test_gather_scatter(cl, shape, dim):
+    n = int(np.prod(shape))
+    x = oracle.uniform(105, n).reshape(shape)
+    r = _rng(n + dim)
+    ishape = list(shape)
+    ishape[dim] = max(1, shape[dim] // 2)
+    index = r.randint(1, shape[dim] + 1, size=ishape)
+    X, I = cl.ClTensor(x), cl.ClTensor(index.astype(F))
+    assert_bit_equal(X.gather(dim + 1, I).float(), cat.gather(x, dim, index), "gather")
+    # scatter needs distinct targets along dim for a defined result: a permutation prefix per line
+    perm = np.argsort(r.rand(*shape), axis=dim) + 1
+    take = [slice(None)] * len(shape)
+    take[dim] = slice(0, ishape[dim])
+    uidx = perm[tuple(take)]
+    src = oracle.uniform(106, int(np.prod(ishape))).reshape(ishape)
+    R = cl.ClTensor(x)
+    R.scatter(dim + 1, cl.ClTensor(uidx.astype(F)), cl.ClTensor(src))
+    assert_bit_equal(R.float(), cat.scatter(x, dim, uidx, src), "scatter")
+    R2 = cl.ClTensor(x)
+    R2.scatter(dim + 1, cl.ClTensor(uidx.astype(F)), 2.5)
+    assert_bit_equal(R2.float(), cat.scatter(x, dim, uidx, 2.5), "scatterFill")
+    # round trip
+    back = R.gather(dim + 1, cl.ClTensor(uidx.astype(F)))
+    assert_bit_equal(back.float(), src, "gather undoes scatter")
+
+
+def test_gather_scatter_views_and_checks(cl):
+    x = oracle.uniform(107, 30 * 20).reshape(30, 20)
+    p = Pair.dense(cl, x).transpose(0, 1)                            # 20 x 30
+    index = _rng(5).randint(1, 21, size=(4, 30))
+    pi = Pair.dense(cl, index.T.astype(F)).transpose(0, 1)           # a strided index tensor
+    assert_bit_equal(p.dev.gather(1, pi.dev).float(), cat.gather(p.view.gather(), 0, index), "gather on views")
+    X = cl.ClTensor(x)
+    with pytest.raises(cl.ClError):
+        X.gather(1, cl.ClTensor(np.ones((2, 19), dtype=F)))          # other dims must match
+    with pytest.raises(cl.ClError):
+        X.gather(3, cl.ClTensor(np.ones((2, 20), dtype=F)))
+    with pytest.raises(cl.ClError):
+        X.scatter(1, cl.ClTensor(np.ones((2, 20), dtype=F)), cl.ClTensor(3, 20))
+
+
+@pytest.mark.parametrize("n", [1, 5, 255, 256, 4095, 4096, 4097, 100003, (1 << 22) + 11])
+def test_masked_select_and_copy(cl, n):
+    x = oracle.uniform(108, n)
+    mask = (oracle.uniform(109, n) > 0.2).astype(F)
+    mask[::97] *= -3.0                                              # any non-zero selects
+    X, M = cl.ClTensor(x), cl.ClTensor(mask)
+    got = X.maskedSelect(M)
+    want = cat.masked_select(x, mask)
+    assert got.nDimension() == 1 and got.size() == (want.size,)
+    assert_bit_equal(got.float(), want, "maskedSelect")
+    src = oracle.uniform(110, max(1, want.size))
+    if want.size:
+        R = cl.ClTensor(x)
+        R.maskedCopy(M, cl.ClTensor(src))
+        assert_bit_equal(R.float(), cat.masked_copy(x, mask, src), "maskedCopy")
+        # select undoes copy
+        assert_bit_equal(R.maskedSelect(M).float(), src[:want.size], "round trip")
+
+
+def test_masked_edge_cases(cl):
+    n = 10000
+    x = oracle.uniform(111, n)
+    X = cl.ClTensor(x)
+    none = X.maskedSelect(cl.ClTensor(np.zeros(n, dtype=F)))
+    assert none.nElement() == 0
+    every = X.maskedSelect(cl.ClTensor(np.ones(n, dtype=F)))
+    assert_bit_equal(every.float(), x, "all selected")
+    # 2-d strided source and mask
+    p = Pair.dense(cl, x.reshape(100, 100)).transpose(0, 1)
+    m = (oracle.uniform(112, n) > 0.0).astype(F).reshape(100, 100)
+    assert_bit_equal(p.dev.maskedSelect(cl.ClTensor(m)).float(), cat.masked_select(p.view.gather(), m), "strided source")
+    with pytest.raises(cl.ClError):
+        X.maskedSelect(cl.ClTensor(n + 1))
+    R = cl.ClTensor(x)
+    with pytest.raises(cl.ClError, match="source nElements"):
+        R.maskedCopy(cl.ClTensor(np.ones(n, dtype=F)), cl.ClTensor(n - 1))

@@ -339,3 +339,29 @@ def test_level12_small_integer_cases(golden):
     assert cat.dot([1, 2, 3], [4, -5, 6]) == 12.0
     assert cat.addr(1.0, np.ones((2, 3)), 2.0, [1, 2], [3, 4, 5]).tolist() == [[7, 9, 11], [13, 17, 21]]
     assert cat.addr(0.5, np.full((2, 2), 4.0), 1.0, [1, -1], [2, 3]).tolist() == [[4, 5], [0, -1]]
+
+
+def test_indexed_movement_hand_cases():
+    from oracle import catalogue as cat
+    a = np.arange(1, 13, dtype=np.float32).reshape(3, 4)             # rows 1..4 / 5..8 / 9..12
+    assert cat.index_select(a, 0, [3, 1, 1]).tolist() == [[9, 10, 11, 12], [1, 2, 3, 4], [1, 2, 3, 4]]
+    assert cat.index_select(a, 1, [4, 2]).tolist() == [[4, 2], [8, 6], [12, 10]]
+    z = np.zeros((3, 2), dtype=np.float32)
+    s = np.array([[1, 2], [3, 4], [5, 6]], dtype=np.float32)
+    assert cat.index_copy(z, 0, [2, 3, 2], s).tolist() == [[0, 0], [5, 6], [3, 4]]     # target 2 named twice: last wins
+    assert cat.index_fill(a, 1, [1, 3], -1.0)[0].tolist() == [-1, 2, -1, 4]
+    g = cat.gather(a, 1, np.array([[1, 1], [4, 2], [3, 3]]))
+    assert g.tolist() == [[1, 1], [8, 6], [11, 11]]
+    g0 = cat.gather(a, 0, np.array([[3, 2, 1, 1]]))
+    assert g0.tolist() == [[9, 6, 3, 4]]
+    sc = cat.scatter(np.zeros((3, 4), dtype=np.float32), 0, np.array([[3, 2, 1, 1]]), np.array([[7, 8, 9, 10]], dtype=np.float32))
+    assert sc.tolist() == [[0, 0, 9, 10], [0, 8, 0, 0], [7, 0, 0, 0]]
+    assert cat.scatter(np.zeros((2, 2), dtype=np.float32), 1, np.array([[2], [1]]), 5.0).tolist() == [[0, 5], [5, 0]]
+    # gather undoes scatter at the scattered positions
+    idx = np.array([[2, 3, 1, 2], [1, 1, 3, 3]])
+    vals = np.array([[1, 2, 3, 4], [5, 6, 7, 8]], dtype=np.float32)
+    assert np.array_equal(cat.gather(cat.scatter(np.zeros((3, 4), dtype=np.float32), 0, idx, vals), 0, idx), vals)
+    m = np.array([[0, 1, 0, 2], [1, 0, 0, 0], [0, 0, -1, 0]], dtype=np.float32)
+    assert cat.masked_select(a, m).tolist() == [2, 4, 5, 11]
+    assert cat.masked_copy(a, m, [-1, -2, -3, -4, -5])[0].tolist() == [1, -1, 3, -2]
+    assert cat.masked_copy(a, m, [-1, -2, -3, -4])[2].tolist() == [9, 10, -4, 12]
