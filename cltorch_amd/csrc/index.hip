@@ -178,29 +178,52 @@ __global__ __launch_bounds__(1024) void mask_offsets(MaskParams P) {
 }
 
 // COPY false: dst[rank] = src[i] for selected i.  COPY true: dst[i] = src[rank].
-template <bool COPY>
+// A block walks its chunk 1024 elements at a time, 4 consecutive elements per
+// thread (one 16-byte access when VEC), so ranks follow element order and every
+// wave reads whole lines; the rank carries from step to step.
+template <bool COPY, bool VEC>
 __global__ __launch_bounds__(kThreads) void mask_move(MaskParams P) {
   __shared__ unsigned lds[kThreads / 64];
-  // a thread owns kPer consecutive elements so ranks follow element order
-  const thcl_u64 first = (thcl_u64)blockIdx.x * kChunk + (thcl_u64)threadIdx.x * kPer;
-  float m[kPer];
-  unsigned c = 0;
+  constexpr int PER = 4, STEP = kThreads * PER;
+  unsigned carry = P.counts[blockIdx.x];
+  const thcl_u64 chunk0 = (thcl_u64)blockIdx.x * kChunk;
+  for (int step = 0; step < kChunk / STEP; step++) {
+    const thcl_u64 first = chunk0 + (thcl_u64)step * STEP + (thcl_u64)threadIdx.x * PER;
+    if (chunk0 + (thcl_u64)step * STEP >= P.n) break;  // uniform: the whole block is past the end
+    float m[PER], x[PER];
+    const bool whole = first + PER <= P.n;
+    if (VEC && whole) {
+      const thcl_f4 mv = __builtin_nontemporal_load((const thcl_f4 *)(P.mask + first));
 #pragma unroll
-  for (int k = 0; k < kPer; k++) {
-    m[k] = (first + k < P.n) ? P.mask[first + k] : 0.0f;
-    c += (m[k] != 0.0f) ? 1u : 0u;
-  }
-  unsigned total;
-  unsigned rank = P.counts[blockIdx.x] + block_exclusive(c, lds, &total);
+      for (int k = 0; k < PER; k++) m[k] = mv[k];
+      if (!COPY) {
+        const thcl_f4 xv = __builtin_nontemporal_load((const thcl_f4 *)(P.src + first));
 #pragma unroll
-  for (int k = 0; k < kPer; k++) {
-    if (m[k] != 0.0f) {
-      if (COPY) {
-        if (rank < P.src_len) P.dst[first + k] = P.src[rank];
-      } else {
-        P.dst[rank] = P.src[first + k];
+        for (int k = 0; k < PER; k++) x[k] = xv[k];
       }
-      rank++;
+    } else {
+#pragma unroll
+      for (int k = 0; k < PER; k++) {
+        m[k] = (first + k < P.n) ? P.mask[first + k] : 0.0f;
+        if (!COPY) x[k] = (first + k < P.n) ? P.src[first + k] : 0.0f;
+      }
+    }
+    unsigned c = 0;
+#pragma unroll
+    for (int k = 0; k < PER; k++) c += (m[k] != 0.0f) ? 1u : 0u;
+    unsigned total;
+    unsigned rank = carry + block_exclusive(c, lds, &total);
+    carry += total;
+#pragma unroll
+    for (int k = 0; k < PER; k++) {
+      if (m[k] != 0.0f) {
+        if (COPY) {
+          if (rank < P.src_len) P.dst[first + k] = P.src[rank];
+        } else {
+          P.dst[rank] = x[k];
+        }
+        rank++;
+      }
     }
   }
 }
@@ -544,7 +567,10 @@ void THClTensor_maskedSelect(THClState *state, THClTensor *tensor, THClTensor *s
   if (total > 0) {
     Dense r(state, tensor, false, true);
     P.dst = thcl_dptr(r.t);
-    hipLaunchKernelGGL((mask_move<false>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
+    if (aligned16(P.mask) && aligned16(P.src))
+      hipLaunchKernelGGL((mask_move<false, true>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
+    else
+      hipLaunchKernelGGL((mask_move<false, false>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
     check("masked select");
     thcl_after_launch(state, rt);
     r.finish();
@@ -573,7 +599,10 @@ void THClTensor_maskedCopy(THClState *state, THClTensor *tensor, THClTensor *mas
   P.dst = thcl_dptr(r.t);
   P.src_len = (thcl_u64)THClTensor_nElement(state, src);
   mask_prefix(state, rt, P, n);
-  hipLaunchKernelGGL((mask_move<true>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
+  if (aligned16(P.mask))
+    hipLaunchKernelGGL((mask_move<true, true>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
+  else
+    hipLaunchKernelGGL((mask_move<true, false>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
   check("masked copy");
   const long total = read_total(rt, P.counts, P.nblocks);
   thcl_after_launch(state, rt);

@@ -149,6 +149,9 @@ def test_masked_edge_cases(cl):
     p = Pair.dense(cl, x.reshape(100, 100)).transpose(0, 1)
     m = (oracle.uniform(112, n) > 0.0).astype(F).reshape(100, 100)
     assert_bit_equal(p.dev.maskedSelect(cl.ClTensor(m)).float(), cat.masked_select(p.view.gather(), m), "strided source")
+    # operands that start 4 bytes off a 16-byte boundary: the scalar path
+    xo, mo = X.narrow(1, 2, n - 1), cl.ClTensor(m.reshape(-1)).narrow(1, 2, n - 1)
+    assert_bit_equal(xo.maskedSelect(mo).float(), cat.masked_select(x[1:], m.reshape(-1)[1:]), "unaligned operands")
     with pytest.raises(cl.ClError):
         X.maskedSelect(cl.ClTensor(n + 1))
     R = cl.ClTensor(x)
