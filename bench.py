@@ -12,8 +12,10 @@ bytes divided by the wall time of a step (inputs already in HBM).  Each kernel
 is also timed with HIP events on the library's stream inside the timed region;
 the ``roofline`` object describes the kernel that takes the largest share (the
 three-operand expression kernel).  ``detail`` carries the other configurations
-(strided map/copy, reductions along a dim, the point-tensor chain, addmm), each
-with its own effective GB/s or TFLOP/s.  The CPU baseline is the TH-semantics
+(strided map/copy, reductions along a dim, the point-tensor chain, addmm) and,
+under ``w_`` names, the operators either side of the path (catalogue ops,
+scans, level-1/2 contractions, indexed movement), each with its own effective
+GB/s or TFLOP/s.  The CPU baseline is the TH-semantics
 restatement (oracle/) on the host's cores over a bounded sample.
 
 Prints ONE JSON line.
@@ -94,12 +96,24 @@ def cpu_baseline(n_sample, seed_base=1, min_seconds=12.0):
         dt = time.perf_counter() - t0
         if dt >= min_seconds or steps >= 200:
             break
+    # second, labelled row: fp32 addmm on the host through PyTorch's CPU BLAS (Torch7's lineal descendant)
+    import torch
+    k = 2048
+    a, b, c = (torch.from_numpy(oracle.normal(20 + i, k * k, 0.0, 1.0 / np.sqrt(k)).reshape(k, k)) for i in range(3))
+    torch.addmm(c, a, b, beta=0.5, alpha=1.0)
+    g0, reps = time.perf_counter(), 0
+    while time.perf_counter() - g0 < 2.0:
+        torch.addmm(c, a, b, beta=0.5, alpha=1.0)
+        reps += 1
+    gemm_tflops = 2.0 * k ** 3 * reps / (time.perf_counter() - g0) * 1e-12
     fmt = lambda v: float(np.float32(v)) if np.isfinite(v) else str(v)
     return {"value": round(48.0 * n_sample * steps / dt * 1e-9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
             "sample": f"{steps} steps on 2^{int(np.log2(n_sample))} elements per tensor ({dt:.1f} s of CPU work): cadd/cmul/map2 as dense "
                       f"OpenMP loops on {oracle.num_threads()} threads, sum (fp64 accumulator) and max serial in element order "
                       f"(max stops at the first NaN, as TH does); Torch7's own map2 calls a Lua closure per element and is far slower",
-            "seconds": round(dt, 3), "steps": steps, "first_step_sum_max": [fmt(first[0]), fmt(first[1])]}
+            "seconds": round(dt, 3), "steps": steps, "first_step_sum_max": [fmt(first[0]), fmt(first[1])],
+            "addmm_cpu": {"value": round(gemm_tflops, 3), "unit": "TFLOP/s", "kind": "torch.addmm on CPU tensors, fp32, 2048^3",
+                          "threads": torch.get_num_threads()}}
 
 
 def main():
@@ -276,6 +290,47 @@ def detail(cl, oracle, T, X, Y, Z, n):
             peak=FP32_MFMA_PEAK_TFLOPS)
     d["c5_addmm_skinny_64x16384x4096"]["hbm_GBs"] = round(
         4.0 * (M * K + K * N + 2 * M * N) / (d["c5_addmm_skinny_64x16384x4096"]["avg_ms"] * 1e-3) * 1e-9, 1)
+    del At, Bs, Cs
+
+    # ---- the callers either side of the path: operator catalogue, scans, level-1/2, indexed movement
+    A.fill(0.75)
+    B = Y
+    measure("w_clamp_2^%d" % int(np.log2(n)), lambda: A.clamp(-0.5, 0.5), 8 * n)
+    measure("w_lt_tensor", lambda: Z.lt(A, B), 12 * n)
+    measure("w_norm2_to_host", lambda: A.norm(2.0), 4 * n)
+    measure("w_dot_to_host", lambda: A.dot(B), 8 * n)
+    measure("w_cumsum_1d", lambda: Z.cumsum(A, 1), 8 * n)
+    G = cl.ClTensor(4096 * 16384).resize(4096, 16384)
+    G.fill(0.5)
+    R = cl.ClTensor(4096, 16384)
+    for dim in (1, 2):
+        measure(f"w_cumsum_4096x16384_dim{dim}", lambda: R.cumsum(G, dim), 8 * 4096 * 16384)
+    del R
+    q = 16384
+    Mq = cl.ClTensor(q * q).resize(q, q)
+    Mq.fill(0.01)
+    v, y = cl.ClTensor(q), cl.ClTensor(q)
+    v.fill(1.0)
+    y.fill(0.0)
+    measure("w_addmv_rowmajor_16384", lambda: y.addmv(0.0, 1.0, Mq, v), 4 * q * q)
+    measure("w_addmv_colmajor_16384", lambda: y.addmv(0.0, 1.0, Mq.t(), v), 4 * q * q)
+    measure("w_addr_16384", lambda: Mq.addr(1.0, 0.5, v, y), 8 * q * q)
+    del Mq
+    rows, width, cnt = 100000, 1024, 65536
+    rs = np.random.RandomState(0)
+    tab = cl.ClTensor(rows * width).resize(rows, width)
+    tab.fill(1.0)
+    idx = cl.ClTensor(rs.randint(1, rows + 1, size=cnt).astype(np.float32))
+    sel = cl.ClTensor(cnt, width)
+    measure("w_indexSelect_rows_65536x1024", lambda: sel.index(tab, 1, idx), 8 * cnt * width)
+    measure("w_indexCopy_rows_65536x1024", lambda: tab.indexCopy(1, idx, sel), 8 * cnt * width)
+    del tab, sel
+    mask = cl.ClTensor((rs.rand(1 << 26) > 0.5).astype(np.float32))
+    src = cl.ClTensor(1 << 26)
+    src.fill(1.0)
+    packed = cl.ClTensor()
+    # mask read twice (count, move), source read once, half of it written
+    measure("w_maskedSelect_2^26_half", lambda: packed.maskedSelect(src, mask), (4 + 4 + 4 + 2) * (1 << 26))
     return d
 
 
