@@ -180,8 +180,8 @@ def main():
                      "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom["achieved"] / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, calibrated on a copy kernel
-                     # (profiles/headline_kernels_2p28_pmc_traffic.txt): 15.996 bytes/element at 2^28 elements
-                     "traffic": int(round(15.996 * n)) if args.log2n == 28 else None,
+                     # (profiles/headline_kernels_2p28_pmc_traffic.txt): 15.999 bytes/element at 2^28 elements
+                     "traffic": int(round(15.999 * n)) if args.log2n == 28 else None,
                      "algorithmic_bytes_per_launch": 16 * n, "avg_launch_ms": dom["avg_ms"]},
         "kernels": kernels,
     }

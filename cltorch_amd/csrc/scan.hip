@@ -97,6 +97,32 @@ __global__ __launch_bounds__(kThreads) void scan_carries(ScanParams P) {
   }
 }
 
+// Same, for few lines with many segments: a wave per (o, i) line, 64 segments
+// per step with a shuffle scan, instead of one thread walking thousands of
+// dependent loads.
+template <bool PROD>
+__global__ __launch_bounds__(kWave) void scan_carries_wave(ScanParams P) {
+  const thcl_u64 line = blockIdx.x;
+  const thcl_u64 i = line % P.I, o = line / P.I;
+  double *p = P.totals + o * P.S * P.I + i;
+  const int lane = threadIdx.x;
+  double carry = Op<PROD>::identity();
+  for (thcl_u64 base = 0; base < P.S; base += kWave) {
+    const thcl_u64 s = base + lane;
+    const double v = s < P.S ? p[s * P.I] : Op<PROD>::identity();
+    double incl = v;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const double up = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl = Op<PROD>::comb(up, incl);
+    }
+    double excl = __shfl_up(incl, 1, kWave);
+    if (lane == 0) excl = Op<PROD>::identity();
+    if (s < P.S) p[s * P.I] = Op<PROD>::comb(carry, excl);
+    carry = Op<PROD>::comb(carry, __shfl(incl, kWave - 1, kWave));
+  }
+}
+
 template <bool PROD>
 __device__ __forceinline__ double wave_inclusive(double v) {
   const int lane = threadIdx.x % kWave;
@@ -251,6 +277,16 @@ void check(const char *what) {
 }
 
 template <bool PROD>
+void launch_carries(hipStream_t stream, const ScanParams &P) {
+  const thcl_u64 lines = P.O * P.I;
+  if (lines < 4096 && P.S >= 32)
+    hipLaunchKernelGGL((scan_carries_wave<PROD>), dim3((unsigned)lines), dim3(kWave), 0, stream, P);
+  else
+    hipLaunchKernelGGL((scan_carries<PROD>), dim3((unsigned)((lines + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P);
+  check("scan carries");
+}
+
+template <bool PROD>
 void run_scan(hipStream_t stream, ScanParams &P, bool rows, bool vec) {
   if (rows) {
     const dim3 grid((unsigned)(P.O * P.S)), block(kThreads);
@@ -258,8 +294,7 @@ void run_scan(hipStream_t stream, ScanParams &P, bool rows, bool vec) {
       if (vec) hipLaunchKernelGGL((scan_row<PROD, 0, true>), grid, block, 0, stream, P);
       else hipLaunchKernelGGL((scan_row<PROD, 0, false>), grid, block, 0, stream, P);
       check("scan totals");
-      hipLaunchKernelGGL((scan_carries<PROD>), dim3((unsigned)((P.O + kThreads - 1) / kThreads)), block, 0, stream, P);
-      check("scan carries");
+      launch_carries<PROD>(stream, P);
     }
     if (vec) hipLaunchKernelGGL((scan_row<PROD, 1, true>), grid, block, 0, stream, P);
     else hipLaunchKernelGGL((scan_row<PROD, 1, false>), grid, block, 0, stream, P);
@@ -270,9 +305,7 @@ void run_scan(hipStream_t stream, ScanParams &P, bool rows, bool vec) {
     if (P.S > 1) {
       hipLaunchKernelGGL((scan_seq<PROD, 0>), grid, block, 0, stream, P);
       check("scan totals");
-      hipLaunchKernelGGL((scan_carries<PROD>), dim3((unsigned)((P.O * P.I + kThreads - 1) / kThreads)), block, 0, stream,
-                         P);
-      check("scan carries");
+      launch_carries<PROD>(stream, P);
     }
     hipLaunchKernelGGL((scan_seq<PROD, 1>), grid, block, 0, stream, P);
     check("scan");
