@@ -114,6 +114,15 @@ void THClTensor_ones(THClState *state, THClTensor *r_, THLongStorage *size) {
   THCL_GUARD_END()
 }
 long THClTensor_numel(THClState *state, THClTensor *t) { return THClTensor_nElement(state, t); }
+// r_ takes the given shape and t's elements in order (src/lib/THClTensorMath.cpp:97-104)
+void THClTensor_reshape(THClState *state, THClTensor *r_, THClTensor *t, THLongStorage *size) {
+  THCL_GUARD_BEGIN
+  thcl_check_same_device(state, 2, r_, t);
+  if (r_->nDimension < 0 && !r_->storage) r_->device = THClTensor_getDevice(state, t);
+  THClTensor_resize(state, r_, size, nullptr);
+  THClTensor_copy(state, r_, t);
+  THCL_GUARD_END()
+}
 
 // ----------------------------------------------------------- scalar forms ---
 void THClTensor_add(THClState *state, THClTensor *self, THClTensor *src, float value) {

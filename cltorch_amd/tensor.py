@@ -225,6 +225,16 @@ class ClTensor:
             self._lib.THLongStorage_free(sd)
         return self._wrap(h)
 
+    def reshape(self, *sizes) -> "ClTensor":
+        """``a:reshape(s1, s2, ...)``: a new dense tensor with a's elements in order (``torch.reshape``)."""
+        res = ClTensor()
+        sz = _long_storage(list(sizes[0]) if len(sizes) == 1 and not isinstance(sizes[0], int) else list(sizes))
+        try:
+            _call("THClTensor_reshape", res._h, self._h, sz)
+        finally:
+            self._lib.THLongStorage_free(sz)
+        return res
+
     def clone(self) -> "ClTensor":
         return self._wrap(_call("THClTensor_newClone", self._h))
 

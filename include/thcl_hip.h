@@ -252,6 +252,7 @@ void THClTensor_fill_gpu(THClState *state, THClTensor *self, THClTensor *value);
 void THClTensor_zeros(THClState *state, THClTensor *r_, THLongStorage *size);
 void THClTensor_ones(THClState *state, THClTensor *r_, THLongStorage *size);
 long THClTensor_numel(THClState *state, THClTensor *t);
+void THClTensor_reshape(THClState *state, THClTensor *r_, THClTensor *t, THLongStorage *size);
 
 void THClTensor_add(THClState *state, THClTensor *self, THClTensor *src, float value);
 void THClTensor_sub(THClState *state, THClTensor *self, THClTensor *src, float value);

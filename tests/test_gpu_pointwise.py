@@ -369,3 +369,14 @@ def test_same_expression_on_every_kernel_family(cl):
         run(Pair.dense(cl, base.reshape(96, 80)).step(1, 2), Pair.dense(cl, other[:7680].reshape(96, 80)).step(1, 2))              # joint scalar
         run(Pair.dense(cl, base.reshape(96, 80)), Pair.dense(cl, other[:7680].reshape(80, 96)).transpose(0, 1))                    # tiled
         run(Pair.dense(cl, base.reshape(96, 80)), Pair(cl, other, 0, (80, 96), (1, 160)))                   # different shapes: generic
+
+
+def test_reshape_copies_in_logical_order(cl):
+    x = oracle.uniform(120, 6 * 8 * 5).reshape(6, 8, 5)
+    p = Pair.dense(cl, x).transpose(0, 2)                       # 5 x 8 x 6 view
+    r = p.dev.reshape(40, 6)
+    assert r.size() == (40, 6) and r.isContiguous()
+    assert_bit_equal(r.float(), p.view.gather().reshape(40, 6), "reshape of a transposed view")
+    with pytest.raises(cl.ClError):
+        p.dev.reshape(7, 7)
+
