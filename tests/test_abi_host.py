@@ -235,6 +235,12 @@ def test_planner_picks_the_kernel_family_for_each_layout(lib):
     assert kind == "tiled" and grid == 512 * (512 // 64) * (256 // 256)             # 64 x 256 tiles, 512 outer slices
     sq = _plan(lib, [((8192, 8192), (8192, 1), 0), ((8192, 8192), (1, 8192), 0)])
     assert sq == ("tiled", (8192 // 128) ** 2)                                      # plain 2-d transpose: 128 x 128 tiles
+    # element counts: dense walks index with 64 bits, strided walks refuse what 32-bit indices cannot reach
+    n = (1 << 31) + 4096
+    assert _plan(lib, [((n,), (1,), 0), ((n,), (1,), 0)])[0] == "dense128"
+    assert _plan(lib, [((n // 2, 2), (1, n // 2), 0)])[0] == "dense128"               # a transposed walk that is dense after sorting dims
+    assert _plan(lib, [((n,), (2,), 0)])[0] == "rejected"                              # gapped: 32-bit linear index would overflow
+    assert _plan(lib, [((n // 2,), (2,), 0)])[0] in ("joint32", "joint128")
     # a rank-1 update: vectors expanded with stride 0 ride the vector kernel, not the transposing tiles
     outer = _plan(lib, [((4096, 4096), (4096, 1), 0), ((4096, 4096), (1, 0), 0), ((4096, 4096), (0, 1), 0)])
     assert outer[0] == "joint128"

@@ -184,3 +184,27 @@ def test_config5_addmm_square_8192_sampled_and_skinny(cl):
     want = oracle.addmm_f64(0.5, pc.view, 1.0, pa.view, pb.view)
     scale = float(np.sqrt(np.mean(want ** 2)))
     assert np.max(np.abs(pc.dev.float() - want)) / scale < 1e-4
+
+
+def test_dense_tensors_beyond_32_bit_element_counts(cl):
+    """The reference caps apply at 2^30 elements (src/lib/THClApply.cpp:136-139).  Dense
+    kernels here index with 64 bits: closed forms on 2^31 + 4096 elements (8 GiB
+    per tensor), and the strided kernels refuse what their 32-bit indices cannot reach."""
+    n = (1 << 31) + 4096
+    X, Y = cl.ClTensor(n), cl.ClTensor(n)
+    assert X.nElement() == n
+    X.fill(1.0)
+    Y.fill(2.0)
+    X.add(Y)
+    assert X.sum() == float(np.float32(3.0 * n))            # fp64 running sum, one rounding
+    assert X.max() == 3.0 and X.min() == 3.0
+    tail = X.narrow(1, n - 999, 1000)                        # the last elements were reached
+    assert tail.float().tolist() == [3.0] * 1000
+    X.narrow(1, n - 4, 1).fill(-5.0)                         # a single element past 2^31
+    assert X.min() == -5.0 and X.sum() == float(np.float32(3.0 * n - 8.0))
+    X.map_on_gpu(Y, "x = x * y")
+    assert X.max() == 6.0 and X.min() == -10.0
+    half = n // 2
+    X.strided((half, 2), (1, half)).add(1.0)                 # a transposed walk over every element: dense after sorting dims
+    assert X.max() == 7.0 and X.min() == -9.0
+
