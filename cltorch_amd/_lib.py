@@ -30,12 +30,13 @@ _SCALARS = {
 
 def _ctype(decl: str):
     """C type text (without the parameter name) -> ctypes type."""
+    is_const = bool(re.search(r"\bconst\b", decl))
     d = decl.replace("const", " ").replace("struct", " ").strip()
     d = re.sub(r"\s+", " ", d)
     if "*" in d:
         base = d.replace("*", "").strip()
-        if base == "char" and d.count("*") == 1:
-            return C.c_char_p
+        if base == "char" and d.count("*") == 1 and is_const:
+            return C.c_char_p          # NUL-terminated text; a plain `char *` is a buffer of elements
         return C.c_void_p
     if d in _SCALARS:
         return _SCALARS[d]

@@ -273,8 +273,62 @@ class ClTensor:
                 self._lib.THFloatTensor_free(ft)
         return out
 
+    _HOST_TYPES = {"Byte": (np.uint8, C.c_ubyte), "Char": (np.int8, C.c_byte), "Short": (np.int16, C.c_short),
+                   "Int": (np.int32, C.c_int), "Double": (np.float64, C.c_double)}
+
+    def _to_host_typed(self, name: str) -> np.ndarray:
+        """``clTensor:double()`` / ``:int()`` / ``:byte()`` ...: through TH<Name>Tensor_copyCl."""
+        dtype, _ = self._HOST_TYPES[name]
+        shape = self.size() if self.nDimension() > 0 else (0,)
+        out = np.empty(shape, dtype=dtype)
+        if out.size:
+            sz = (C.c_long * out.ndim)(*out.shape)
+            ht = getattr(self._lib, f"TH{name}Tensor_newWithData")(out.ctypes.data_as(C.c_void_p), out.size, 0, out.ndim, sz, None)
+            try:
+                _call(f"TH{name}Tensor_copyCl", ht, self._h)
+            finally:
+                getattr(self._lib, f"TH{name}Tensor_free")(ht)
+        return out
+
+    def _from_host_typed(self, name: str, arr: np.ndarray) -> "ClTensor":
+        dtype, _ = self._HOST_TYPES[name]
+        arr = np.asarray(arr, dtype=dtype)
+        strides = tuple(s // arr.itemsize for s in arr.strides)
+        if any(s < 0 for s in strides) or not arr.flags.aligned:
+            arr = np.ascontiguousarray(arr)
+            strides = tuple(s // arr.itemsize for s in arr.strides)
+        sz, st = (C.c_long * max(arr.ndim, 1))(*arr.shape), (C.c_long * max(arr.ndim, 1))(*strides)
+        span = 1 + sum((n - 1) * s for n, s in zip(arr.shape, strides)) if arr.size else 0
+        ht = getattr(self._lib, f"TH{name}Tensor_newWithData")(arr.ctypes.data_as(C.c_void_p), span, 0, arr.ndim, sz, st)
+        try:
+            _call(f"THClTensor_copy{name}", self._h, ht)
+        finally:
+            getattr(self._lib, f"TH{name}Tensor_free")(ht)
+        return self
+
     def double(self) -> np.ndarray:
-        return self.float().astype(np.float64)
+        return self._to_host_typed("Double")
+
+    def int(self) -> np.ndarray:
+        return self._to_host_typed("Int")
+
+    def short(self) -> np.ndarray:
+        return self._to_host_typed("Short")
+
+    def char(self) -> np.ndarray:
+        return self._to_host_typed("Char")
+
+    def byte(self) -> np.ndarray:
+        return self._to_host_typed("Byte")
+
+    def copyFrom(self, arr: np.ndarray) -> "ClTensor":
+        """``cl:copy(hostTensor)`` for a host array of any of TH's element types (element counts must match)."""
+        kinds = {np.dtype(np.uint8): "Byte", np.dtype(np.int8): "Char", np.dtype(np.int16): "Short",
+                 np.dtype(np.int32): "Int", np.dtype(np.float64): "Double"}
+        arr = np.asarray(arr)
+        if arr.dtype in kinds:
+            return self._from_host_typed(kinds[arr.dtype], arr)
+        return self.copy(arr)
 
     def long(self) -> np.ndarray:
         return self.float().astype(np.int64)
@@ -450,8 +504,11 @@ class ClTensor:
     def eq(self, *args): return self._compare("eq", args)
     def ne(self, *args): return self._compare("ne", args)
 
-    def maskedFill(self, mask: "ClTensor", value: float) -> "ClTensor":
-        _call("THClTensor_maskedFill", self._h, mask._h, C.c_float(value))
+    def maskedFill(self, mask, value: float) -> "ClTensor":
+        if isinstance(mask, ClTensor):
+            _call("THClTensor_maskedFill", self._h, mask._h, C.c_float(value))
+        else:
+            self._with_byte_mask(mask, lambda m: _call("THClTensor_maskedFillByte", self._h, m, C.c_float(value)))
         return self
 
     # ---- user expressions ---------------------------------------------------
@@ -639,12 +696,28 @@ class ClTensor:
     def maskedSelect(self, *args) -> "ClTensor":
         """``a:maskedSelect(mask)`` -> new vector; ``res:maskedSelect(a, mask)``."""
         res, src, mask = (ClTensor(), self, args[0]) if len(args) == 1 else (self, args[0], args[1])
-        _call("THClTensor_maskedSelect", res._h, src._h, mask._h)
+        if isinstance(mask, ClTensor):
+            _call("THClTensor_maskedSelect", res._h, src._h, mask._h)
+        else:
+            self._with_byte_mask(mask, lambda m: _call("THClTensor_maskedSelectByte", res._h, src._h, m))
         return res
 
-    def maskedCopy(self, mask: "ClTensor", src: "ClTensor") -> "ClTensor":
-        _call("THClTensor_maskedCopy", self._h, mask._h, src._h)
+    def maskedCopy(self, mask, src: "ClTensor") -> "ClTensor":
+        if isinstance(mask, ClTensor):
+            _call("THClTensor_maskedCopy", self._h, mask._h, src._h)
+        else:
+            self._with_byte_mask(mask, lambda m: _call("THClTensor_maskedCopyByte", self._h, m, src._h))
         return self
+
+    def _with_byte_mask(self, mask, call):
+        """A host ``torch.ByteTensor`` mask (numpy uint8 / bool array): the ``*Byte`` entry points."""
+        arr = np.ascontiguousarray(np.asarray(mask).astype(np.uint8))
+        sz = (C.c_long * max(arr.ndim, 1))(*arr.shape)
+        bt = self._lib.THByteTensor_newWithData(arr.ctypes.data_as(C.c_void_p), arr.size, 0, arr.ndim, sz, None)
+        try:
+            return call(bt)
+        finally:
+            self._lib.THByteTensor_free(bt)
 
     def dot(self, other: "ClTensor") -> float:
         """``a:dot(b)`` (``src/TensorMath.lua:932-936``)."""

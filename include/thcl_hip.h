@@ -67,6 +67,44 @@ typedef struct THLongTensor {
   char flag;
 } THLongTensor;
 
+/* host tensors of the other element types: same layout, element type aside */
+#define THCL_DECLARE_HOST_TENSOR(Name, T)                                        \
+  typedef struct TH##Name##Storage {                                             \
+    T *data;                                                                     \
+    long size;                                                                   \
+    int refcount;                                                                \
+    char flag;                                                                   \
+    void *allocator;                                                             \
+    void *allocatorContext;                                                      \
+    struct TH##Name##Storage *view;                                              \
+  } TH##Name##Storage;                                                           \
+  typedef struct TH##Name##Tensor {                                              \
+    long *size;                                                                  \
+    long *stride;                                                                \
+    int nDimension;                                                              \
+    TH##Name##Storage *storage;                                                  \
+    long storageOffset;                                                          \
+    int refcount;                                                                \
+    char flag;                                                                   \
+  } TH##Name##Tensor;
+THCL_DECLARE_HOST_TENSOR(Byte, unsigned char)
+THCL_DECLARE_HOST_TENSOR(Char, char)
+THCL_DECLARE_HOST_TENSOR(Short, short)
+THCL_DECLARE_HOST_TENSOR(Int, int)
+THCL_DECLARE_HOST_TENSOR(Double, double)
+#undef THCL_DECLARE_HOST_TENSOR
+/* borrow `data` (not freed with the tensor): strided host views for the copies below */
+THByteTensor *THByteTensor_newWithData(unsigned char *data, long storageSize, long storageOffset, int nDimension, const long *size, const long *stride);
+THCharTensor *THCharTensor_newWithData(char *data, long storageSize, long storageOffset, int nDimension, const long *size, const long *stride);
+THShortTensor *THShortTensor_newWithData(short *data, long storageSize, long storageOffset, int nDimension, const long *size, const long *stride);
+THIntTensor *THIntTensor_newWithData(int *data, long storageSize, long storageOffset, int nDimension, const long *size, const long *stride);
+THDoubleTensor *THDoubleTensor_newWithData(double *data, long storageSize, long storageOffset, int nDimension, const long *size, const long *stride);
+void THByteTensor_free(THByteTensor *t);
+void THCharTensor_free(THCharTensor *t);
+void THShortTensor_free(THShortTensor *t);
+void THIntTensor_free(THIntTensor *t);
+void THDoubleTensor_free(THDoubleTensor *t);
+
 THLongStorage *THLongStorage_newWithSize(long size);
 void THLongStorage_free(THLongStorage *s);
 void THLongStorage_set(THLongStorage *s, long i, long v);
@@ -241,6 +279,18 @@ void THClTensor_copyFloat(THClState *state, THClTensor *self, THFloatTensor *src
 void THClTensor_copyLong(THClState *state, THClTensor *self, THLongTensor *src);
 void THFloatTensor_copyCl(THClState *state, THFloatTensor *self, THClTensor *src);
 void THLongTensor_copyCl(THClState *state, THLongTensor *self, THClTensor *src);
+/* the other host element types convert through float, as in the reference
+ * (src/lib/THClTensorCopy.h:8-22, src/lib/THClTensorCopy.cpp:38-66,93-128) */
+void THClTensor_copyByte(THClState *state, THClTensor *self, THByteTensor *src);
+void THClTensor_copyChar(THClState *state, THClTensor *self, THCharTensor *src);
+void THClTensor_copyShort(THClState *state, THClTensor *self, THShortTensor *src);
+void THClTensor_copyInt(THClState *state, THClTensor *self, THIntTensor *src);
+void THClTensor_copyDouble(THClState *state, THClTensor *self, THDoubleTensor *src);
+void THByteTensor_copyCl(THClState *state, THByteTensor *self, THClTensor *src);
+void THCharTensor_copyCl(THClState *state, THCharTensor *self, THClTensor *src);
+void THShortTensor_copyCl(THClState *state, THShortTensor *self, THClTensor *src);
+void THIntTensor_copyCl(THClState *state, THIntTensor *self, THClTensor *src);
+void THDoubleTensor_copyCl(THClState *state, THDoubleTensor *self, THClTensor *src);
 
 /* ------------------------------------------------------------------------- */
 /* Pointwise (reference: src/lib/THClTensorMath.h:7-28,98-155)                */
@@ -421,6 +471,10 @@ void THClTensor_scatterFill(THClState *state, THClTensor *self, long dim, THClTe
 /* mask: a ClTensor of 0 / non-0 with as many elements as the tensor it selects from */
 void THClTensor_maskedSelect(THClState *state, THClTensor *tensor, THClTensor *src, THClTensor *mask);
 void THClTensor_maskedCopy(THClState *state, THClTensor *tensor, THClTensor *mask, THClTensor *src);
+/* host byte masks: uploaded as floats, then the forms above (src/lib/THClTensorMath.h:117-119) */
+void THClTensor_maskedFillByte(THClState *state, THClTensor *tensor, THByteTensor *mask, float value);
+void THClTensor_maskedCopyByte(THClState *state, THClTensor *tensor, THByteTensor *mask, THClTensor *src);
+void THClTensor_maskedSelectByte(THClState *state, THClTensor *tensor, THClTensor *src, THByteTensor *mask);
 
 /* ------------------------------------------------------------------------- */
 /* User kernels compiled at run time: the C side of torch.ClKernel.  The      */

@@ -157,3 +157,45 @@ def test_masked_edge_cases(cl):
     R = cl.ClTensor(x)
     with pytest.raises(cl.ClError, match="source nElements"):
         R.maskedCopy(cl.ClTensor(np.ones(n, dtype=F)), cl.ClTensor(n - 1))
+
+
+def test_host_element_types_and_byte_masks(cl):
+    """copyByte/Char/Short/Int/Double both ways (src/lib/THClTensorCopy.h:8-22) and the
+    byte-mask forms of the masked operators (src/lib/THClTensorMasked.cpp:248-281)."""
+    vals = np.array([[0, 1, 2.75, -3.5], [100, -128, 127, 255], [65000.5, -7, 8, 9]], dtype=F)
+    X = cl.ClTensor(vals)
+    assert np.array_equal(X.double(), vals.astype(np.float64)) and X.double().dtype == np.float64
+    assert np.array_equal(X.int(), vals.astype(np.int32))                 # C conversion: truncation toward zero
+    small = cl.ClTensor(np.array([[0, 1, 2.75], [-3.5, 100, 127]], dtype=F))
+    assert np.array_equal(small.short(), np.array([[0, 1, 2], [-3, 100, 127]], dtype=np.int16))
+    assert np.array_equal(small.char(), np.array([[0, 1, 2], [-3, 100, 127]], dtype=np.int8))
+    pos = cl.ClTensor(np.array([0, 1, 2.75, 200, 255], dtype=F))
+    assert np.array_equal(pos.byte(), np.array([0, 1, 2, 200, 255], dtype=np.uint8))
+    for dtype in (np.uint8, np.int8, np.int16, np.int32, np.float64):
+        h = (np.arange(24).reshape(4, 6) % 100).astype(dtype)
+        T = cl.ClTensor(4, 6)
+        T.copyFrom(h)
+        assert_bit_equal(T.float(), h.astype(F), f"from {dtype.__name__}")
+        T2 = cl.ClTensor(6, 4)
+        T2.copyFrom(h.T)                                                  # strided host view
+        assert_bit_equal(T2.float(), h.T.astype(F), f"from transposed {dtype.__name__}")
+        dst = Pair.dense(cl, np.zeros((6, 4), dtype=F)).transpose(0, 1)   # strided device view
+        dst.dev.copyFrom(h)
+        assert_bit_equal(dst.dev.float(), h.astype(F), f"into a transposed view from {dtype.__name__}")
+    d = np.array([1e-3, 1.0000001, 16777217.0, -2.5e38], dtype=np.float64)
+    D = cl.ClTensor(4)
+    D.copyFrom(d)
+    assert_bit_equal(D.float(), d.astype(F), "double -> float rounding")
+    with pytest.raises(cl.ClError):
+        cl.ClTensor(5).copyFrom(np.zeros(4, dtype=np.int32))
+    # byte masks
+    x = oracle.uniform(121, 5000).reshape(50, 100)
+    m = oracle.uniform(122, 5000).reshape(50, 100) > 0.1
+    Xm = cl.ClTensor(x)
+    assert_bit_equal(Xm.maskedSelect(m).float(), cat.masked_select(x, m), "maskedSelectByte")
+    Xm.maskedFill(m, 4.0)
+    assert_bit_equal(Xm.float(), cat.masked_fill(x, m, 4.0), "maskedFillByte")
+    src = oracle.uniform(123, int(m.sum()))
+    Xc = cl.ClTensor(x)
+    Xc.maskedCopy(m, cl.ClTensor(src))
+    assert_bit_equal(Xc.float(), cat.masked_copy(x, m, src), "maskedCopyByte")
