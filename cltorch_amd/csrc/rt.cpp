@@ -4,8 +4,10 @@
 
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
+#include <unistd.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -271,6 +273,55 @@ int thcl_rt_compile_check(const char *source, const char *arch, size_t *code_byt
   return rc;
 }
 
+// Optional on-disk cache of compiled code objects, for processes that meet the
+// same expressions again: THCL_KERNEL_CACHE_DIR names a directory; a file per
+// (source text, architecture, compiler version) holds the code object.  Off
+// when the variable is unset.  Files are written under a temporary name and
+// renamed, so concurrent processes never read a partial file.
+static std::string disk_cache_path(const char *source, const std::string &arch) {
+  const char *dir = getenv("THCL_KERNEL_CACHE_DIR");
+  if (!dir || !dir[0]) return std::string();
+  int major = 0, minor = 0;
+  hiprtcVersion(&major, &minor);
+  unsigned long long h = 1469598103934665603ull;  // FNV-1a over everything that shapes the code
+  auto mix = [&](const char *p) {
+    for (; *p; p++) h = (h ^ (unsigned char)*p) * 1099511628211ull;
+    h = (h ^ 0xffu) * 1099511628211ull;
+  };
+  mix(source);
+  mix(arch.c_str());
+  mix("-O3 -ffp-contract=off -std=c++17 -packed-fp32-ops");
+  char name[96];
+  snprintf(name, sizeof(name), "/thcl_%016llx_%zu_rtc%d.%d.hsaco", h, strlen(source), major, minor);
+  return std::string(dir) + name;
+}
+static bool disk_cache_read(const std::string &path, std::vector<char> &code) {
+  if (path.empty()) return false;
+  FILE *f = fopen(path.c_str(), "rb");
+  if (!f) return false;
+  fseek(f, 0, SEEK_END);
+  const long n = ftell(f);
+  fseek(f, 0, SEEK_SET);
+  bool ok = n > 0;
+  if (ok) {
+    code.resize((size_t)n);
+    ok = fread(code.data(), 1, (size_t)n, f) == (size_t)n;
+  }
+  fclose(f);
+  return ok;
+}
+static void disk_cache_write(const std::string &path, const std::vector<char> &code) {
+  if (path.empty()) return;
+  char suffix[48];
+  snprintf(suffix, sizeof(suffix), ".tmp%ld", (long)getpid());
+  const std::string tmp = path + suffix;
+  FILE *f = fopen(tmp.c_str(), "wb");
+  if (!f) return;  // an unwritable cache directory only costs the next process a compile
+  const bool ok = fwrite(code.data(), 1, code.size(), f) == code.size();
+  fclose(f);
+  if (!ok || rename(tmp.c_str(), path.c_str()) != 0) remove(tmp.c_str());
+}
+
 int thcl_rt_kernel_cached(thcl_rt *rt, const char *key) { return rt->modules.count(key) ? 1 : 0; }
 
 // Modules are cached by `key`, entry points by (key, entry): one source holds
@@ -287,9 +338,19 @@ thcl_rt_kernel *thcl_rt_kernel_get(thcl_rt *rt, const char *key, const char *sou
     std::string arch = rt->props.arch;
     size_t colon = arch.find(':');
     if (colon != std::string::npos) arch = arch.substr(0, colon);
-    if (rtc_compile(source, arch.c_str(), code) != 0) return nullptr;
+    const std::string cached = disk_cache_path(source, arch);
+    hipError_t e = hipErrorInvalidValue;
     mod = new RtModule();
-    hipError_t e = hipModuleLoadData(&mod->module, code.data());
+    if (disk_cache_read(cached, code)) e = hipModuleLoadData(&mod->module, code.data());
+    if (e != hipSuccess) {  // nothing cached, or a file this runtime cannot load: compile
+      (void)hipGetLastError();
+      if (rtc_compile(source, arch.c_str(), code) != 0) {
+        delete mod;
+        return nullptr;
+      }
+      e = hipModuleLoadData(&mod->module, code.data());
+      if (e == hipSuccess) disk_cache_write(cached, code);
+    }
     if (e != hipSuccess) {
       fail("loading runtime-compiled code", e);
       delete mod;

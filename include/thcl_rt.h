@@ -63,7 +63,9 @@ float *thcl_rt_host_word(thcl_rt *rt);
 
 /* Runtime-compiled kernels (hipRTC), cached per context by `key`.  `source`
  * is complete HIP source; `entry` the extern "C" kernel name.  On a compile
- * error returns NULL and thcl_rt_error() holds the compiler log. */
+ * error returns NULL and thcl_rt_error() holds the compiler log.  With the
+ * environment variable THCL_KERNEL_CACHE_DIR set, compiled code objects are
+ * also kept in that directory and loaded from it by later processes. */
 thcl_rt_kernel *thcl_rt_kernel_get(thcl_rt *rt, const char *key, const char *source, const char *entry);
 int thcl_rt_kernel_cached(thcl_rt *rt, const char *key);
 int thcl_rt_launch(thcl_rt *rt, thcl_rt_kernel *k, unsigned gx, unsigned gy, unsigned gz, unsigned bx,

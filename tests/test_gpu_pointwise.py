@@ -1,6 +1,8 @@
 """GPU parity: pointwise apply, expressions and copies against the CPU oracle,
 bit for bit, through the C ABI (ctypes mirror of the Lua methods).  Modelled on
 the reference's own cases (src/test/unit_tensor.lua:225-359,583-635,759-775)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -380,3 +382,29 @@ def test_reshape_copies_in_logical_order(cl):
     with pytest.raises(cl.ClError):
         p.dev.reshape(7, 7)
 
+
+
+def test_compiled_kernels_persist_in_the_optional_disk_cache(cl, tmp_path):
+    """THCL_KERNEL_CACHE_DIR: the first process compiles and stores the code object, the
+    second loads it (same results, file untouched)."""
+    import subprocess
+    import sys
+    code = ("import numpy as np, cltorch_amd as cl\n"
+            "x = cl.ClTensor(np.arange(8, dtype=np.float32))\n"
+            "x.apply_on_gpu('x = x*3 + 0.125')\n"
+            "print(x.float().tolist())\n")
+    env = dict(os.environ, THCL_KERNEL_CACHE_DIR=str(tmp_path), PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    want = str([float(v * 3 + 0.125) for v in range(8)])
+    first = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert first.returncode == 0 and want in first.stdout, first.stderr[-500:]
+    files = sorted(tmp_path.glob("thcl_*.hsaco"))
+    assert len(files) == 1 and files[0].stat().st_size > 1000
+    stamp = files[0].stat().st_mtime_ns
+    second = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert second.returncode == 0 and want in second.stdout, second.stderr[-500:]
+    assert sorted(tmp_path.glob("thcl_*")) == files and files[0].stat().st_mtime_ns == stamp
+    # a damaged file is recompiled over, not trusted
+    files[0].write_bytes(b"not a code object")
+    third = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert third.returncode == 0 and want in third.stdout, third.stderr[-500:]
+    assert files[0].stat().st_size > 1000
