@@ -219,7 +219,7 @@ def pmc_workload(cl, n):
 def detail(cl, oracle, T, X, Y, Z, n):
     """The other benchmark configurations, a few launches each."""
     d = {}
-    reps = 10
+    reps = 20
 
     def measure(name, fn, work, unit="GB/s", reps=reps, peak=HBM_PEAK_GBS):
         fn()
@@ -280,7 +280,7 @@ def detail(cl, oracle, T, X, Y, Z, n):
     k = 8192
     sd = 1.0 / np.sqrt(k)
     Am, Bm, Cm = (cl.ClTensor(oracle.normal(s, k * k, 0.0, sd)).resize(k, k) for s in (8, 9, 10))
-    measure("c5_addmm_8192", lambda: Cm.addmm(0.5, 1.0, Am, Bm), 2.0 * k ** 3, "TFLOP/s", reps=5, peak=FP32_MFMA_PEAK_TFLOPS)
+    measure("c5_addmm_8192", lambda: Cm.addmm(0.5, 1.0, Am, Bm), 2.0 * k ** 3, "TFLOP/s", reps=10, peak=FP32_MFMA_PEAK_TFLOPS)
     del Am, Bm, Cm
     M, N, K = 64, 16384, 4096
     At = cl.ClTensor(oracle.normal(11, K * M, 0.0, sd)).resize(K, M)
