@@ -134,11 +134,14 @@ __device__ __forceinline__ double wave_inclusive(double v) {
   return v;
 }
 
-// I == 1: block (o, s) walks its segment of row o, 4 consecutive elements per thread per step.
+// I == 1: block (o, s) walks its segment of row o.  A step covers UNR runs of
+// 1024 elements; in each run a thread holds 4 consecutive elements (one 16-byte
+// access), so every wave reads whole lines, and the UNR runs share one pair of
+// barriers and keep UNR loads in flight per thread.
 template <bool PROD, int PHASE, bool VEC>
 __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
-  constexpr int WAVES = kThreads / kWave, PER = 4, STEP = kThreads * PER;
-  __shared__ double wave_tot[WAVES];
+  constexpr int WAVES = kThreads / kWave, PER = 4, RUN = kThreads * PER, UNR = 4, STEP = RUN * UNR;
+  __shared__ double wave_tot[UNR][WAVES];
   const thcl_u64 o = blockIdx.x / P.S, s = blockIdx.x % P.S;
   const thcl_u64 r0 = s * P.seg;
   thcl_u64 r1 = r0 + P.seg;
@@ -149,43 +152,56 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
   double carry = Op<PROD>::identity();
   if (PHASE == 1 && P.S > 1) carry = P.totals[blockIdx.x];
   for (thcl_u64 base = r0; base < r1; base += STEP) {
-    const thcl_u64 j = base + (thcl_u64)threadIdx.x * PER;
-    float x[PER];
-    if (VEC && j + PER <= r1) {
-      const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
+    float x[UNR][PER];
 #pragma unroll
-      for (int c = 0; c < PER; c++) x[c] = v[c];
-    } else {
-#pragma unroll
-      for (int c = 0; c < PER; c++) x[c] = (j + c < r1) ? row[j + c] : (PROD ? 1.0f : 0.0f);
-    }
-    double a[PER];
-    a[0] = (double)x[0];
-#pragma unroll
-    for (int c = 1; c < PER; c++) a[c] = Op<PROD>::comb(a[c - 1], (double)x[c]);
-    const double incl = wave_inclusive<PROD>(a[PER - 1]);
-    __syncthreads();  // wave_tot of the previous step has been read
-    if (lane == kWave - 1) wave_tot[wave] = incl;
-    __syncthreads();
-    double before = carry;  // everything ahead of this thread's first element
-#pragma unroll
-    for (int w = 0; w < WAVES; w++) {
-      if (w < wave) before = Op<PROD>::comb(before, wave_tot[w]);
-      carry = Op<PROD>::comb(carry, wave_tot[w]);
-    }
-    if (PHASE == 1) {
-      // lanes ahead in this wave: the exclusive prefix is the neighbour's inclusive one
-      const double prev = __shfl_up(incl, 1, kWave);
-      if (lane > 0) before = Op<PROD>::comb(before, prev);
+    for (int u = 0; u < UNR; u++) {
+      const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
       if (VEC && j + PER <= r1) {
-        thcl_f4 v;
+        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
 #pragma unroll
-        for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[c]);
-        __builtin_nontemporal_store(v, (thcl_f4 *)(orow + j));
+        for (int c = 0; c < PER; c++) x[u][c] = v[c];
       } else {
 #pragma unroll
-        for (int c = 0; c < PER; c++)
-          if (j + c < r1) orow[j + c] = (float)Op<PROD>::comb(before, a[c]);
+        for (int c = 0; c < PER; c++) x[u][c] = (j + c < r1) ? row[j + c] : (PROD ? 1.0f : 0.0f);
+      }
+    }
+    double a[UNR][PER], incl[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; u++) {
+      a[u][0] = (double)x[u][0];
+#pragma unroll
+      for (int c = 1; c < PER; c++) a[u][c] = Op<PROD>::comb(a[u][c - 1], (double)x[u][c]);
+      incl[u] = wave_inclusive<PROD>(a[u][PER - 1]);
+    }
+    __syncthreads();  // wave_tot of the previous step has been read
+    if (lane == kWave - 1) {
+#pragma unroll
+      for (int u = 0; u < UNR; u++) wave_tot[u][wave] = incl[u];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < UNR; u++) {
+      double before = carry;  // everything ahead of this thread's first element of run u
+#pragma unroll
+      for (int w = 0; w < WAVES; w++) {
+        if (w < wave) before = Op<PROD>::comb(before, wave_tot[u][w]);
+        carry = Op<PROD>::comb(carry, wave_tot[u][w]);
+      }
+      if (PHASE == 1) {
+        // lanes ahead in this wave: the exclusive prefix is the neighbour's inclusive one
+        const double prev = __shfl_up(incl[u], 1, kWave);
+        if (lane > 0) before = Op<PROD>::comb(before, prev);
+        const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
+        if (VEC && j + PER <= r1) {
+          thcl_f4 v;
+#pragma unroll
+          for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[u][c]);
+          __builtin_nontemporal_store(v, (thcl_f4 *)(orow + j));
+        } else {
+#pragma unroll
+          for (int c = 0; c < PER; c++)
+            if (j + c < r1) orow[j + c] = (float)Op<PROD>::comb(before, a[u][c]);
+        }
       }
     }
   }
@@ -363,7 +379,7 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     }
     if (S < 1) S = 1;
     thcl_u64 seg = (P.R + S - 1) / S;
-    if (rows) seg = (seg + 1023) / 1024 * 1024;  // whole steps, so vector accesses stay aligned
+    if (rows) seg = (seg + 4095) / 4096 * 4096;  // whole steps, so vector accesses stay aligned
     S = (P.R + seg - 1) / seg;
     P.S = S;
     P.seg = seg;
