@@ -292,6 +292,25 @@ def detail(cl, oracle, T, X, Y, Z, n):
         4.0 * (M * K + K * N + 2 * M * N) / (d["c5_addmm_skinny_64x16384x4096"]["avg_ms"] * 1e-3) * 1e-9, 1)
     del At, Bs, Cs
 
+    # the reference's own perf script times 900 calls of cmul / add / sum on 6400- and 64000-element
+    # tensors (src/test/test-perf.lua:43-106): per-call cost where launches, not bytes, dominate
+    lat = {}
+    for m_small in (6400, 64000):
+        sa, sb, spt = cl.ClTensor(m_small), cl.ClTensor(m_small), cl.ClTensor()
+        sa.fill(1.0)
+        sb.fill(1.0)
+        for name, fn in (("cmul", lambda: sa.cmul(sb)), ("add", lambda: sa.add(sb)), ("sum_to_point_tensor", lambda: spt.sum(sa)),
+                         ("sum_to_host", lambda: sa.sum())):
+            fn()
+            cl.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(900):
+                fn()
+            cl.synchronize()
+            lat[f"{name}_{m_small}"] = round((time.perf_counter() - t0) / 900 * 1e6, 2)
+    d["small_tensor_us_per_call"] = dict(lat, note="900 calls through the Python mirror, one synchronisation at the end "
+                                                   "(sum_to_host waits for every result)")
+
     # ---- the callers either side of the path: operator catalogue, scans, level-1/2, indexed movement
     A.fill(0.75)
     B = Y

@@ -332,15 +332,11 @@ float THClTensor_dot(THClState *state, THClTensor *self, THClTensor *src) {
   THClTensor *a = THClTensor_newContiguous(state, self);
   THClTensor *b = THClTensor_newContiguous(state, src);
   thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, self));
-  size_t sb = 0;
-  char *scratch = (char *)thcl_rt_scratch(rt, &sb);
-  float *dres = (float *)(scratch + sb - 256);
   float result = 0.f;
   try {
-    thcl_dot_dense(state, rt, thcl_dptr(a), thcl_dptr(b), n, dres);
-    float *hw = thcl_rt_host_word(rt);
-    THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, dres, sizeof(float)) == 0, "%s", thcl_rt_error());
-    result = hw[0];
+    thcl_dot_dense(state, rt, thcl_dptr(a), thcl_dptr(b), n, thcl_rt_host_word_device(rt));
+    THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
+    result = thcl_rt_host_word(rt)[0];
   } catch (...) {
     THClTensor_free(state, a);
     THClTensor_free(state, b);

@@ -495,18 +495,15 @@ void THLongTensor_copyCl(THClState *state, THLongTensor *self, THClTensor *src) 
 
 // -------------------------------------------------------------- reductions ---
 static float reduce_all_to_host(THClState *state, ThclReduce kind, THClTensor *self, float exponent = 0.f) {
-  // result lands in the device scratch block, then one word comes back: the
-  // only synchronising step (src/lib/THClTensorMath.cpp:346-368)
   THCL_CHECK(self->storage != nullptr || self->nDimension <= 0, "tensor has no storage");
   int device = THClTensor_getDevice(state, self);
   thcl_rt *rt = thcl_ctx(state, device);
-  size_t sb = 0;
-  char *scratch = (char *)thcl_rt_scratch(rt, &sb);
-  float *dres = (float *)(scratch + sb - 256);  // last 256 bytes of the block are the result slot
-  thcl_reduce_all(state, kind, self, dres, exponent);
-  float *hw = thcl_rt_host_word(rt);
-  THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, dres, sizeof(float)) == 0, "%s", thcl_rt_error());
-  return hw[0];
+  // the last block stores the scalar straight into pinned host memory; waiting
+  // for the stream is the only synchronising step, no copy follows
+  // (the reference: blocking read-back of the scratch buffer, src/lib/THClTensorMath.cpp:346-368)
+  thcl_reduce_all(state, kind, self, thcl_rt_host_word_device(rt), exponent);
+  THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
+  return thcl_rt_host_word(rt)[0];
 }
 static void reduce_all_to_point(THClState *state, ThclReduce kind, THClTensor *self, THClTensor *src) {
   thcl_check_same_device(state, 2, self, src);

@@ -30,6 +30,7 @@ struct thcl_rt {
   void *scratch = nullptr;
   size_t scratch_bytes = 0;
   float *host_word = nullptr;
+  float *host_word_dev = nullptr;  // the same words as the device addresses them
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
   thcl_rt_props props{};
@@ -119,7 +120,8 @@ thcl_rt *thcl_rt_get(int device) {
   }
   e = hipMalloc(&rt->scratch, kScratchBytes);
   if (e == hipSuccess) e = hipMemset(rt->scratch, 0, kScratchBytes);
-  if (e == hipSuccess) e = hipHostMalloc((void **)&rt->host_word, 64 * sizeof(float), hipHostMallocDefault);
+  if (e == hipSuccess) e = hipHostMalloc((void **)&rt->host_word, 64 * sizeof(float), hipHostMallocMapped);
+  if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&rt->host_word_dev, rt->host_word, 0);
   if (e == hipSuccess) e = hipDeviceSynchronize();
   if (e != hipSuccess) {
     fail("scratch allocation", e);
@@ -211,6 +213,7 @@ void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes) {
 }
 
 float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
+float *thcl_rt_host_word_device(thcl_rt *rt) { return rt->host_word_dev; }
 
 void *thcl_rt_workspace(thcl_rt *rt, size_t bytes) {
   if (bytes <= rt->workspace_bytes) return rt->workspace;

@@ -60,6 +60,9 @@ void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes);
 void *thcl_rt_workspace(thcl_rt *rt, size_t bytes);
 /* pinned host words for handing scalars back */
 float *thcl_rt_host_word(thcl_rt *rt);
+/* the same words at the address kernels use: a kernel may leave a scalar there
+ * directly, and the host reads it after thcl_rt_sync (no copy in between) */
+float *thcl_rt_host_word_device(thcl_rt *rt);
 
 /* Runtime-compiled kernels (hipRTC), cached per context by `key`.  `source`
  * is complete HIP source; `entry` the extern "C" kernel name.  On a compile
