@@ -37,14 +37,17 @@ void thcl_clear_error();
 
 // Entry points call one another; only the outermost one turns an exception
 // into a recorded error, inner ones let it propagate.
+void thcl_profile_enter(const char *entry);  // names the launches that follow (per-kernel profiling)
 struct ThclGuardScope {
   static thread_local int depth;
-  ThclGuardScope() { ++depth; }
+  explicit ThclGuardScope(const char *entry) {
+    if (++depth == 1) thcl_profile_enter(entry);
+  }
   ~ThclGuardScope() { --depth; }
   bool outer() const { return depth == 1; }
 };
 #define THCL_GUARD_BEGIN                  \
-  ThclGuardScope guard_scope_;            \
+  ThclGuardScope guard_scope_(__func__);  \
   if (guard_scope_.outer()) thcl_clear_error(); \
   try {
 #define THCL_GUARD_END(...)              \

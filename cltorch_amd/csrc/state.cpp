@@ -2,7 +2,10 @@
 // `TH` host types the C ABI mentions.
 #include <cstdio>
 #include <cstdlib>
+#include <algorithm>
 #include <cstring>
+#include <map>
+#include <string>
 #include <vector>
 
 #include "internal.h"
@@ -16,6 +19,43 @@ void *g_handler_data = nullptr;
 }  // namespace
 
 thread_local int ThclGuardScope::depth = 0;
+
+// ---------------------------------------------------------------- profiling ---
+// The reference's `cltorch.setProfiling(1)` / `dumpProfiling()` report OpenCL
+// event timings per kernel (src/init.cpp:149-178).  Here every launch made
+// while profiling is on sits between two HIP events on the library's stream
+// and is booked under the entry point that made it.
+namespace {
+struct ProfRecord {
+  const char *entry;
+  thcl_rt_timer *timer;
+};
+std::vector<ProfRecord> g_prof_records;
+bool g_prof_on = false;
+thread_local const char *tl_entry = "";
+thread_local thcl_rt_timer *tl_open = nullptr;  // started, waiting for the launch it will time
+
+void prof_open(thcl_rt *rt) {
+  if (!g_prof_on || tl_open) return;
+  tl_open = thcl_rt_timer_new(rt);
+  if (tl_open) thcl_rt_timer_start(tl_open);
+}
+void prof_close(thcl_rt *rt) {
+  if (!tl_open) return;
+  thcl_rt_timer_stop(tl_open);
+  g_prof_records.push_back({tl_entry, tl_open});
+  tl_open = nullptr;
+  prof_open(rt);  // an entry point may launch again
+}
+}  // namespace
+
+void thcl_profile_enter(const char *entry) {
+  tl_entry = entry;
+  if (tl_open) {  // opened by the previous call but never followed by a launch
+    thcl_rt_timer_free(tl_open);
+    tl_open = nullptr;
+  }
+}
 
 void thcl_throw(const char *fmt, ...) {
   char buf[2048];
@@ -246,10 +286,12 @@ thcl_rt *thcl_ctx(THClState *state, int device) {
     sp->data = thcl_rt_host_word(rt);
     state->scratchSpaceByDevice[device] = sp;
   }
+  prof_open(state->clByDevice[device]);
   return state->clByDevice[device];
 }
 
 void thcl_after_launch(THClState *state, thcl_rt *rt) {
+  prof_close(rt);
   if (state->addFinish) THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
 }
 
@@ -270,3 +312,44 @@ void thcl_check_same_device(THClState *state, int n, ...) {
   va_end(ap);
   THCL_CHECK(ok, "tensors are on different devices");
 }
+
+extern "C" {
+// `cltorch.setProfiling(on)` (src/init.cpp:166-178)
+void THClState_setProfiling(THClState *state, int on) {
+  (void)state;
+  g_prof_on = on != 0;
+}
+// `cltorch.dumpProfiling()` (src/init.cpp:149-157): waits for the device, writes one
+// line per entry point -- launches, total and mean milliseconds -- into `buf`
+// (always NUL-terminated within `cap`), forgets the records, and returns the
+// number of characters the full report needs.
+long THClState_dumpProfiling(THClState *state, char *buf, long cap) {
+  THCL_GUARD_BEGIN
+  for (int d = 0; d < state->allocatedDevices; d++)
+    if (state->clByDevice[d]) THCL_CHECK(thcl_rt_sync(state->clByDevice[d]) == 0, "%s", thcl_rt_error());
+  std::map<std::string, std::pair<long, double>> agg;
+  for (auto &r : g_prof_records) {
+    auto &a = agg[r.entry];
+    a.first += 1;
+    a.second += (double)thcl_rt_timer_ms(r.timer);
+    thcl_rt_timer_free(r.timer);
+  }
+  g_prof_records.clear();
+  std::vector<std::pair<std::string, std::pair<long, double>>> rows(agg.begin(), agg.end());
+  std::sort(rows.begin(), rows.end(), [](const auto &x, const auto &y) { return x.second.second > y.second.second; });
+  std::string out = "entry point, launches, total ms, mean ms\n";
+  char line[256];
+  for (auto &r : rows) {
+    snprintf(line, sizeof(line), "%s, %ld, %.4f, %.4f\n", r.first.c_str(), r.second.first, r.second.second,
+             r.second.second / (double)r.second.first);
+    out += line;
+  }
+  if (buf && cap > 0) {
+    const size_t n = out.size() < (size_t)cap - 1 ? out.size() : (size_t)cap - 1;
+    memcpy(buf, out.data(), n);
+    buf[n] = 0;
+  }
+  return (long)out.size();
+  THCL_GUARD_END(-1)
+}
+}  // extern "C"

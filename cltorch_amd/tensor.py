@@ -69,6 +69,18 @@ def synchronize() -> None:
 finish = synchronize
 
 
+def setProfiling(on) -> None:
+    """``cltorch.setProfiling(1)``: time every launch with device events."""
+    _call("THClState_setProfiling", C.c_int(1 if on else 0))
+
+
+def dumpProfiling() -> str:
+    """``cltorch.dumpProfiling()``: per entry point -- launches, total and mean ms; clears the records."""
+    buf = C.create_string_buffer(1 << 16)
+    _call("THClState_dumpProfiling", buf, C.c_long(len(buf)))
+    return buf.value.decode()
+
+
 def getDeviceCount() -> int:
     return int(_call("THClState_getNumDevices"))
 

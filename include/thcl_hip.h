@@ -157,6 +157,13 @@ struct thcl_rt *THClState_getClv2(THClState *state, int device);
 /* src/lib/THClGeneral.h:128-131 */
 struct THClScratchSpace *THClState_getDeviceScratchSpace(THClState *state, int device, int stream);
 size_t THClState_getDeviceScratchSpaceSize(THClState *state, int device);
+/* `cltorch.setProfiling(on)` / `cltorch.dumpProfiling()` (src/init.cpp:149-178): while on,
+ * every launch is timed with HIP events and booked under the entry point that
+ * made it.  dumpProfiling waits for the device, writes "entry point, launches,
+ * total ms, mean ms" lines into buf (NUL-terminated within cap), forgets the
+ * records and returns the length of the full report. */
+void THClState_setProfiling(THClState *state, int on);
+long THClState_dumpProfiling(THClState *state, char *buf, long cap);
 /* `cltorch.synchronize()` / `cltorch.finish()`: src/init.cpp:72-78 */
 void THClState_synchronize(THClState *state);
 

@@ -213,3 +213,27 @@ def test_dim_argument_checks(cl):
         X.max(0)
     with pytest.raises(cl.ClError):
         cl.ClTensor(np.zeros(3, dtype=F)).s()              # not a point tensor
+
+
+def test_profiling_books_launches_under_their_entry_points(cl):
+    """cltorch.setProfiling / dumpProfiling (src/init.cpp:149-178)."""
+    x = cl.ClTensor(np.ones(1 << 20, dtype=F))
+    y = cl.ClTensor(np.ones(1 << 20, dtype=F))
+    cl.dumpProfiling()                                   # forget whatever came before
+    cl.setProfiling(1)
+    for _ in range(5):
+        x.add(y)
+    x.cmul(y)
+    total = x.sum()
+    g = cl.ClTensor(np.ones((4096, 64), dtype=F))
+    g.sum(1)                                             # a split column reduction: main kernel (+ fold)
+    cl.setProfiling(0)
+    x.add(y)                                             # not recorded
+    report = cl.dumpProfiling()
+    rows = {l.split(",")[0]: [float(v) for v in l.split(",")[1:]] for l in report.strip().splitlines()[1:]}
+    assert rows["THClTensor_cadd"][0] == 5 and rows["THClTensor_cmul"][0] == 1
+    assert rows["THClTensor_sumall"][0] == 1 and rows["THClTensor_sum"][0] >= 1
+    assert all(r[1] > 0 and abs(r[2] - r[1] / r[0]) < 1e-3 for r in rows.values())
+    assert 0.001 < rows["THClTensor_cadd"][2] < 5.0      # milliseconds per launch: microseconds, not seconds
+    assert total == 6.0 * (1 << 20)
+    assert cl.dumpProfiling().strip().count("\n") == 0    # records were cleared
