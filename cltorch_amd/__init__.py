@@ -6,8 +6,8 @@ pointwise / copy / reduce / addmm path.  ``ClTensor`` mirrors the Lua methods
 on top of it.  Importing this package does not touch a GPU; the first tensor
 does, and raises if no device or no built library is present.
 """
-from .tensor import (ClError, ClKernel, ClTensor, dumpProfiling, setProfiling, finish, ger, getDeviceCount, mm, mv, setAddFinish, state,  # noqa: F401
+from .tensor import (ClError, ClKernel, ClTensor, dumpProfiling, emptyCache, memoryStats, setProfiling, finish, ger, getDeviceCount, mm, mv, setAddFinish, state,  # noqa: F401
                      synchronize)
 from . import _lib  # noqa: F401
 
-__all__ = ["ClTensor", "ClError", "ClKernel", "mm", "mv", "ger", "synchronize", "finish", "setProfiling", "dumpProfiling", "getDeviceCount", "setAddFinish", "state"]
+__all__ = ["ClTensor", "ClError", "ClKernel", "mm", "mv", "ger", "synchronize", "finish", "setProfiling", "dumpProfiling", "memoryStats", "emptyCache", "getDeviceCount", "setAddFinish", "state"]

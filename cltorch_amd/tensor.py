@@ -69,6 +69,23 @@ def synchronize() -> None:
 finish = synchronize
 
 
+def memoryStats(device: int = 1) -> dict:
+    """Bytes in live tensors, bytes kept in the block cache, and how many requests
+    went to the driver or were served from the cache (device is 1-based)."""
+    st = state()
+    rt = st.lib.THClState_getClv2(st.ptr, device - 1)
+    live, cached = C.c_size_t(0), C.c_size_t(0)
+    mallocs, hits = C.c_ulonglong(0), C.c_ulonglong(0)
+    st.lib.thcl_rt_memory_stats(rt, C.byref(live), C.byref(cached), C.byref(mallocs), C.byref(hits))
+    return {"live_bytes": live.value, "cached_bytes": cached.value, "device_mallocs": mallocs.value, "cache_hits": hits.value}
+
+
+def emptyCache(device: int = 1) -> None:
+    """Hands every cached block back to the driver."""
+    st = state()
+    st.lib.thcl_rt_empty_cache(st.lib.THClState_getClv2(st.ptr, device - 1))
+
+
 def setProfiling(on) -> None:
     """``cltorch.setProfiling(1)``: time every launch with device events."""
     _call("THClState_setProfiling", C.c_int(1 if on else 0))

@@ -43,8 +43,15 @@ const thcl_rt_props *thcl_rt_get_props(thcl_rt *rt);
 const char *thcl_rt_error(void);
 
 /* buffers */
+/* Released blocks are kept and handed out again (safe because each context has
+ * one in-order stream); at most half the device's memory, or THCL_ALLOC_CACHE_MB
+ * megabytes (0: no caching), stays cached, and the cache is emptied when the
+ * driver runs out of memory. */
 void *thcl_rt_malloc(thcl_rt *rt, size_t bytes);
 int thcl_rt_free(thcl_rt *rt, void *dptr);
+int thcl_rt_empty_cache(thcl_rt *rt);
+void thcl_rt_memory_stats(thcl_rt *rt, size_t *live_bytes, size_t *cached_bytes, unsigned long long *device_mallocs,
+                          unsigned long long *cache_hits);
 int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
 int thcl_rt_memcpy_d2h(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
 int thcl_rt_memcpy_d2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* queued            */

@@ -208,3 +208,34 @@ def test_dense_tensors_beyond_32_bit_element_counts(cl):
     X.strided((half, 2), (1, half)).add(1.0)                 # a transposed walk over every element: dense after sorting dims
     assert X.max() == 7.0 and X.min() == -9.0
 
+
+
+def test_released_blocks_are_reused_without_stalling_or_mixing_owners(cl):
+    """The block cache: a tensor's memory goes to the next request of its size while
+    the old owner's kernels may still be queued; stream order keeps both right."""
+    n = 1 << 26
+    cl.synchronize()
+    cl.emptyCache()
+    before = cl.memoryStats()
+    results = []
+    for i in range(12):
+        t = cl.ClTensor(n)                       # from the second round on: the block the previous t released
+        t.fill(float(i + 1))
+        pt = cl.ClTensor()
+        pt.sum(t)                                # queued; t is released before it has run
+        results.append(pt)
+        del t
+    after = cl.memoryStats()
+    assert [r.s() for r in results] == [float(n) * (i + 1) for i in range(12)]
+    assert after["device_mallocs"] - before["device_mallocs"] <= 3 + 12   # one big block (+ the point tensors), not twelve
+    assert after["cache_hits"] - before["cache_hits"] >= 11
+    assert after["cached_bytes"] >= 4 * n
+    # a smaller request may take a block up to a quarter larger, not more
+    small = cl.ClTensor(n // 2)
+    assert cl.memoryStats()["cached_bytes"] >= 4 * n              # the 256 MiB block was not handed to a 128 MiB request
+    del small
+    cl.emptyCache()
+    assert cl.memoryStats()["cached_bytes"] == 0
+    x = cl.ClTensor(n)
+    x.fill(2.0)
+    assert x.sum() == 2.0 * n
