@@ -408,3 +408,21 @@ def test_compiled_kernels_persist_in_the_optional_disk_cache(cl, tmp_path):
     third = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
     assert third.returncode == 0 and want in third.stdout, third.stderr[-500:]
     assert files[0].stat().st_size > 1000
+
+
+def test_denormal_operands_and_results_are_kept(cl):
+    """Subnormal fp32 values are neither flushed on input nor on output, in fixed
+    operators and in run-time compiled expressions alike."""
+    x = np.array([1e-39, 3e-42, 1.1754944e-38, -2e-40, 1e-20, 5e-45, 0.0, -0.0], dtype=F)
+    y = np.array([0.5, 3.0, 0.5, 2.0, 1e-20, 0.5, 1e-45, -1.0], dtype=F)
+    X, Y = cl.ClTensor(x), cl.ClTensor(y)
+    with np.errstate(all="ignore"):
+        assert_bit_equal(X.clone().cmul(Y).float(), x * y, "cmul")
+        assert_bit_equal(X.clone().add(Y).float(), x + y, "add")
+        assert_bit_equal(X.clone().cdiv(Y).float(), x / y, "cdiv")
+        assert_bit_equal(X.clone().abs().sqrt().float(), np.sqrt(np.abs(x)), "sqrt")
+        assert_bit_equal(X.clone().mul(0.25).float(), x * F(0.25), "mul scalar")
+        want = expr_host.evaluate("x = x*y + x", x.copy(), y)
+        assert_bit_equal(X.clone().map_on_gpu(Y, "x = x*y + x").float(), want, "expression")
+    assert X.sum() == float(np.float32(x.astype(np.float64).sum()))
+    assert X.min() == float(x.min()) and X.max() == float(x.max())
