@@ -279,3 +279,15 @@ def test_user_kernel_renders_and_compiles_for_gfx950(lib):
     assert size.value > 1000
     lib.THClKernel_free(None, k)
 
+
+def test_gemm_tile_choice(lib):
+    """128x128 tiles unless that leaves fewer than 4 tiles per CU; ragged or small dims use 64-wide tiles."""
+    def tile(m, n, cus=256):
+        bm, bn = C.c_int(0), C.c_int(0)
+        lib.thcl_dbg_gemm_tile(C.c_long(m), C.c_long(n), C.c_int(cus), C.byref(bm), C.byref(bn))
+        return bm.value, bn.value
+    assert tile(8192, 8192) == (128, 128) and tile(4096, 4096) == (128, 128)
+    assert tile(3072, 3072) == (128, 64) and tile(2048, 2048) == (64, 64) and tile(1024, 1024) == (64, 64)
+    assert tile(16384, 64) == (128, 64)          # the skinny configuration after the row-major swap
+    assert tile(100, 100) == (64, 64) and tile(200, 4096) == (64, 128)
+
