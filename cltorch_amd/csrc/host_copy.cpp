@@ -174,6 +174,36 @@ THCL_HOST_TYPE(Int, int)
 THCL_HOST_TYPE(Double, double)
 #undef THCL_HOST_TYPE
 
+// whole storages, host element types other than float (src/lib/THClStorageCopy.cpp:45-60,75-94)
+#define THCL_HOST_STORAGE(Name, T)                                                                           \
+  void THClStorage_copy##Name(THClState *state, THClStorage *self, TH##Name##Storage *src) {               \
+    THCL_GUARD_BEGIN                                                                                         \
+    THCL_ARGCHECK(self->size == src->size, 2, "size does not match");                                        \
+    std::vector<float> f((size_t)src->size);                                                                 \
+    for (long i = 0; i < src->size; i++) f[(size_t)i] = (float)src->data[i];                                 \
+    if (src->size > 0) THClStorage_rawCopy(state, self, f.data());                                           \
+    THCL_GUARD_END()                                                                                         \
+  }                                                                                                          \
+  void TH##Name##Storage_copyCl(THClState *state, TH##Name##Storage *self, THClStorage *src) {             \
+    THCL_GUARD_BEGIN                                                                                         \
+    THCL_ARGCHECK(self->size == src->size, 2, "size does not match");                                        \
+    std::vector<float> f((size_t)src->size);                                                                 \
+    THFloatStorage fs;                                                                                       \
+    memset(&fs, 0, sizeof(fs));                                                                              \
+    fs.data = f.data();                                                                                      \
+    fs.size = src->size;                                                                                     \
+    if (src->size > 0) THFloatStorage_copyCl(state, &fs, src);                                               \
+    for (long i = 0; i < src->size; i++) self->data[i] = (T)f[(size_t)i];                                    \
+    THCL_GUARD_END()                                                                                         \
+  }
+THCL_HOST_STORAGE(Byte, unsigned char)
+THCL_HOST_STORAGE(Char, char)
+THCL_HOST_STORAGE(Short, short)
+THCL_HOST_STORAGE(Int, int)
+THCL_HOST_STORAGE(Long, long)
+THCL_HOST_STORAGE(Double, double)
+#undef THCL_HOST_STORAGE
+
 #ifndef THCL_EXTERNAL_TH
 #define THCL_HOST_STANDIN(Name, T)                                                                           \
   TH##Name##Tensor *TH##Name##Tensor_newWithData(T *data, long storageSize, long storageOffset, int nDimension, \

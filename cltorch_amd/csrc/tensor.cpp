@@ -529,4 +529,77 @@ float THClTensor_get2d(THClState *state, const THClTensor *t, long x0, long x1) 
   THCL_GUARD_END(0.f)
 }
 
+// ---- the rest of the header / storage interface (src/lib/THClTensor.h:31-145,
+//      src/lib/THClStorage.h:28-59, src/lib/THClStorageCopy.h:9-30)
+void THClTensor_setFlag(THClState *, THClTensor *self, const char flag) { self->flag |= flag; }
+void THClTensor_clearFlag(THClState *, THClTensor *self, const char flag) { self->flag &= ~flag; }
+void THClStorage_setFlag(THClState *, THClStorage *s, const char flag) { s->flag |= flag; }
+void THClStorage_clearFlag(THClState *, THClStorage *s, const char flag) { s->flag &= ~flag; }
+
+void THClTensor_resize5d(THClState *state, THClTensor *self, long s0, long s1, long s2, long s3, long s4) {
+  THCL_GUARD_BEGIN
+  long size[5] = {s0, s1, s2, s3, s4};
+  header_resize(state, self, 5, size, nullptr);
+  THCL_GUARD_END()
+}
+// drops `dimension` when its size is 1 (src/lib/THClTensor.cpp:528-548)
+void THClTensor_squeeze1d(THClState *state, THClTensor *self, THClTensor *src, int dimension) {
+  THCL_GUARD_BEGIN
+  if (!src) src = self;
+  THCL_ARGCHECK(dimension >= 0 && dimension < src->nDimension, 3, "dimension out of range");
+  THClTensor_set(state, self, src);
+  if (src->size[dimension] == 1 && src->nDimension > 1) {
+    for (int d = dimension; d < self->nDimension - 1; d++) {
+      self->size[d] = self->size[d + 1];
+      self->stride[d] = self->stride[d + 1];
+    }
+    self->nDimension--;
+  }
+  THCL_GUARD_END()
+}
+void THClTensor_set3d(THClState *state, THClTensor *t, long x0, long x1, long x2, float value) {
+  THCL_GUARD_BEGIN
+  THCL_ARGCHECK(t->nDimension == 3, 1, "tensor must have three dimensions");
+  THCL_ARGCHECK(x0 >= 0 && x0 < t->size[0] && x1 >= 0 && x1 < t->size[1] && x2 >= 0 && x2 < t->size[2], 2, "out of range");
+  THClStorage_set(state, t->storage, t->storageOffset + x0 * t->stride[0] + x1 * t->stride[1] + x2 * t->stride[2], value);
+  THCL_GUARD_END()
+}
+float THClTensor_get3d(THClState *state, const THClTensor *t, long x0, long x1, long x2) {
+  THCL_GUARD_BEGIN
+  THCL_ARGCHECK(t->nDimension == 3, 1, "tensor must have three dimensions");
+  THCL_ARGCHECK(x0 >= 0 && x0 < t->size[0] && x1 >= 0 && x1 < t->size[1] && x2 >= 0 && x2 < t->size[2], 2, "out of range");
+  return THClStorage_get(state, t->storage, t->storageOffset + x0 * t->stride[0] + x1 * t->stride[1] + x2 * t->stride[2]);
+  THCL_GUARD_END(0.f)
+}
+void THClTensor_set4d(THClState *state, THClTensor *t, long x0, long x1, long x2, long x3, float value) {
+  THCL_GUARD_BEGIN
+  THCL_ARGCHECK(t->nDimension == 4, 1, "tensor must have four dimensions");
+  THCL_ARGCHECK(x0 >= 0 && x0 < t->size[0] && x1 >= 0 && x1 < t->size[1] && x2 >= 0 && x2 < t->size[2] && x3 >= 0 &&
+                    x3 < t->size[3],
+                2, "out of range");
+  THClStorage_set(state, t->storage,
+                  t->storageOffset + x0 * t->stride[0] + x1 * t->stride[1] + x2 * t->stride[2] + x3 * t->stride[3], value);
+  THCL_GUARD_END()
+}
+float THClTensor_get4d(THClState *state, const THClTensor *t, long x0, long x1, long x2, long x3) {
+  THCL_GUARD_BEGIN
+  THCL_ARGCHECK(t->nDimension == 4, 1, "tensor must have four dimensions");
+  THCL_ARGCHECK(x0 >= 0 && x0 < t->size[0] && x1 >= 0 && x1 < t->size[1] && x2 >= 0 && x2 < t->size[2] && x3 >= 0 &&
+                    x3 < t->size[3],
+                2, "out of range");
+  return THClStorage_get(state, t->storage,
+                         t->storageOffset + x0 * t->stride[0] + x1 * t->stride[1] + x2 * t->stride[2] + x3 * t->stride[3]);
+  THCL_GUARD_END(0.f)
+}
+// device to device, whole storages (src/lib/THClStorageCopy.cpp:17-25)
+void THClStorage_copy(THClState *state, THClStorage *self, THClStorage *src) {
+  THCL_GUARD_BEGIN
+  THCL_ARGCHECK(self->size == src->size, 2, "size does not match");
+  THCL_CHECK(self->device == src->device, "copy between devices is not implemented");
+  if (self->size > 0 && self != src)
+    THCL_CHECK(thcl_rt_memcpy_d2d(self->cl, self->wrapper, src->wrapper, (size_t)self->size * sizeof(float)) == 0, "%s",
+               thcl_rt_error());
+  THCL_GUARD_END()
+}
+
 }  // extern "C"

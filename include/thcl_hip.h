@@ -202,6 +202,23 @@ void THClStorage_retain(THClState *state, THClStorage *s);
 void THClStorage_free(THClState *state, THClStorage *s);
 void THClStorage_resize(THClState *state, THClStorage *s, long size);
 void THClStorage_fill(THClState *state, THClStorage *s, float value);
+void THClStorage_setFlag(THClState *state, THClStorage *s, const char flag);
+void THClStorage_clearFlag(THClState *state, THClStorage *s, const char flag);
+/* whole-storage copies: device to device, and host storages of every element
+ * type both ways (src/lib/THClStorageCopy.h:9-30) */
+void THClStorage_copy(THClState *state, THClStorage *self, THClStorage *src);
+void THClStorage_copyByte(THClState *state, THClStorage *self, THByteStorage *src);
+void THClStorage_copyChar(THClState *state, THClStorage *self, THCharStorage *src);
+void THClStorage_copyShort(THClState *state, THClStorage *self, THShortStorage *src);
+void THClStorage_copyInt(THClState *state, THClStorage *self, THIntStorage *src);
+void THClStorage_copyLong(THClState *state, THClStorage *self, THLongStorage *src);
+void THClStorage_copyDouble(THClState *state, THClStorage *self, THDoubleStorage *src);
+void THByteStorage_copyCl(THClState *state, THByteStorage *self, THClStorage *src);
+void THCharStorage_copyCl(THClState *state, THCharStorage *self, THClStorage *src);
+void THShortStorage_copyCl(THClState *state, THShortStorage *self, THClStorage *src);
+void THIntStorage_copyCl(THClState *state, THIntStorage *self, THClStorage *src);
+void THLongStorage_copyCl(THClState *state, THLongStorage *self, THClStorage *src);
+void THDoubleStorage_copyCl(THClState *state, THDoubleStorage *self, THClStorage *src);
 /* src/lib/THClStorageCopy.h:9-10,27 */
 void THClStorage_rawCopy(THClState *state, THClStorage *s, float *src);
 void THClStorage_copyFloat(THClState *state, THClStorage *s, THFloatStorage *src);
@@ -250,6 +267,14 @@ THClTensor *THClTensor_newUnfold(THClState *state, THClTensor *tensor, int dimen
 void THClTensor_resize(THClState *state, THClTensor *self, THLongStorage *size, THLongStorage *stride);
 void THClTensor_resizeAs(THClState *state, THClTensor *self, THClTensor *src);
 void THClTensor_resize0d(THClState *state, THClTensor *self);
+void THClTensor_setFlag(THClState *state, THClTensor *self, const char flag);
+void THClTensor_clearFlag(THClState *state, THClTensor *self, const char flag);
+void THClTensor_resize5d(THClState *state, THClTensor *self, long size0, long size1, long size2, long size3, long size4);
+void THClTensor_squeeze1d(THClState *state, THClTensor *self, THClTensor *src, int dimension);
+void THClTensor_set3d(THClState *state, THClTensor *tensor, long x0, long x1, long x2, float value);
+float THClTensor_get3d(THClState *state, const THClTensor *tensor, long x0, long x1, long x2);
+void THClTensor_set4d(THClState *state, THClTensor *tensor, long x0, long x1, long x2, long x3, float value);
+float THClTensor_get4d(THClState *state, const THClTensor *tensor, long x0, long x1, long x2, long x3);
 void THClTensor_resize1d(THClState *state, THClTensor *self, long size0);
 void THClTensor_resize2d(THClState *state, THClTensor *self, long size0, long size1);
 void THClTensor_resize3d(THClState *state, THClTensor *self, long size0, long size1, long size2);

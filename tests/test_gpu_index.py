@@ -199,3 +199,49 @@ def test_host_element_types_and_byte_masks(cl):
     Xc = cl.ClTensor(x)
     Xc.maskedCopy(m, cl.ClTensor(src))
     assert_bit_equal(Xc.float(), cat.masked_copy(x, m, src), "maskedCopyByte")
+
+
+def test_header_and_storage_interface_extras(cl):
+    """resize5d, squeeze1d, 3-d / 4-d element access, whole-storage copies of every host
+    element type (src/lib/THClTensor.h:31-145, src/lib/THClStorageCopy.h:9-30)."""
+    import ctypes as C
+    from cltorch_amd.tensor import _call
+    t = cl.ClTensor()
+    _call("THClTensor_resize5d", t._h, 2, 1, 3, 1, 4)
+    assert t.size() == (2, 1, 3, 1, 4) and t.isContiguous()
+    u = cl.ClTensor()
+    _call("THClTensor_squeeze1d", u._h, t._h, C.c_int(1))
+    assert u.size() == (2, 3, 1, 4)
+    _call("THClTensor_squeeze1d", u._h, u._h, C.c_int(0))            # size 2: nothing to drop
+    assert u.size() == (2, 3, 1, 4)
+    u.zero()
+    _call("THClTensor_set4d", u._h, 1, 2, 0, 3, C.c_float(7.5))
+    lib = cl.state().lib
+    lib.THClTensor_get4d.restype = C.c_float
+    assert _call("THClTensor_get4d", u._h, 1, 2, 0, 3) == 7.5 and u.float()[1, 2, 0, 3] == 7.5 and u.sum() == 7.5
+    v = cl.ClTensor(3, 4, 5).zero().transpose(1, 3)
+    _call("THClTensor_set3d", v._h, 4, 1, 2, C.c_float(-2.0))
+    assert _call("THClTensor_get3d", v._h, 4, 1, 2) == -2.0 and v.float()[4, 1, 2] == -2.0
+    with pytest.raises(cl.ClError):
+        _call("THClTensor_get3d", v._h, 5, 0, 0)
+    # whole storages
+    a = cl.ClTensor(np.arange(10, dtype=F))
+    b = cl.ClTensor(10).zero()
+    sa = lib.THClTensor_storage(cl.state().ptr, a._h)
+    sb = lib.THClTensor_storage(cl.state().ptr, b._h)
+    _call("THClStorage_copy", sb, sa)
+    assert b.float().tolist() == list(range(10))
+
+    class _Storage(C.Structure):
+        _fields_ = [("data", C.c_void_p), ("size", C.c_long), ("refcount", C.c_int), ("flag", C.c_char),
+                    ("allocator", C.c_void_p), ("allocatorContext", C.c_void_p), ("view", C.c_void_p)]
+    for name, dtype in (("Byte", np.uint8), ("Char", np.int8), ("Short", np.int16), ("Int", np.int32), ("Long", np.int64),
+                        ("Double", np.float64)):
+        h = (np.arange(10) * 3 % 100).astype(dtype)
+        hs = _Storage(h.ctypes.data, 10, 1, b"\x00", None, None, None)
+        _call(f"THClStorage_copy{name}", sb, C.byref(hs))
+        assert b.float().tolist() == h.astype(F).tolist(), name
+        out = np.zeros(10, dtype=dtype)
+        os_ = _Storage(out.ctypes.data, 10, 1, b"\x00", None, None, None)
+        _call(f"TH{name}Storage_copyCl", C.byref(os_), sa)
+        assert out.tolist() == list(range(10)), name
