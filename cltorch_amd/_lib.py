@@ -23,7 +23,7 @@ class LibraryMissing(RuntimeError):
 
 
 _SCALARS = {
-    "void": None, "int": C.c_int, "unsigned": C.c_uint, "long": C.c_long, "float": C.c_float,
+    "void": None, "int": C.c_int, "unsigned": C.c_uint, "unsigned int": C.c_uint, "long": C.c_long, "float": C.c_float,
     "double": C.c_double, "char": C.c_char, "size_t": C.c_size_t, "int64_t": C.c_int64,
 }
 
@@ -65,6 +65,8 @@ def parse_declarations(path: str) -> Dict[str, Tuple[object, List[object]]]:
         if args and args != "void":
             for a in args.split(","):
                 a = a.strip()
+                if a == "...":          # variadic tail: ctypes passes extra arguments as given
+                    continue
                 # strip the parameter name (last identifier) unless the type ends in '*'
                 mm = re.match(r"^(.*?)(\b\w+)$", a)
                 if mm and mm.group(1).strip():

@@ -263,6 +263,18 @@ size_t THClState_getDeviceScratchSpaceSize(THClState *state, int device) {
   THCL_GUARD_END(0)
 }
 
+struct thcl_rt *THClState_getCl(THClState *state) { return THClState_getClv2(state, state->currentDevice); }
+struct thcl_rt *THClState_getClAndDevice(THClState *state, int *p_device) {
+  if (p_device) *p_device = state->currentDevice;
+  return THClState_getClv2(state, state->currentDevice);
+}
+struct THClScratchSpace *THClState_getCurrentDeviceScratchSpace(THClState *state) {
+  return THClState_getDeviceScratchSpace(state, state->currentDevice, 0);
+}
+size_t THClState_getCurrentDeviceScratchSpaceSize(THClState *state) {
+  return THClState_getDeviceScratchSpaceSize(state, state->currentDevice);
+}
+
 void THClState_synchronize(THClState *state) {
   THCL_GUARD_BEGIN
   for (int d = 0; d < state->allocatedDevices; d++)

@@ -5,6 +5,7 @@
 // is a refcounted header (sizes, strides, offset) over a storage; narrow /
 // select / transpose / unfold only rewrite the header
 // (src/lib/THClTensor.cpp:389-520).
+#include <cstdarg>
 #include <cstdlib>
 #include <cstdio>
 #include <cstring>
@@ -135,6 +136,7 @@ THClStorage *THClStorage_newv2(THClState *state, int device) {
   return storage_new(state, device, 0);
   THCL_GUARD_END(nullptr)
 }
+THClStorage *THClStorage_new(THClState *state) { return THClStorage_newv2(state, state->currentDevice); }
 THClStorage *THClStorage_newWithSize(THClState *state, int device, long size) {
   THCL_GUARD_BEGIN
   return storage_new(state, device, size);
@@ -243,6 +245,27 @@ THClTensor *THClTensor_newv2(THClState *state, int device) {
   return header_new(device);
   THCL_GUARD_END(nullptr)
 }
+THClTensor *THClTensor_new(THClState *state) { return THClTensor_newv2(state, state->currentDevice); }
+
+int THClTensor_checkGPU(THClState *, unsigned int nTensors, ...) {
+  va_list args;
+  va_start(args, nTensors);
+  int first = -1, same = 1;
+  for (unsigned int i = 0; i < nTensors; i++) {
+    const THClTensor *t = va_arg(args, const THClTensor *);
+    if (!t) continue;
+    if (first < 0) first = t->device;
+    if (t->device != first) same = 0;
+  }
+  va_end(args);
+  return same;
+}
+
+struct thcl_rt *THClTensor_getCl(THClState *, const THClTensor *tensor) {
+  return tensor->storage ? tensor->storage->cl : nullptr;
+}
+void *THClTensor_wrapper(THClState *, const THClTensor *self) { return self->storage ? self->storage->wrapper : nullptr; }
+
 THClTensor *THClTensor_newWithTensor(THClState *state, THClTensor *tensor) {
   THCL_GUARD_BEGIN
   THClTensor *t = header_new(tensor->device);

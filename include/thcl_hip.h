@@ -157,6 +157,12 @@ struct thcl_rt *THClState_getClv2(THClState *state, int device);
 /* src/lib/THClGeneral.h:128-131 */
 struct THClScratchSpace *THClState_getDeviceScratchSpace(THClState *state, int device, int stream);
 size_t THClState_getDeviceScratchSpaceSize(THClState *state, int device);
+/* Forms the reference keeps for old callers, all acting on the current device
+ * (src/lib/THClGeneral.h:105-106,128,130; src/lib/THClGeneral.cpp:119-133,178-185). */
+struct thcl_rt *THClState_getCl(THClState *state);
+struct thcl_rt *THClState_getClAndDevice(THClState *state, int *p_device);
+struct THClScratchSpace *THClState_getCurrentDeviceScratchSpace(THClState *state);
+size_t THClState_getCurrentDeviceScratchSpaceSize(THClState *state);
 /* `cltorch.setProfiling(on)` / `cltorch.dumpProfiling()` (src/init.cpp:149-178): while on,
  * every launch is timed with HIP events and booked under the entry point that
  * made it.  dumpProfiling waits for the device, writes "entry point, launches,
@@ -197,6 +203,8 @@ long THClStorage_size(THClState *state, const THClStorage *s);
 void THClStorage_set(THClState *state, THClStorage *s, long index, float value);
 float THClStorage_get(THClState *state, const THClStorage *s, long index);
 THClStorage *THClStorage_newv2(THClState *state, int device);
+/* on the current device (src/lib/THClStorage.cpp:93-96) */
+THClStorage *THClStorage_new(THClState *state);
 THClStorage *THClStorage_newWithSize(THClState *state, int device, long size);
 void THClStorage_retain(THClState *state, THClStorage *s);
 void THClStorage_free(THClState *state, THClStorage *s);
@@ -249,6 +257,16 @@ THLongStorage *THClTensor_newStrideOf(THClState *state, THClTensor *self);
 float *THClTensor_data(THClState *state, const THClTensor *self);
 
 THClTensor *THClTensor_newv2(THClState *state, int device);
+/* on the current device (src/lib/THClTensor.cpp:92-95) */
+THClTensor *THClTensor_new(THClState *state);
+/* 1 when every non-NULL tensor of the nTensors that follow lives on one device
+ * (src/lib/THClTensor.cpp:844-873) */
+int THClTensor_checkGPU(THClState *state, unsigned int nTensors, ...);
+/* the runtime context of the tensor's storage (src/lib/THClTensor.cpp:900-902) and the
+ * device address of that storage's first element, NULL without a storage
+ * (src/lib/THClTensor.cpp:66-72: the reference hands out its buffer wrapper) */
+struct thcl_rt *THClTensor_getCl(THClState *state, const THClTensor *tensor);
+void *THClTensor_wrapper(THClState *state, const THClTensor *self);
 THClTensor *THClTensor_newWithTensor(THClState *state, THClTensor *tensor);
 THClTensor *THClTensor_newWithStorage(THClState *state, int device, THClStorage *storage, long storageOffset,
                                       THLongStorage *size, THLongStorage *stride);

@@ -245,3 +245,32 @@ def test_header_and_storage_interface_extras(cl):
         os_ = _Storage(out.ctypes.data, 10, 1, b"\x00", None, None, None)
         _call(f"TH{name}Storage_copyCl", C.byref(os_), sa)
         assert out.tolist() == list(range(10)), name
+
+
+def test_current_device_forms(cl):
+    """The forms without a device argument act on the current device
+    (src/lib/THClGeneral.cpp:119-133,178-185, src/lib/THClTensor.cpp:66-72,92-95,844-902,
+    src/lib/THClStorage.cpp:93-96)."""
+    import ctypes as C
+    st = cl.state()
+    lib, sp = st.lib, st.ptr
+    cur = lib.THClState_getDevice(sp)
+    ctx = lib.THClState_getClv2(sp, cur)
+    assert lib.THClState_getCl(sp) == ctx
+    dev = C.c_int(-5)
+    assert lib.THClState_getClAndDevice(sp, C.byref(dev)) == ctx and dev.value == cur
+    assert lib.THClState_getClAndDevice(sp, None) == ctx
+    assert lib.THClState_getCurrentDeviceScratchSpace(sp) == lib.THClState_getDeviceScratchSpace(sp, cur, 0)
+    assert lib.THClState_getCurrentDeviceScratchSpaceSize(sp) == lib.THClState_getDeviceScratchSpaceSize(sp, cur) > 0
+    t = lib.THClTensor_new(sp)
+    s = lib.THClStorage_new(sp)
+    assert lib.THClTensor_getDevice(sp, t) == cur and lib.THClStorage_size(sp, s) == 0
+    assert lib.THClTensor_wrapper(sp, t) is None and lib.THClTensor_getCl(sp, t) is None
+    a = cl.ClTensor(np.arange(6, dtype=F)).narrow(1, 3, 2)
+    assert lib.THClTensor_getCl(sp, a._h) == ctx
+    base = lib.THClTensor_wrapper(sp, a._h)
+    assert lib.THClTensor_data(sp, a._h) == base + 2 * 4
+    assert lib.THClTensor_checkGPU(sp, C.c_uint(3), C.c_void_p(a._h), C.c_void_p(None), C.c_void_p(t)) == 1
+    assert lib.THClTensor_checkGPU(sp, C.c_uint(0)) == 1
+    lib.THClTensor_free(sp, t)
+    lib.THClStorage_free(sp, s)
