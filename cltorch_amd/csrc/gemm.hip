@@ -161,40 +161,55 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   const int k_end = (k_begin + P.kchunk < P.k) ? (k_begin + P.kchunk) : P.k;
   const int KT = (k_end - k_begin + BK - 1) / BK;
 
-  la.load(P.a, P.lda, m0, k_begin, P.m, k_end);
-  lb.load(P.b, P.ldb, n0, k_begin, P.n, k_end);
+  // Two register sets: while slab kt is multiplied out of LDS, slab kt+1 waits in one
+  // set (it goes to the other LDS buffer at the end of the step) and the loads of
+  // slab kt+2 are in flight into the other set, so a load has two steps to land.
+  // Loads are issued unconditionally (past the end they re-read the last slab) so
+  // that the wait counts the compiler derives stay exact.
+  TileLoader<BM, AKC, EDGE> la1;
+  TileLoader<BN, BKC, EDGE> lb1;
+  const int last = KT > 0 ? KT - 1 : 0;
+  auto slab_k = [&](int kt) { return k_begin + (kt < last ? kt : last) * BK; };
+  la.load(P.a, P.lda, m0, slab_k(0), P.m, k_end);
+  lb.load(P.b, P.ldb, n0, slab_k(0), P.n, k_end);
+  la1.load(P.a, P.lda, m0, slab_k(1), P.m, k_end);
+  lb1.load(P.b, P.ldb, n0, slab_k(1), P.n, k_end);
   la.store(lds);
   lb.store(lds + AF);
   __syncthreads();
 
-  for (int kt = 0; kt < KT; kt++) {
-    const int cur = kt & 1;
+  auto step = [&](int kt, int cur, auto &issue_a, auto &issue_b, auto &keep_a, auto &keep_b) {
     float *As = lds + cur * (AF + BF);
     float *Bs = As + AF;
-    if (kt + 1 < KT) {
-      la.load(P.a, P.lda, m0, k_begin + (kt + 1) * BK, P.m, k_end);
-      lb.load(P.b, P.ldb, n0, k_begin + (kt + 1) * BK, P.n, k_end);
+    issue_a.load(P.a, P.lda, m0, slab_k(kt + 2), P.m, k_end);
+    issue_b.load(P.b, P.ldb, n0, slab_k(kt + 2), P.n, k_end);
+    __builtin_amdgcn_sched_barrier(0);   // keep the loads at the top of the step
+    {
+#pragma unroll
+      for (int kg = 0; kg < BK / 8; kg++) {
+        float fa[MT][4], fb[NT][4];
+        read_frags<BM, AKC, MT>(As, wm0, kg, fa);
+        read_frags<BN, BKC, NT>(Bs, wn0, kg, fb);
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+          for (int i = 0; i < MT; i++)
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+      }
     }
-#pragma unroll
-    for (int kg = 0; kg < BK / 8; kg++) {
-      float fa[MT][4], fb[NT][4];
-      read_frags<BM, AKC, MT>(As, wm0, kg, fa);
-      read_frags<BN, BKC, NT>(Bs, wn0, kg, fb);
-#pragma unroll
-      for (int s = 0; s < 4; s++)
-#pragma unroll
-        for (int i = 0; i < MT; i++)
-#pragma unroll
-          for (int j = 0; j < NT; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < KT) {
-      float *An = lds + (cur ^ 1) * (AF + BF);
-      la.store(An);
-      lb.store(An + AF);
-    }
+    float *An = lds + (cur ^ 1) * (AF + BF);
+    keep_a.store(An);
+    keep_b.store(An + AF);
     __syncthreads();
+  };
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
+    step(kt, 0, la, lb, la1, lb1);
+    step(kt + 1, 1, la1, lb1, la, lb);
   }
+  if (kt < KT) step(kt, 0, la, lb, la1, lb1);
 
   // epilogue: lane holds rows 8*(r/4) + 4*(lane/32) + (r%4) of column lane%32
   const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
