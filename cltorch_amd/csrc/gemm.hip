@@ -315,7 +315,31 @@ static void choose_tile(long m, long n, int cus, int &bm, int &bn) {
     if ((m / 128) * (n / 64) < cus4) bm = 64;
   }
 }
-// host-only hook for tests: the tile a product of this shape would use
+// Few tiles and a long K: slice K over blockIdx.y so every CU has work; the slices'
+// partial products are summed in slice order by a second kernel.  Below one tile per
+// CU any K from 1024 up is sliced; between one and two tiles per CU only K >= 2048
+// (512x2048x4096: 96 -> 108 TFLOP/s, while 1024^3 loses 10 % when sliced).
+static void choose_ksplit(long tiles, long k, int cus, int &ksplit, int &kchunk) {
+  ksplit = 1;
+  kchunk = (int)(k > 0 ? k : 0);
+  if (!((tiles < cus && k >= 1024) || (tiles < 2L * cus && k >= 2048))) return;
+  long want = (2L * cus + tiles - 1) / tiles;
+  const long max_by_k = k / 256;  // at least 16 slabs per slice
+  if (want > max_by_k) want = max_by_k;
+  if (want > 32) want = 32;
+  if (want <= 1) return;
+  const long chunk = ((k + want - 1) / want + BK - 1) / BK * BK;
+  const long slices = (k + chunk - 1) / chunk;
+  if (slices > 1) {
+    ksplit = (int)slices;
+    kchunk = (int)chunk;
+  }
+}
+// host-only hooks for tests: the tile and the K slicing a product of this shape would use
+extern "C" void thcl_dbg_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk) {
+  choose_tile(m, n, cus, *bm, *bn);
+  choose_ksplit(((m + *bm - 1) / *bm) * ((n + *bn - 1) / *bn), k, cus, *ksplit, *kchunk);
+}
 extern "C" void thcl_dbg_gemm_tile(long m, long n, int cus, int *bm, int *bn) { choose_tile(m, n, cus, *bm, *bn); }
 
 void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m, long n, long k, float alpha,
@@ -349,30 +373,10 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   P.tiles_m = (int)((m + bm - 1) / bm);
   P.tiles_n = (int)((n + bn - 1) / bn);
   P.group_m = P.tiles_m < 8 ? P.tiles_m : 8;
-  // Few tiles and a long K: slice K over blockIdx.y so every CU has work; the
-  // slices' partial products are summed in slice order by a second kernel.
-  P.ksplit = 1;
-  P.kchunk = P.k;
-  {
-    const int cus = thcl_rt_get_props(rt)->compute_units;
-    const long tiles = (long)P.tiles_m * P.tiles_n;
-    if (tiles < cus && k >= 1024) {
-      long want = (2L * cus + tiles - 1) / tiles;
-      long max_by_k = k / 256;  // at least 16 slabs per slice
-      if (want > max_by_k) want = max_by_k;
-      if (want > 32) want = 32;
-      if (want > 1) {
-        long chunk = ((k + want - 1) / want + BK - 1) / BK * BK;
-        P.kchunk = (int)chunk;
-        P.ksplit = (int)((k + chunk - 1) / chunk);
-        if (P.ksplit > 1) {
-          P.work = (float *)thcl_rt_workspace(rt, (size_t)P.ksplit * m * n * sizeof(float));
-          THCL_CHECK(P.work != nullptr, "gemm workspace: %s", thcl_rt_error());
-        } else {
-          P.kchunk = P.k;
-        }
-      }
-    }
+  choose_ksplit((long)P.tiles_m * P.tiles_n, k, thcl_rt_get_props(rt)->compute_units, P.ksplit, P.kchunk);
+  if (P.ksplit > 1) {
+    P.work = (float *)thcl_rt_workspace(rt, (size_t)P.ksplit * m * n * sizeof(float));
+    THCL_CHECK(P.work != nullptr, "gemm workspace: %s", thcl_rt_error());
   }
   dim3 grid((unsigned)(P.tiles_m * P.tiles_n), (unsigned)P.ksplit);
 #define GO(BM_, BN_)                                                   \

@@ -291,3 +291,23 @@ def test_gemm_tile_choice(lib):
     assert tile(16384, 64) == (128, 64)          # the skinny configuration after the row-major swap
     assert tile(100, 100) == (64, 64) and tile(200, 4096) == (64, 128)
 
+
+
+def test_gemm_k_slicing(lib):
+    """K is sliced when there are too few tiles for the chip: below one tile per CU from K = 1024 up, below
+    two tiles per CU from K = 2048 up; slices are multiples of the K slab (16) and at least 256 long."""
+    def plan(m, n, k, cus=256):
+        bm, bn, ks, kc = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
+        lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(k), C.c_int(cus), C.byref(bm), C.byref(bn),
+                               C.byref(ks), C.byref(kc))
+        return bm.value, bn.value, ks.value, kc.value
+    assert plan(8192, 8192, 8192) == (128, 128, 1, 8192)
+    assert plan(16384, 64, 4096) == (128, 64, 4, 1024)           # skinny: 128 tiles on 256 CUs
+    assert plan(2048, 512, 4096) == (64, 64, 2, 2048)            # 256 tiles: one per CU, long K
+    assert plan(1024, 1024, 1024) == (64, 64, 1, 1024)           # 256 tiles but K too short to pay for a second pass
+    assert plan(64, 64, 100000)[2] == 32                         # capped
+    bm, bn, ks, kc = plan(128, 128, 1000)
+    assert ks == 1 and kc == 1000
+    for k in (1024, 1040, 3000, 5555):
+        _, _, ks, kc = plan(64, 64, k)
+        assert kc % 16 == 0 and (ks - 1) * kc < k <= ks * kc and (ks == 1 or kc >= 256)

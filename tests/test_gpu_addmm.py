@@ -146,3 +146,40 @@ def test_large_square_sampled(cl):
     two = cl.ClTensor(np.zeros((n, n), dtype=F)).addmm(0.0, 2.0, A, B).float()
     one = cl.mm(A, B).float()
     assert np.array_equal(two, 2 * one)                      # scaling by 2 is exact
+
+
+def test_sliced_products_repeat_bit_exactly(cl):
+    """K-sliced products sum their slices in slice order: every repetition gives the same
+    bits, also with other reductions in between, with ragged shapes, with beta = 0 over
+    NaNs, and into a result with gaps between its rows."""
+    rng = np.random.RandomState(5)
+    for (M, N, K) in ((64, 2048, 4096), (100, 260, 3000), (512, 512, 2048)):
+        a = rng.standard_normal((M, K)).astype(F) / np.sqrt(K)
+        b = rng.standard_normal((K, N)).astype(F)
+        c0 = rng.standard_normal((M, N)).astype(F)
+        A, B = cl.ClTensor(a), cl.ClTensor(b)
+        want = 0.25 * c0.astype(np.float64) + 2.0 * (a.astype(np.float64) @ b.astype(np.float64))
+        first = None
+        red = cl.ClTensor(rng.standard_normal((2048, 300)).astype(F))
+        red_want = red.float().astype(np.float64).sum(axis=0)
+        for rep in range(6):
+            Cd = cl.ClTensor(c0)
+            Cd.addmm(0.25, 2.0, A, B)
+            got = Cd.float()
+            assert rel_err(got, want) < RTOL
+            if first is None:
+                first = got
+            assert np.array_equal(first.view(np.uint32), got.view(np.uint32)), (M, N, K, rep)
+            s = red.sum(1).float().ravel()
+            assert np.allclose(s, red_want, rtol=1e-5, atol=1e-4)
+        # beta = 0 never reads the old contents
+        Cn = cl.ClTensor(np.full((M, N), np.nan, dtype=F))
+        Cn.addmm(0.0, 1.0, A, B)
+        assert rel_err(Cn.float(), a.astype(np.float64) @ b.astype(np.float64)) < RTOL
+        # rows of the result 8 elements apart from dense: a narrowed view of a wider tensor
+        wide = cl.ClTensor(np.zeros((M, N + 8), dtype=F))
+        view = wide.narrow(2, 1, N)
+        view.copy(cl.ClTensor(c0))
+        view.addmm(0.25, 2.0, A, B)
+        w = wide.float()
+        assert np.array_equal(w[:, :N].view(np.uint32), first.view(np.uint32)) and not w[:, N:].any()
