@@ -170,6 +170,20 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
         no++;
       }
       t.nouter = no;
+      // 128-bit accesses when every operand allows them.  Measured on MI355X: +50 % with
+      // three operands, +15..70 % when edge tiles are partial, +3..7 % on plain 2-d
+      // transposes, but -4 % on two-operand planes of full tiles under outer dims,
+      // which therefore keep the 32-bit body.
+      const bool ragged = (J.sizes[A] % tileA != 0) || (J.sizes[B] % tileB != 0);
+      bool v4 = (J.sizes[A] % 4 == 0) && (J.sizes[B] % 4 == 0) && (n >= 3 || ragged || J.dims == 2);
+      for (int i = 0; i < n && v4; i++) {
+        if ((((uintptr_t)p[i]) & 15u) != 0) v4 = false;
+        if (i > 0 && !t.via_lds[i] && J.strides[i][A] != 1) v4 = false;   // repeated along A: scalar kernel
+        const int unit = (i > 0 && t.via_lds[i]) ? B : A;   // the one dim this operand walks with stride 1
+        for (int d = 0; d < J.dims && v4; d++)
+          if (d != unit && J.strides[i][d] % 4 != 0) v4 = false;
+      }
+      t.vec4 = v4 ? 1u : 0u;
       if (blocks < (1l << 31)) {
         plan.kind = K_TILED;
         plan.grid = (unsigned)blocks;

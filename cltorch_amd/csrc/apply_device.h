@@ -395,6 +395,7 @@ struct ThclTileParams {
   thcl_u32 ostride[3][THCL_TILE_MAX_OUTER];
   thcl_u32 shape;     // index into THCL_TILE_SHAPE_A/B
   thcl_u32 diagonal;  // 1: shift the B tile coordinate by the A tile coordinate
+  thcl_u32 vec4;      // 1: sizes, strides and bases allow 128-bit accesses on every operand
 };
 
 template <class Op, int NT, int TA, int TB>
@@ -494,9 +495,139 @@ __device__ __forceinline__ void thcl_apply_tiled_body(const ThclTileParams &P, f
   }
 }
 
+// picks element e (0..3, differs per lane) of a 4-vector
+__device__ __forceinline__ float thcl_pick4(const thcl_f4 &v, int e) {
+  return e == 0 ? v[0] : e == 1 ? v[1] : e == 2 ? v[2] : v[3];
+}
+
+// The same tiling with 128-bit global accesses: phase 1 reads 4 values along B per
+// lane, phase 2 reads, computes and writes 4 values along A per lane.  LDS is
+// addressed one float at a time (the pitch is odd); each lane walks its 4 values
+// starting at a different one (by its group of 8 lanes) so the 32 lanes of a pass
+// fall on 32 different banks.  Needs sizeA, sizeB and every stride that is not 1
+// to be multiples of 4, 16-byte aligned bases and no operand repeated along A.
+template <class Op, int NT, int TA, int TB>
+__device__ __forceinline__ void thcl_apply_tiled_body_v4(const ThclTileParams &P, float (*lds)[THCL_TILE_LDS_FLOATS]) {
+  static_assert(TA * (TB + 1) <= THCL_TILE_LDS_FLOATS, "tile does not fit its LDS array");
+  constexpr int PITCH = TB + 1;
+  const float p1 = P.pt[0] ? *P.pt[0] : 0.f;
+  const float p2 = P.pt[1] ? *P.pt[1] : 0.f;
+  const float v1 = P.val[0], v2 = P.val[1];
+  thcl_u32 bid = blockIdx.x;
+  thcl_u32 q = thcl_div(bid, P.tilesA);
+  const thcl_u32 ta = bid - q * P.tilesA.d;
+  const thcl_u32 a0 = ta * TA;
+  bid = q;
+  q = thcl_div(bid, P.tilesB);
+  thcl_u32 tb = bid - q * P.tilesB.d;
+  if (P.diagonal) {
+    tb += ta;
+    tb -= thcl_div(tb, P.tilesB) * P.tilesB.d;
+  }
+  const thcl_u32 b0 = tb * TB;
+  bid = q;
+  thcl_u64 base[3] = {0, 0, 0};
+  for (int d = P.nouter - 1; d >= 0; d--) {
+    q = thcl_div(bid, P.osize[d]);
+    const thcl_u32 r = bid - q * P.osize[d].d;
+    base[0] += (thcl_u64)r * P.ostride[0][d];
+    if (NT > 1) base[1] += (thcl_u64)r * P.ostride[1][d];
+    if (NT > 2) base[2] += (thcl_u64)r * P.ostride[2][d];
+    bid = q;
+  }
+  const bool full = (a0 + TA <= P.sizeA) && (b0 + TB <= P.sizeB);
+  const int rot = (int)((threadIdx.x & 31u) >> 3);
+  // phase 1: lanes along B, 4 values each
+  {
+    constexpr int BQ = TB / 4, ROWS = THCL_TILE_THREADS / BQ;
+    const thcl_u32 l4 = threadIdx.x % BQ, row = threadIdx.x / BQ;
+#pragma unroll
+    for (int t = 1; t < NT; t++) {
+      if (P.via_lds[t]) {
+        const float *src = P.p[t] + base[t] + (thcl_u64)(a0 + row) * P.strideA[t] + (b0 + 4 * l4);
+        const thcl_u64 step = (thcl_u64)ROWS * P.strideA[t];
+        const bool bok = b0 + 4 * l4 < P.sizeB;
+#pragma unroll
+        for (int i = 0; i < TA / ROWS; i++) {
+          if (full || (bok && a0 + row + ROWS * i < P.sizeA)) {
+            const thcl_f4 v = thcl_ld((const thcl_f4 *)src);
+            float *dst = &lds[t - 1][(row + ROWS * i) * PITCH + 4 * l4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+              const int e = (c + rot) & 3;
+              dst[e] = thcl_pick4(v, e);
+            }
+          }
+          src += step;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // phase 2: lanes along A, 4 values each
+  {
+    constexpr int AQ = TA / 4, ROWS = THCL_TILE_THREADS / AQ;
+    const thcl_u32 l4 = threadIdx.x % AQ, row = threadIdx.x / AQ;
+    float *op = P.p[0] + base[0] + (a0 + 4 * l4) + (thcl_u64)(b0 + row) * P.strideB[0];
+    const thcl_u64 ostep = (thcl_u64)ROWS * P.strideB[0];
+    const float *q1 = nullptr, *q2 = nullptr;
+    thcl_u64 step1 = 0, step2 = 0;
+    if (NT > 1 && !P.via_lds[1]) {
+      q1 = P.p[1] + base[1] + (a0 + 4 * l4) + (thcl_u64)(b0 + row) * P.strideB[1];
+      step1 = (thcl_u64)ROWS * P.strideB[1];
+    }
+    if (NT > 2 && !P.via_lds[2]) {
+      q2 = P.p[2] + base[2] + (a0 + 4 * l4) + (thcl_u64)(b0 + row) * P.strideB[2];
+      step2 = (thcl_u64)ROWS * P.strideB[2];
+    }
+    const bool aok = a0 + 4 * l4 < P.sizeA;
+    auto gather = [&](const float *plane, thcl_u32 bl) {
+      float t[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) t[j] = plane[(4 * l4 + ((j + rot) & 3)) * PITCH + bl];
+      // t[j] holds element (j + rot) & 3
+      thcl_f4 r;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int j = (c - rot) & 3;
+        r[c] = j == 0 ? t[0] : j == 1 ? t[1] : j == 2 ? t[2] : t[3];
+      }
+      return r;
+    };
+#pragma unroll 4
+    for (int i = 0; i < TB / ROWS; i++) {
+      const thcl_u32 bl = row + ROWS * i;
+      if (full || (aok && b0 + bl < P.sizeB)) {
+        thcl_f4 oo = thcl_ld((const thcl_f4 *)op), x = {0.f, 0.f, 0.f, 0.f}, y = {0.f, 0.f, 0.f, 0.f};
+        if (NT > 1) x = P.via_lds[1] ? gather(lds[0], bl) : thcl_ld((const thcl_f4 *)q1);
+        if (NT > 2) y = P.via_lds[2] ? gather(lds[NT > 2 ? 1 : 0], bl) : thcl_ld((const thcl_f4 *)q2);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          float o = oo[c];
+          thcl_apply_one<Op>(o, x[c], y[c], v1, v2, p1, p2);
+          oo[c] = o;
+        }
+        thcl_st(oo, (thcl_f4 *)op);
+      }
+      op += ostep;
+      if (NT > 1) q1 += step1;
+      if (NT > 2) q2 += step2;
+    }
+  }
+}
+
 template <class Op, int NT>
 __device__ __forceinline__ void thcl_apply_tiled(const ThclTileParams &P) {
   __shared__ float lds[NT > 2 ? 2 : 1][THCL_TILE_LDS_FLOATS];
+  if (P.vec4) {
+    if (P.shape == 0)
+      thcl_apply_tiled_body_v4<Op, NT, THCL_TILE_SHAPE_A(0), THCL_TILE_SHAPE_B(0)>(P, lds);
+    else if (P.shape == 1)
+      thcl_apply_tiled_body_v4<Op, NT, THCL_TILE_SHAPE_A(1), THCL_TILE_SHAPE_B(1)>(P, lds);
+    else
+      thcl_apply_tiled_body_v4<Op, NT, THCL_TILE_SHAPE_A(2), THCL_TILE_SHAPE_B(2)>(P, lds);
+    return;
+  }
   if (P.shape == 0)
     thcl_apply_tiled_body<Op, NT, THCL_TILE_SHAPE_A(0), THCL_TILE_SHAPE_B(0)>(P, lds);
   else if (P.shape == 1)

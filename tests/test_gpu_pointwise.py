@@ -312,7 +312,8 @@ def test_host_roundtrip_of_strided_views(cl):
 
 # ------------------------------------------------- transposed operands (LDS tiles) ---
 @pytest.mark.parametrize("shape", [(130, 70), (64, 128), (200, 300), (3, 150, 90), (5, 17, 260), (2, 3, 70, 129),
-                                   (64, 300), (300, 64), (256, 1024), (2, 512, 1024), (3, 1024, 272)])
+                                   (64, 300), (300, 64), (256, 1024), (2, 512, 1024), (3, 1024, 272),
+                                   (1000, 3000), (4, 128, 132), (100, 60), (2, 3, 68, 260)])
 def test_transposed_operand_meets_dense_one(cl, shape):
     """Operands whose unit-stride dims differ: the library stages the transposed
     ones through LDS tiles; full tiles, ragged edges and outer dims, each of the
@@ -349,6 +350,34 @@ def test_transposed_operand_meets_dense_one(cl, shape):
     oracle.pointwise("addcmul", acc2.view, srcT.view, zT.view, 2.0)
     assert_bit_equal(acc2.device_storage(), acc2.host_storage, f"addcmul T,T {shape}")
     assert_bit_equal(srcT.device_storage(), y, "input modified")
+
+
+def test_transposed_operand_alignment_and_repeats(cl):
+    """The 128-bit form of the tiled kernels needs aligned bases and strides; views that
+    start an odd number of elements in, rows an odd pitch apart, and operands repeated
+    along an outer dim or along the destination's unit-stride dim all give the same
+    results through whichever form takes them."""
+    rng = np.random.RandomState(77)
+    buf_y = rng.standard_normal(4 + 136 * 260).astype(F)
+    buf_z = rng.standard_normal(4 + 132 * 264).astype(F)
+    for off_y, pitch_y, off_z in ((0, 136, 0), (1, 136, 0), (0, 133, 0), (4, 136, 3), (0, 136, 4)):
+        # destination 128 x 256 dense; y = transposed view of a 256 x pitch buffer; z dense rows of pitch 264
+        dst = Pair.dense(cl, rng.standard_normal((128, 256)).astype(F))
+        py = Pair(cl, buf_y, off_y, (128, 256), (1, pitch_y))
+        pz = Pair(cl, buf_z, off_z, (128, 256), (264, 1))
+        dst.dev.map2_on_gpu(py.dev, pz.dev, "x = x + 2*y - z")
+        want = expr_host.evaluate("x = x + 2*y - z", dst.view.gather(), py.view.gather(), pz.view.gather())
+        assert_bit_equal(dst.device_storage(), want, f"offsets {off_y},{off_z} pitch {pitch_y}")
+    # y repeated along the outer dim (stride 0), z repeated along the destination's unit-stride dim
+    dst = Pair.dense(cl, rng.standard_normal((3, 64, 128)).astype(F))
+    py = Pair(cl, buf_y, 0, (3, 64, 128), (0, 1, 136))
+    pz = Pair(cl, buf_z, 0, (3, 64, 128), (64, 1, 0))
+    dst.dev.map2_on_gpu(py.dev, pz.dev, "x = x*y + z")
+    want = expr_host.evaluate("x = x*y + z", dst.view.gather(), py.view.gather(), pz.view.gather())
+    assert_bit_equal(dst.device_storage(), want, "repeated operands")
+    dst2 = Pair.dense(cl, np.zeros((3, 64, 128), dtype=F))
+    dst2.dev.copy(py.dev)
+    assert_bit_equal(dst2.device_storage(), py.view.gather(), "copy of a repeated transposed operand")
 
 
 def test_same_expression_on_every_kernel_family(cl):
