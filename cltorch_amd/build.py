@@ -70,9 +70,6 @@ def _compile(name: str) -> str:
 
 
 def build(verbose: bool = False, jobs: int = 8) -> str:
-    extra = os.environ.get("THCL_EXTRA_CXXFLAGS", "").split()   # tuning builds only
-    if extra:
-        COMMON.extend(extra)
     os.makedirs(OBJ, exist_ok=True)
     embed_skeleton()
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:

@@ -329,21 +329,12 @@ float THClTensor_dot(THClState *state, THClTensor *self, THClTensor *src) {
   const long n = THClTensor_nElement(state, self);
   THCL_ARGCHECK(n == THClTensor_nElement(state, src), 2, "sizes do not match");
   if (n == 0) return 0.f;
-  THClTensor *a = THClTensor_newContiguous(state, self);
-  THClTensor *b = THClTensor_newContiguous(state, src);
+  ThclTemp a(state, THClTensor_newContiguous(state, self));
+  ThclTemp b(state, THClTensor_newContiguous(state, src));
   thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, self));
-  float result = 0.f;
-  try {
-    thcl_dot_dense(state, rt, thcl_dptr(a), thcl_dptr(b), n, thcl_rt_host_word_device(rt));
-    THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
-    result = thcl_rt_host_word(rt)[0];
-  } catch (...) {
-    THClTensor_free(state, a);
-    THClTensor_free(state, b);
-    throw;
-  }
-  THClTensor_free(state, a);
-  THClTensor_free(state, b);
+  thcl_dot_dense(state, rt, thcl_dptr(a.t), thcl_dptr(b.t), n, thcl_rt_host_word_device(rt));
+  THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
+  const float result = thcl_rt_host_word(rt)[0];
   return result;
   THCL_GUARD_END(0.f)
 }
@@ -367,15 +358,9 @@ void THClTensor_addmv(THClState *state, THClTensor *r_, float beta, THClTensor *
     THClBlas_gemv(state, 't', mat->size[1], mat->size[0], alpha, mat, mat->stride[0], vec, vec->stride[0], beta, r_,
                   r_->stride[0]);
   } else {
-    THClTensor *cmat = THClTensor_newContiguous(state, mat);
-    try {
-      THClBlas_gemv(state, 't', mat->size[1], mat->size[0], alpha, cmat, cmat->stride[0], vec, vec->stride[0], beta, r_,
-                    r_->stride[0]);
-    } catch (...) {
-      THClTensor_free(state, cmat);
-      throw;
-    }
-    THClTensor_free(state, cmat);
+    ThclTemp cmat(state, THClTensor_newContiguous(state, mat));
+    THClBlas_gemv(state, 't', mat->size[1], mat->size[0], alpha, cmat.t, cmat.t->stride[0], vec, vec->stride[0], beta, r_,
+                  r_->stride[0]);
   }
   THCL_GUARD_END()
 }

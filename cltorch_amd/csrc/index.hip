@@ -257,7 +257,11 @@ struct Dense {  // a dense stand-in for a tensor that kernels write or read
     }
   }
   ~Dense() {
-    if (t != orig) THClTensor_free(state, t);  // error path: drop the stand-in
+    if (t == orig) return;
+    try {
+      THClTensor_free(state, t);  // error path: drop the stand-in
+    } catch (...) {  // a destructor must not throw
+    }
   }
 };
 

@@ -139,4 +139,25 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
 
 // ------------------------------------------------------------------ misc ---
 // contiguous device fill / copy kernels used by storage-level calls
+// A temporary tensor that is released when the scope ends, also by an exception.
+// give_to() copies it into the tensor it stood in for and releases it.
+struct ThclTemp {
+  THClState *state;
+  THClTensor *t;
+  ThclTemp(THClState *s, THClTensor *x) : state(s), t(x) {}
+  ThclTemp(const ThclTemp &) = delete;
+  ThclTemp &operator=(const ThclTemp &) = delete;
+  ~ThclTemp() {
+    if (!t) return;
+    try {
+      THClTensor_free(state, t);
+    } catch (...) {  // a destructor must not throw; the failed release is already recorded
+    }
+  }
+  void give_to(THClTensor *dst) {
+    THClTensor *x = t;
+    t = nullptr;
+    THClTensor_freeCopyTo(state, x, dst);
+  }
+};
 void thcl_fill_contig(thcl_rt *rt, float *dst, float value, long n);

@@ -807,12 +807,13 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
 
   // kernels write dense outputs; strided destinations get a dense stand-in
   THClTensor *vdense = values, *idense = indices_f32;
+  ThclTemp v_hold(state, nullptr), i_hold(state, nullptr);
   if (!THClTensor_isContiguous(state, values)) {
-    vdense = THClTensor_newv2(state, device);
+    v_hold.t = vdense = THClTensor_newv2(state, device);
     THClTensor_resize(state, vdense, &oshape, nullptr);
   }
   if (indices_f32 && !THClTensor_isContiguous(state, indices_f32)) {
-    idense = THClTensor_newv2(state, device);
+    i_hold.t = idense = THClTensor_newv2(state, device);
     THClTensor_resize(state, idense, &oshape, nullptr);
   }
 
@@ -910,6 +911,6 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
 #undef DISPATCH_VALUES
 #undef DISPATCH
   thcl_after_launch(state, rt);
-  if (vdense != values) THClTensor_freeCopyTo(state, vdense, values);
-  if (idense != indices_f32) THClTensor_freeCopyTo(state, idense, indices_f32);
+  if (vdense != values) v_hold.give_to(values);
+  if (idense != indices_f32) i_hold.give_to(indices_f32);
 }

@@ -336,11 +336,13 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
   thcl_check_same_device(state, 2, self, src);
   THCL_ARGCHECK(src->nDimension > 0, 2, "cannot scan an empty tensor");
   THCL_ARGCHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
-  THClTensor *srcc = THClTensor_newContiguous(state, src);  // before resizing self: they may be the same tensor
+  ThclTemp src_hold(state, THClTensor_newContiguous(state, src));  // before resizing self: they may be the same tensor
+  THClTensor *srcc = src_hold.t;
   THClTensor_resizeAs(state, self, src);
+  ThclTemp self_hold(state, nullptr);
   THClTensor *selfc = self;
   if (!THClTensor_isContiguous(state, self)) {
-    selfc = THClTensor_newv2(state, THClTensor_getDevice(state, self));
+    self_hold.t = selfc = THClTensor_newv2(state, THClTensor_getDevice(state, self));
     THClTensor_resizeAs(state, selfc, self);
   }
   thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, src));
@@ -399,8 +401,7 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     }
     thcl_after_launch(state, rt);
   }
-  THClTensor_free(state, srcc);
-  if (selfc != self) THClTensor_freeCopyTo(state, selfc, self);
+  if (selfc != self) self_hold.give_to(self);
 }
 
 extern "C" {
