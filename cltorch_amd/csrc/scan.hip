@@ -18,6 +18,8 @@
 // the scan proper with each segment's carry-in.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <cstring>
 
 #include "apply_device.h"
@@ -151,20 +153,9 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   double carry = Op<PROD>::identity();
   if (PHASE == 1 && P.S > 1) carry = P.totals[blockIdx.x];
-  for (thcl_u64 base = r0; base < r1; base += STEP) {
-    float x[UNR][PER];
-#pragma unroll
-    for (int u = 0; u < UNR; u++) {
-      const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
-      if (VEC && j + PER <= r1) {
-        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
-#pragma unroll
-        for (int c = 0; c < PER; c++) x[u][c] = v[c];
-      } else {
-#pragma unroll
-        for (int c = 0; c < PER; c++) x[u][c] = (j + c < r1) ? row[j + c] : (PROD ? 1.0f : 0.0f);
-      }
-    }
+  // one step over x (4 runs of 1024 elements starting at base); FULL: every element is inside the segment
+  auto work = [&](float (&x)[UNR][PER], thcl_u64 base, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
     double a[UNR][PER], incl[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; u++) {
@@ -192,7 +183,7 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
         const double prev = __shfl_up(incl[u], 1, kWave);
         if (lane > 0) before = Op<PROD>::comb(before, prev);
         const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
-        if (VEC && j + PER <= r1) {
+        if (VEC && (FULL || j + PER <= r1)) {
           thcl_f4 v;
 #pragma unroll
           for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[u][c]);
@@ -204,6 +195,47 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
         }
       }
     }
+  };
+  thcl_u64 base = r0;
+  if (VEC && base + STEP <= r1) {
+    // Whole steps: the next step's loads are issued before this step's work and carry
+    // no bounds tests, so they stay in flight across the step's two barriers.
+    auto fetch = [&](float (&x)[UNR][PER], thcl_u64 at) {
+#pragma unroll
+      for (int u = 0; u < UNR; u++) {
+        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + at + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER));
+#pragma unroll
+        for (int c = 0; c < PER; c++) x[u][c] = v[c];
+      }
+    };
+    float x[UNR][PER], xn[UNR][PER];
+    fetch(x, base);
+    for (; base + 2 * STEP <= r1; base += STEP) {
+      fetch(xn, base + STEP);
+      work(x, base, std::true_type());
+#pragma unroll
+      for (int u = 0; u < UNR; u++)
+#pragma unroll
+        for (int c = 0; c < PER; c++) x[u][c] = xn[u][c];
+    }
+    work(x, base, std::true_type());
+    base += STEP;
+  }
+  for (; base < r1; base += STEP) {
+    float x[UNR][PER];
+#pragma unroll
+    for (int u = 0; u < UNR; u++) {
+      const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
+      if (VEC && j + PER <= r1) {
+        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
+#pragma unroll
+        for (int c = 0; c < PER; c++) x[u][c] = v[c];
+      } else {
+#pragma unroll
+        for (int c = 0; c < PER; c++) x[u][c] = (j + c < r1) ? row[j + c] : (PROD ? 1.0f : 0.0f);
+      }
+    }
+    work(x, base, std::false_type());
   }
   if (PHASE == 0 && threadIdx.x == 0) P.totals[blockIdx.x] = carry;
 }
