@@ -133,48 +133,65 @@ __device__ __forceinline__ unsigned block_exclusive(unsigned v, unsigned *lds, u
   return before + incl - v;
 }
 
+template <bool VEC>
 __global__ __launch_bounds__(kThreads) void mask_count(MaskParams P) {
   __shared__ unsigned lds[kThreads / 64];
   const thcl_u64 base = (thcl_u64)blockIdx.x * kChunk;
   unsigned c = 0;
+  if (VEC && base + kChunk <= P.n) {  // whole chunk: 128-bit loads (the order inside a chunk does not matter for a count)
+    thcl_f4 v[kPer / 4];
 #pragma unroll
-  for (int k = 0; k < kPer; k++) {
-    const thcl_u64 i = base + (thcl_u64)k * kThreads + threadIdx.x;
-    if (i < P.n) c += (__builtin_nontemporal_load(P.mask + i) != 0.0f) ? 1u : 0u;
+    for (int k = 0; k < kPer / 4; k++)
+      v[k] = __builtin_nontemporal_load((const thcl_f4 *)(P.mask + base) + k * kThreads + threadIdx.x);
+#pragma unroll
+    for (int k = 0; k < kPer / 4; k++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) c += (v[k][e] != 0.0f) ? 1u : 0u;
+  } else {
+#pragma unroll
+    for (int k = 0; k < kPer; k++) {
+      const thcl_u64 i = base + (thcl_u64)k * kThreads + threadIdx.x;
+      if (i < P.n) c += (__builtin_nontemporal_load(P.mask + i) != 0.0f) ? 1u : 0u;
+    }
   }
   unsigned total;
   (void)block_exclusive(c, lds, &total);
   if (threadIdx.x == 0) P.counts[blockIdx.x] = total;
 }
 
+// counts -> exclusive offsets, total at counts[nblocks].  One block: each thread sums a
+// run of adjacent counts, the 1024 run sums are scanned once, and the run is walked
+// again to leave the offsets.
 __global__ __launch_bounds__(1024) void mask_offsets(MaskParams P) {
   __shared__ unsigned lds[1024 / 64];
-  __shared__ unsigned carry_s;
-  if (threadIdx.x == 0) carry_s = 0;
-  __syncthreads();
-  for (thcl_u32 base = 0; base < P.nblocks; base += 1024) {
-    const thcl_u32 i = base + threadIdx.x;
-    const unsigned v = i < P.nblocks ? P.counts[i] : 0u;
-    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-    unsigned incl = v;
+  const thcl_u32 per = (P.nblocks + 1023u) / 1024u;
+  const thcl_u32 lo = threadIdx.x * per;
+  thcl_u32 hi = lo + per;
+  if (hi > P.nblocks) hi = P.nblocks;
+  unsigned sum = 0;
+  for (thcl_u32 i = lo; i < hi; i++) sum += P.counts[i];
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  unsigned incl = sum;
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const unsigned up = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += up;
-    }
-    if (lane == 63) lds[wave] = incl;
-    __syncthreads();
-    unsigned before = carry_s, all = 0;
-    for (int w = 0; w < 1024 / 64; w++) {
-      if (w < wave) before += lds[w];
-      all += lds[w];
-    }
-    if (i < P.nblocks) P.counts[i] = before + incl - v;
-    __syncthreads();
-    if (threadIdx.x == 0) carry_s += all;
-    __syncthreads();
+  for (int d = 1; d < 64; d <<= 1) {
+    const unsigned up = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += up;
   }
-  if (threadIdx.x == 0) P.counts[P.nblocks] = carry_s;
+  if (lane == 63) lds[wave] = incl;
+  __syncthreads();
+  unsigned before = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < 1024 / 64; w++) {
+    if (w < wave) before += lds[w];
+    all += lds[w];
+  }
+  before += incl - sum;
+  for (thcl_u32 i = lo; i < hi; i++) {
+    const unsigned v = P.counts[i];
+    P.counts[i] = before;
+    before += v;
+  }
+  if (threadIdx.x == 0) P.counts[P.nblocks] = all;
 }
 
 // COPY false: dst[rank] = src[i] for selected i.  COPY true: dst[i] = src[rank].
@@ -529,7 +546,8 @@ static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long 
   P.nblocks = (thcl_u32)nb;
   P.counts = (unsigned *)thcl_rt_workspace(rt, (size_t)(nb + 1) * sizeof(unsigned));
   THCL_CHECK(P.counts != nullptr, "%s", thcl_rt_error());
-  hipLaunchKernelGGL(mask_count, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
+  if (aligned16(P.mask)) hipLaunchKernelGGL(mask_count<true>, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
+  else hipLaunchKernelGGL(mask_count<false>, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
   check("mask count");
   hipLaunchKernelGGL(mask_offsets, dim3(1), dim3(1024), 0, stream, P);
   check("mask offsets");
