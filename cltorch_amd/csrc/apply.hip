@@ -302,10 +302,11 @@ void launch_fixed(const KernelSet &ks, ApplyPlan &plan) {
 }
 
 void launch_expr(THClState *state, const std::string &expr, int nt, ApplyPlan &plan) {
-  std::string key = std::to_string(nt) + "|" + expr;
+  // one module per (expression, kernel family): a first use compiles only what it launches
+  std::string key = std::to_string(nt) + "|" + std::to_string((int)plan.kind) + "|" + expr;
   std::string entry = thcl_expr_tag(expr, nt) + kKindSuffix[plan.kind];
   std::string source;
-  if (!thcl_rt_kernel_cached(plan.rt, key.c_str())) source = thcl_expr_source(expr, nt);
+  if (!thcl_rt_kernel_cached(plan.rt, key.c_str())) source = thcl_expr_source(expr, nt, (int)plan.kind);
   thcl_rt_kernel *k = thcl_rt_kernel_get(plan.rt, key.c_str(), source.c_str(), entry.c_str());
   THCL_CHECK(k != nullptr, "%s", thcl_rt_error());
   void *params = nullptr;

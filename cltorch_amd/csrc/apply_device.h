@@ -636,25 +636,38 @@ __device__ __forceinline__ void thcl_apply_tiled(const ThclTileParams &P) {
     thcl_apply_tiled_body<Op, NT, THCL_TILE_SHAPE_A(2), THCL_TILE_SHAPE_B(2)>(P, lds);
 }
 
-// Entry points for one operator; K is a name prefix.
-#define THCL_DEFINE_APPLY_KERNELS(K, Op, NT)                                                             \
+// Entry points for one operator; K is a name prefix.  One macro per kernel family, so
+// that a run-time compiled expression builds only the family a launch needs.
+#define THCL_DEFINE_APPLY_CONTIG_V4(K, Op, NT)                                                                  \
   extern "C" __global__ __launch_bounds__(THCL_CONTIG_THREADS_FOR(NT)) void K##_contig_v4(ThclContigParams P) { \
-    thcl_apply_contig_v4<Op, NT>(P);                                                                     \
-  }                                                                                                      \
-  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_contig_s(ThclContigParams P) {   \
-    thcl_apply_contig_s<Op, NT>(P);                                                                      \
-  }                                                                                                      \
-  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_v4(ThclJointParams P) {    \
-    thcl_apply_joint<Op, NT, 4, THCL_JOINT_V4_UNROLL>(P);                                                                      \
-  }                                                                                                      \
-  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_s(ThclJointParams P) {     \
-    thcl_apply_joint<Op, NT, 1, THCL_JOINT_S_UNROLL>(P);                                                                      \
-  }                                                                                                      \
-  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_generic(ThclGenericParams P) {   \
-    thcl_apply_generic<Op, NT>(P);                                                                       \
-  }                                                                                                      \
-  extern "C" __global__ __launch_bounds__(THCL_TILE_THREADS) void K##_tiled(ThclTileParams P) {         \
-    thcl_apply_tiled<Op, NT>(P);                                                                         \
+    thcl_apply_contig_v4<Op, NT>(P);                                                                            \
   }
+#define THCL_DEFINE_APPLY_CONTIG_S(K, Op, NT)                                                          \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_contig_s(ThclContigParams P) { \
+    thcl_apply_contig_s<Op, NT>(P);                                                                    \
+  }
+#define THCL_DEFINE_APPLY_JOINT_V4(K, Op, NT)                                                         \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_v4(ThclJointParams P) { \
+    thcl_apply_joint<Op, NT, 4, THCL_JOINT_V4_UNROLL>(P);                                             \
+  }
+#define THCL_DEFINE_APPLY_JOINT_S(K, Op, NT)                                                         \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_joint_s(ThclJointParams P) { \
+    thcl_apply_joint<Op, NT, 1, THCL_JOINT_S_UNROLL>(P);                                             \
+  }
+#define THCL_DEFINE_APPLY_GENERIC(K, Op, NT)                                                            \
+  extern "C" __global__ __launch_bounds__(THCL_APPLY_THREADS) void K##_generic(ThclGenericParams P) { \
+    thcl_apply_generic<Op, NT>(P);                                                                      \
+  }
+#define THCL_DEFINE_APPLY_TILED(K, Op, NT)                                                       \
+  extern "C" __global__ __launch_bounds__(THCL_TILE_THREADS) void K##_tiled(ThclTileParams P) { \
+    thcl_apply_tiled<Op, NT>(P);                                                                 \
+  }
+#define THCL_DEFINE_APPLY_KERNELS(K, Op, NT) \
+  THCL_DEFINE_APPLY_CONTIG_V4(K, Op, NT)     \
+  THCL_DEFINE_APPLY_CONTIG_S(K, Op, NT)      \
+  THCL_DEFINE_APPLY_JOINT_V4(K, Op, NT)      \
+  THCL_DEFINE_APPLY_JOINT_S(K, Op, NT)       \
+  THCL_DEFINE_APPLY_GENERIC(K, Op, NT)       \
+  THCL_DEFINE_APPLY_TILED(K, Op, NT)
 
 #endif  // THCL_APPLY_DEVICE_H

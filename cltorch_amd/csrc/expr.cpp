@@ -124,7 +124,7 @@ std::string thcl_expr_tag(const std::string &rewritten, int ntensors) {
   return buf;
 }
 
-std::string thcl_expr_source(const std::string &rewritten, int ntensors) {
+std::string thcl_expr_source(const std::string &rewritten, int ntensors, int family) {
   THCL_CHECK(ntensors >= 1 && ntensors <= 3, "expression kernels take 1 to 3 tensors");
   std::string src;
   src.reserve(sizeof(kSkeleton) + sizeof(kPrelude) + rewritten.size() + 1024);
@@ -140,7 +140,11 @@ std::string thcl_expr_source(const std::string &rewritten, int ntensors) {
   src += "    (void)out; (void)in1; (void)in2; (void)val1; (void)val2; (void)pointTensor1; (void)pointTensor2;\n";
   src += "    " + rewritten + ";\n";
   src += "  }\n};\n";
-  src += "THCL_DEFINE_APPLY_KERNELS(" + thcl_expr_tag(rewritten, ntensors) + ", ThclUserOp, " + std::to_string(ntensors) + ")\n";
+  static const char *const kFamilyMacro[] = {"THCL_DEFINE_APPLY_CONTIG_V4", "THCL_DEFINE_APPLY_CONTIG_S", "THCL_DEFINE_APPLY_JOINT_V4",
+                                             "THCL_DEFINE_APPLY_JOINT_S",   "THCL_DEFINE_APPLY_GENERIC",  "THCL_DEFINE_APPLY_TILED"};
+  THCL_CHECK(family >= -1 && family < 6, "internal: no kernel family %d", family);
+  src += std::string(family < 0 ? "THCL_DEFINE_APPLY_KERNELS" : kFamilyMacro[family]) + "(" + thcl_expr_tag(rewritten, ntensors) +
+         ", ThclUserOp, " + std::to_string(ntensors) + ")\n";
   return src;
 }
 
@@ -157,12 +161,15 @@ int thcl_dbg_rewrite_expr(const char *expr, int ntensors, char *buf, size_t bufl
     return -1;
   }
 }
-int thcl_dbg_compile_expr(const char *expr, int ntensors, const char *arch, size_t *code_bytes) {
+int thcl_dbg_compile_expr_family(const char *expr, int ntensors, int family, const char *arch, size_t *code_bytes) {
   try {
-    std::string src = thcl_expr_source(thcl_rewrite_expr(expr, ntensors), ntensors);
+    std::string src = thcl_expr_source(thcl_rewrite_expr(expr, ntensors), ntensors, family);
     return thcl_rt_compile_check(src.c_str(), arch, code_bytes);
   } catch (const std::exception &) {
     return -2;
   }
+}
+int thcl_dbg_compile_expr(const char *expr, int ntensors, const char *arch, size_t *code_bytes) {
+  return thcl_dbg_compile_expr_family(expr, ntensors, -1, arch, code_bytes);
 }
 }

@@ -109,7 +109,8 @@ void thcl_apply_expr(THClState *state, const std::string &expr, ApplyCall &call)
 // The text transformation applied to user expressions (x/y/z -> pointers,
 // float literals suffixed); exposed for host-side tests.
 std::string thcl_rewrite_expr(const char *expr, int ntensors);
-std::string thcl_expr_source(const std::string &rewritten, int ntensors);
+// family: index of the kernel family to build (the order of the plan kinds), -1 for all six
+std::string thcl_expr_source(const std::string &rewritten, int ntensors, int family);
 std::string thcl_expr_tag(const std::string &rewritten, int ntensors);
 std::string thcl_apply_config_defines();
 
