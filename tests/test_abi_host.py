@@ -311,3 +311,27 @@ def test_gemm_k_slicing(lib):
     for k in (1024, 1040, 3000, 5555):
         _, _, ks, kc = plan(64, 64, k)
         assert kc % 16 == 0 and (ks - 1) * kc < k <= ks * kc and (ks == 1 or kc >= 256)
+
+
+def test_torch7_file_framing_known_bytes():
+    """The bytes written for a 2 x 3 tensor at offset 1 of a 7-element storage, assembled by hand from
+    the field order of src/torch/generic/Tensor.cpp:1290-1304 and Storage.cpp:255-266 inside Torch7's
+    object framing; then the reader's error paths."""
+    import struct
+    from cltorch_amd import serialize as S
+    data = np.array([9, 1, 2, 3, 4, 5, 6], dtype=np.float32)
+    want = b"".join([
+        struct.pack("<ii", 4, 1), struct.pack("<i", 3), b"V 1", struct.pack("<i", 14), b"torch.ClTensor",
+        struct.pack("<i", 2), struct.pack("<qq", 2, 3), struct.pack("<qq", 3, 1), struct.pack("<q", 2),
+        struct.pack("<ii", 4, 2), struct.pack("<i", 3), b"V 1", struct.pack("<i", 15), b"torch.ClStorage",
+        struct.pack("<q", 7), data.tobytes()])
+    got = S.encode_tensor([2, 3], [3, 1], 1, data)
+    assert got == want
+    sizes, strides, off, storage, tclass, sclass = S.decode_tensor(got)
+    assert (sizes, strides, off, tclass, sclass) == ([2, 3], [3, 1], 1, "torch.ClTensor", "torch.ClStorage")
+    assert np.array_equal(storage, data)
+    empty = S.encode_tensor([], [], 0, None)
+    assert empty.endswith(struct.pack("<q", 1) + struct.pack("<i", 0)) and S.decode_tensor(empty)[3] is None
+    for bad in (got[:-2], got[:40], got.replace(b"torch.ClTensor", b"torch.XxTensor"), struct.pack("<ii", 3, 1) + got[8:]):
+        with pytest.raises(ValueError):
+            S.decode_tensor(bad)

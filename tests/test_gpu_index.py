@@ -274,3 +274,22 @@ def test_current_device_forms(cl):
     assert lib.THClTensor_checkGPU(sp, C.c_uint(0)) == 1
     lib.THClTensor_free(sp, t)
     lib.THClStorage_free(sp, s)
+
+
+def test_save_and_load(cl, tmp_path):
+    """torch.save / torch.load of a ClTensor (src/test/unit_tensor.lua:1033-1052: values with NaN
+    and infinities come back as they were), and a strided view keeps its sizes, strides and offset."""
+    a = cl.ClTensor(np.array([3, 5, 4.7, np.nan, np.inf], dtype=F))
+    path = str(tmp_path / "out.dat")
+    cl.save(path, a)
+    b = cl.load(path)
+    assert b.size() == a.size()
+    assert np.array_equal(a.float().view(np.uint32), b.float().view(np.uint32))
+    base = cl.ClTensor(np.arange(60, dtype=F).reshape(3, 4, 5))
+    v = base.transpose(1, 3).narrow(2, 2, 2)
+    cl.save(path, v)
+    w = cl.load(path)
+    assert (w.size(), w.stride(), w.storageOffset()) == (v.size(), v.stride(), v.storageOffset())
+    assert np.array_equal(w.float(), v.float())
+    cl.save(path, cl.ClTensor())
+    assert cl.load(path).nElement() == 0
