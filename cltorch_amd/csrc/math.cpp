@@ -212,8 +212,10 @@ static void addc(THClState *state, THClTensor *self, THClTensor *t, float value,
   if (self != t) {
     THClTensor_resizeAs(state, self, t);
     THClTensor_copy(state, self, t);
+  } else {
+    // element counts must agree, shapes need not: self keeps its own
+    THCL_ARGCHECK(THClTensor_nElement(state, self) == THClTensor_nElement(state, src1), 1, "sizes do not match");
   }
-  THClTensor_resizeAs(state, self, src1);
   THCL_ARGCHECK(THClTensor_nElement(state, src1) == THClTensor_nElement(state, src2), 3, "sizes do not match");
   ApplyCall c;
   c.n = 3;
