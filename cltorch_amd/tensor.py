@@ -773,6 +773,77 @@ class ClTensor:
     def addr(self, *args) -> "ClTensor":
         return self._addblas("addr", args)
 
+    # ---- Lua operators (src/TensorOperator.c:5-250): each makes a new tensor ------------
+    def _copy_of(self) -> "ClTensor":
+        r = ClTensor(device=_call("THClTensor_getDevice", self._h))
+        _call("THClTensor_resizeAs", r._h, self._h)
+        _call("THClTensor_copy", r._h, self._h)
+        return r
+
+    def __add__(self, other) -> "ClTensor":
+        r = self._copy_of()
+        if isinstance(other, ClTensor):
+            _call("THClTensor_cadd", r._h, r._h, C.c_float(1.0), other._h)
+        else:
+            _call("THClTensor_add", r._h, r._h, C.c_float(other))
+        return r
+
+    __radd__ = __add__
+
+    def __sub__(self, other) -> "ClTensor":
+        r = self._copy_of()
+        if isinstance(other, ClTensor):
+            _call("THClTensor_cadd", r._h, r._h, C.c_float(-1.0), other._h)
+        else:
+            _call("THClTensor_add", r._h, r._h, C.c_float(-other))
+        return r
+
+    def __rsub__(self, number) -> "ClTensor":
+        """``number - tensor``: a tensor filled with the number, then ``cadd`` with -1."""
+        r = ClTensor(device=_call("THClTensor_getDevice", self._h))
+        _call("THClTensor_resizeAs", r._h, self._h)
+        _call("THClTensor_fill", r._h, C.c_float(number))
+        _call("THClTensor_cadd", r._h, r._h, C.c_float(-1.0), self._h)
+        return r
+
+    def __neg__(self) -> "ClTensor":
+        r = self._copy_of()
+        _call("THClTensor_mul", r._h, r._h, C.c_float(-1.0))
+        return r
+
+    def __mul__(self, other):
+        """number: scaled copy; vector * vector: dot (a number); matrix * vector: mv; matrix * matrix: mm."""
+        if not isinstance(other, ClTensor):
+            r = self._copy_of()
+            _call("THClTensor_mul", r._h, r._h, C.c_float(other))
+            return r
+        dt, ds = self.nDimension(), other.nDimension()
+        if dt == 1 and ds == 1:
+            return self.dot(other)
+        if dt == 2 and ds == 1:
+            return mv(self, other)
+        if dt == 2 and ds == 2:
+            r = ClTensor(self.size(1), other.size(2)).zero()
+            _call("THClTensor_addmm", r._h, C.c_float(1.0), r._h, C.c_float(1.0), self._h, other._h)
+            return r
+        raise ClError(f"multiplication between {dt}D and {ds}D tensors not yet supported")
+
+    def __rmul__(self, number) -> "ClTensor":
+        return self.__mul__(number)
+
+    def __truediv__(self, number) -> "ClTensor":
+        """``tensor / number``: a copy multiplied by ``1 / number`` (the reciprocal is taken in double)."""
+        if isinstance(number, ClTensor):
+            raise ClError("number expected")
+        r = self._copy_of()
+        _call("THClTensor_mul", r._h, r._h, C.c_float(1.0 / number))
+        return r
+
+    def __str__(self):
+        """``tostring(clTensor)``: the host copy in Torch7's text form."""
+        from .printing import tensor_tostring
+        return tensor_tostring(self.float() if self.nDimension() > 0 else np.zeros(()), "torch.ClTensor")
+
     def __repr__(self):
         return f"ClTensor(size={self.size()}, stride={self.stride()})"
 

@@ -335,3 +335,21 @@ def test_torch7_file_framing_known_bytes():
     for bad in (got[:-2], got[:40], got.replace(b"torch.ClTensor", b"torch.XxTensor"), struct.pack("<ii", 3, 1) + got[8:]):
         with pytest.raises(ValueError):
             S.decode_tensor(bad)
+
+
+def test_text_form_matches_the_reference_expected_strings():
+    """tostring of tensors and storages against every expected string the reference's tests hold."""
+    import json
+    from cltorch_amd.printing import storage_tostring, tensor_tostring
+    gold = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")))["tostring"]
+    for case in gold["tensors"]:
+        assert tensor_tostring(np.array(case["values"], dtype=np.float32), case["type"]) == case["text"], case
+    for case in gold["storages"]:
+        assert storage_tostring(np.array(case["values"], dtype=np.float32), case["type"]) == case["text"], case
+    # forms without an expected string in the reference: structure only
+    wide = tensor_tostring(np.arange(60, dtype=np.float32).reshape(2, 30))
+    assert wide.startswith("Columns 1 to 20\n") and "\nColumns 21 to 30\n" in wide and wide.endswith("[torch.ClTensor of size 2x30]\n")
+    nd = tensor_tostring(np.zeros((2, 2, 2), dtype=np.float32))
+    assert nd.startswith("(1,.,.) = \n  0  0\n  0  0\n\n(2,.,.) = \n") and nd.endswith("[torch.ClTensor of size 2x2x2]\n")
+    assert tensor_tostring(np.array([1e-3, 5.0, 123456.0])).splitlines()[0] == " 1.0000e-03"
+    assert tensor_tostring(np.zeros(())) == "[torch.ClTensor with no dimension]\n"

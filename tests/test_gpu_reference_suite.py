@@ -69,3 +69,69 @@ def test_inplace_and_outplace_compare(cl, op):         # unit_tensor.lua:222-306
     assert np.array_equal(getattr(cl.ClTensor(), op)(A, 3.0).float(), fn(a, F(3.0)).astype(F))
     r = getattr(A, op)(B)                              # the method form returns a new tensor and leaves a as it was
     assert np.array_equal(r.float(), fn(a, b).astype(F)) and np.array_equal(A.float(), a)
+
+
+def test_basic_and_clone_text(cl):                     # unit_tensor.lua:164-199
+    c = cl.ClTensor([7, 4, 5])
+    assert str(c) == " 7\n 4\n 5\n[torch.ClTensor of size 3]\n"
+    c = cl.ClTensor([[3, 1, 6], [2.1, 5.2, 3.9]])
+    d = cl.ClTensor(2, 3).copy(c)
+    want = " 3.0000  1.0000  6.0000\n 2.1000  5.2000  3.9000\n[torch.ClTensor of size 2x3]\n"
+    assert str(c) == want and str(d) == want
+    c = cl.ClTensor([[7, 4, 5], [3, 1, 4]])
+    d = c.clone().fill(3)
+    assert str(c) == " 7  4  5\n 3  1  4\n[torch.ClTensor of size 2x3]\n"          # the clone's fill left c alone
+    assert str(d) == " 3  3  3\n 3  3  3\n[torch.ClTensor of size 2x3]\n"
+
+
+C0 = np.array([[4, 2, -1], [3.1, 1.2, 4.9]], dtype=F)
+D0 = np.array([[3, 5, -2], [2.1, 2.2, 3.9]], dtype=F)
+
+
+def test_operators(cl):                                # unit_tensor.lua:349-375,401-405; src/TensorOperator.c
+    c, d = cl.ClTensor(C0), cl.ClTensor(D0)
+    v = F(3.4)
+    assert np.array_equal((c + 3.4).float(), C0 + v) and np.array_equal((3.4 + c).float(), C0 + v)
+    assert np.array_equal((c - 3.4).float(), C0 + (-v))
+    assert np.array_equal((3.4 - c).float(), v + F(-1) * C0)
+    assert np.array_equal((c * 3.4).float(), C0 * v) and np.array_equal((3.4 * c).float(), C0 * v)
+    assert np.array_equal((c / 3.4).float(), C0 * F(1.0 / 3.4))       # a multiplication by the reciprocal
+    assert np.array_equal((c + d).float(), C0 + D0) and np.array_equal((c - d).float(), C0 + F(-1) * D0)
+    assert np.array_equal((-c).float(), -C0)
+    assert np.array_equal(c.float(), C0) and np.array_equal(d.float(), D0)                # operands untouched
+    # tensor * tensor by dimensions: dot, mv, mm
+    a = cl.ClTensor([1, 2, 3]); b = cl.ClTensor([4, -5, 6])
+    assert a * b == 12
+    m = cl.ClTensor([[1, 2, -1], [3, 4, 0]])
+    assert np.array_equal((m * a).float(), np.array([2, 11], dtype=F))
+    n = cl.ClTensor([[0, 1], [1, 2], [4, 5]])
+    assert np.array_equal((m * n).float(), np.array([[-2, 0], [4, 11]], dtype=F))
+    with pytest.raises(cl.ClError):
+        cl.ClTensor(2, 2, 2).zero() * m
+
+
+def test_perelement(cl):                               # unit_tensor.lua:377-411
+    c, d = cl.ClTensor(C0), cl.ClTensor(D0)
+    assert np.array_equal(c.add(d).float(), C0 + D0)
+    c = cl.ClTensor(C0)
+    assert np.array_equal(c.cmul(d).float(), C0 * D0)
+    c = cl.ClTensor(C0)
+    assert np.array_equal(cl.ClTensor().clamp(c, 1.5, 4.5).float(), np.clip(C0, F(1.5), F(4.5)))
+
+
+@pytest.mark.parametrize("name", ["add", "mul", "div", "pow", "lt", "le", "gt", "ge", "ne", "eq"])
+def test_outplace_with_a_number(cl, name):             # unit_tensor.lua:337-347
+    c = cl.ClTensor(C0)
+    got = getattr(cl.ClTensor(), name)(c, 3.4).float()
+    v = F(3.4)
+    with np.errstate(invalid="ignore"):
+        want = {"add": lambda: C0 + v, "mul": lambda: C0 * v, "div": lambda: C0 * F(1.0 / 3.4),
+                "pow": lambda: np.power(C0, v), "lt": lambda: (C0 < v).astype(F), "le": lambda: (C0 <= v).astype(F),
+                "gt": lambda: (C0 > v).astype(F), "ge": lambda: (C0 >= v).astype(F), "ne": lambda: (C0 != v).astype(F),
+                "eq": lambda: (C0 == v).astype(F)}[name]()
+    if name in ("pow", "div"):
+        ok = ~np.isnan(want)
+        assert np.array_equal(np.isnan(got), np.isnan(want)) and np.allclose(got[ok], want[ok], rtol=2e-6, atol=2e-4)
+    else:
+        assert np.array_equal(got, want)
+    assert np.array_equal(c.float(), C0)
