@@ -254,6 +254,148 @@ class ClTensor:
             self._lib.THLongStorage_free(sd)
         return self._wrap(h)
 
+    # ---- header-only views the Lua binding borrows from torch (src/Tensor.lua:74-81) --------
+    def _view_of(self, sizes, strides) -> "ClTensor":
+        return self.strided(list(sizes), list(strides), self.storageOffset())
+
+    def sub(self, *bounds) -> "ClTensor":
+        """``a:sub(i1, j1 [, i2, j2 ...])``: a narrow per leading dim; negative bounds count from the end."""
+        t = self
+        for d in range(0, len(bounds), 2):
+            n = t.size(d // 2 + 1)
+            lo, hi = bounds[d], bounds[d + 1]
+            lo = lo + n + 1 if lo < 0 else lo
+            hi = hi + n + 1 if hi < 0 else hi
+            if not (1 <= lo <= hi <= n):
+                raise ClError("sub: index out of range")
+            t = t.narrow(d // 2 + 1, lo, hi - lo + 1)
+        return t
+
+    def expand(self, *sizes) -> "ClTensor":
+        """``a:expand(s1, s2, ...)``: dims of size 1 repeat with stride 0; the other sizes must match."""
+        sizes = list(sizes[0]) if len(sizes) == 1 and isinstance(sizes[0], (list, tuple)) else list(sizes)
+        have, st = self.size(), self.stride()
+        if len(sizes) != len(have):
+            raise ClError("the number of dimensions provided must equal tensor:dim()")
+        strides = []
+        for d, (want, got) in enumerate(zip(sizes, have)):
+            if got == 1:
+                strides.append(0 if want != 1 else st[d])
+            elif want == got:
+                strides.append(st[d])
+            else:
+                raise ClError("incorrect size: only supporting singleton expansion (size=1)")
+        return self._view_of(sizes, strides)
+
+    def expandAs(self, other: "ClTensor") -> "ClTensor":
+        return self.expand(*other.size())
+
+    def view(self, *sizes) -> "ClTensor":
+        """``a:view(s1, s2, ...)`` of a contiguous tensor; one size may be -1."""
+        sizes = list(sizes[0]) if len(sizes) == 1 and isinstance(sizes[0], (list, tuple)) else list(sizes)
+        if not self.isContiguous():
+            raise ClError("expecting a contiguous tensor")
+        n = self.nElement()
+        if sizes.count(-1) > 1:
+            raise ClError("only one dimension can be at -1")
+        if -1 in sizes:
+            rest = int(np.prod([x for x in sizes if x != -1]))
+            if rest == 0 or n % rest:
+                raise ClError("input view size not compatible with input tensor size")
+            sizes[sizes.index(-1)] = n // rest
+        if int(np.prod(sizes)) != n:
+            raise ClError("Wrong size for view. Input size: %d. Output size: %s" % (n, "x".join(map(str, sizes))))
+        strides = [1] * len(sizes)
+        for d in range(len(sizes) - 2, -1, -1):
+            strides[d] = strides[d + 1] * sizes[d + 1]
+        return self._view_of(sizes, strides)
+
+    def viewAs(self, other: "ClTensor") -> "ClTensor":
+        return self.view(*other.size())
+
+    def permute(self, *order) -> "ClTensor":
+        """``a:permute(d1, d2, ...)``: dim i of the result is dim ``order[i]`` of a."""
+        nd = self.nDimension()
+        if sorted(order) != list(range(1, nd + 1)):
+            raise ClError("Invalid permutation")
+        sz, st = self.size(), self.stride()
+        return self._view_of([sz[o - 1] for o in order], [st[o - 1] for o in order])
+
+    def split(self, size: int, dim: int = 1):
+        """``a:split(size, dim)``: narrow views of at most ``size`` along dim."""
+        n = self.size(dim)
+        return [self.narrow(dim, lo, min(size, n - lo + 1)) for lo in range(1, n + 1, size)]
+
+    def chunk(self, parts: int, dim: int = 1):
+        return self.split(-(-self.size(dim) // parts), dim)
+
+    def repeatTensor(self, *sizes) -> "ClTensor":
+        """``a:repeatTensor(r1, r2, ...)``: a new tensor tiling a; built as torch does, by unfolding the
+        result into blocks of a's shape and copying an expanded view of a into them."""
+        sizes = list(sizes[0]) if len(sizes) == 1 and isinstance(sizes[0], (list, tuple)) else list(sizes)
+        if len(sizes) < self.nDimension():
+            raise ClError("Number of dimensions of repeat dims can not be smaller than number of dimensions of tensor")
+        src = self.contiguous()
+        xsize = [1] * (len(sizes) - self.nDimension()) + list(self.size())
+        x = src.view(*xsize)
+        result = ClTensor(*[a * b for a, b in zip(xsize, sizes)])
+        blocks = result
+        for d, s in enumerate(xsize):
+            blocks = blocks.unfold(d + 1, s, s)
+        x = x.view(*([1] * len(xsize) + xsize))
+        blocks.copy(x.expandAs(blocks))
+        return result
+
+    # ---- Lua indexing (src/torch/generic/Tensor.cpp:782-1148) -----------------------------
+    def __getitem__(self, key):
+        """``a[i]``: the number at i of a vector, else ``select(1, i)``; ``a[mask]``: ``maskedSelect``;
+        ``a[{i, {lo, hi}, ...}]`` as a tuple of ints and (lo, hi) pairs: select / narrow per dim."""
+        if isinstance(key, ClTensor):
+            return self.maskedSelect(key)
+        if isinstance(key, (int, np.integer)):
+            key = int(key) + self.size(1) + 1 if key < 0 else int(key)
+            if self.nDimension() == 1:
+                return float(_call("THClTensor_get1d", self._h, key - 1))
+            return self.select(1, key)
+        return self._index_view(key)
+
+    def _index_view(self, key) -> "ClTensor":
+        t, d = self, 1
+        for k in key:
+            if isinstance(k, (int, np.integer)):
+                k = int(k) + t.size(d) + 1 if k < 0 else int(k)
+                if t.nDimension() > 1:
+                    t = t.select(d, k)          # the dim goes away, d now names the next one
+                else:
+                    t = t.narrow(1, k, 1)
+                    d += 1
+            else:
+                lo, hi = (k + (None,))[:2] if len(k) == 1 else k
+                n = t.size(d)
+                lo = 1 if lo is None else (lo + n + 1 if lo < 0 else lo)
+                hi = n if hi is None else (hi + n + 1 if hi < 0 else hi)
+                t = t.narrow(d, lo, hi - lo + 1)
+                d += 1
+        return t
+
+    def __setitem__(self, key, value) -> None:
+        """``a[i] = v``, ``a[mask] = v`` (``maskedFill``), ``a[{...}] = number or tensor``."""
+        if isinstance(key, ClTensor):
+            if isinstance(value, ClTensor):
+                self.maskedCopy(key, value)
+            else:
+                self.maskedFill(key, value)
+            return
+        if isinstance(key, (int, np.integer)) and self.nDimension() == 1 and not isinstance(value, ClTensor):
+            key = int(key) + self.size(1) + 1 if key < 0 else int(key)
+            _call("THClTensor_set1d", self._h, key - 1, C.c_float(value))
+            return
+        view = self[key] if not isinstance(key, (int, np.integer)) else self.select(1, int(key) + self.size(1) + 1 if key < 0 else int(key))
+        if isinstance(value, ClTensor):
+            view.copy(value)
+        else:
+            view.fill(value)
+
     def reshape(self, *sizes) -> "ClTensor":
         """``a:reshape(s1, s2, ...)``: a new dense tensor with a's elements in order (``torch.reshape``)."""
         res = ClTensor()
@@ -867,6 +1009,86 @@ def ger(v1: ClTensor, v2: ClTensor) -> ClTensor:
     r = ClTensor(v1.size(1), v2.size(1)).zero()
     _call("THClTensor_addr", r._h, C.c_float(1.0), r._h, C.c_float(1.0), v1._h, v2._h)
     return r
+
+
+class _HostStorageStruct(C.Structure):  # TH<Type>Storage: data*, size, refcount, flag, allocator, allocatorContext, view
+    _fields_ = [("data", C.c_void_p), ("size", C.c_long), ("refcount", C.c_int), ("flag", C.c_char),
+                ("allocator", C.c_void_p), ("allocatorContext", C.c_void_p), ("view", C.c_void_p)]
+
+
+class ClStorage:
+    """``torch.ClStorage``: ``ClStorage()``, ``ClStorage(n)``, ``ClStorage{...}`` (a list), with ``fill``,
+    ``resize``, ``copy`` (from another ClStorage or a host array: ``torch.Storage`` in the Lua tests),
+    ``s[i]`` / ``s[i] = v`` (1-based), ``#s`` and ``tostring`` (src/torch/generic/Storage.cpp,
+    src/test/unit_storage.lua:24-73)."""
+
+    _COPY_IN = {np.dtype(np.float32): "Float", np.dtype(np.float64): "Double", np.dtype(np.int64): "Long",
+                np.dtype(np.int32): "Int", np.dtype(np.int16): "Short", np.dtype(np.int8): "Char",
+                np.dtype(np.uint8): "Byte"}
+
+    def __init__(self, arg=None, device: int = 0):
+        self._lib = state().lib
+        if arg is None:
+            self._h = _call("THClStorage_newv2", device)
+        elif isinstance(arg, (int, np.integer)):
+            self._h = _call("THClStorage_newWithSize", device, C.c_long(int(arg)))
+        else:
+            data = np.ascontiguousarray(arg, dtype=np.float32).reshape(-1)
+            self._h = _call("THClStorage_newWithSize", device, C.c_long(data.size))
+            self.copy(data)
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None) and _state is not None:
+                self._lib.THClStorage_free(_state.ptr, self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    def size(self) -> int:
+        return int(_call("THClStorage_size", self._h))
+
+    __len__ = size
+
+    def fill(self, value: float) -> "ClStorage":
+        _call("THClStorage_fill", self._h, C.c_float(value))
+        return self
+
+    def resize(self, n: int) -> "ClStorage":
+        _call("THClStorage_resize", self._h, C.c_long(n))
+        return self
+
+    def copy(self, src) -> "ClStorage":
+        """From a ClStorage, or from a host array of any of the seven element types (sizes must match)."""
+        if isinstance(src, ClStorage):
+            _call("THClStorage_copy", self._h, src._h)
+            return self
+        arr = np.ascontiguousarray(src)
+        if arr.dtype not in self._COPY_IN:
+            arr = arr.astype(np.float64)
+        arr = arr.reshape(-1)
+        host = _HostStorageStruct(arr.ctypes.data, arr.size, 1, b"\x00", None, None, None)
+        _call("THClStorage_copy" + self._COPY_IN[arr.dtype], self._h, C.byref(host))
+        return self
+
+    def to_host(self, dtype=np.float32) -> np.ndarray:
+        """``hostStorage:copy(clStorage)``: the elements as a host array of the given type."""
+        out = np.zeros(self.size(), dtype=dtype)
+        host = _HostStorageStruct(out.ctypes.data, out.size, 1, b"\x00", None, None, None)
+        _call("TH" + self._COPY_IN[np.dtype(dtype)] + "Storage_copyCl", C.byref(host), self._h)
+        return out
+
+    def __getitem__(self, i: int) -> float:
+        fn = self._lib.THClStorage_get
+        fn.restype = C.c_float
+        return float(_call("THClStorage_get", self._h, C.c_long(i - 1)))
+
+    def __setitem__(self, i: int, value: float) -> None:
+        _call("THClStorage_set", self._h, C.c_long(i - 1), C.c_float(value))
+
+    def __str__(self) -> str:
+        from .printing import storage_tostring
+        return storage_tostring(self.to_host(), "torch.ClStorage")
 
 
 class ClKernel:

@@ -135,3 +135,161 @@ def test_outplace_with_a_number(cl, name):             # unit_tensor.lua:337-347
     else:
         assert np.array_equal(got, want)
     assert np.array_equal(c.float(), C0)
+
+
+def test_borrowed_torch_views(cl):                     # src/Tensor.lua:74-81: expand, view, permute, split, chunk, repeatTensor
+    rng = np.random.RandomState(11)
+    a = rng.standard_normal((3, 1, 5)).astype(F)
+    A = cl.ClTensor(a)
+    e = A.expand(3, 4, 5)
+    assert e.stride()[1] == 0 and np.array_equal(e.float(), np.broadcast_to(a, (3, 4, 5)))
+    assert np.array_equal(cl.ClTensor(3, 4, 5).zero().add(e).float(), np.broadcast_to(a, (3, 4, 5)))   # read through stride 0
+    assert np.array_equal(A.expandAs(cl.ClTensor(3, 2, 5)).float(), np.broadcast_to(a, (3, 2, 5)))
+    with pytest.raises(cl.ClError):
+        A.expand(4, 4, 5)
+    assert np.array_equal(A.view(5, 3).float(), a.reshape(5, 3)) and A.view(-1, 5).size() == (3, 5)
+    assert A.viewAs(cl.ClTensor(15)).size() == (15,)
+    with pytest.raises(cl.ClError):
+        A.transpose(1, 3).view(15)
+    b = rng.standard_normal((2, 3, 4)).astype(F)
+    B = cl.ClTensor(b)
+    assert np.array_equal(B.permute(3, 1, 2).float(), b.transpose(2, 0, 1))
+    assert np.array_equal(B.permute(3, 1, 2).contiguous().float(), b.transpose(2, 0, 1))
+    parts = cl.ClTensor(np.arange(70, dtype=F).reshape(7, 10)).split(3, 1)
+    assert [p.size(1) for p in parts] == [3, 3, 1] and parts[2].float()[0, 0] == 60
+    assert [p.size(2) for p in cl.ClTensor(7, 10).chunk(4, 2)] == [3, 3, 3, 1]
+    assert np.array_equal(B.repeatTensor(2, 1, 3).float(), np.tile(b, (2, 1, 3)))
+    assert np.array_equal(cl.ClTensor([1, 2, 3]).repeatTensor(2, 2).float(), np.tile(np.array([1, 2, 3], dtype=F), (2, 2)))
+    assert np.array_equal(B.sub(2, 2, 1, -2).float(), b[1:2, 0:2])
+
+
+def test_lua_indexing(cl):                             # src/torch/generic/Tensor.cpp:782-1148; unit_tensor.lua:1009-1023
+    rng = np.random.RandomState(12)
+    x0 = rng.standard_normal((13, 19)).astype(F)
+    x = cl.ClTensor(x0)
+    assert np.array_equal(x[x.gt(0.5)].float(), x0[x0 > 0.5])
+    xt = x.t()
+    assert np.array_equal(xt[xt.gt(0.5)].float(), x0.T[x0.T > 0.5])
+    assert np.array_equal(x[3].float(), x0[2]) and x[3][4] == x0[2, 3]
+    assert np.array_equal(x[(2, (5, 9))].float(), x0[1, 4:9]) and np.array_equal(x[((2, 4), (1, 3))].float(), x0[1:4, 0:3])
+    x[2] = 7.0
+    x[((5, 6), (1, 2))] = -1.0
+    x[(9, (3, 5))] = cl.ClTensor([1, 2, 3])
+    want = x0.copy(); want[1] = 7; want[4:6, 0:2] = -1; want[8, 2:5] = [1, 2, 3]
+    assert np.array_equal(x.float(), want)
+    x[x.lt(-1.5)] = 0.0
+    want[want < -1.5] = 0
+    assert np.array_equal(x.float(), want)
+    v = cl.ClTensor([4, 5, 6])
+    v[2] = 9.5
+    assert v[2] == 9.5 and v[-1] == 6 and v.float().tolist() == [4, 9.5, 6]
+
+
+def test_remaining_reference_cases(cl):                # unit_tensor.lua:522-604,700-760,862-960
+    rng = np.random.RandomState(13)
+    a, b, c = (rng.uniform(-0.5, 0.5, (60, 50)).astype(F) for _ in range(3))
+    A, B, Cc = cl.ClTensor(a), cl.ClTensor(b), cl.ClTensor(c)
+    assert np.array_equal(cl.ClTensor().add(A, B).float(), a + b) and np.array_equal((A + B).float(), a + b)
+    assert np.array_equal(cl.ClTensor().cmul(A, B).float(), a * b)
+    v = F(1.234)
+    assert np.array_equal(cl.ClTensor().addcmul(A, 1.234, B, Cc).float(), a + v * b * c)
+    assert np.array_equal(A.clone().addcmul(1.234, B, Cc).float(), a + v * b * c)
+    assert np.array_equal(cl.ClTensor().addcdiv(A, 1.234, B, Cc).float(), a + v * b / c)
+    assert np.array_equal((-A).float(), -a) and np.array_equal(A.clone().neg().float(), -a)
+    assert np.array_equal((A - B).float(), a + F(-1) * b) and np.array_equal(A.clone().csub(B).float(), a - b)
+    # both expression syntaxes, and the apply2 / apply3 names
+    small = rng.uniform(-0.5, 0.5, (6, 4)).astype(F)
+    r1 = cl.ClTensor(small).apply_on_gpu("*out = sqrt(*out + 3) + exp(*out)").float()
+    r2 = cl.ClTensor(small).apply_on_gpu("x = sqrt(x + 3) + exp(x)").float()
+    assert np.array_equal(r1, r2) and np.allclose(r1, np.sqrt(small + 3) + np.exp(small), rtol=1e-6)
+    m1 = A.clone().map_on_gpu(B, "*out = sqrt(*out * *out + *in1 * *in1 + 3 + exp(*in1))").float()
+    m2 = A.clone().apply2_on_gpu(B, "x = sqrt(x * x + y * y + 3 + exp(y))").float()
+    assert np.array_equal(m1, m2) and np.allclose(m1, np.sqrt(a * a + b * b + 3 + np.exp(b)), rtol=1e-6)
+    t1 = A.clone().map2_on_gpu(B, Cc, "*out = sqrt(*out * *out + *in1 * *in1 + *in2 + 3 + exp(*in2))").float()
+    t2 = A.clone().apply3_on_gpu(B, Cc, "x = sqrt(x * x + y * y + z + 3 + exp(z))").float()
+    assert np.array_equal(t1, t2) and np.allclose(t1, np.sqrt(a * a + b * b + c + 3 + np.exp(c)), rtol=1e-6)
+    # reductions
+    a64 = a.astype(np.float64)
+    assert abs(A.sum() - a64.sum()) < 1e-3 and abs(A.t().sum() - a64.sum()) < 1e-3
+    assert abs(A.mean() - a64.mean()) < 1e-6
+    assert np.isclose(A.prod(), np.prod(a64), rtol=1e-4, atol=0)
+    pos = cl.ClTensor(np.abs(a) * 3)
+    p64 = np.abs(a64) * 3
+    assert np.isclose(pos.norm(), np.sqrt((p64 ** 2).sum()), rtol=1e-6) and np.isclose(pos.norm(1), p64.sum(), rtol=1e-6)
+    assert np.allclose(pos.norm(1, 2).float(), p64.sum(axis=1, keepdims=True), rtol=1e-5)
+    assert np.allclose(pos.norm(2, 1).float(), np.sqrt((p64 ** 2).sum(axis=0, keepdims=True)), rtol=1e-5)
+    for d in (1, 2):
+        assert np.allclose(A.sum(d).float(), a64.sum(axis=d - 1, keepdims=True), rtol=1e-5, atol=1e-5)
+        assert np.allclose(A.mean(d).float(), a64.mean(axis=d - 1, keepdims=True), rtol=1e-5, atol=1e-6)
+        assert np.allclose(A.prod(d).float(), a64.prod(axis=d - 1, keepdims=True), rtol=1e-4, atol=1e-30)
+        assert np.allclose(A.t().sum(d).float(), a64.T.sum(axis=d - 1, keepdims=True), rtol=1e-5, atol=1e-5)
+        for view, ref in ((A.narrow(1, 10, 30).t(), a64[9:39].T), (A.narrow(2, 10, 30).t(), a64[:, 9:39].T)):
+            assert np.allclose(view.sum(d).float(), ref.sum(axis=d - 1, keepdims=True), rtol=1e-5, atol=1e-5)
+    s = rng.uniform(-0.5, 0.5, (5, 2)).astype(F)
+    S = cl.ClTensor(s)
+    for d in (1, 2):
+        vals, idx = S.max(d)
+        assert np.array_equal(vals.float(), s.max(axis=d - 1, keepdims=True))
+        assert np.array_equal(idx.float(), s.argmax(axis=d - 1).reshape(vals.size()) + 1)
+        vals, idx = S.min(d)
+        assert np.array_equal(vals.float(), s.min(axis=d - 1, keepdims=True))
+        assert np.array_equal(idx.float(), s.argmin(axis=d - 1).reshape(vals.size()) + 1)
+    # select + fill through views (test_indexselect), cumulative ops without a dim argument
+    X = cl.ClTensor(a)
+    X.select(1, 2).fill(2)
+    X.select(2, 5).fill(5)
+    w = a.copy(); w[1] = 2; w[:, 4] = 5
+    assert np.array_equal(X.float(), w)
+    assert np.allclose(A.cumsum().float(), np.cumsum(a64, axis=0), rtol=1e-5, atol=1e-6)
+    assert np.allclose(A.cumprod(2).float(), np.cumprod(a64, axis=1), rtol=1e-4, atol=1e-30)
+    # gather on a narrowed and on a transposed tensor with indices held in a ClTensor
+    g = np.arange(1, 241, dtype=F).reshape(60, 4)
+    G = cl.ClTensor(g)
+    idx = cl.ClTensor([[2, 1, 3, 1]])
+    assert np.array_equal(G.gather(1, idx).float(), np.array([[g[1, 0], g[0, 1], g[2, 2], g[0, 3]]], dtype=F))
+    assert np.array_equal(G.t().gather(2, idx.t()).float(), np.array([[g[1, 0]], [g[0, 1]], [g[2, 2]], [g[0, 3]]], dtype=F))
+    gn = g[19:39]
+    assert np.array_equal(G.narrow(1, 20, 20).gather(1, idx).float(), np.array([[gn[1, 0], gn[0, 1], gn[2, 2], gn[0, 3]]], dtype=F))
+    # scatter of a tensor and of a number
+    xs = np.arange(1, 11, dtype=F).reshape(2, 5)
+    ind = np.array([[1, 2, 3, 1, 1], [3, 1, 1, 2, 3]])
+    z = np.zeros((3, 5), dtype=F); zf = np.zeros((3, 5), dtype=F)
+    for i in range(2):
+        for j in range(5):
+            z[ind[i, j] - 1, j] = xs[i, j]
+            zf[ind[i, j] - 1, j] = F(3.4567)
+    assert np.array_equal(cl.ClTensor(3, 5).zero().scatter(1, cl.ClTensor(ind.astype(F)), cl.ClTensor(xs)).float(), z)
+    assert np.array_equal(cl.ClTensor(3, 5).zero().scatter(1, cl.ClTensor(ind.astype(F)), 3.4567).float(), zf)
+    # maskedSelect into a given result, transposed source
+    xm = rng.standard_normal((13, 19)).astype(F)
+    mask = (rng.uniform(size=(19, 13)) < 0.5)
+    out = cl.ClTensor()
+    out.maskedSelect(cl.ClTensor(xm).t(), cl.ClTensor(mask.astype(F)))
+    assert np.array_equal(out.float(), xm.T[mask])
+    assert np.array_equal(A.clone().cmin(B).float(), np.minimum(a, b))
+
+
+def test_storage_basic_and_get(cl):                    # src/test/unit_storage.lua:24-73
+    assert str(cl.ClStorage()) == "[torch.ClStorage of size 0]\n"
+    assert str(cl.ClStorage(3)).endswith("[torch.ClStorage of size 3]\n")
+    assert str(cl.ClStorage([4, 9, 2])) == " 4\n 9\n 2\n[torch.ClStorage of size 3]\n"
+    assert str(cl.ClStorage([1.5, 2.4, 5.3])) == " 1.5000\n 2.4000\n 5.3000\n[torch.ClStorage of size 3]\n"
+    c = cl.ClStorage([4, 9, 2]).fill(7)
+    assert str(c) == " 7\n 7\n 7\n[torch.ClStorage of size 3]\n"
+    c = cl.ClStorage([4, 9, 2]).copy(np.array([1.5, 2.4, 5.3]))                       # from a host double storage
+    assert str(c) == " 1.5000\n 2.4000\n 5.3000\n[torch.ClStorage of size 3]\n"
+    assert cl.storage_tostring(cl.ClStorage([4, 9, 2]).to_host(np.float64), "torch.DoubleStorage") == \
+        " 4\n 9\n 2\n[torch.DoubleStorage of size 3]\n"
+    c = cl.ClStorage([4, 9, 2])
+    d = cl.ClStorage(3).copy(c)
+    assert str(d) == " 4\n 9\n 2\n[torch.ClStorage of size 3]\n" and len(d) == 3 and d.size() == 3
+    c.resize(5)
+    assert len(c) == 5
+    assert str(c.fill(1)) == " 1\n 1\n 1\n 1\n 1\n[torch.ClStorage of size 5]\n"
+    acl = cl.ClStorage(10000)
+    acl[2] = 72
+    acl[500] = 104
+    acl[7500] = 1040
+    assert (acl[2], acl[500], acl[7500]) == (72, 104, 1040)
+    with pytest.raises(cl.ClError):
+        cl.ClStorage(3).copy(np.zeros(4))                                              # sizes must match
