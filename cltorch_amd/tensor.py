@@ -103,9 +103,87 @@ def getDeviceCount() -> int:
 
 
 def setAddFinish(flag: int) -> None:
-    # THClState.addFinish is the 6th int of the struct (src/lib/THClGeneral.h:76-93)
-    ints = C.cast(state().buf, C.POINTER(C.c_int))
-    ints[5] = int(flag)
+    _state_int(5, flag)
+
+
+def getDevice() -> int:
+    """``cltorch.getDevice()`` (1-based, src/init.cpp:44-50)."""
+    return int(_call("THClState_getDevice")) + 1
+
+
+def setDevice(device: int) -> None:
+    """``cltorch.setDevice(device)`` (1-based, src/init.cpp:52-59)."""
+    _call("THClState_setDevice", C.c_int(device - 1))
+
+
+class _RtProps(C.Structure):  # thcl_rt_props of include/thcl_rt.h
+    _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int), ("wavefront", C.c_int),
+                ("max_threads_per_block", C.c_int), ("clock_khz", C.c_int), ("lds_bytes_per_block", C.c_int),
+                ("total_mem", C.c_size_t)]
+
+
+def getDeviceProperties(device: int) -> dict:
+    """``cltorch.getDeviceProperties(device)``: the reference's keys (src/init.cpp:79-121) where HIP has a
+    counterpart, plus the code-object architecture and the wavefront width."""
+    st = state()
+    if device < 1 or device > getDeviceCount():
+        raise ClError("Device doesnt exist")
+    fn = st.lib.thcl_rt_get_props
+    fn.restype = C.POINTER(_RtProps)
+    p = fn(st.lib.THClState_getClv2(st.ptr, device - 1)).contents
+    st.check()
+    return {"deviceName": p.name.decode(), "deviceType": "GPU", "platformVendor": "Advanced Micro Devices, Inc.",
+            "maxComputeUnits": p.compute_units, "maxWorkGroupSize": p.max_threads_per_block,
+            "maxClockFrequency": p.clock_khz // 1000, "globalMemSizeMB": p.total_mem // (1 << 20),
+            "maxMemAllocSizeMB": p.total_mem // (1 << 20), "localMemSizeKB": p.lds_bytes_per_block // 1024,
+            "deviceVersion": p.arch.decode(), "wavefrontSize": p.wavefront}
+
+
+def _state_int(index: int, value: int) -> None:
+    # THClState starts with ints: initialized, allowNonGpus, allocatedDevices, currentDevice, trace, addFinish,
+    # detailedTimings (include/thcl_hip.h, field order of src/lib/THClGeneral.h:76-93)
+    C.cast(state().buf, C.POINTER(C.c_int))[index] = int(value)
+
+
+def setTrace(flag: int) -> None:
+    """``cltorch.setTrace(1)`` (src/init.cpp:61-67): the state's trace flag."""
+    _state_int(4, flag)
+
+
+def setDetailedTimings(flag: int) -> None:
+    _state_int(6, flag)
+
+
+def setEnableTiming(flag) -> None:
+    """``cltorch.setEnableTiming`` / ``setTiming``: the reference's host-side timers map onto launch profiling."""
+    setProfiling(flag)
+
+
+setTiming = setEnableTiming
+
+
+def dumpTimings() -> str:
+    """``cltorch.dumpTimings()``: same records as :func:`dumpProfiling`."""
+    return dumpProfiling()
+
+
+def about() -> str:
+    """``cltorch.about()`` (src/init.cpp:180-196)."""
+    return "cltorch_amd: cltorch's tensor operator API on AMD Instinct GPUs through HIP\n"
+
+
+_rng = np.random.RandomState(5489)
+
+
+def manualSeed(seed: int) -> None:
+    """``torch.manualSeed(seed)`` for the host-side generator behind ``uniform`` / ``bernoulli`` / ``normal``."""
+    global _rng
+    _rng = np.random.RandomState(int(seed) & 0xFFFFFFFF)
+
+
+def _uniform01(n: int) -> np.ndarray:
+    # one 32-bit Mersenne-Twister word per value, scaled by 2^-32 (Torch7's THRandom_uniform)
+    return _rng.randint(0, 1 << 32, size=n, dtype=np.uint64).astype(np.float64) * (1.0 / 4294967296.0)
 
 
 def _long_storage(values: Sequence[int]):
@@ -914,6 +992,21 @@ class ClTensor:
 
     def addr(self, *args) -> "ClTensor":
         return self._addblas("addr", args)
+
+    # ---- random fills (src/Random.lua:6-24): drawn on the host, then copied over ----------
+    def uniform(self, a: float = 0.0, b: float = 1.0) -> "ClTensor":
+        vals = _uniform01(self.nElement()) * (b - a) + a
+        return self.copy(ClTensor(vals.astype(np.float32).reshape(self.size())))
+
+    def bernoulli(self, p: float = 0.5) -> "ClTensor":
+        vals = (_uniform01(self.nElement()) <= p).astype(np.float32)
+        return self.copy(ClTensor(vals.reshape(self.size())))
+
+    def normal(self, mean: float = 0.0, stdv: float = 1.0) -> "ClTensor":
+        n = self.nElement()
+        u1, u2 = _uniform01(n), _uniform01(n)
+        vals = np.sqrt(-2.0 * np.log(1.0 - u2)) * np.cos(2.0 * np.pi * u1) * stdv + mean
+        return self.copy(ClTensor(vals.astype(np.float32).reshape(self.size())))
 
     # ---- Lua operators (src/TensorOperator.c:5-250): each makes a new tensor ------------
     def _copy_of(self) -> "ClTensor":

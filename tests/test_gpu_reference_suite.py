@@ -293,3 +293,30 @@ def test_storage_basic_and_get(cl):                    # src/test/unit_storage.l
     assert (acl[2], acl[500], acl[7500]) == (72, 104, 1040)
     with pytest.raises(cl.ClError):
         cl.ClStorage(3).copy(np.zeros(4))                                              # sizes must match
+
+
+def test_device_functions_and_random_fills(cl):        # src/test/test-device.lua, src/init.cpp:44-121, src/Random.lua
+    n = cl.getDeviceCount()
+    assert n >= 1 and cl.getDevice() == 1
+    props = cl.getDeviceProperties(1)
+    assert props["deviceType"] == "GPU" and props["maxComputeUnits"] > 0 and props["globalMemSizeMB"] > 1024
+    assert props["maxWorkGroupSize"] == 1024 and props["deviceVersion"].startswith("gfx")
+    with pytest.raises(cl.ClError):
+        cl.getDeviceProperties(n + 1)
+    cl.setDevice(1)
+    assert np.array_equal(cl.ClTensor([7, -4, 5]).abs().float(), np.array([7, 4, 5], dtype=F))
+    cl.setTrace(1); cl.setTrace(0)
+    assert "cltorch" in cl.about()
+    # host-side draws: ranges, means, and the same seed giving the same values
+    cl.manualSeed(123)
+    u = cl.ClTensor(200, 50).uniform(-2, 3).float()
+    assert u.min() >= -2 and u.max() < 3 and abs(u.mean() - 0.5) < 0.05
+    cl.manualSeed(123)
+    assert np.array_equal(cl.ClTensor(200, 50).uniform(-2, 3).float(), u)
+    b = cl.ClTensor(10000).bernoulli(0.3).float()
+    assert set(np.unique(b)) <= {0.0, 1.0} and abs(b.mean() - 0.3) < 0.03
+    g = cl.ClTensor(20000).normal(1.0, 2.0).float()
+    assert abs(g.mean() - 1.0) < 0.06 and abs(g.std() - 2.0) < 0.06
+    # the first word of the Mersenne Twister seeded with 5489 is 3499211612 (the generator's published test value)
+    cl.manualSeed(5489)
+    assert cl.ClTensor(1).uniform().float()[0] == F(3499211612 / 4294967296.0)
