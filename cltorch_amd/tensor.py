@@ -1210,7 +1210,8 @@ class ClKernel:
         name = spec.get("name")
         funcs = spec.get("funcs")
         self._lib = state().lib
-        self._h = _call("THClKernel_new", name.encode() if name else None, (spec.get("src") or "").encode(),
+        self._src = spec.get("src") or ""
+        self._h = _call("THClKernel_new", name.encode() if name else None, self._src.encode(),
                         funcs.encode() if funcs else None, C.c_int(n), names, types, dirs)
         if not self._h:
             raise ClError("kernel construction failed")
@@ -1225,6 +1226,17 @@ class ClKernel:
 
     def getRenderedKernel(self) -> str:
         return self._lib.THClKernel_getRenderedKernel(self._h).decode()
+
+    def getRawKernel(self) -> str:
+        """The body as it was given (src/UserKernel.cpp:304-308)."""
+        return self._src
+
+    def print(self) -> str:
+        """``k:print()`` (src/UserKernel.cpp:292-303): both sources under the reference's headings."""
+        text = ("Original source\n===============\n" + self._src + "\n\n" +
+                "Generated source\n================\n" + self.getRenderedKernel() + "\n")
+        print(text, end="")
+        return text
 
     def run(self, params: dict, options: Optional[dict] = None) -> None:
         options = options or {}

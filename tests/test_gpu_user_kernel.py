@@ -99,3 +99,21 @@ def test_errors(cl):
     t = cl.ClTensor(64)
     ok.run({"a": t})
     assert t.float().tolist() == [1.0] * 64
+
+
+def test_reference_script(cl, capsys):
+    """src/test/test_userkernel.lua: more work-items than elements, the bound test in the body, print()."""
+    src = """
+   int linearId = get_global_id(0);
+   if(linearId < nElements) {
+     output_data[linearId] = input_data[linearId] + 3.0f;
+   }
+"""
+    k = cl.ClKernel({"input": {"nElements": "int", "input": "torch.ClTensor"}, "output": {"output": "torch.ClTensor"}, "src": src})
+    text = k.print()
+    assert capsys.readouterr().out == text
+    assert text.startswith("Original source\n===============\n" + src) and "Generated source\n================\n" in text
+    assert k.getRawKernel() == src and "input_data" in k.getRenderedKernel()
+    x, y = cl.ClTensor([3, 5, 2]), cl.ClTensor([6, 4, 2])
+    k.run({"nElements": 3, "input": x, "output": y}, {"numWorkgroups": 10, "workgroupSize": 32})
+    assert y.float().tolist() == [6, 8, 5] and x.float().tolist() == [3, 5, 2]
