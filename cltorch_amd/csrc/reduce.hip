@@ -518,19 +518,43 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
       thcl_u32 r = r_begin + wave;
       const float *ptr = P.in + off + (thcl_u64)r * P.rstride;
       const thcl_u64 step = (thcl_u64)WAVES * P.rstride;
-      for (; r + (FLY - 1) * WAVES < r_end; r += FLY * WAVES) {
-        if (VEC == 4) {
-          thcl_f4 v[FLY];
+      if (VEC == 4) {
+        // whole batches of FLY rows: the next batch is requested before the current one
+        // is consumed, so the wave always has loads in flight
+        if (r + (FLY - 1) * WAVES < r_end) {
+          thcl_f4 v[FLY], w[FLY];
+          auto fetch = [&](thcl_f4 (&x)[FLY]) {
 #pragma unroll
-          for (int f = 0; f < FLY; f++) {
-            v[f] = __builtin_nontemporal_load((const thcl_f4 *)ptr);
-            ptr += step;
+            for (int f = 0; f < FLY; f++) {
+              x[f] = __builtin_nontemporal_load((const thcl_f4 *)ptr);
+              ptr += step;
+            }
+          };
+          auto consume = [&](const thcl_f4 (&x)[FLY]) {
+#pragma unroll
+            for (int f = 0; f < FLY; f++)
+#pragma unroll
+              for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], x[f][c], (int)(r + f * WAVES), P.exponent);
+            r += FLY * WAVES;
+          };
+          fetch(v);
+          // two batches per turn, each requested while the other is consumed
+          while (r + (3 * FLY - 1) * WAVES < r_end) {
+            fetch(w);
+            consume(v);
+            fetch(v);
+            consume(w);
           }
-#pragma unroll
-          for (int f = 0; f < FLY; f++)
-#pragma unroll
-            for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v[f][c], (int)(r + f * WAVES), P.exponent);
-        } else {
+          if (r + (2 * FLY - 1) * WAVES < r_end) {
+            fetch(w);
+            consume(v);
+            consume(w);
+          } else {
+            consume(v);
+          }
+        }
+      } else {
+        for (; r + (FLY - 1) * WAVES < r_end; r += FLY * WAVES) {
           float v[FLY];
 #pragma unroll
           for (int f = 0; f < FLY; f++) {
