@@ -291,6 +291,26 @@ void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes) {
   return rt->scratch;
 }
 
+void *thcl_rt_host_alloc(size_t bytes) {
+  void *p = nullptr;
+  hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    g_err = std::string("hipHostMalloc: ") + hipGetErrorString(e);
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return p;
+}
+int thcl_rt_host_free(void *ptr) {
+  if (!ptr) return 0;
+  hipError_t e = hipHostFree(ptr);
+  if (e != hipSuccess) {
+    g_err = std::string("hipHostFree: ") + hipGetErrorString(e);
+    return -1;
+  }
+  return 0;
+}
+
 float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
 float *thcl_rt_host_word_device(thcl_rt *rt) { return rt->host_word_dev; }
 

@@ -106,6 +106,37 @@ def setAddFinish(flag: int) -> None:
     _state_int(5, flag)
 
 
+class _PinnedOwner:
+    def __init__(self, lib, ptr):
+        self.lib, self.ptr = lib, ptr
+
+    def __del__(self):
+        try:
+            if self.ptr and self.lib is not None:
+                self.lib.thcl_rt_host_free(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+def pinned_array(shape, dtype=np.float32) -> np.ndarray:
+    """A numpy array in page-locked host memory: copies between it and a ClTensor run at the link's
+    rate instead of the pageable-memory rate.  The memory is released with the array."""
+    st = state()
+    getDeviceCount()                                  # initialises the runtime
+    count = int(np.prod(shape)) if np.ndim(shape) else int(shape)
+    nbytes = max(count, 1) * np.dtype(dtype).itemsize
+    fn = st.lib.thcl_rt_host_alloc
+    fn.restype = C.c_void_p
+    ptr = fn(C.c_size_t(nbytes))
+    if not ptr:
+        raise ClError("pinned allocation failed: " + st.lib.thcl_rt_error().decode())
+    owner = _PinnedOwner(st.lib, ptr)
+    buf = (C.c_char * nbytes).from_address(ptr)
+    buf._owner = owner                                # keeps the allocation alive as long as any view of it
+    return np.frombuffer(buf, dtype=dtype, count=count).reshape(shape)
+
+
 def getDevice() -> int:
     """``cltorch.getDevice()`` (1-based, src/init.cpp:44-50)."""
     return int(_call("THClState_getDevice")) + 1

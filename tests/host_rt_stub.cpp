@@ -90,6 +90,8 @@ void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes) {
   if (bytes) *bytes = 65536;
   return rt->scratch;
 }
+void *thcl_rt_host_alloc(size_t bytes) { return malloc(bytes ? bytes : 1); }
+int thcl_rt_host_free(void *ptr) { free(ptr); return 0; }
 float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
 float *thcl_rt_host_word_device(thcl_rt *rt) { return rt->host_word; }
 thcl_rt_timer *thcl_rt_timer_new(thcl_rt *) { return new thcl_rt_timer(); }
