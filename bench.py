@@ -128,6 +128,9 @@ def main():
     ap.add_argument("--pmc-workload", action="store_true",
                     help="run each headline kernel twice plus a same-size copy (counter calibration) and exit; "
                          "meant to run under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --kernel-trace`")
+    ap.add_argument("--pmc-gemm", action="store_true",
+                    help="run the two addmm configurations a few times and exit; meant to run under "
+                         "`rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE --kernel-trace`")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -137,6 +140,8 @@ def main():
     import oracle
     if args.pmc_workload:
         return pmc_workload(cl, 1 << args.log2n)
+    if args.pmc_gemm:
+        return pmc_gemm(cl, oracle)
     T = Timers(cl)
     n = 1 << args.log2n
     X, Y, Z = (cl.ClTensor(oracle.uniform(s, n)) for s in (1, 2, 3))
@@ -191,6 +196,27 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(1 << args.cpu_log2n)
     print(json.dumps(out))
+
+
+def pmc_gemm(cl, oracle):
+    """Launches for a matrix-core counter run: config 5's square product five times (the clock
+    settles over the first launches) and its skinny product thirty times."""
+    k = 8192
+    sd = 1.0 / np.sqrt(k)
+    Am, Bm, Cm = (cl.ClTensor(oracle.normal(s, k * k, 0.0, sd)).resize(k, k) for s in (8, 9, 10))
+    for _ in range(5):
+        Cm.addmm(0.5, 1.0, Am, Bm)
+    cl.synchronize()
+    del Am, Bm, Cm
+    M, N, K = 64, 16384, 4096
+    sd = 1.0 / np.sqrt(K)
+    At = cl.ClTensor(oracle.normal(11, K * M, 0.0, sd)).resize(K, M)
+    Bs = cl.ClTensor(oracle.normal(12, K * N, 0.0, sd)).resize(K, N)
+    Cs = cl.ClTensor(oracle.normal(13, M * N, 0.0, sd)).resize(M, N)
+    for _ in range(30):
+        Cs.addmm(0.5, 1.0, At.t(), Bs)
+    cl.synchronize()
+    print(json.dumps({"pmc_gemm": "done"}))
 
 
 def pmc_workload(cl, n):
