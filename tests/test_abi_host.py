@@ -353,3 +353,44 @@ def test_text_form_matches_the_reference_expected_strings():
     assert nd.startswith("(1,.,.) = \n  0  0\n  0  0\n\n(2,.,.) = \n") and nd.endswith("[torch.ClTensor of size 2x2x2]\n")
     assert tensor_tostring(np.array([1e-3, 5.0, 123456.0])).splitlines()[0] == " 1.0000e-03"
     assert tensor_tostring(np.zeros(())) == "[torch.ClTensor with no dimension]\n"
+
+
+def test_public_structs_keep_the_reference_field_layout(tmp_path):
+    """LuaJIT code reads THClStorage / THClTensor fields directly (src/FFI.lua:6-33): the public header
+    must give every field the offset the reference's declaration gives it.  Both are compiled by gcc:
+    the header as shipped, and the reference's field list restated here with opaque pointers."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc not found")
+    src = tmp_path / "layout.c"
+    src.write_text(r'''
+#include <stddef.h>
+#include <stdio.h>
+#include "thcl_hip.h"
+typedef struct RefStorage { int device; float *data; void *cl; void *wrapper; long size; int refcount; char flag;
+                            void *allocator; void *allocatorContext; struct RefStorage *view; } RefStorage;
+typedef struct RefTensor { long *size; long *stride; int nDimension; RefStorage *storage; long storageOffset;
+                           int refcount; char flag; int device; } RefTensor;
+#define CHECK(T, R, f) if (offsetof(T, f) != offsetof(R, f)) { printf("%s.%s at %zu, reference %zu\n", #T, #f, offsetof(T, f), offsetof(R, f)); bad = 1; }
+int main(void) {
+  int bad = 0;
+  CHECK(THClStorage, RefStorage, device) CHECK(THClStorage, RefStorage, data) CHECK(THClStorage, RefStorage, cl)
+  CHECK(THClStorage, RefStorage, wrapper) CHECK(THClStorage, RefStorage, size) CHECK(THClStorage, RefStorage, refcount)
+  CHECK(THClStorage, RefStorage, flag) CHECK(THClStorage, RefStorage, allocator) CHECK(THClStorage, RefStorage, allocatorContext)
+  CHECK(THClStorage, RefStorage, view)
+  CHECK(THClTensor, RefTensor, size) CHECK(THClTensor, RefTensor, stride) CHECK(THClTensor, RefTensor, nDimension)
+  CHECK(THClTensor, RefTensor, storage) CHECK(THClTensor, RefTensor, storageOffset) CHECK(THClTensor, RefTensor, refcount)
+  CHECK(THClTensor, RefTensor, flag) CHECK(THClTensor, RefTensor, device)
+  if (sizeof(THClStorage) != sizeof(RefStorage) || sizeof(THClTensor) != sizeof(RefTensor)) { printf("sizes differ\n"); bad = 1; }
+  printf("%zu %zu\n", sizeof(THClStorage), sizeof(THClTensor));
+  return bad;
+}
+''')
+    exe = tmp_path / "layout"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-I", os.path.join(root, "include"), str(src), "-o", str(exe)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr          # also: the public header is valid C99 on its own
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout
