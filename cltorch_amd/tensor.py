@@ -479,10 +479,12 @@ class ClTensor:
                     t = t.narrow(1, k, 1)
                     d += 1
             else:
-                lo, hi = (k + (None,))[:2] if len(k) == 1 else k
+                k = tuple(k)                    # (): the whole dim, (i,): i alone with the dim kept, (lo, hi): a range
                 n = t.size(d)
-                lo = 1 if lo is None else (lo + n + 1 if lo < 0 else lo)
-                hi = n if hi is None else (hi + n + 1 if hi < 0 else hi)
+                lo = k[0] if len(k) > 0 else 1
+                hi = k[1] if len(k) > 1 else (lo if len(k) == 1 else n)
+                lo = lo + n + 1 if lo < 0 else lo
+                hi = hi + n + 1 if hi < 0 else hi
                 t = t.narrow(d, lo, hi - lo + 1)
                 d += 1
         return t

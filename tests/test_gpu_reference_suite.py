@@ -172,6 +172,7 @@ def test_lua_indexing(cl):                             # src/torch/generic/Tenso
     assert np.array_equal(xt[xt.gt(0.5)].float(), x0.T[x0.T > 0.5])
     assert np.array_equal(x[3].float(), x0[2]) and x[3][4] == x0[2, 3]
     assert np.array_equal(x[(2, (5, 9))].float(), x0[1, 4:9]) and np.array_equal(x[((2, 4), (1, 3))].float(), x0[1:4, 0:3])
+    assert np.array_equal(x[((), (3,))].float(), x0[:, 2:3]) and x[((2,), ())].size() == (1, 19)
     x[2] = 7.0
     x[((5, 6), (1, 2))] = -1.0
     x[(9, (3, 5))] = cl.ClTensor([1, 2, 3])
