@@ -542,8 +542,10 @@ class ClTensor:
     def float(self) -> np.ndarray:
         """``clTensor:float()``: a host copy shaped like the tensor."""
         nd = self.nDimension()
-        if nd == 0:
-            return np.array(self.s(), dtype=np.float32)
+        if nd <= 0:
+            # no dimensions: an empty tensor, or a point tensor, whose one value ``s()`` reads; as in Lua,
+            # the host copy of either has no elements
+            return np.empty((0,), dtype=np.float32)
         shape = self.size()
         out = np.empty(shape if nd > 0 else (0,), dtype=np.float32)
         if out.size:

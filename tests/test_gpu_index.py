@@ -142,7 +142,7 @@ def test_masked_edge_cases(cl):
     x = oracle.uniform(111, n)
     X = cl.ClTensor(x)
     none = X.maskedSelect(cl.ClTensor(np.zeros(n, dtype=F)))
-    assert none.nElement() == 0
+    assert none.nElement() == 0 and none.nDimension() == 0 and none.float().shape == (0,)
     every = X.maskedSelect(cl.ClTensor(np.ones(n, dtype=F)))
     assert_bit_equal(every.float(), x, "all selected")
     # 2-d strided source and mask
