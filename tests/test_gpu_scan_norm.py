@@ -73,6 +73,28 @@ def test_scan_closed_forms_views_and_in_place(cl):
         cl.ClTensor(x).cumsum(3)
 
 
+def test_scan_of_long_rows(cl):
+    """Rows too few to fill the chip are cut into segments: segment totals, a scan of the totals, then the
+    scan proper.  2^25 + 5000 elements end in a ragged segment; the result is the same on every run."""
+    n = (1 << 25) + 5000
+    ones = cl.ClTensor(n)
+    ones.fill(1.0)
+    assert np.array_equal(ones.cumsum().float(), np.arange(1, n + 1, dtype=np.float64).astype(F))
+    x = oracle.uniform(66, n)
+    X = cl.ClTensor(x)
+    first = X.cumsum().float()
+    _scan_close(first, cat.cumulate(x, 0), "cumsum of 2^25 + 5000 elements")
+    for _ in range(3):
+        assert_bit_equal(X.cumsum().float(), first, "repeat of the same scan")
+    # an odd length and a source that starts 4 bytes off a 16-byte boundary: the scalar path
+    xo = X.narrow(1, 2, n - 2)
+    _scan_close(xo.cumsum().float(), cat.cumulate(x[1:n - 1], 0), "unaligned source")
+    # three long rows; products that stay near 1
+    y = oracle.uniform(67, 3 * 70 * 4096, 0.999, 1.001).reshape(3, 70 * 4096)
+    _scan_close(cl.ClTensor(y).cumprod(2).float(), cat.cumulate(y, 1, prod=True), "cumprod of 3 long rows")
+    _scan_close(cl.ClTensor(y).cumsum(2).float(), cat.cumulate(y, 1), "cumsum of 3 long rows")
+
+
 def test_mean_and_norms(cl):
     x = oracle.normal(64, 300 * 700).reshape(300, 700)
     x[5, :40] = 0.0
