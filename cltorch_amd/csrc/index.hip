@@ -98,80 +98,81 @@ __global__ __launch_bounds__(kThreads) void fill_int(int *p, int v, thcl_u32 n) 
 // ---------------------------------------------------------------- masked ---
 // Stream compaction in three passes over blocks of kChunk elements: count the
 // selected elements of every block, turn the counts into offsets (one block,
-// the list is short), then every block re-derives its elements' ranks and moves them.
+// the list is short), then every block derives its elements' ranks and moves them.
+// The first pass also leaves the mask as one bit per element, so the last pass
+// reads 1/32 of the mask's bytes and finds ranks by counting bits, with no
+// exchange between threads.
+//
+// Bit layout: a chunk is 4 steps of 1024 elements; in a step thread t holds elements
+// 4t .. 4t+3.  Word [chunk][step][wave][e] has bit l set when element e of lane l of
+// that wave is selected.
 constexpr int kPer = 16, kChunk = kThreads * kPer;
+constexpr int kMaskPer = 4, kMaskStep = kThreads * kMaskPer, kMaskSteps = kChunk / kMaskStep, kMaskWaves = kThreads / 64;
+constexpr int kWordsPerStep = kMaskWaves * kMaskPer, kWordsPerChunk = kMaskSteps * kWordsPerStep;
 
 struct MaskParams {
   const float *mask;
   const float *src;   // select: [n] values; copy: the packed source
   float *dst;         // select: packed output; copy: [n] destination
-  unsigned *counts;   // per block, then exclusive offsets; counts[nblocks] = total
+  unsigned *counts;   // per block, then exclusive offsets inside the block's group of 4096
+  unsigned *groups;   // per group of 4096 blocks: total, then exclusive offset; groups[ngroups] = grand total
+  thcl_u32 ngroups;
+  unsigned long long *bits;  // [nblocks][kWordsPerChunk]
   thcl_u64 n;
   thcl_u32 nblocks;
   thcl_u64 src_len;   // copy: elements available in src
 };
 
-__device__ __forceinline__ unsigned block_exclusive(unsigned v, unsigned *lds, unsigned *total) {
-  // exclusive prefix of v over the block's threads
-  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-  unsigned incl = v;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const unsigned up = __shfl_up(incl, d, 64);
-    if (lane >= d) incl += up;
-  }
-  __syncthreads();
-  if (lane == 63) lds[wave] = incl;
-  __syncthreads();
-  unsigned before = 0, all = 0;
-#pragma unroll
-  for (int w = 0; w < kThreads / 64; w++) {
-    if (w < wave) before += lds[w];
-    all += lds[w];
-  }
-  *total = all;
-  return before + incl - v;
-}
-
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void mask_count(MaskParams P) {
-  __shared__ unsigned lds[kThreads / 64];
-  const thcl_u64 base = (thcl_u64)blockIdx.x * kChunk;
-  unsigned c = 0;
-  if (VEC && base + kChunk <= P.n) {  // whole chunk: 128-bit loads (the order inside a chunk does not matter for a count)
-    thcl_f4 v[kPer / 4];
+  __shared__ unsigned lds[kMaskWaves];
+  const thcl_u64 chunk0 = (thcl_u64)blockIdx.x * kChunk;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  float m[kMaskSteps][kMaskPer];
 #pragma unroll
-    for (int k = 0; k < kPer / 4; k++)
-      v[k] = __builtin_nontemporal_load((const thcl_f4 *)(P.mask + base) + k * kThreads + threadIdx.x);
+  for (int step = 0; step < kMaskSteps; step++) {
+    const thcl_u64 first = chunk0 + (thcl_u64)step * kMaskStep + (thcl_u64)threadIdx.x * kMaskPer;
+    if (VEC && first + kMaskPer <= P.n) {
+      const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(P.mask + first));
 #pragma unroll
-    for (int k = 0; k < kPer / 4; k++)
+      for (int e = 0; e < kMaskPer; e++) m[step][e] = v[e];
+    } else {
 #pragma unroll
-      for (int e = 0; e < 4; e++) c += (v[k][e] != 0.0f) ? 1u : 0u;
-  } else {
-#pragma unroll
-    for (int k = 0; k < kPer; k++) {
-      const thcl_u64 i = base + (thcl_u64)k * kThreads + threadIdx.x;
-      if (i < P.n) c += (__builtin_nontemporal_load(P.mask + i) != 0.0f) ? 1u : 0u;
+      for (int e = 0; e < kMaskPer; e++) m[step][e] = (first + e < P.n) ? P.mask[first + e] : 0.0f;
     }
   }
-  unsigned total;
-  (void)block_exclusive(c, lds, &total);
-  if (threadIdx.x == 0) P.counts[blockIdx.x] = total;
+  unsigned c = 0;                // the wave's selected elements (the same in every lane)
+  unsigned long long mine = 0;   // lane 4 * step + e keeps word (step, e) of this wave
+#pragma unroll
+  for (int step = 0; step < kMaskSteps; step++) {
+#pragma unroll
+    for (int e = 0; e < kMaskPer; e++) {
+      const unsigned long long b = __ballot(m[step][e] != 0.0f);
+      c += (unsigned)__popcll(b);
+      if (lane == step * kMaskPer + e) mine = b;
+    }
+  }
+  if (lane < kMaskSteps * kMaskPer)
+    P.bits[(thcl_u64)blockIdx.x * kWordsPerChunk + (lane / kMaskPer) * kWordsPerStep + wave * kMaskPer + lane % kMaskPer] = mine;
+  if (lane == 0) lds[wave] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned total = 0;
+#pragma unroll
+    for (int w = 0; w < kMaskWaves; w++) total += lds[w];
+    P.counts[blockIdx.x] = total;
+  }
 }
 
-// counts -> exclusive offsets, total at counts[nblocks].  One block: each thread sums a
-// run of adjacent counts, the 1024 run sums are scanned once, and the run is walked
-// again to leave the offsets.
-__global__ __launch_bounds__(1024) void mask_offsets(MaskParams P) {
-  __shared__ unsigned lds[1024 / 64];
-  const thcl_u32 per = (P.nblocks + 1023u) / 1024u;
-  const thcl_u32 lo = threadIdx.x * per;
-  thcl_u32 hi = lo + per;
-  if (hi > P.nblocks) hi = P.nblocks;
-  unsigned sum = 0;
-  for (thcl_u32 i = lo; i < hi; i++) sum += P.counts[i];
+// Block counts -> exclusive offsets in two levels.  mask_scan_groups: a block of 1024
+// threads turns 4096 adjacent counts into offsets within the group (4 per thread, one
+// 16-byte access) and leaves the group's total.  mask_scan_totals: one block turns
+// the group totals into group offsets and leaves the grand total behind them.
+constexpr int kGroup = 4096;
+
+__device__ __forceinline__ unsigned block1024_exclusive(unsigned v, unsigned *lds, unsigned *total) {
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
-  unsigned incl = sum;
+  unsigned incl = v;
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
     const unsigned up = __shfl_up(incl, d, 64);
@@ -185,63 +186,134 @@ __global__ __launch_bounds__(1024) void mask_offsets(MaskParams P) {
     if (w < wave) before += lds[w];
     all += lds[w];
   }
-  before += incl - sum;
-  for (thcl_u32 i = lo; i < hi; i++) {
-    const unsigned v = P.counts[i];
-    P.counts[i] = before;
-    before += v;
+  __syncthreads();  // lds may be reused
+  *total = all;
+  return before + incl - v;
+}
+
+__global__ __launch_bounds__(1024) void mask_scan_groups(MaskParams P) {
+  __shared__ unsigned lds[1024 / 64];
+  const thcl_u64 i0 = (thcl_u64)blockIdx.x * kGroup + (thcl_u64)threadIdx.x * 4;
+  unsigned v[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) v[k] = (i0 + k < P.nblocks) ? P.counts[i0 + k] : 0u;
+  unsigned total;
+  unsigned run = block1024_exclusive(v[0] + v[1] + v[2] + v[3], lds, &total);
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    if (i0 + k < P.nblocks) P.counts[i0 + k] = run;
+    run += v[k];
   }
-  if (threadIdx.x == 0) P.counts[P.nblocks] = all;
+  if (threadIdx.x == 0) P.groups[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(1024) void mask_scan_totals(MaskParams P) {
+  __shared__ unsigned lds[1024 / 64];
+  unsigned carry = 0;
+  for (thcl_u32 g0 = 0; g0 < P.ngroups; g0 += 1024) {
+    const thcl_u32 g = g0 + threadIdx.x;
+    const unsigned v = g < P.ngroups ? P.groups[g] : 0u;
+    unsigned total;
+    const unsigned excl = block1024_exclusive(v, lds, &total);
+    if (g < P.ngroups) P.groups[g] = carry + excl;
+    carry += total;
+  }
+  if (threadIdx.x == 0) P.groups[P.ngroups] = carry;
 }
 
 // COPY false: dst[rank] = src[i] for selected i.  COPY true: dst[i] = src[rank].
-// A block walks its chunk 1024 elements at a time, 4 consecutive elements per
-// thread (one 16-byte access when VEC), so ranks follow element order and every
-// wave reads whole lines; the rank carries from step to step.
+// VEC: the full-length operand (src when selecting, dst when copying) allows 16-byte accesses.
+// A block takes a chunk, 4 steps of 1024 elements with 4 consecutive elements per thread.
+// Every wave reads the chunk's 64 bit words, one per lane; a shuffle scan of their
+// population counts gives the rank in front of every (step, wave), and an element's rank
+// adds the set bits of earlier lanes (4 words) and of earlier elements of its own lane.
+// The chunk's selected elements are adjacent in the packed tensor: they pass through LDS,
+// so the packed side is read or written as one run, and every global read of the block is
+// requested before the first one is waited for.  When copying into a chunk with an eighth
+// or more of its elements selected, whole 16-byte groups of dst are rewritten instead of
+// single elements.
 template <bool COPY, bool VEC>
 __global__ __launch_bounds__(kThreads) void mask_move(MaskParams P) {
-  __shared__ unsigned lds[kThreads / 64];
-  constexpr int PER = 4, STEP = kThreads * PER;
-  unsigned carry = P.counts[blockIdx.x];
+  __shared__ float stage[kChunk];
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const unsigned long long below = (1ull << lane) - 1ull;
   const thcl_u64 chunk0 = (thcl_u64)blockIdx.x * kChunk;
-  for (int step = 0; step < kChunk / STEP; step++) {
-    const thcl_u64 first = chunk0 + (thcl_u64)step * STEP + (thcl_u64)threadIdx.x * PER;
-    if (chunk0 + (thcl_u64)step * STEP >= P.n) break;  // uniform: the whole block is past the end
-    float m[PER], x[PER];
-    const bool whole = first + PER <= P.n;
-    if (VEC && whole) {
-      const thcl_f4 mv = __builtin_nontemporal_load((const thcl_f4 *)(P.mask + first));
+  const thcl_u64 block_rank = (thcl_u64)P.counts[blockIdx.x] + (thcl_u64)P.groups[blockIdx.x / kGroup];
+  const unsigned long long word = P.bits[(thcl_u64)blockIdx.x * kWordsPerChunk + lane];  // kWordsPerChunk == 64
+  // exclusive prefix of the words' population counts, in word order = (step, wave, e) order
+  const unsigned pc = (unsigned)__popcll(word);
+  unsigned incl = pc;
 #pragma unroll
-      for (int k = 0; k < PER; k++) m[k] = mv[k];
-      if (!COPY) {
-        const thcl_f4 xv = __builtin_nontemporal_load((const thcl_f4 *)(P.src + first));
+  for (int d = 1; d < 64; d <<= 1) {
+    const unsigned up = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += up;
+  }
+  const unsigned excl = incl - pc;
+  const unsigned chunk_total = __shfl(incl, 63, 64);
+  if (chunk_total == 0) return;  // uniform over the block
+  const bool groups16 = COPY && VEC && chunk_total >= kChunk / 8;
+
+  // a vector that is not whole (at most one in the tensor) is requested from the start of the
+  // tensor instead (n >= 4 when VEC) and its elements are handled one by one below
+  thcl_f4 x[kMaskSteps];
+  if (VEC && (!COPY || groups16)) {
+    const float *full = COPY ? P.dst : P.src;
 #pragma unroll
-        for (int k = 0; k < PER; k++) x[k] = xv[k];
+    for (int step = 0; step < kMaskSteps; step++) {
+      thcl_u64 first = chunk0 + (thcl_u64)step * kMaskStep + (thcl_u64)threadIdx.x * kMaskPer;
+      if (first + kMaskPer > P.n) first = 0;
+      x[step] = COPY ? *(const thcl_f4 *)(full + first) : __builtin_nontemporal_load((const thcl_f4 *)(full + first));
+    }
+  }
+  if (COPY) {
+    // the chunk's run of the packed source, as far as the source reaches
+    for (unsigned j = threadIdx.x; j < chunk_total; j += kThreads)
+      stage[j] = (block_rank + j < P.src_len) ? P.src[block_rank + j] : 0.0f;
+    __syncthreads();
+  }
+#pragma unroll
+  for (int step = 0; step < kMaskSteps; step++) {
+    const int w0 = step * kWordsPerStep + wave * kMaskPer;   // this wave's first word of the step
+    unsigned long long b[kMaskPer];
+#pragma unroll
+    for (int e = 0; e < kMaskPer; e++) b[e] = __shfl(word, w0 + e, 64);
+    unsigned rank = __shfl(excl, w0, 64);   // inside the chunk
+#pragma unroll
+    for (int e = 0; e < kMaskPer; e++) rank += (unsigned)__popcll(b[e] & below);
+    const thcl_u64 first = chunk0 + (thcl_u64)step * kMaskStep + (thcl_u64)threadIdx.x * kMaskPer;
+    const bool whole = first + kMaskPer <= P.n;
+    if (!COPY) {
+#pragma unroll
+      for (int e = 0; e < kMaskPer; e++) {
+        if ((b[e] >> lane) & 1ull) stage[rank++] = (VEC && whole) ? x[step][e] : P.src[first + e];
       }
+    } else if (groups16 && whole) {
+      thcl_f4 d = x[step];
+      bool any = false;
+#pragma unroll
+      for (int e = 0; e < kMaskPer; e++) {
+        if ((b[e] >> lane) & 1ull) {
+          if (block_rank + rank < P.src_len) {
+            d[e] = stage[rank];
+            any = true;
+          }
+          rank++;
+        }
+      }
+      if (any) *(thcl_f4 *)(P.dst + first) = d;
     } else {
 #pragma unroll
-      for (int k = 0; k < PER; k++) {
-        m[k] = (first + k < P.n) ? P.mask[first + k] : 0.0f;
-        if (!COPY) x[k] = (first + k < P.n) ? P.src[first + k] : 0.0f;
-      }
-    }
-    unsigned c = 0;
-#pragma unroll
-    for (int k = 0; k < PER; k++) c += (m[k] != 0.0f) ? 1u : 0u;
-    unsigned total;
-    unsigned rank = carry + block_exclusive(c, lds, &total);
-    carry += total;
-#pragma unroll
-    for (int k = 0; k < PER; k++) {
-      if (m[k] != 0.0f) {
-        if (COPY) {
-          if (rank < P.src_len) P.dst[first + k] = P.src[rank];
-        } else {
-          P.dst[rank] = x[k];
+      for (int e = 0; e < kMaskPer; e++) {
+        if ((b[e] >> lane) & 1ull) {
+          if (block_rank + rank < P.src_len) P.dst[first + e] = stage[rank];
+          rank++;
         }
-        rank++;
       }
     }
+  }
+  if (!COPY) {
+    __syncthreads();
+    for (unsigned j = threadIdx.x; j < chunk_total; j += kThreads) P.dst[block_rank + j] = stage[j];
   }
 }
 
@@ -544,20 +616,28 @@ static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long 
   THCL_CHECK(nb < (1l << 31) - 1, THCL_DIM_WARNING);
   P.n = (thcl_u64)n;
   P.nblocks = (thcl_u32)nb;
-  P.counts = (unsigned *)thcl_rt_workspace(rt, (size_t)(nb + 1) * sizeof(unsigned));
-  THCL_CHECK(P.counts != nullptr, "%s", thcl_rt_error());
+  // the bit words first (8-byte aligned), then the counts and the group totals
+  const long ng = (nb + kGroup - 1) / kGroup;
+  P.ngroups = (thcl_u32)ng;
+  const size_t bit_bytes = (size_t)nb * kWordsPerChunk * sizeof(unsigned long long);
+  char *w = (char *)thcl_rt_workspace(rt, bit_bytes + (size_t)(nb + ng + 1) * sizeof(unsigned));
+  THCL_CHECK(w != nullptr, "%s", thcl_rt_error());
+  P.bits = (unsigned long long *)w;
+  P.counts = (unsigned *)(w + bit_bytes);
+  P.groups = P.counts + nb;
   if (aligned16(P.mask)) hipLaunchKernelGGL(mask_count<true>, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
   else hipLaunchKernelGGL(mask_count<false>, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
   check("mask count");
-  hipLaunchKernelGGL(mask_offsets, dim3(1), dim3(1024), 0, stream, P);
+  hipLaunchKernelGGL(mask_scan_groups, dim3((unsigned)ng), dim3(1024), 0, stream, P);
+  hipLaunchKernelGGL(mask_scan_totals, dim3(1), dim3(1024), 0, stream, P);
   check("mask offsets");
   (void)state;
   return P.counts;
 }
 
-static long read_total(thcl_rt *rt, const unsigned *counts, thcl_u32 nblocks) {
+static long read_total(thcl_rt *rt, const MaskParams &P) {
   float *hw = thcl_rt_host_word(rt);  // a pinned 4-byte word: carries the count's bits
-  THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, counts + nblocks, sizeof(unsigned)) == 0, "%s", thcl_rt_error());
+  THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, P.groups + P.ngroups, sizeof(unsigned)) == 0, "%s", thcl_rt_error());
   unsigned total;
   memcpy(&total, hw, sizeof(total));
   return (long)total;
@@ -584,12 +664,12 @@ void THClTensor_maskedSelect(THClState *state, THClTensor *tensor, THClTensor *s
   P.mask = thcl_dptr(m.t);
   P.src = thcl_dptr(s.t);
   mask_prefix(state, rt, P, n);
-  const long total = read_total(rt, P.counts, P.nblocks);  // the one synchronising step: the result's size
+  const long total = read_total(rt, P);  // the one synchronising step: the result's size
   THClTensor_resize1d(state, tensor, total);
   if (total > 0) {
     Dense r(state, tensor, false, true);
     P.dst = thcl_dptr(r.t);
-    if (aligned16(P.mask) && aligned16(P.src))
+    if (aligned16(P.src) && n >= 4)
       hipLaunchKernelGGL((mask_move<false, true>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
     else
       hipLaunchKernelGGL((mask_move<false, false>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
@@ -621,12 +701,12 @@ void THClTensor_maskedCopy(THClState *state, THClTensor *tensor, THClTensor *mas
   P.dst = thcl_dptr(r.t);
   P.src_len = (thcl_u64)THClTensor_nElement(state, src);
   mask_prefix(state, rt, P, n);
-  if (aligned16(P.mask))
+  if (aligned16(P.dst))
     hipLaunchKernelGGL((mask_move<true, true>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
   else
     hipLaunchKernelGGL((mask_move<true, false>), dim3(P.nblocks), dim3(kThreads), 0, (hipStream_t)thcl_rt_stream(rt), P);
   check("masked copy");
-  const long total = read_total(rt, P.counts, P.nblocks);
+  const long total = read_total(rt, P);
   thcl_after_launch(state, rt);
   s.finish();
   m.finish();

@@ -118,7 +118,7 @@ def test_gather_scatter_views_and_checks(cl):
         X.scatter(1, cl.ClTensor(np.ones((2, 20), dtype=F)), cl.ClTensor(3, 20))
 
 
-@pytest.mark.parametrize("n", [1, 5, 255, 256, 4095, 4096, 4097, 100003, (1 << 22) + 11])
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 6, 255, 256, 1023, 1025, 4095, 4096, 4097, 100003, (1 << 22) + 11, (1 << 24) + 3 * 4099])
 def test_masked_select_and_copy(cl, n):
     x = oracle.uniform(108, n)
     mask = (oracle.uniform(109, n) > 0.2).astype(F)
