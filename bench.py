@@ -374,8 +374,9 @@ def detail(cl, oracle, T, X, Y, Z, n):
     src = cl.ClTensor(1 << 26)
     src.fill(1.0)
     packed = cl.ClTensor()
-    # mask read twice (count, move), source read once, half of it written
-    measure("w_maskedSelect_2^26_half", lambda: packed.maskedSelect(src, mask), (4 + 4 + 4 + 2) * (1 << 26))
+    # algorithmic bytes: mask and source read once, half of the source written (the call also
+    # waits for the count, which sizes the result)
+    measure("w_maskedSelect_2^26_half", lambda: packed.maskedSelect(src, mask), (4 + 4 + 2) * (1 << 26))
     return d
 
 
