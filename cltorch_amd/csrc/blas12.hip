@@ -7,8 +7,8 @@
 // All three are bound by HBM: gemv reads the matrix once (4 bytes per 2
 // flops), so the kernels are streaming reductions, with fp64 accumulators
 // like the other sums of this library.  The rank-1 update is a pointwise
-// operator over the matrix with the vectors as stride-0 views, and runs on the
-// apply engine.
+// operator over the matrix: a dedicated kernel when the matrix has unit stride
+// along one dim, otherwise the apply engine with the vectors as stride-0 views.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -185,6 +185,76 @@ void check(const char *what) {
 bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 
 // 1-d vector as an (rows x cols) view that repeats it along the other dim
+// Rank-1 update of a matrix whose lines are contiguous: a[l][c] = beta * a[l][c] + alpha * u[l] * v[c]
+// with c along the contiguous dim.  A thread owns 4 adjacent columns (one 16-byte access) and 8 lines,
+// so its 8 reads are in flight together and its part of v is read once.  UFIRST: the product is
+// (alpha * u[l]) * v[c], otherwise (alpha * v[c]) * u[l] -- the association of the operator string
+// the generic path would compile, so both paths give the same bits.
+struct Rank1Params {
+  float *a;
+  const float *u, *v;
+  thcl_u64 lines, cols, pitch;
+  long incu, incv;
+  float beta, alpha;
+};
+template <bool UFIRST>
+__global__ __launch_bounds__(kThreads) void rank1_update(Rank1Params P) {
+  constexpr int LINES = 8, LANES = 64, GROUPS = kThreads / LANES;
+  const thcl_u64 c = ((thcl_u64)blockIdx.x * LANES + threadIdx.x % LANES) * 4;
+  const thcl_u64 l0 = (thcl_u64)blockIdx.y * (GROUPS * LINES) + threadIdx.x / LANES;
+  if (c >= P.cols) return;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) v[e] = P.v[(long)(c + e) * P.incv];
+  thcl_f4 a[LINES];
+  float u[LINES];
+#pragma unroll
+  for (int k = 0; k < LINES; k++) {
+    thcl_u64 l = l0 + (thcl_u64)k * GROUPS;
+    if (l >= P.lines) l = P.lines - 1;  // read again, not stored
+    a[k] = __builtin_nontemporal_load((const thcl_f4 *)(P.a + l * P.pitch + c));
+    u[k] = P.u[(long)l * P.incu];
+  }
+#pragma unroll
+  for (int k = 0; k < LINES; k++) {
+    const thcl_u64 l = l0 + (thcl_u64)k * GROUPS;
+    if (l >= P.lines) break;
+    thcl_f4 r;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float prod = UFIRST ? (P.alpha * u[k]) * v[e] : (P.alpha * v[e]) * u[k];
+      r[e] = (P.beta == 1.f) ? a[k][e] + prod : P.beta * a[k][e] + prod;
+    }
+    __builtin_nontemporal_store(r, (thcl_f4 *)(P.a + l * P.pitch + c));
+  }
+}
+
+// true when the update ran here; false: the caller takes the generic pointwise path
+bool rank1_fast(THClState *state, thcl_rt *rt, float *a, thcl_u64 lines, thcl_u64 cols, thcl_u64 pitch, const float *u, long incu,
+                const float *v, long incv, float beta, float alpha, bool ufirst) {
+  if (cols % 4 != 0 || pitch % 4 != 0 || (((uintptr_t)a) & 15u) != 0 || pitch < cols) return false;
+  const thcl_u64 gx = (cols / 4 + 63) / 64, gy = (lines + 31) / 32;
+  if (gx >= (1ull << 31) || gy >= 65536) return false;
+  Rank1Params P;
+  P.a = a;
+  P.u = u;
+  P.v = v;
+  P.lines = lines;
+  P.cols = cols;
+  P.pitch = pitch;
+  P.incu = incu;
+  P.incv = incv;
+  P.beta = beta;
+  P.alpha = alpha;
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
+  if (ufirst) hipLaunchKernelGGL(rank1_update<true>, dim3((unsigned)gx, (unsigned)gy), dim3(kThreads), 0, stream, P);
+  else hipLaunchKernelGGL(rank1_update<false>, dim3((unsigned)gx, (unsigned)gy), dim3(kThreads), 0, stream, P);
+  hipError_t e = hipGetLastError();
+  THCL_CHECK(e == hipSuccess, "rank-1 update launch failed: %s", hipGetErrorString(e));
+  thcl_after_launch(state, rt);
+  return true;
+}
+
 THClTensor *expanded(THClState *state, THClTensor *vec, long rows, long cols, bool along_rows) {
   long sz[2] = {rows, cols};
   long st[2] = {along_rows ? vec->stride[0] : 0, along_rows ? 0 : vec->stride[0]};
@@ -380,6 +450,19 @@ void THClTensor_addr(THClState *state, THClTensor *r_, float beta, THClTensor *t
     THClTensor_copy(state, r_, t);
   }
   if (r_->size[0] == 0 || r_->size[1] == 0) return;
+  {
+    // the generic path's operator is beta * out + (alpha * vec1[i]) * vec2[j]
+    thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, r_));
+    const long rows = r_->size[0], cols = r_->size[1];
+    if (r_->stride[1] == 1 && r_->stride[0] >= cols && cols > 1 &&
+        rank1_fast(state, rt, thcl_dptr(r_), (thcl_u64)rows, (thcl_u64)cols, (thcl_u64)r_->stride[0], thcl_dptr(vec1), vec1->stride[0],
+                   thcl_dptr(vec2), vec2->stride[0], beta, alpha, true))
+      return;
+    if (r_->stride[0] == 1 && r_->stride[1] >= rows && rows > 1 &&
+        rank1_fast(state, rt, thcl_dptr(r_), (thcl_u64)cols, (thcl_u64)rows, (thcl_u64)r_->stride[1], thcl_dptr(vec2), vec2->stride[0],
+                   thcl_dptr(vec1), vec1->stride[0], beta, alpha, false))
+      return;
+  }
   THClTensor *v1 = expanded(state, vec1, r_->size[0], r_->size[1], true);
   THClTensor *v2 = expanded(state, vec2, r_->size[0], r_->size[1], false);
   ApplyCall c;

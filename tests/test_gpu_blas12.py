@@ -89,6 +89,27 @@ def test_addmv_beta_zero_ignores_old_contents_and_checks_shapes(cl):
         cl.ClTensor().addmv(cl.ClTensor(t), cl.ClTensor(v), cl.ClTensor(v))
 
 
+def test_addr_kernel_and_generic_path_agree_bit_for_bit(cl):
+    """A matrix with unit stride along one dim, 16-byte aligned, takes the rank-1 kernel; the same values in a
+    view that starts 4 bytes off a 16-byte boundary take the pointwise engine.  Same association, same bits."""
+    rows, cols = 1000, 1000
+    t = oracle.normal(83, rows * cols).reshape(rows, cols)
+    a, b = oracle.normal(84, rows), oracle.normal(85, cols)
+    A, B = cl.ClTensor(a), cl.ClTensor(b)
+    wide = np.zeros((rows, cols + 4), dtype=F)
+    wide[:, 1:cols + 1] = t
+    for beta, alpha in ((1.0, 0.5), (0.9, -1.25)):
+        fast = cl.ClTensor(t)
+        fast.addr(beta, alpha, A, B)
+        slow = cl.ClTensor(wide).narrow(2, 2, cols)
+        slow.addr(beta, alpha, A, B)
+        assert np.array_equal(fast.float().view(np.uint32), slow.float().view(np.uint32)), (beta, alpha)
+        # column-major: the transposed view of a (cols x rows) matrix
+        fast_t = cl.ClTensor(np.ascontiguousarray(t.T)).t()
+        fast_t.addr(beta, alpha, A, B)
+        assert np.array_equal(fast_t.float().view(np.uint32), slow.float().view(np.uint32)), (beta, alpha, "column-major")
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 1), (2, 3), (130, 70), (64, 256), (1000, 1000), (5, 50000), (50000, 5)])
 def test_addr_layouts(cl, rows, cols):
     t = oracle.normal(80, rows * cols).reshape(rows, cols)
