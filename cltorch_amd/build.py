@@ -25,7 +25,7 @@ SOURCES = ["rt.cpp", "state.cpp", "tensor.cpp", "layout.cpp", "expr.cpp", "math.
 
 COMMON = ["-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function", "-Wno-unused-const-variable",
           "-I", os.path.join(ROOT, "include"), "-I", CSRC]
-# packed fp32 instructions stay off on this hardware pool
+# packed fp32 instructions stay out of the generated code
 DEVICE = [f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_ONLY = ["-x", "c++", "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include"]
 

@@ -346,7 +346,8 @@ static int rtc_compile(const char *source, const char *arch, std::vector<char> &
   }
   std::string archopt = std::string("--offload-arch=") + arch;
   // Contraction stays off so a*b+c rounds twice like the host arithmetic it is
-  // compared with; packed fp32 instructions are disabled on this hardware pool.
+  // compared with; packed fp32 instructions are kept out of the generated code,
+  // as in the library's own build.
   const char *opts[] = {archopt.c_str(), "-O3", "-ffp-contract=off", "-std=c++17",
                         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
   int nopts = (int)(sizeof(opts) / sizeof(opts[0]));
