@@ -409,6 +409,34 @@ float THClTensor_dot(THClState *state, THClTensor *self, THClTensor *src) {
   THCL_GUARD_END(0.f)
 }
 
+// dot of n elements at x[xoffset + i * incx] and y[yoffset + i * incy]; the two "wrappers" are what
+// storage->wrapper holds, device addresses of the storages' first elements
+// (src/lib/THClBlas.cpp:149-213, where they are the storages' buffer objects)
+float THClBlas_dot(THClState *state, long n, void *xwrapper, long xoffset, long incx, void *ywrapper, long yoffset,
+                   long incy) {
+  THCL_GUARD_BEGIN
+  if (n <= 0) return 0.f;
+  if (n == 1) incx = incy = 1;
+  THCL_CHECK(n <= INT32_MAX && incx <= INT32_MAX && incy <= INT32_MAX,
+             "dot only supports n, incx and incy up to signed integer limits: %d", INT32_MAX);
+  THCL_CHECK(xwrapper && ywrapper && xoffset >= 0 && yoffset >= 0 && incx > 0 && incy > 0, "dot: invalid operand");
+  const int device = THClState_getDevice(state);
+  // borrowed views: storages that are not reference-counted and own nothing
+  THClStorage sx, sy;
+  memset(&sx, 0, sizeof(sx));
+  sx.device = device;
+  sx.cl = thcl_ctx(state, device);
+  sy = sx;
+  sx.wrapper = xwrapper;
+  sx.size = xoffset + (n - 1) * incx + 1;
+  sy.wrapper = ywrapper;
+  sy.size = yoffset + (n - 1) * incy + 1;
+  ThclTemp x(state, THClTensor_newWithStorage1d(state, device, &sx, xoffset, n, incx));
+  ThclTemp y(state, THClTensor_newWithStorage1d(state, device, &sy, yoffset, n, incy));
+  return THClTensor_dot(state, x.t, y.t);
+  THCL_GUARD_END(0.f)
+}
+
 // r_ = beta * t + alpha * mat * vec  (src/lib/THClTensorMathBlas.cpp:43-105)
 void THClTensor_addmv(THClState *state, THClTensor *r_, float beta, THClTensor *t, float alpha, THClTensor *mat,
                       THClTensor *vec) {

@@ -283,6 +283,30 @@ THClTensor *THClTensor_newWithStorage(THClState *state, int device, THClStorage 
   return t;
   THCL_GUARD_END(nullptr)
 }
+// sizes and strides spelled out, -1 from the first dimension that is not there
+// (src/lib/THClTensor.cpp:136-171)
+THClTensor *THClTensor_newWithStorage4d(THClState *state, int device, THClStorage *storage, long storageOffset, long size0,
+                                        long stride0, long size1, long stride1, long size2, long stride2, long size3,
+                                        long stride3) {
+  THCL_GUARD_BEGIN
+  long size[4] = {size0, size1, size2, size3}, stride[4] = {stride0, stride1, stride2, stride3};
+  THClTensor *t = header_new(device);
+  header_set(state, t, storage, storageOffset, 4, size, stride);
+  return t;
+  THCL_GUARD_END(nullptr)
+}
+THClTensor *THClTensor_newWithStorage1d(THClState *state, int device, THClStorage *storage, long storageOffset, long size0,
+                                        long stride0) {
+  return THClTensor_newWithStorage4d(state, device, storage, storageOffset, size0, stride0, -1, -1, -1, -1, -1, -1);
+}
+THClTensor *THClTensor_newWithStorage2d(THClState *state, int device, THClStorage *storage, long storageOffset, long size0,
+                                        long stride0, long size1, long stride1) {
+  return THClTensor_newWithStorage4d(state, device, storage, storageOffset, size0, stride0, size1, stride1, -1, -1, -1, -1);
+}
+THClTensor *THClTensor_newWithStorage3d(THClState *state, int device, THClStorage *storage, long storageOffset, long size0,
+                                        long stride0, long size1, long stride1, long size2, long stride2) {
+  return THClTensor_newWithStorage4d(state, device, storage, storageOffset, size0, stride0, size1, stride1, size2, stride2, -1, -1);
+}
 THClTensor *THClTensor_newWithSize(THClState *state, int device, THLongStorage *size, THLongStorage *stride) {
   return THClTensor_newWithStorage(state, device, nullptr, 0, size, stride);
 }
@@ -385,6 +409,27 @@ void THClTensor_setStorage(THClState *state, THClTensor *self, THClStorage *stor
   int nd = size ? (int)size->size : (stride ? (int)stride->size : 0);
   header_set(state, self, storage, storageOffset, nd, size ? size->data : nullptr, stride ? stride->data : nullptr);
   THCL_GUARD_END()
+}
+
+// (src/lib/THClTensor.cpp:342-386)
+void THClTensor_setStorage4d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset, long size0,
+                             long stride0, long size1, long stride1, long size2, long stride2, long size3, long stride3) {
+  THCL_GUARD_BEGIN
+  long size[4] = {size0, size1, size2, size3}, stride[4] = {stride0, stride1, stride2, stride3};
+  header_set(state, self, storage, storageOffset, 4, size, stride);
+  THCL_GUARD_END()
+}
+void THClTensor_setStorage1d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset, long size0,
+                             long stride0) {
+  THClTensor_setStorage4d(state, self, storage, storageOffset, size0, stride0, -1, -1, -1, -1, -1, -1);
+}
+void THClTensor_setStorage2d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset, long size0,
+                             long stride0, long size1, long stride1) {
+  THClTensor_setStorage4d(state, self, storage, storageOffset, size0, stride0, size1, stride1, -1, -1, -1, -1);
+}
+void THClTensor_setStorage3d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset, long size0,
+                             long stride0, long size1, long stride1, long size2, long stride2) {
+  THClTensor_setStorage4d(state, self, storage, storageOffset, size0, stride0, size1, stride1, size2, stride2, -1, -1);
 }
 
 void THClTensor_narrow(THClState *state, THClTensor *self, THClTensor *src, int dim, long first, long size) {

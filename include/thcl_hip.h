@@ -270,6 +270,16 @@ void *THClTensor_wrapper(THClState *state, const THClTensor *self);
 THClTensor *THClTensor_newWithTensor(THClState *state, THClTensor *tensor);
 THClTensor *THClTensor_newWithStorage(THClState *state, int device, THClStorage *storage, long storageOffset,
                                       THLongStorage *size, THLongStorage *stride);
+/* sizes and strides spelled out; -1 from the first dimension that is not there (src/lib/THClTensor.h:53-66) */
+THClTensor *THClTensor_newWithStorage1d(THClState *state, int device, THClStorage *storage, long storageOffset,
+                                        long size0, long stride0);
+THClTensor *THClTensor_newWithStorage2d(THClState *state, int device, THClStorage *storage, long storageOffset,
+                                        long size0, long stride0, long size1, long stride1);
+THClTensor *THClTensor_newWithStorage3d(THClState *state, int device, THClStorage *storage, long storageOffset,
+                                        long size0, long stride0, long size1, long stride1, long size2, long stride2);
+THClTensor *THClTensor_newWithStorage4d(THClState *state, int device, THClStorage *storage, long storageOffset,
+                                        long size0, long stride0, long size1, long stride1, long size2, long stride2,
+                                        long size3, long stride3);
 THClTensor *THClTensor_newWithSize(THClState *state, int device, THLongStorage *size, THLongStorage *stride);
 THClTensor *THClTensor_newWithSize1d(THClState *state, int device, long size0);
 THClTensor *THClTensor_newWithSize2d(THClState *state, int device, long size0, long size1);
@@ -301,6 +311,16 @@ void THClTensor_resize4d(THClState *state, THClTensor *self, long size0, long si
 void THClTensor_set(THClState *state, THClTensor *self, THClTensor *src);
 void THClTensor_setStorage(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset,
                            THLongStorage *size, THLongStorage *stride);
+/* (src/lib/THClTensor.h:93-106) */
+void THClTensor_setStorage1d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset,
+                             long size0, long stride0);
+void THClTensor_setStorage2d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset,
+                             long size0, long stride0, long size1, long stride1);
+void THClTensor_setStorage3d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset,
+                             long size0, long stride0, long size1, long stride1, long size2, long stride2);
+void THClTensor_setStorage4d(THClState *state, THClTensor *self, THClStorage *storage, long storageOffset,
+                             long size0, long stride0, long size1, long stride1, long size2, long stride2,
+                             long size3, long stride3);
 void THClTensor_narrow(THClState *state, THClTensor *self, THClTensor *src, int dimension, long firstIndex, long size);
 void THClTensor_select(THClState *state, THClTensor *self, THClTensor *src, int dimension, long sliceIndex);
 void THClTensor_transpose(THClState *state, THClTensor *self, THClTensor *src, int dimension1, int dimension2);
@@ -499,6 +519,10 @@ void THClTensor_addmv(THClState *state, THClTensor *self, float beta, THClTensor
                       THClTensor *vec);
 void THClTensor_addr(THClState *state, THClTensor *self, float beta, THClTensor *t, float alpha, THClTensor *vec1,
                      THClTensor *vec2);
+/* (src/lib/THClBlas.h:21-23) xwrapper / ywrapper: what storage->wrapper holds, the device address of the
+ * storage's first element; offsets and increments in elements */
+float THClBlas_dot(THClState *state, long n, void *xwrapper, long xoffset, long incx, void *ywrapper, long yoffset,
+                   long incy);
 void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, THClTensor *a, long lda, THClTensor *x,
                    long incx, float beta, THClTensor *y, long incy);
 void THClBlas_ger(THClState *state, long m, long n, float alpha, THClTensor *x, long incx, THClTensor *y, long incy,

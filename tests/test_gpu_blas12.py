@@ -47,6 +47,26 @@ def test_dot_lengths_and_views(cl, n):
         cl.ClTensor(a).dot(cl.ClTensor(n + 1))
 
 
+def test_blas_dot_on_storage_addresses(cl):
+    """THClBlas_dot takes what storage->wrapper holds plus an offset and an increment per operand
+    (src/lib/THClBlas.cpp:149-213)."""
+    import ctypes as C
+    lib, st = cl.state().lib, cl.state().ptr
+    lib.THClBlas_dot.restype = C.c_float
+    lib.THClTensor_wrapper.restype = C.c_void_p
+    a, b = oracle.uniform(86, 5000), oracle.uniform(87, 5000)
+    A, B = cl.ClTensor(a), cl.ClTensor(b)
+    wa, wb = C.c_void_p(lib.THClTensor_wrapper(st, A._h)), C.c_void_p(lib.THClTensor_wrapper(st, B._h))
+    L = C.c_long
+    for n, xo, ix, yo, iy in ((5000, 0, 1, 0, 1), (1000, 3, 2, 7, 4), (1, 4999, 9, 4999, 9), (0, 0, 1, 0, 1)):
+        got = lib.THClBlas_dot(st, L(n), wa, L(xo), L(ix), wb, L(yo), L(iy))
+        cl.state().check()
+        if n == 1:
+            ix = iy = 1
+        want = float(cat.dot(a[xo:xo + n * ix:ix], b[yo:yo + n * iy:iy])) if n else 0.0
+        assert abs(got - want) <= 1e-5 * max(abs(want), 1e-2), (n, xo, ix, yo, iy, got, want)
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 1), (2, 3), (7, 130), (130, 7), (64, 64), (300, 1000), (1000, 300), (4096, 33),
                                        (33, 4096), (5, 70000), (70000, 5), (2048, 2048)])
 def test_addmv_layouts(cl, rows, cols):

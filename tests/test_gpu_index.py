@@ -247,6 +247,51 @@ def test_header_and_storage_interface_extras(cl):
         assert out.tolist() == list(range(10)), name
 
 
+def test_views_over_a_storage_with_sizes_spelled_out(cl):
+    """newWithStorage1d..4d and setStorage1d..4d: sizes and strides as plain arguments, -1 for the
+    dimensions that are not there and for strides to be derived (src/lib/THClTensor.cpp:136-171,342-386)."""
+    import ctypes as C
+    from cltorch_amd.tensor import _call
+    lib, st = cl.state().lib, cl.state().ptr
+    base = cl.ClTensor(np.arange(24, dtype=F))
+    storage = C.c_void_p(lib.THClTensor_storage(st, base._h))
+    L = C.c_long
+    for name in ("THClTensor_newWithStorage1d", "THClTensor_newWithStorage2d", "THClTensor_newWithStorage3d", "THClTensor_newWithStorage4d"):
+        getattr(lib, name).restype = C.c_void_p
+    host = np.arange(24, dtype=F)
+
+    def view(handle):
+        t = cl.ClTensor()
+        _call("THClTensor_set", t._h, C.c_void_p(handle))
+        lib.THClTensor_free(st, C.c_void_p(handle))
+        return t
+
+    v1 = view(lib.THClTensor_newWithStorage1d(st, C.c_int(0), storage, L(2), L(5), L(4)))
+    assert v1.size() == (5,) and v1.stride() == (4,) and v1.float().tolist() == host[2::4][:5].tolist()
+    v2 = view(lib.THClTensor_newWithStorage2d(st, C.c_int(0), storage, L(0), L(4), L(6), L(6), L(1)))
+    assert v2.size() == (4, 6) and np.array_equal(v2.float(), host.reshape(4, 6))
+    v2t = view(lib.THClTensor_newWithStorage2d(st, C.c_int(0), storage, L(0), L(6), L(1), L(4), L(6)))
+    assert np.array_equal(v2t.float(), host.reshape(4, 6).T)
+    v3 = view(lib.THClTensor_newWithStorage3d(st, C.c_int(0), storage, L(0), L(2), L(-1), L(3), L(-1), L(4), L(-1)))
+    assert v3.size() == (2, 3, 4) and v3.stride() == (12, 4, 1) and np.array_equal(v3.float(), host.reshape(2, 3, 4))
+    v4 = view(lib.THClTensor_newWithStorage4d(st, C.c_int(0), storage, L(0), L(2), L(12), L(2), L(6), L(3), L(2), L(2), L(1)))
+    assert v4.size() == (2, 2, 3, 2) and np.array_equal(v4.float(), host.reshape(2, 2, 3, 2))
+    assert v4.sum() == float(host.sum())                      # kernels see the same elements
+    t = cl.ClTensor()
+    _call("THClTensor_setStorage1d", t._h, storage, L(20), L(4), L(1))
+    assert t.float().tolist() == [20.0, 21.0, 22.0, 23.0]
+    _call("THClTensor_setStorage2d", t._h, storage, L(1), L(3), L(8), L(2), L(3))
+    assert np.array_equal(t.float(), np.array([[1, 4], [9, 12], [17, 20]], dtype=F))
+    _call("THClTensor_setStorage3d", t._h, storage, L(0), L(2), L(12), L(2), L(6), L(6), L(1))
+    assert np.array_equal(t.float(), host.reshape(2, 2, 6))
+    _call("THClTensor_setStorage4d", t._h, storage, L(0), L(1), L(-1), L(2), L(-1), L(3), L(-1), L(4), L(-1))
+    assert t.size() == (1, 2, 3, 4) and t.isContiguous()
+    t.fill(-1.0)                                              # the view writes through to the shared storage
+    assert base.float().tolist() == [-1.0] * 24
+    with pytest.raises(cl.ClError):
+        _call("THClTensor_setStorage1d", t._h, storage, L(-1), L(4), L(1))
+
+
 def test_current_device_forms(cl):
     """The forms without a device argument act on the current device
     (src/lib/THClGeneral.cpp:119-133,178-185, src/lib/THClTensor.cpp:66-72,92-95,844-902,
