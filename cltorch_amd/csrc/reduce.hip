@@ -365,6 +365,7 @@ struct ReduceDimParams {
   thcl_u32 split;        // blocks sharing one slice's reduction (column kernel)
   thcl_u32 fused;        // split > 1: the last block of a tile folds its partials (else a second kernel does)
   thcl_u32 rows_per_split;
+  thcl_u32 ub_log2;      // column kernel: a wave spans 2^ub_log2 units side by side and 64 >> ub_log2 rows
   float exponent;        // p of the |x|^p sum
   ThclGenericOperand L;  // layout of the slice starts (the view without `dim`)
 };
@@ -413,7 +414,8 @@ struct Slot<KIND, true> {
 };
 
 // Reduced dim is dense in memory: LPR lanes walk one slice, VEC floats each.
-// LPR in {8, 64, 256}; a block holds 256/LPR slices.
+// LPR in {1, 8, 64, 256}; a block holds 256/LPR slices.  blockIdx.y cuts long slices
+// into pieces of rows_per_split elements (a multiple of 4) that leave partials.
 template <int KIND, bool ARG, int LPR, int VEC>
 __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
   typedef Slot<KIND, ARG> S;
@@ -422,14 +424,16 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
   __shared__ T lds[kThreads / kWave];
   const int sub = threadIdx.x % LPR, row_in_block = threadIdx.x / LPR;
   const thcl_u32 ngroups = (P.nslices + ROWS - 1) / ROWS;
+  const thcl_u32 r0 = blockIdx.y * P.rows_per_split;
+  const thcl_u32 len = (P.R - r0 < P.rows_per_split) ? (P.R - r0) : P.rows_per_split;
   for (thcl_u32 g = blockIdx.x; g < ngroups; g += gridDim.x) {
     const thcl_u32 s = g * ROWS + row_in_block;
     T acc = S::init();
     if (s < P.nslices) {
-      const float *row = P.in + thcl_generic_offset(s, P.L);
+      const float *row = P.in + thcl_generic_offset(s, P.L) + r0;
       if (VEC == 4) {
         const thcl_f4 *row4 = (const thcl_f4 *)row;
-        const thcl_u32 r4 = P.R >> 2;
+        const thcl_u32 r4 = len >> 2;
         constexpr int FLY = 4;  // independent loads issued before any is consumed
         thcl_u32 i = sub;
         for (; i + (FLY - 1) * LPR < r4; i += FLY * LPR) {
@@ -439,31 +443,34 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
 #pragma unroll
           for (int f = 0; f < FLY; f++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) acc = S::take(acc, v[f][c], (int)((i + f * LPR) * 4 + c), P.exponent);
+            for (int c = 0; c < 4; c++) acc = S::take(acc, v[f][c], (int)(r0 + (i + f * LPR) * 4 + c), P.exponent);
         }
         for (; i < r4; i += LPR) {
           const thcl_f4 v = __builtin_nontemporal_load(row4 + i);
 #pragma unroll
-          for (int c = 0; c < 4; c++) acc = S::take(acc, v[c], (int)(i * 4 + c), P.exponent);
+          for (int c = 0; c < 4; c++) acc = S::take(acc, v[c], (int)(r0 + i * 4 + c), P.exponent);
         }
       } else {
         constexpr int FLY = 4;
         thcl_u32 i = sub;
-        for (; i + (FLY - 1) * LPR < P.R; i += FLY * LPR) {
+        for (; i + (FLY - 1) * LPR < len; i += FLY * LPR) {
           float v[FLY];
 #pragma unroll
           for (int f = 0; f < FLY; f++) v[f] = row[i + f * LPR];
 #pragma unroll
-          for (int f = 0; f < FLY; f++) acc = S::take(acc, v[f], (int)(i + f * LPR), P.exponent);
+          for (int f = 0; f < FLY; f++) acc = S::take(acc, v[f], (int)(r0 + i + f * LPR), P.exponent);
         }
-        for (; i < P.R; i += LPR) acc = S::take(acc, row[i], (int)i, P.exponent);
+        for (; i < len; i += LPR) acc = S::take(acc, row[i], (int)(r0 + i), P.exponent);
       }
       // the first position this thread met
-      acc = S::seal(acc, (int)(VEC == 4 ? sub * 4 : sub), (VEC == 4 ? (thcl_u32)sub < (P.R >> 2) : (thcl_u32)sub < P.R));
+      acc = S::seal(acc, (int)(r0 + (VEC == 4 ? sub * 4 : sub)), (VEC == 4 ? (thcl_u32)sub < (len >> 2) : (thcl_u32)sub < len));
     }
     if (LPR <= kWave) {
       acc = S::reduce(acc, LPR);
-      if (sub == 0 && s < P.nslices) S::store(P, s, acc);
+      if (sub == 0 && s < P.nslices) {
+        if (P.split > 1) ((T *)P.partials)[(thcl_u64)blockIdx.y * P.nslices + s] = acc;
+        else S::store(P, s, acc);
+      }
     } else {
       acc = S::reduce(acc, kWave);
       const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -473,14 +480,16 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
       if (threadIdx.x == 0) {
         T r = lds[0];
         for (int w = 1; w < kThreads / kWave; w++) r = S::comb(r, lds[w]);
-        S::store(P, s, r);
+        if (P.split > 1) ((T *)P.partials)[(thcl_u64)blockIdx.y * P.nslices + s] = r;
+        else S::store(P, s, r);
       }
     }
   }
 }
 
-// Reduced dim is strided: lanes lie along the slices (64 lanes x VEC adjacent
-// slices), the 4 waves of a block interleave over the reduced dim and meet in
+// Reduced dim is strided: lanes lie along the slices (UB lanes x VEC adjacent
+// slices; UB = 64 unless the slices are fewer, then the wave's other lanes take
+// further rows), the 4 waves of a block interleave over the reduced dim and meet in
 // LDS; blockIdx.y splits long reductions, leaving partials for the finisher.
 template <int KIND, bool ARG, int VEC>
 __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
@@ -489,12 +498,15 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
   constexpr int WAVES = kThreads / kWave;
   __shared__ T lds[WAVES][kWave * VEC];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const thcl_u32 ntiles = (P.nunits + kWave - 1) / kWave;
+  const thcl_u32 UB = 1u << P.ub_log2, RL = kWave >> P.ub_log2;  // units and rows across a wave
+  const thcl_u32 ul = lane & (UB - 1), rl = lane >> P.ub_log2;
+  const thcl_u32 ntiles = (P.nunits + UB - 1) / UB;
   const thcl_u32 r_begin = blockIdx.y * P.rows_per_split;
   thcl_u32 r_end = r_begin + P.rows_per_split;
   if (r_end > P.R) r_end = P.R;
+  const thcl_u32 RSTEP = WAVES * RL;  // rows between a lane's consecutive elements
   for (thcl_u32 tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-    const thcl_u32 u = tile * kWave + lane;
+    const thcl_u32 u = tile * UB + ul;
     T acc[VEC];
 #pragma unroll
     for (int c = 0; c < VEC; c++) acc[c] = S::init();
@@ -515,13 +527,13 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
       // this wave takes rows r_begin + wave, + WAVES, ...; FLY of them are loaded
       // before any is consumed, the address advances by a constant step
       constexpr int FLY = 8;
-      thcl_u32 r = r_begin + wave;
+      thcl_u32 r = r_begin + wave * RL + rl;
       const float *ptr = P.in + off + (thcl_u64)r * P.rstride;
-      const thcl_u64 step = (thcl_u64)WAVES * P.rstride;
+      const thcl_u64 step = (thcl_u64)RSTEP * P.rstride;
       if (VEC == 4) {
         // whole batches of FLY rows: the next batch is requested before the current one
         // is consumed, so the wave always has loads in flight
-        if (r + (FLY - 1) * WAVES < r_end) {
+        if (r + (FLY - 1) * RSTEP < r_end) {
           thcl_f4 v[FLY], w[FLY];
           auto fetch = [&](thcl_f4 (&x)[FLY]) {
 #pragma unroll
@@ -534,18 +546,18 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
 #pragma unroll
             for (int f = 0; f < FLY; f++)
 #pragma unroll
-              for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], x[f][c], (int)(r + f * WAVES), P.exponent);
-            r += FLY * WAVES;
+              for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], x[f][c], (int)(r + f * RSTEP), P.exponent);
+            r += FLY * RSTEP;
           };
           fetch(v);
           // two batches per turn, each requested while the other is consumed
-          while (r + (3 * FLY - 1) * WAVES < r_end) {
+          while (r + (3 * FLY - 1) * RSTEP < r_end) {
             fetch(w);
             consume(v);
             fetch(v);
             consume(w);
           }
-          if (r + (2 * FLY - 1) * WAVES < r_end) {
+          if (r + (2 * FLY - 1) * RSTEP < r_end) {
             fetch(w);
             consume(v);
             consume(w);
@@ -554,7 +566,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
           }
         }
       } else {
-        for (; r + (FLY - 1) * WAVES < r_end; r += FLY * WAVES) {
+        for (; r + (FLY - 1) * RSTEP < r_end; r += FLY * RSTEP) {
           float v[FLY];
 #pragma unroll
           for (int f = 0; f < FLY; f++) {
@@ -562,10 +574,10 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
             ptr += step;
           }
 #pragma unroll
-          for (int f = 0; f < FLY; f++) acc[0] = S::take(acc[0], v[f], (int)(r + f * WAVES), P.exponent);
+          for (int f = 0; f < FLY; f++) acc[0] = S::take(acc[0], v[f], (int)(r + f * RSTEP), P.exponent);
         }
       }
-      for (; r < r_end; r += WAVES) {
+      for (; r < r_end; r += RSTEP) {
         if (VEC == 4) {
           const thcl_f4 v0 = *(const thcl_f4 *)ptr;
 #pragma unroll
@@ -576,17 +588,25 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
         ptr += step;
       }
 #pragma unroll
-      for (int c = 0; c < VEC; c++) acc[c] = S::seal(acc[c], (int)(r_begin + wave), r_begin + wave < r_end);
+      for (int c = 0; c < VEC; c++)
+        acc[c] = S::seal(acc[c], (int)(r_begin + wave * RL + rl), r_begin + wave * RL + rl < r_end);
+    }
+    // the wave's row lanes of one unit meet first (lanes UB apart)
+    for (thcl_u32 m = UB; m < (thcl_u32)kWave; m <<= 1) {
+#pragma unroll
+      for (int c = 0; c < VEC; c++) acc[c] = S::comb(acc[c], shfl_xor_t(acc[c], (int)m));
     }
     __syncthreads();
+    if (rl == 0) {
 #pragma unroll
-    for (int c = 0; c < VEC; c++) lds[wave][lane * VEC + c] = acc[c];
+      for (int c = 0; c < VEC; c++) lds[wave][ul * VEC + c] = acc[c];
+    }
     __syncthreads();
-    if (wave == 0 && u < P.nunits) {
+    if (wave == 0 && rl == 0 && u < P.nunits) {
 #pragma unroll
       for (int c = 0; c < VEC; c++) {
-        T r = lds[0][lane * VEC + c];
-        for (int w = 1; w < WAVES; w++) r = S::comb(r, lds[w][lane * VEC + c]);
+        T r = lds[0][ul * VEC + c];
+        for (int w = 1; w < WAVES; w++) r = S::comb(r, lds[w][ul * VEC + c]);
         const thcl_u32 s = u * VEC + c;
         if (P.split > 1) store_shared((T *)P.partials + (thcl_u64)blockIdx.y * P.nslices + s, r);
         else S::store(P, s, r);
@@ -610,8 +630,8 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
   __syncthreads();
   if (!s_last) return;
   const T *partials = (const T *)P.partials;
-  for (thcl_u32 j = threadIdx.x; j < kWave * VEC; j += kThreads) {
-    const thcl_u32 s = blockIdx.x * (kWave * VEC) + j;
+  for (thcl_u32 j = threadIdx.x; j < UB * VEC; j += kThreads) {
+    const thcl_u32 s = blockIdx.x * (UB * VEC) + j;
     if (s < P.nslices) {
       T t = S::init();
       thcl_u32 k = 0;
@@ -628,6 +648,61 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
     }
   }
   if (threadIdx.x == 0) P.ticket[blockIdx.x] = 0u;
+}
+
+// Reduced dim is strided and short (R <= 32): a thread owns a unit of VEC adjacent slices and
+// walks all of R itself, 4 rows requested at a time; adjacent threads read adjacent units.
+template <int KIND, bool ARG, int VEC>
+__global__ __launch_bounds__(kThreads) void reduce_cols_short(ReduceDimParams P) {
+  typedef Slot<KIND, ARG> S;
+  typedef typename S::T T;
+  for (thcl_u32 u = blockIdx.x * kThreads + threadIdx.x; u < P.nunits; u += gridDim.x * kThreads) {
+    thcl_u64 off = 0;
+    {
+      thcl_u32 i = u;
+      for (int d = P.L.dims - 1; d > 0; d--) {
+        const thcl_u32 q = thcl_div(i, P.L.size[d]);
+        const thcl_u32 r = i - q * P.L.size[d].d;
+        off += (thcl_u64)((d == P.L.dims - 1) ? r * VEC : r) * P.L.stride[d];
+        i = q;
+      }
+      off += (thcl_u64)((P.L.dims == 1) ? i * VEC : i) * P.L.stride[0];
+    }
+    const float *ptr = P.in + off;
+    T acc[VEC];
+#pragma unroll
+    for (int c = 0; c < VEC; c++) acc[c] = S::init();
+    constexpr int FLY = 4;
+    thcl_u32 r = 0;
+    for (; r + FLY <= P.R; r += FLY) {
+      float x[FLY][VEC];
+#pragma unroll
+      for (int f = 0; f < FLY; f++) {
+        if (VEC == 4) {
+          const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(ptr + (thcl_u64)(r + f) * P.rstride));
+#pragma unroll
+          for (int c = 0; c < VEC; c++) x[f][c] = v[c];
+        } else {
+          x[f][0] = ptr[(thcl_u64)(r + f) * P.rstride];
+        }
+      }
+#pragma unroll
+      for (int f = 0; f < FLY; f++)
+#pragma unroll
+        for (int c = 0; c < VEC; c++) acc[c] = S::take(acc[c], x[f][c], (int)(r + f), P.exponent);
+    }
+    for (; r < P.R; r++) {
+      if (VEC == 4) {
+        const thcl_f4 v = *(const thcl_f4 *)(ptr + (thcl_u64)r * P.rstride);
+#pragma unroll
+        for (int c = 0; c < VEC; c++) acc[c] = S::take(acc[c], v[c], (int)r, P.exponent);
+      } else {
+        acc[0] = S::take(acc[0], ptr[(thcl_u64)r * P.rstride], (int)r, P.exponent);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < VEC; c++) S::store(P, u * VEC + c, S::seal(acc[c], 0, P.R > 0));
+  }
 }
 
 // Folds the [split][nslices] partials.  A block owns 16 adjacent slices; its 16
@@ -695,9 +770,12 @@ void launch_dim(bool rows, int lpr, int vec, dim3 grid, hipStream_t stream, cons
   if (rows) {
 #define ROWS_CASE(L, V) \
   if (lpr == L && vec == V) { hipLaunchKernelGGL((reduce_rows<KIND, ARG, L, V>), grid, block, 0, stream, P); return; }
-    ROWS_CASE(8, 1) ROWS_CASE(8, 4) ROWS_CASE(64, 1) ROWS_CASE(64, 4) ROWS_CASE(256, 1) ROWS_CASE(256, 4)
+    ROWS_CASE(1, 1) ROWS_CASE(1, 4) ROWS_CASE(8, 1) ROWS_CASE(8, 4) ROWS_CASE(64, 1) ROWS_CASE(64, 4) ROWS_CASE(256, 1) ROWS_CASE(256, 4)
 #undef ROWS_CASE
     thcl_throw("internal: no row-reduction kernel for lanes=%d vec=%d", lpr, vec);
+  } else if (lpr < 0) {  // short reduced dim: a thread per unit
+    if (vec == 4) hipLaunchKernelGGL((reduce_cols_short<KIND, ARG, 4>), grid, block, 0, stream, P);
+    else hipLaunchKernelGGL((reduce_cols_short<KIND, ARG, 1>), grid, block, 0, stream, P);
   } else {
     if (vec == 4) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 4>), grid, block, 0, stream, P);
     else hipLaunchKernelGGL((reduce_cols<KIND, ARG, 1>), grid, block, 0, stream, P);
@@ -828,6 +906,12 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   const long R = src->size[dim];
   THCL_CHECK(nslices < (1l << 31) && R < (1l << 31), THCL_DIM_WARNING);
   THCL_CHECK(thcl_fits_32bit(src), THCL_DIM_WARNING);
+  // a dimension of size 1: every slice is its one element, at position 1
+  if (R == 1 && idx_i64_dev == nullptr && (kind == RED_SUM || kind == RED_PROD || kind == RED_MAX || kind == RED_MIN)) {
+    THClTensor_copy(state, values, src);
+    if (indices_f32) THClTensor_fill(state, indices_f32, 1.0f);
+    return;
+  }
 
   // kernels write dense outputs; strided destinations get a dense stand-in
   THClTensor *vdense = values, *idense = indices_f32;
@@ -867,12 +951,29 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   int lpr = 0, vec = 1;
   dim3 grid(1, 1, 1);
   if (rows) {
-    lpr = R >= 2048 ? 256 : (R >= 128 ? 64 : 8);
+    // lanes per slice: a whole block for long slices, a thread for the shortest ones
+    lpr = R >= 2048 ? 256 : (R >= 128 ? 64 : (R > 16 ? 8 : 1));
     bool v4 = (R % 4 == 0) && aligned16(P.in);
     for (int d = 0; d < L.dims && v4; d++) v4 = (L.strides[d] % 4 == 0) || L.sizes[d] == 1;
     vec = v4 ? 4 : 1;
     const long groups = (nslices + (kThreads / lpr) - 1) / (kThreads / lpr);
     grid.x = (unsigned)(groups > (1l << 22) ? (1l << 22) : groups);
+    // few long slices: cut them into pieces of at least 8192 elements until the chip is full
+    if (lpr == 256 && groups < (long)cus * 4) {
+      long split = ((long)cus * 8 + groups - 1) / groups;
+      if (split > R / 8192) split = R / 8192;
+      if (split > 1024) split = 1024;
+      if (split * nslices > partial_cap) split = partial_cap / nslices;
+      if (split > 1) {
+        long rps = ((R + split - 1) / split + 1023) / 1024 * 1024;  // whole passes of the block's 256 x 4 elements
+        split = (R + rps - 1) / rps;
+        if (split > 1) {
+          P.split = (thcl_u32)split;
+          P.rows_per_split = (thcl_u32)rps;
+          grid.y = (unsigned)split;
+        }
+      }
+    }
   } else {
     const int last = L.dims - 1;
     bool v4 = L.strides[last] == 1 && (L.sizes[last] % 4 == 0) && (src->stride[dim] % 4 == 0) && aligned16(P.in);
@@ -880,13 +981,24 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     vec = v4 ? 4 : 1;
     if (v4) P.L.size[last] = thcl_make_divisor(L.sizes[last] / 4);
     P.nunits = (thcl_u32)(nslices / vec);
-    const long tiles = (P.nunits + kWave - 1) / kWave;
+    // a short reduced dim with enough slices to fill the chip: a thread per unit, no exchange
+    if (R <= 32 && (long)P.nunits >= (long)cus * 1024) {
+      lpr = -1;
+      const long blocks = ((long)P.nunits + kThreads - 1) / kThreads;
+      grid.x = (unsigned)(blocks > (1l << 22) ? (1l << 22) : blocks);
+    } else {
+    // fewer units than lanes: the wave's spare lanes take further rows
+    unsigned ub_log2 = 6;
+    while (ub_log2 > 0 && (1u << (ub_log2 - 1)) >= P.nunits) ub_log2--;
+    P.ub_log2 = ub_log2;
+    const long ub = 1l << ub_log2, row_lanes = kWave >> ub_log2;
+    const long tiles = (P.nunits + ub - 1) / ub;
     // enough blocks to fill the chip: split the reduced dim when slices are few
     long split = 1;
     const long target = (long)cus * 4;
     if (tiles < target) {
       split = (target + tiles - 1) / tiles;
-      const long max_by_rows = (R + 31) / 32;  // at least 32 rows per block
+      const long max_by_rows = (R + 32 * row_lanes - 1) / (32 * row_lanes);  // at least 32 rows per lane
       if (split > max_by_rows) split = max_by_rows;
       if (split > 256) split = 256;
       if (split * nslices > partial_cap) split = partial_cap / nslices;
@@ -901,13 +1013,14 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     P.fused = (split > 1 && split <= 32 && tiles <= (long)kColTickets) ? 1u : 0u;
     grid.x = (unsigned)(tiles > (1l << 20) ? (1l << 20) : tiles);
     grid.y = (unsigned)split;
+    }
   }
 
 #define DISPATCH(K)                                                       \
   if (arg) launch_dim<K, true>(rows, lpr, vec, grid, stream, P);          \
   else launch_dim<K, false>(rows, lpr, vec, grid, stream, P);             \
   check_launch("reduce-dim");                                             \
-  if (!rows && P.split > 1 && !P.fused) {                                 \
+  if (P.split > 1 && !P.fused) {                                          \
     unsigned fg = (unsigned)((nslices + kFinSlices - 1) / kFinSlices);    \
     if (arg) launch_finish<K, true>(fg, stream, P);                       \
     else launch_finish<K, false>(fg, stream, P);                          \
@@ -916,7 +1029,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
 #define DISPATCH_VALUES(K)                                                \
   launch_dim<K, false>(rows, lpr, vec, grid, stream, P);                  \
   check_launch("reduce-dim");                                             \
-  if (!rows && P.split > 1 && !P.fused) {                                 \
+  if (P.split > 1 && !P.fused) {                                          \
     unsigned fg = (unsigned)((nslices + kFinSlices - 1) / kFinSlices);    \
     launch_finish<K, false>(fg, stream, P);                               \
     check_launch("reduce-dim finish");                                    \

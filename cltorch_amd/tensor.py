@@ -821,19 +821,23 @@ class ClTensor:
             return self
         raise ClError(f"invalid arguments to {name}")
 
-    def sum(self, *args):
+    def _along(self, name: str, args):
+        """``a:sum(dim)`` -> new tensor; ``res:sum(a, dim)`` -> res (the result slot first, as the wrapper
+        table orders them: ``src/TensorMath.lua:943-953``); anything else is a whole-tensor form."""
         if len(args) == 1 and not isinstance(args[0], ClTensor):
             res = ClTensor()
-            _call("THClTensor_sum", res._h, self._h, C.c_long(args[0] - 1))
+            _call(f"THClTensor_{name}", res._h, self._h, C.c_long(args[0] - 1))
             return res
-        return self._reduce("sum", args)
+        if len(args) == 2 and isinstance(args[0], ClTensor) and not isinstance(args[1], ClTensor):
+            _call(f"THClTensor_{name}", self._h, args[0]._h, C.c_long(args[1] - 1))
+            return self
+        return self._reduce(name, args)
+
+    def sum(self, *args):
+        return self._along("sum", args)
 
     def prod(self, *args):
-        if len(args) == 1 and not isinstance(args[0], ClTensor):
-            res = ClTensor()
-            _call("THClTensor_prod", res._h, self._h, C.c_long(args[0] - 1))
-            return res
-        return self._reduce("prod", args)
+        return self._along("prod", args)
 
     def _scan(self, name: str, args):
         """``a:cumsum()`` / ``a:cumsum(dim)`` -> new tensor (dim defaults to 1); ``res:cumsum(a, dim)``
@@ -855,6 +859,9 @@ class ClTensor:
         """``a:mean()`` -> number, ``a:mean(dim)`` -> new tensor (``src/TensorMath.lua:1104-1111``)."""
         if len(args) == 0:
             return float(_call("THClTensor_meanall", self._h))
+        if len(args) == 2:                                    # res:mean(a, dim)
+            _call("THClTensor_mean", self._h, args[0]._h, C.c_long(args[1] - 1))
+            return self
         res = ClTensor()
         _call("THClTensor_mean", res._h, self._h, C.c_long(args[0] - 1))
         return res

@@ -120,7 +120,11 @@ def _check_dim(cl, pair, dim0):
 
 
 @pytest.mark.parametrize("shape", [(5, 2), (60, 50), (3, 2000), (2000, 3), (7, 128), (129, 64), (33, 4096), (4096, 33),
-                                   (17, 9, 13), (4, 300, 8), (2, 3, 4, 5), (1, 77), (77, 1), (256, 2048)])
+                                   (17, 9, 13), (4, 300, 8), (2, 3, 4, 5), (1, 77), (77, 1), (256, 2048),
+                                   # few long slices (cut into pieces over blocks), slices of 1..16 elements (a thread each),
+                                   # fewer than 64 column units (a wave's spare lanes take further rows)
+                                   (1, 1 << 20), (3, 300001), (5, 1 << 18), (1 << 20, 1), (300000, 3), (1 << 18, 4), (70000, 16),
+                                   (100000, 12), (40000, 40), (2, 50000, 8), (3, 20000, 5), (70000, 100), (20000, 252)])
 def test_reduce_dim_shapes(cl, shape):
     x = oracle.normal(6, int(np.prod(shape))).reshape(shape)
     p = Pair.dense(cl, x)
