@@ -64,6 +64,17 @@ void THClTensor_addmm(THClState *state, THClTensor *r_, float beta, THClTensor *
     THClTensor_copy(state, r_, t);
   }
 
+  // a result with one column or one row is a matrix-vector product: bound by reading the matrix once,
+  // which the gemv kernels do at several times the rate of a 64-wide GEMM tile with one live line
+  if ((r_->size[0] == 1 || r_->size[1] == 1) && m1->size[1] > 0) {
+    const bool column = r_->size[1] == 1;
+    ThclTemp out(state, THClTensor_newSelect(state, r_, column ? 1 : 0, 0));
+    ThclTemp vec(state, column ? THClTensor_newSelect(state, m2, 1, 0) : THClTensor_newSelect(state, m1, 0, 0));
+    ThclTemp mat(state, column ? THClTensor_newWithTensor(state, m1) : THClTensor_newTranspose(state, m2, 0, 1));
+    THClTensor_addmv(state, out.t, beta, out.t, alpha, mat.t, vec.t);
+    return;
+  }
+
   // result layout decides whether the product is computed as is or transposed
   THClTensor *r = r_;
   int fast;

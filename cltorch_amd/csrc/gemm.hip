@@ -39,6 +39,8 @@ struct GemmParams {
   int ksplit;   // blockIdx.y slices of K; > 1: raw partial products go to `work`
   int kchunk;   // K per slice (multiple of BK)
   float *work;  // [ksplit][n][m] dense partials
+  // edge kernels: the operand's 16-byte groups along its contiguous dim are whole and aligned
+  int vec_a, vec_b, vec_c;
 };
 
 // One operand tile in LDS.  KC: contiguous along k in global memory.
@@ -54,7 +56,8 @@ struct TileLoader {
   f4 r[NV];
 
   // g: operand base; ld: leading dim; mn0: first row/col of the tile; k0: first k; lim_mn/lim_k: extents
-  __device__ __forceinline__ void load(const float *g, int ld, int mn0, int k0, int lim_mn, int lim_k) {
+  // vec (edge kernels): a 16-byte group is either inside the operand or outside, and aligned
+  __device__ __forceinline__ void load(const float *g, int ld, int mn0, int k0, int lim_mn, int lim_k, bool vec) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = threadIdx.x + 256 * p;
@@ -63,6 +66,10 @@ struct TileLoader {
         const float *src = g + (size_t)(mn0 + mn) * ld + k0 + kq * 4;
         if (!EDGE) {
           r[p] = *(const f4 *)src;
+        } else if (vec) {
+          const bool in = mn0 + mn < lim_mn && k0 + kq * 4 < lim_k;
+          const f4 v = *(const f4 *)(in ? src : g);
+          r[p] = in ? v : f4{0.f, 0.f, 0.f, 0.f};
         } else {
 #pragma unroll
           for (int c = 0; c < 4; c++)
@@ -73,6 +80,10 @@ struct TileLoader {
         const float *src = g + (size_t)(k0 + kk) * ld + mn0 + q * 4;
         if (!EDGE) {
           r[p] = *(const f4 *)src;
+        } else if (vec) {
+          const bool in = k0 + kk < lim_k && mn0 + q * 4 < lim_mn;
+          const f4 v = *(const f4 *)(in ? src : g);
+          r[p] = in ? v : f4{0.f, 0.f, 0.f, 0.f};
         } else {
 #pragma unroll
           for (int c = 0; c < 4; c++)
@@ -170,10 +181,11 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   TileLoader<BN, BKC, EDGE> lb1;
   const int last = KT > 0 ? KT - 1 : 0;
   auto slab_k = [&](int kt) { return k_begin + (kt < last ? kt : last) * BK; };
-  la.load(P.a, P.lda, m0, slab_k(0), P.m, k_end);
-  lb.load(P.b, P.ldb, n0, slab_k(0), P.n, k_end);
-  la1.load(P.a, P.lda, m0, slab_k(1), P.m, k_end);
-  lb1.load(P.b, P.ldb, n0, slab_k(1), P.n, k_end);
+  const bool va = P.vec_a != 0, vb = P.vec_b != 0;
+  la.load(P.a, P.lda, m0, slab_k(0), P.m, k_end, va);
+  lb.load(P.b, P.ldb, n0, slab_k(0), P.n, k_end, vb);
+  la1.load(P.a, P.lda, m0, slab_k(1), P.m, k_end, va);
+  lb1.load(P.b, P.ldb, n0, slab_k(1), P.n, k_end, vb);
   la.store(lds);
   lb.store(lds + AF);
   __syncthreads();
@@ -181,8 +193,8 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   auto step = [&](int kt, int cur, auto &issue_a, auto &issue_b, auto &keep_a, auto &keep_b) {
     float *As = lds + cur * (AF + BF);
     float *Bs = As + AF;
-    issue_a.load(P.a, P.lda, m0, slab_k(kt + 2), P.m, k_end);
-    issue_b.load(P.b, P.ldb, n0, slab_k(kt + 2), P.n, k_end);
+    issue_a.load(P.a, P.lda, m0, slab_k(kt + 2), P.m, k_end, va);
+    issue_b.load(P.b, P.ldb, n0, slab_k(kt + 2), P.n, k_end, vb);
     __builtin_amdgcn_sched_barrier(0);   // keep the loads at the top of the step
     {
 #pragma unroll
@@ -225,7 +237,7 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
         for (int rq = 0; rq < 4; rq++) {
           const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
           float *wp = w + (size_t)col * P.m + row;
-          if (!EDGE) {
+          if (!EDGE || (P.m % 4 == 0 && col < P.n && row < P.m)) {  // the partials are dense: pitch m, 16-byte aligned base
             f4 v;
 #pragma unroll
             for (int c = 0; c < 4; c++) v[c] = acc[i][j][rq * 4 + c];
@@ -248,7 +260,7 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
       for (int rq = 0; rq < 4; rq++) {
         const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
         float *cp = P.c + (size_t)col * P.ldc + row;
-        if (!EDGE) {
+        if (!EDGE || (P.vec_c && col < P.n && row < P.m)) {
           f4 v;
 #pragma unroll
           for (int c = 0; c < 4; c++) v[c] = P.alpha * acc[i][j][rq * 4 + c];
@@ -326,7 +338,7 @@ static void choose_ksplit(long tiles, long k, int cus, int &ksplit, int &kchunk)
   long want = (2L * cus + tiles - 1) / tiles;
   const long max_by_k = k / 256;  // at least 16 slabs per slice
   if (want > max_by_k) want = max_by_k;
-  if (want > 32) want = 32;
+  if (want > 512) want = 512;  // want * tiles stays near 2 * cus, so the partials stay near 2 * cus tiles
   if (want <= 1) return;
   const long chunk = ((k + want - 1) / want + BK - 1) / BK * BK;
   const long slices = (k + chunk - 1) / chunk;
@@ -370,6 +382,11 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   choose_tile(m, n, thcl_rt_get_props(rt)->compute_units, bm, bn);
   const bool fast = (m % bm == 0) && (n % bn == 0) && (k % BK == 0) && k > 0 && (lda % 4 == 0) && (ldb % 4 == 0) &&
                     (ldc % 4 == 0) && al16(a) && al16(b) && al16(c);
+  // an operand's contiguous dim is m for a 'n', k for a 't'; n for b 't', k for b 'n'
+  const long a_run = ta ? k : m, b_run = tb ? n : k;
+  P.vec_a = (lda % 4 == 0 && a_run % 4 == 0 && al16(a)) ? 1 : 0;
+  P.vec_b = (ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) ? 1 : 0;
+  P.vec_c = (ldc % 4 == 0 && m % 4 == 0 && al16(c)) ? 1 : 0;
   P.tiles_m = (int)((m + bm - 1) / bm);
   P.tiles_n = (int)((n + bn - 1) / bn);
   P.group_m = P.tiles_m < 8 ? P.tiles_m : 8;

@@ -305,7 +305,8 @@ def test_gemm_k_slicing(lib):
     assert plan(16384, 64, 4096) == (128, 64, 4, 1024)           # skinny: 128 tiles on 256 CUs
     assert plan(2048, 512, 4096) == (64, 64, 2, 2048)            # 256 tiles: one per CU, long K
     assert plan(1024, 1024, 1024) == (64, 64, 1, 1024)           # 256 tiles but K too short to pay for a second pass
-    assert plan(64, 64, 100000)[2] == 32                         # capped
+    assert plan(64, 64, 100000)[2] == 368                        # one tile: as many slices of at least 256 as fit
+    assert plan(32, 32, 1 << 20)[2] == 512                       # capped
     bm, bn, ks, kc = plan(128, 128, 1000)
     assert ks == 1 and kc == 1000
     for k in (1024, 1040, 3000, 5555):

@@ -52,7 +52,11 @@ def test_shapes_row_major(cl, M, N, K):
 @pytest.mark.parametrize("ta", [False, True])
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("tc", [False, True])
-@pytest.mark.parametrize("M,N,K", [(128, 256, 64), (70, 90, 50)])
+@pytest.mark.parametrize("M,N,K", [(128, 256, 64), (70, 90, 50),
+                                   # one row or one column: the matrix-vector kernels; ragged sizes: the edge kernels with
+                                   # and without whole 16-byte groups
+                                   (1, 3000, 700), (3000, 1, 700), (1, 1, 5000), (1, 64, 4096), (200, 1000, 300), (201, 999, 301),
+                                   (32, 32, 40000)])
 def test_every_operand_layout(cl, ta, tb, tc, M, N, K):
     """Each operand either dense or the transpose of a dense array: all
     'n'/'t' combinations of the gemm, with the result row- or column-major."""
