@@ -469,6 +469,13 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
   thcl_check_same_device(state, 2, self, src);
   THCL_ARGCHECK(src->nDimension > 0, 2, "cannot scan an empty tensor");
   THCL_ARGCHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
+  if (src->size[dim] == 1) {  // every line has one element: the scan is the source itself
+    if (self != src) {
+      THClTensor_resizeAs(state, self, src);
+      THClTensor_copy(state, self, src);
+    }
+    return;
+  }
   ThclTemp src_hold(state, THClTensor_newContiguous(state, src));  // before resizing self: they may be the same tensor
   THClTensor *srcc = src_hold.t;
   THClTensor_resizeAs(state, self, src);
