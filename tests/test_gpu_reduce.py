@@ -195,6 +195,37 @@ def test_positions_when_every_element_is_the_start_value(cl, shape):
             assert (wi == 1).sum() >= min(shape[1 - d], 2) - 2
 
 
+@pytest.mark.parametrize("shape,dim0", [((3, 200001), 1), ((200001, 3), 0), ((1, 1 << 19), 1), ((70, 40000), 1), ((40000, 70), 0)])
+def test_positions_on_long_slices_cut_over_blocks(cl, shape, dim0):
+    """Few long slices are reduced by many blocks whose partial (value, position) pairs are folded afterwards:
+    ties keep the lowest position and the first NaN wins, wherever the pieces' borders fall."""
+    rs = np.random.RandomState(41)
+    R = shape[dim0]
+    for mode in ("ties", "nan", "constant"):
+        if mode == "ties":
+            x = rs.randint(-3, 4, size=shape).astype(F)
+        elif mode == "nan":
+            x = rs.standard_normal(shape).astype(F)
+            for _ in range(4):
+                x[tuple(int(rs.randint(n)) for n in shape)] = np.nan
+        else:
+            x = np.full(shape, F(-1.25))
+        X = cl.ClTensor(x)
+        rows = np.moveaxis(x, dim0, -1).reshape(-1, R)
+        for kind in ("max", "min"):
+            want = np.empty(rows.shape[0], dtype=np.int64)
+            for k, row in enumerate(rows):
+                nans = np.isnan(row)
+                want[k] = int(np.argmax(nans)) if nans.any() else int(np.argmax(row) if kind == "max" else np.argmin(row))
+            vals, pos = getattr(X, kind)(dim0 + 1)
+            got = np.moveaxis(pos.long(), dim0, -1).reshape(-1) - 1
+            assert np.array_equal(got, want), (mode, kind)
+            got_v = np.moveaxis(vals.float(), dim0, -1).reshape(-1)
+            assert_bit_equal(got_v, rows[np.arange(rows.shape[0]), want], f"{mode} {kind} values")
+            _, pos64 = getattr(X, f"{kind}_long")(dim0 + 1)
+            assert np.array_equal(np.moveaxis(pos64, dim0, -1).reshape(-1) - 1, want)
+
+
 def test_results_into_existing_strided_tensors(cl):
     x = oracle.uniform(19, 40 * 24).reshape(40, 24)
     X = cl.ClTensor(x)
