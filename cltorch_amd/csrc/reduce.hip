@@ -305,7 +305,17 @@ __global__ __launch_bounds__(kThreads) void reduce_all_strided(ReduceAllParams P
   typedef typename Acc<KIND>::T T;
   __shared__ T lds[kThreads / kWave];
   T acc = Acc<KIND>::init();
-  for (thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x; i < P.n; i += (thcl_u64)gridDim.x * kThreads)
+  const thcl_u64 all = (thcl_u64)gridDim.x * kThreads;
+  thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x;
+  constexpr int FLY = 8;  // independent loads per thread and turn
+  for (; i + (FLY - 1) * all < P.n; i += FLY * all) {
+    float v[FLY];
+#pragma unroll
+    for (int k = 0; k < FLY; k++) v[k] = P.in[thcl_generic_offset((thcl_u32)(i + k * all), P.L)];
+#pragma unroll
+    for (int k = 0; k < FLY; k++) acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(v[k], P.exponent));
+  }
+  for (; i < P.n; i += all)
     acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(P.in[thcl_generic_offset((thcl_u32)i, P.L)], P.exponent));
   acc = block_reduce<KIND, T>(acc, lds);
   finish_all<KIND>(acc, P, lds);
@@ -813,17 +823,31 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
   P.ticket = (unsigned *)(scratch + kTicketOff);
   P.out = out;
   P.exponent = exponent;
-  const bool dense = THClTensor_isContiguous(state, src);
+  // The order in which elements are folded is free, so the view is walked in memory order: dims sorted
+  // by stride and merged.  A transposed or permuted view of a whole block of memory becomes dense.
+  Layout walk;
+  {
+    THClTensor *one[1] = {src};
+    const JointLayout J = thcl_joint_collapse(1, one);
+    walk.dims = J.dims;
+    for (int d = 0; d < J.dims; d++) {
+      walk.sizes[d] = J.sizes[d];
+      walk.strides[d] = J.strides[0][d];
+    }
+  }
+  const bool dense = walk.contiguous();
   const int cus = thcl_rt_get_props(rt)->compute_units;
   long want;
   if (dense) {
     want = (n / 4 + kThreads * 4 - 1) / (kThreads * 4);
   } else {
     THCL_CHECK(n < (1l << 31), THCL_DIM_WARNING);
-    fill_operand(P.L, thcl_collapse(src));
-    want = (n + kThreads - 1) / kThreads;
+    fill_operand(P.L, walk);
+    want = (n + kThreads * 8 - 1) / (kThreads * 8);
   }
-  long cap = (long)cus * 2;  // two resident blocks per CU keep HBM busy; fewer blocks, fewer tickets
+  // dense: two resident blocks per CU keep HBM busy (fewer blocks, fewer tickets); strided walks read
+  // 4 bytes per lane and need more of them in flight
+  long cap = (long)cus * (dense ? 2 : 8);
   const long max_partials = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
   if (cap > max_partials) cap = max_partials;
   unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));
