@@ -370,6 +370,25 @@ def detail(cl, oracle, T, X, Y, Z, n):
     measure("w_indexSelect_rows_65536x1024", lambda: sel.index(tab, 1, idx), 8 * cnt * width)
     measure("w_indexCopy_rows_65536x1024", lambda: tab.indexCopy(1, idx, sel), 8 * cnt * width)
     del tab, sel
+    # shapes that leave a plain slice-per-block or element-order walk idle: few long slices, a handful of
+    # columns, a whole-tensor sum over a transposed view, a ragged product
+    few = cl.ClTensor(64 << 20).resize(64, 1 << 20)
+    few.fill(0.5)
+    res = cl.ClTensor()
+    measure("w_sum_dim2_64x2^20", lambda: res.sum(few, 2), 4 * (64 << 20))
+    measure("w_max_dim2_64x2^20", lambda: few.max(2), 4 * (64 << 20))
+    tall = few.resize(1 << 24, 4)
+    measure("w_sum_dim1_2^24x4", lambda: res.sum(tall, 1), 4 * (64 << 20))
+    sq = tall.resize(8192, 8192).t()
+    measure("w_sumall_transposed_8192^2", lambda: res.sum(sq), 4 * (64 << 20))
+    del few, tall, sq
+    ra, rb, rc = cl.ClTensor(3000, 7000), cl.ClTensor(7000, 5000), cl.ClTensor(3000, 5000)
+    ra.fill(0.01)
+    rb.fill(0.02)
+    rc.fill(0.0)
+    measure("w_addmm_3000x5000x7000", lambda: rc.addmm(0.0, 1.0, ra, rb), 2.0 * 3000 * 5000 * 7000, "TFLOP/s", reps=6,
+            peak=FP32_MFMA_PEAK_TFLOPS)
+    del ra, rb, rc
     mask = cl.ClTensor((rs.rand(1 << 26) > 0.5).astype(np.float32))
     src = cl.ClTensor(1 << 26)
     src.fill(1.0)
