@@ -31,7 +31,9 @@ struct GemvParams {
   thcl_u64 lda;
   long incx, incy;
   float alpha, beta;
-  thcl_u32 split, per_split;
+  thcl_u32 split, per_split;  // blocks sharing one output's contraction, and the length each takes
+  thcl_u32 outputs;           // n for 't', m for 'n'
+  thcl_u32 ub_log2;           // 'n' kernel: a wave spans 2^ub_log2 units of outputs and 64 >> ub_log2 columns
 };
 
 __device__ __forceinline__ void store_result(const GemvParams &P, thcl_u32 i, double acc) {
@@ -41,19 +43,22 @@ __device__ __forceinline__ void store_result(const GemvParams &P, thcl_u32 i, do
 }
 
 // trans = 't': y[j] = alpha * dot(A[:, j], x) + beta * y[j].  Column j is m
-// contiguous floats; LPR lanes walk it (8, 64 or a whole block).
+// contiguous floats; LPR lanes walk it (1, 8, 64 or a whole block).  blockIdx.y cuts
+// long columns into pieces of per_split elements (a multiple of 4) that leave partials.
 template <int LPR, bool VEC>
 __global__ __launch_bounds__(kThreads) void gemv_t(GemvParams P) {
   constexpr int COLS = kThreads / LPR;
   __shared__ double lds[kThreads / kWave];
   const int sub = threadIdx.x % LPR;
   const thcl_u32 j = blockIdx.x * COLS + threadIdx.x / LPR;
+  const thcl_u32 i0 = blockIdx.y * P.per_split;
+  const thcl_u32 len = (P.m - i0 < P.per_split) ? (P.m - i0) : P.per_split;
   double acc = 0.0;
   if (j < P.n) {
-    const float *col = P.a + (thcl_u64)j * P.lda;
+    const float *col = P.a + (thcl_u64)j * P.lda + i0;
     if (VEC) {  // m % 4 == 0, 16-byte aligned columns, incx == 1
-      const thcl_f4 *c4 = (const thcl_f4 *)col, *x4 = (const thcl_f4 *)P.x;
-      const thcl_u32 m4 = P.m >> 2;
+      const thcl_f4 *c4 = (const thcl_f4 *)col, *x4 = (const thcl_f4 *)(P.x + i0);
+      const thcl_u32 m4 = len >> 2;
       constexpr int FLY = 4;
       thcl_u32 i = sub;
       for (; i + (FLY - 1) * LPR < m4; i += FLY * LPR) {
@@ -74,14 +79,17 @@ __global__ __launch_bounds__(kThreads) void gemv_t(GemvParams P) {
         for (int c = 0; c < 4; c++) acc += (double)v[c] * (double)w[c];
       }
     } else {
-      for (thcl_u32 i = sub; i < P.m; i += LPR) acc += (double)col[i] * (double)P.x[(long)i * P.incx];
+      for (thcl_u32 i = sub; i < len; i += LPR) acc += (double)col[i] * (double)P.x[(long)(i0 + i) * P.incx];
     }
   }
   // fold the LPR lanes of a column
 #pragma unroll
   for (int d = (LPR < kWave ? LPR : kWave) >> 1; d > 0; d >>= 1) acc += __shfl_xor(acc, d, kWave);
   if (LPR <= kWave) {
-    if (sub == 0 && j < P.n) store_result(P, j, acc);
+    if (sub == 0 && j < P.n) {
+      if (P.split > 1) P.partials[(thcl_u64)blockIdx.y * P.n + j] = acc;
+      else store_result(P, j, acc);
+    }
   } else {
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     if (lane == 0) lds[wave] = acc;
@@ -89,21 +97,26 @@ __global__ __launch_bounds__(kThreads) void gemv_t(GemvParams P) {
     if (threadIdx.x == 0 && j < P.n) {
       double r = lds[0];
       for (int w = 1; w < kThreads / kWave; w++) r += lds[w];
-      store_result(P, j, r);
+      if (P.split > 1) P.partials[(thcl_u64)blockIdx.y * P.n + j] = r;
+      else store_result(P, j, r);
     }
   }
 }
 
 // trans = 'n': y[i] = alpha * sum_j A[i + j*lda] * x[j] + beta * y[i].  Lanes lie
-// along i (VEC rows each), the 4 waves of a block interleave over j and meet in
-// LDS; blockIdx.y splits long contractions, leaving partials for gemv_n_finish.
+// along i (VEC rows each; with fewer than 64 units of rows the wave's other lanes take
+// further columns), the 4 waves of a block interleave over j and meet in
+// LDS; blockIdx.y splits long contractions, leaving partials for gemv_finish.
 template <int VEC>
 __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
   constexpr int WAVES = kThreads / kWave;
   __shared__ double lds[WAVES][kWave * VEC];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const thcl_u32 UB = 1u << P.ub_log2, RL = kWave >> P.ub_log2;
+  const thcl_u32 ul = lane & (UB - 1), rl = lane >> P.ub_log2;
+  const thcl_u32 JSTEP = WAVES * RL;  // columns between a lane's consecutive elements
   const thcl_u32 units = (P.m + VEC - 1) / VEC;
-  const thcl_u32 u = blockIdx.x * kWave + lane;
+  const thcl_u32 u = blockIdx.x * UB + ul;
   const thcl_u32 j0 = blockIdx.y * P.per_split;
   thcl_u32 j1 = j0 + P.per_split;
   if (j1 > P.n) j1 = P.n;
@@ -112,17 +125,17 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
   for (int c = 0; c < VEC; c++) acc[c] = 0.0;
   if (u < units) {
     constexpr int FLY = 4;
-    thcl_u32 j = j0 + wave;
+    thcl_u32 j = j0 + wave * RL + rl;
     const float *ptr = P.a + (thcl_u64)j * P.lda + (thcl_u64)u * VEC;
-    const thcl_u64 step = (thcl_u64)WAVES * P.lda;
-    for (; j + (FLY - 1) * WAVES < j1; j += FLY * WAVES) {
+    const thcl_u64 step = (thcl_u64)JSTEP * P.lda;
+    for (; j + (FLY - 1) * JSTEP < j1; j += FLY * JSTEP) {
       float xs[FLY];
       if (VEC == 4) {
         thcl_f4 v[FLY];
 #pragma unroll
         for (int f = 0; f < FLY; f++) {
           v[f] = __builtin_nontemporal_load((const thcl_f4 *)ptr);
-          xs[f] = P.x[(long)(j + f * WAVES) * P.incx];
+          xs[f] = P.x[(long)(j + f * JSTEP) * P.incx];
           ptr += step;
         }
 #pragma unroll
@@ -134,14 +147,14 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
 #pragma unroll
         for (int f = 0; f < FLY; f++) {
           v[f] = *ptr;
-          xs[f] = P.x[(long)(j + f * WAVES) * P.incx];
+          xs[f] = P.x[(long)(j + f * JSTEP) * P.incx];
           ptr += step;
         }
 #pragma unroll
         for (int f = 0; f < FLY; f++) acc[0] += (double)v[f] * (double)xs[f];
       }
     }
-    for (; j < j1; j += WAVES) {
+    for (; j < j1; j += JSTEP) {
       const double xj = (double)P.x[(long)j * P.incx];
       if (VEC == 4) {
         const thcl_f4 v = *(const thcl_f4 *)ptr;
@@ -153,14 +166,21 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
       ptr += step;
     }
   }
+  // the wave's column lanes of one unit meet first (lanes UB apart)
+  for (thcl_u32 d = UB; d < (thcl_u32)kWave; d <<= 1) {
 #pragma unroll
-  for (int c = 0; c < VEC; c++) lds[wave][lane * VEC + c] = acc[c];
+    for (int c = 0; c < VEC; c++) acc[c] += __shfl_xor(acc[c], (int)d, kWave);
+  }
+  if (rl == 0) {
+#pragma unroll
+    for (int c = 0; c < VEC; c++) lds[wave][ul * VEC + c] = acc[c];
+  }
   __syncthreads();
-  if (wave == 0 && u < units) {
+  if (wave == 0 && rl == 0 && u < units) {
 #pragma unroll
     for (int c = 0; c < VEC; c++) {
-      double r = lds[0][lane * VEC + c];
-      for (int w = 1; w < WAVES; w++) r += lds[w][lane * VEC + c];
+      double r = lds[0][ul * VEC + c];
+      for (int w = 1; w < WAVES; w++) r += lds[w][ul * VEC + c];
       const thcl_u32 i = u * VEC + c;
       if (i < P.m) {
         if (P.split > 1) P.partials[(thcl_u64)blockIdx.y * P.m + i] = r;
@@ -170,11 +190,12 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
   }
 }
 
-__global__ __launch_bounds__(kThreads) void gemv_n_finish(GemvParams P) {
+// folds the [split][outputs] partials in split order
+__global__ __launch_bounds__(kThreads) void gemv_finish(GemvParams P) {
   const thcl_u32 i = blockIdx.x * kThreads + threadIdx.x;
-  if (i >= P.m) return;
+  if (i >= P.outputs) return;
   double r = 0.0;
-  for (thcl_u32 k = 0; k < P.split; k++) r += P.partials[(thcl_u64)k * P.m + i];
+  for (thcl_u32 k = 0; k < P.split; k++) r += P.partials[(thcl_u64)k * P.outputs + i];
   store_result(P, i, r);
 }
 
@@ -301,28 +322,55 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
   P.alpha = alpha;
   P.beta = beta;
   P.split = 1;
-  P.per_split = (thcl_u32)n;
+  P.per_split = (thcl_u32)(t ? m : n);
+  P.outputs = (thcl_u32)outputs;
+  const long cus = thcl_rt_get_props(rt)->compute_units;
   const bool rows_aligned = aligned16(P.a) && (lda % 4 == 0) && (m % 4 == 0);
   if (t) {
     const bool vec = rows_aligned && incx == 1 && aligned16(P.x);
+    // few long columns: cut them into pieces of at least 8192 elements until the chip is full
+    if (m >= 2048 && n < cus * 4) {
+      long split = (cus * 8 + n - 1) / n;
+      if (split > m / 8192) split = m / 8192;
+      if (split > 1024) split = 1024;
+      if (split > 1) {
+        const long per = ((m + split - 1) / split + 1023) / 1024 * 1024;
+        split = (m + per - 1) / per;
+        if (split > 1) {
+          P.split = (thcl_u32)split;
+          P.per_split = (thcl_u32)per;
+          P.partials = (double *)thcl_rt_workspace(rt, (size_t)split * (size_t)n * sizeof(double));
+          THCL_CHECK(P.partials != nullptr, "%s", thcl_rt_error());
+        }
+      }
+    }
 #define GEMV_T(L)                                                                                        \
   {                                                                                                      \
-    const dim3 grid((unsigned)((n + (kThreads / L) - 1) / (kThreads / L)));                              \
+    const dim3 grid((unsigned)((n + (kThreads / L) - 1) / (kThreads / L)), P.split);                     \
     if (vec) hipLaunchKernelGGL((gemv_t<L, true>), grid, dim3(kThreads), 0, stream, P);                  \
     else hipLaunchKernelGGL((gemv_t<L, false>), grid, dim3(kThreads), 0, stream, P);                     \
   }
-    if (m >= 2048) GEMV_T(256) else if (m >= 128) GEMV_T(64) else GEMV_T(8)
+    if (m >= 2048) GEMV_T(256) else if (m >= 128) GEMV_T(64) else if (m > 16) GEMV_T(8) else GEMV_T(1)
 #undef GEMV_T
     check("gemv");
+    if (P.split > 1) {
+      hipLaunchKernelGGL(gemv_finish, dim3((unsigned)((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P);
+      check("gemv finish");
+    }
   } else {
     const int vecw = rows_aligned ? 4 : 1;
     const long units = (m + vecw - 1) / vecw;
-    const long tiles = (units + kWave - 1) / kWave;
-    const long target = (long)thcl_rt_get_props(rt)->compute_units * 4;
+    // fewer units than lanes: the wave's spare lanes take further columns
+    unsigned ub_log2 = 6;
+    while (ub_log2 > 0 && (1l << (ub_log2 - 1)) >= units) ub_log2--;
+    P.ub_log2 = ub_log2;
+    const long ub = 1l << ub_log2, col_lanes = kWave >> ub_log2;
+    const long tiles = (units + ub - 1) / ub;
+    const long target = cus * 4;
     long split = 1;
     if (tiles < target) {
       split = (target + tiles - 1) / tiles;
-      const long most = (n + 31) / 32;  // at least 32 columns per block
+      const long most = (n + 32 * col_lanes - 1) / (32 * col_lanes);  // at least 32 columns per lane
       if (split > most) split = most;
       if (split > 256) split = 256;
       if (split < 1) split = 1;
@@ -341,7 +389,7 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
     else hipLaunchKernelGGL((gemv_n<1>), grid, dim3(kThreads), 0, stream, P);
     check("gemv");
     if (split > 1) {
-      hipLaunchKernelGGL(gemv_n_finish, dim3((unsigned)((m + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P);
+      hipLaunchKernelGGL(gemv_finish, dim3((unsigned)((m + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P);
       check("gemv finish");
     }
   }

@@ -68,7 +68,11 @@ def test_blas_dot_on_storage_addresses(cl):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (2, 3), (7, 130), (130, 7), (64, 64), (300, 1000), (1000, 300), (4096, 33),
-                                       (33, 4096), (5, 70000), (70000, 5), (2048, 2048)])
+                                       (33, 4096), (5, 70000), (70000, 5), (2048, 2048),
+                                       # few long lines (cut over blocks), lines of 1..16 elements (a thread each), fewer than
+                                       # 64 units of outputs (spare lanes take further columns)
+                                       (3, 300001), (300001, 3), (4, 1 << 20), (1 << 20, 4), (16, 100000), (100000, 16),
+                                       (40, 50000), (50000, 40), (1, 1 << 20), (1 << 20, 1)])
 def test_addmv_layouts(cl, rows, cols):
     m = oracle.normal(73, rows * cols).reshape(rows, cols)
     v, t = oracle.normal(74, cols), oracle.normal(75, rows)
