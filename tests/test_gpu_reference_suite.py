@@ -22,6 +22,11 @@ def test_matrixwide(cl):                               # unit_tensor.lua:488-496
     assert c.max() == 9 and c.min() == 2 and c.sum() == 30
     assert np.array_equal(c.sum(1).float(), a.sum(axis=0, keepdims=True))
     assert np.array_equal(c.sum(2).float(), a.sum(axis=1, keepdims=True))
+    # the result slot first, as torch.sum(res, src, dim) orders them (src/TensorMath.lua:943-953)
+    res = cl.ClTensor()
+    assert res.sum(c, 2) is res and np.array_equal(res.float(), a.sum(axis=1, keepdims=True))
+    assert np.array_equal(res.prod(c, 1).float(), a.prod(axis=0, keepdims=True))
+    assert np.allclose(res.mean(c, 2).float(), a.mean(axis=1, keepdims=True))
 
 
 def test_intpower_and_powerofneg(cl):                  # unit_tensor.lua:506-520
