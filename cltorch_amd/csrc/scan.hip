@@ -253,18 +253,24 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
   if (PHASE == 0 && threadIdx.x == 0) P.totals[blockIdx.x] = carry;
 }
 
-// I > 1 with too few columns for a thread per column: a block walks a strip of 32 columns
-// down all of R, 256 rows a step.  A thread holds 8 consecutive rows of 4 adjacent columns
-// (one 16-byte access per row; the 8 threads that share a row read 128 contiguous bytes),
-// so 32 rows per column are combined side by side: thread totals, a shuffle scan over the 8
-// row groups of a wave, the 4 waves' totals through LDS, then the rows are finished from the
-// registers.  One barrier a step; the next step's rows are requested before this step's work.
-template <bool PROD>
+// I > 1 with too few columns for a thread per column: a block walks a strip of 4 * TC columns
+// down its segment of R, (256 / TC) * 8 rows a step.  A thread holds 8 consecutive rows of 4
+// adjacent columns (one 16-byte access per row; the TC threads that share a row read 16 * TC
+// contiguous bytes), so 256 / TC rows per column are combined side by side: thread totals, a
+// shuffle scan over the row groups of a wave, the 4 waves' totals through LDS, then the rows are
+// finished from the registers.  One barrier a step; the next step's rows are requested before
+// this step's work.  TC = 8 for wide tensors; with 4 to 28 columns TC = 1, 2, 4 or 8 covers the whole
+// width and consecutive rows are adjacent in memory, so a step reads one contiguous run.  PHASE 0 leaves the segment's
+// totals, PHASE 1 scans (from the segment's carry when the lines are cut into segments).
+template <bool PROD, int TC, int PHASE>
 __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
-  constexpr int TC = 8, K = 8, WAVES = kThreads / kWave, ROWS = kThreads / TC * K, CW = TC * 4;
+  // rows per thread: 8; 2 on the narrowest strips, where a thread's 8 rows would be 128 or 256 contiguous
+  // bytes read 16 at a time (measured 0.6 TB/s on 4 columns against 2.0 with 2 rows)
+  constexpr int K = TC >= 4 ? 8 : 2;
+  constexpr int WAVES = kThreads / kWave, ROWS = kThreads / TC * K, CW = TC * 4;
   __shared__ double wave_tot[2][WAVES][CW];
   const thcl_u64 strips = (P.I / 4 + TC - 1) / TC;
-  const thcl_u64 o = blockIdx.x / strips, strip = blockIdx.x % strips;
+  const thcl_u64 strip = blockIdx.x % strips, seg_id = (blockIdx.x / strips) % P.S, o = blockIdx.x / (strips * P.S);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int tc = threadIdx.x % TC, tr = threadIdx.x / TC;
   const thcl_u64 col = (strip * TC + tc) * 4;
@@ -273,33 +279,36 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
   const float *src = P.in + first;
   float *dst = P.out + first;
   const float fill = PROD ? 1.0f : 0.0f;
+  const thcl_u64 rbegin = seg_id * P.seg;
+  const thcl_u64 rend = (rbegin + P.seg < P.R) ? rbegin + P.seg : P.R;
   // rows past the end are read from the last row (so that every load is issued) and replaced
   auto fetch = [&](thcl_f4 (&x)[K], thcl_u64 r0) {
 #pragma unroll
     for (int k = 0; k < K; k++) {
       const thcl_u64 r = r0 + (thcl_u64)tr * K + k;
-      x[k] = __builtin_nontemporal_load((const thcl_f4 *)(src + (r < P.R ? r : P.R - 1) * P.I));
+      x[k] = __builtin_nontemporal_load((const thcl_f4 *)(src + (r < rend ? r : rend - 1) * P.I));
     }
   };
+  double *tot = P.totals + (o * P.S + seg_id) * P.I + (live ? col : 0);
   double carry[4];
 #pragma unroll
-  for (int c = 0; c < 4; c++) carry[c] = Op<PROD>::identity();
+  for (int c = 0; c < 4; c++) carry[c] = (PHASE == 1 && P.S > 1) ? tot[c] : Op<PROD>::identity();
   thcl_f4 x[K], xn[K];
-  fetch(x, 0);
+  fetch(x, rbegin);
   int buf = 0;
-  for (thcl_u64 r0 = 0; r0 < P.R; r0 += ROWS, buf ^= 1) {
+  for (thcl_u64 r0 = rbegin; r0 < rend; r0 += ROWS, buf ^= 1) {
     fetch(xn, r0 + ROWS);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int k = 0; k < K; k++)
-      if (r0 + (thcl_u64)tr * K + k >= P.R) x[k] = thcl_f4{fill, fill, fill, fill};
+      if (r0 + (thcl_u64)tr * K + k >= rend) x[k] = thcl_f4{fill, fill, fill, fill};
     double incl[4];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
       double t = (double)x[0][c];
 #pragma unroll
       for (int k = 1; k < K; k++) t = Op<PROD>::comb(t, (double)x[k][c]);
-      // the 8 row groups of this wave sit TC lanes apart
+      // the row groups of this wave sit TC lanes apart
 #pragma unroll
       for (int d = TC; d < kWave; d <<= 1) {
         const double up = __shfl_up(t, d, kWave);
@@ -325,19 +334,25 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
       if (lane >= TC) before = Op<PROD>::comb(before, prev);
       incl[c] = before;  // from here on: the running value of column c
     }
+    if (PHASE == 1) {
 #pragma unroll
-    for (int k = 0; k < K; k++) {
-      thcl_f4 v;
+      for (int k = 0; k < K; k++) {
+        thcl_f4 v;
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        incl[c] = Op<PROD>::comb(incl[c], (double)x[k][c]);
-        v[c] = (float)incl[c];
+        for (int c = 0; c < 4; c++) {
+          incl[c] = Op<PROD>::comb(incl[c], (double)x[k][c]);
+          v[c] = (float)incl[c];
+        }
+        const thcl_u64 r = r0 + (thcl_u64)tr * K + k;
+        if (live && r < rend) __builtin_nontemporal_store(v, (thcl_f4 *)(dst + r * P.I));
       }
-      const thcl_u64 r = r0 + (thcl_u64)tr * K + k;
-      if (live && r < P.R) __builtin_nontemporal_store(v, (thcl_f4 *)(dst + r * P.I));
     }
 #pragma unroll
     for (int k = 0; k < K; k++) x[k] = xn[k];
+  }
+  if (PHASE == 0 && tr == 0 && live) {
+#pragma unroll
+    for (int c = 0; c < 4; c++) tot[c] = carry[c];
   }
 }
 
@@ -509,12 +524,28 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     // is a strip for every other CU and the lines are long enough to amortise a block's start.  On 256
     // CUs, 2^26 elements: 16384 columns 4.9 TB/s against 3.7 in three passes, 8192 columns 5.2,
     // 4096 columns (128 strips) 4.2 against 3.8, 2048 columns 2.5 against 3.7.
-    const thcl_u64 strips = P.O * ((P.I / 4 + 7) / 8);
-    const bool strip = !rows && !shortrows && P.I % 4 == 0 && P.R >= 1024 && P.O * P.I < (thcl_u64)cus * 512 &&
-                       strips * 2 >= (thcl_u64)cus && strips < (1ull << 31) &&
-                       ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
+    const bool aligned = ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
+    const bool few_lines = !rows && !shortrows && P.I % 4 == 0 && aligned && P.O * P.I < (thcl_u64)cus * 512;
+    thcl_u64 strips = P.O * ((P.I / 4 + 7) / 8);
+    bool strip = few_lines && P.R >= 1024 && strips * 2 >= (thcl_u64)cus && strips < (1ull << 31);
+    // A handful of columns (4 to 28): the thread-per-column kernel would read 16 to 112 bytes per row
+    // and line segment.  Strips as wide as the tensor read whole runs of rows instead; the lines are
+    // cut into segments (three passes) to fill the chip.  2^26 elements in rows of 4 / 8 / 16 columns:
+    // 0.8 -> 2.0, 1.7 -> 2.1, 2.5 -> 3.0 TB/s.
+    int strip_tc = 8;
+    bool narrow = false;
+    if (!strip && few_lines && P.I <= 28 && P.R >= 16384) {
+      strip_tc = P.I <= 4 ? 1 : (P.I <= 8 ? 2 : (P.I <= 16 ? 4 : 8));
+      strips = P.O;
+      strip = narrow = true;
+    }
     thcl_u64 S = 1;
-    if (shortrows || strip) {
+    if (narrow) {
+      const thcl_u64 want = (thcl_u64)cus * 8;  // blocks
+      if (P.O < want) S = (want + P.O - 1) / P.O;
+      const thcl_u64 most = P.R / 4096;  // a few steps of the block at least
+      if (S > most) S = most;
+    } else if (shortrows || strip) {
       S = 1;
     } else if (rows) {
       // Segments cost a second read of the input (12 bytes an element instead of 8), which pays
@@ -539,16 +570,33 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     THCL_CHECK(P.O * P.S < (1ull << 31) && (P.O * P.S * P.I + kThreads - 1) / kThreads < (1ull << 31), THCL_DIM_WARNING);
     if (S > 1) P.totals = (double *)thcl_rt_workspace(rt, (size_t)(P.O * P.S * P.I) * sizeof(double));
     THCL_CHECK(S == 1 || P.totals != nullptr, "%s", thcl_rt_error());
-    const bool vec = (rows || shortrows) && (P.R % 4 == 0) && ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
+    const bool vec = (rows || shortrows) && (P.R % 4 == 0) && aligned;
     if (shortrows) {
       THCL_CHECK(P.O < (1ull << 31), THCL_DIM_WARNING);
       if (prod) run_short<true>(stream, P, vec);
       else run_short<false>(stream, P, vec);
       check("scan");
     } else if (strip) {
-      const dim3 grid((unsigned)strips), block(kThreads);
-      if (prod) hipLaunchKernelGGL((scan_strip<true>), grid, block, 0, stream, P);
-      else hipLaunchKernelGGL((scan_strip<false>), grid, block, 0, stream, P);
+      const dim3 grid((unsigned)(strips * P.S)), block(kThreads);
+#define STRIP_PHASE(PH)                                                                                        \
+  switch (strip_tc * 2 + (prod ? 1 : 0)) {                                                                     \
+    case 2: hipLaunchKernelGGL((scan_strip<false, 1, PH>), grid, block, 0, stream, P); break;                  \
+    case 3: hipLaunchKernelGGL((scan_strip<true, 1, PH>), grid, block, 0, stream, P); break;                   \
+    case 4: hipLaunchKernelGGL((scan_strip<false, 2, PH>), grid, block, 0, stream, P); break;                  \
+    case 5: hipLaunchKernelGGL((scan_strip<true, 2, PH>), grid, block, 0, stream, P); break;                   \
+    case 8: hipLaunchKernelGGL((scan_strip<false, 4, PH>), grid, block, 0, stream, P); break;                  \
+    case 9: hipLaunchKernelGGL((scan_strip<true, 4, PH>), grid, block, 0, stream, P); break;                   \
+    case 16: hipLaunchKernelGGL((scan_strip<false, 8, PH>), grid, block, 0, stream, P); break;                 \
+    default: hipLaunchKernelGGL((scan_strip<true, 8, PH>), grid, block, 0, stream, P); break;                  \
+  }
+      if (P.S > 1) {
+        STRIP_PHASE(0)
+        check("scan totals");
+        if (prod) launch_carries<true>(stream, P);
+        else launch_carries<false>(stream, P);
+      }
+      STRIP_PHASE(1)
+#undef STRIP_PHASE
       check("scan");
     } else if (prod) {
       run_scan<true>(stream, P, rows, vec);
