@@ -447,10 +447,15 @@ float THClTensor_dot(THClState *state, THClTensor *self, THClTensor *src) {
   const long n = THClTensor_nElement(state, self);
   THCL_ARGCHECK(n == THClTensor_nElement(state, src), 2, "sizes do not match");
   if (n == 0) return 0.f;
-  ThclTemp a(state, THClTensor_newContiguous(state, self));
-  ThclTemp b(state, THClTensor_newContiguous(state, src));
   thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, self));
-  thcl_dot_dense(state, rt, thcl_dptr(a.t), thcl_dptr(b.t), n, thcl_rt_host_word_device(rt));
+  // The order of the products is free: same-shaped views that are dense when walked in memory order
+  // (both transposed or permuted alike) are multiplied where they lie; others through dense stand-ins.
+  THClTensor *pair[2] = {self, src};
+  const JointLayout J = thcl_joint_collapse(2, pair);
+  const bool in_place = J.valid && J.dims == 1 && J.strides[0][0] == 1 && J.strides[1][0] == 1;
+  ThclTemp a(state, in_place ? nullptr : THClTensor_newContiguous(state, self));
+  ThclTemp b(state, in_place ? nullptr : THClTensor_newContiguous(state, src));
+  thcl_dot_dense(state, rt, thcl_dptr(in_place ? self : a.t), thcl_dptr(in_place ? src : b.t), n, thcl_rt_host_word_device(rt));
   THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
   const float result = thcl_rt_host_word(rt)[0];
   return result;

@@ -45,6 +45,14 @@ def test_dot_lengths_and_views(cl, n):
         assert abs(pa.dev.dot(pb.dev) - want) <= 1e-5 * max(abs(want), np.sqrt(n) * 1e-2)
     with pytest.raises(cl.ClError):
         cl.ClTensor(a).dot(cl.ClTensor(n + 1))
+    if n >= 4096 and n % 64 == 0:
+        # both operands transposed alike: multiplied where they lie; one transposed, one not: through dense copies
+        qa, qb = Pair.dense(cl, a.reshape(64, n // 64)).transpose(0, 1), Pair.dense(cl, b.reshape(64, n // 64)).transpose(0, 1)
+        want = float(cat.dot(qa.view.gather(), qb.view.gather()))
+        assert abs(qa.dev.dot(qb.dev) - want) <= 1e-5 * max(abs(want), np.sqrt(n) * 1e-2)
+        qc = Pair.dense(cl, b.reshape(n // 64, 64))
+        want = float(cat.dot(qa.view.gather(), qc.view.gather()))
+        assert abs(qa.dev.dot(qc.dev) - want) <= 1e-5 * max(abs(want), np.sqrt(n) * 1e-2)
 
 
 def test_blas_dot_on_storage_addresses(cl):
