@@ -501,15 +501,16 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
 // slices; UB = 64 unless the slices are fewer, then the wave's other lanes take
 // further rows), the 4 waves of a block interleave over the reduced dim and meet in
 // LDS; blockIdx.y splits long reductions, leaving partials for the finisher.
-template <int KIND, bool ARG, int VEC>
+template <int KIND, bool ARG, int VEC, bool NARROW>
 __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
   typedef Slot<KIND, ARG> S;
   typedef typename S::T T;
   constexpr int WAVES = kThreads / kWave;
   __shared__ T lds[WAVES][kWave * VEC];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const thcl_u32 UB = 1u << P.ub_log2, RL = kWave >> P.ub_log2;  // units and rows across a wave
-  const thcl_u32 ul = lane & (UB - 1), rl = lane >> P.ub_log2;
+  // units and rows across a wave; constants in the common case of 64 units or more
+  const thcl_u32 UB = NARROW ? (1u << P.ub_log2) : (thcl_u32)kWave, RL = NARROW ? ((thcl_u32)kWave >> P.ub_log2) : 1u;
+  const thcl_u32 ul = NARROW ? (lane & (UB - 1)) : (thcl_u32)lane, rl = NARROW ? ((thcl_u32)lane >> P.ub_log2) : 0u;
   const thcl_u32 ntiles = (P.nunits + UB - 1) / UB;
   const thcl_u32 r_begin = blockIdx.y * P.rows_per_split;
   thcl_u32 r_end = r_begin + P.rows_per_split;
@@ -602,9 +603,11 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
         acc[c] = S::seal(acc[c], (int)(r_begin + wave * RL + rl), r_begin + wave * RL + rl < r_end);
     }
     // the wave's row lanes of one unit meet first (lanes UB apart)
-    for (thcl_u32 m = UB; m < (thcl_u32)kWave; m <<= 1) {
+    if (NARROW) {
+      for (thcl_u32 m = UB; m < (thcl_u32)kWave; m <<= 1) {
 #pragma unroll
-      for (int c = 0; c < VEC; c++) acc[c] = S::comb(acc[c], shfl_xor_t(acc[c], (int)m));
+        for (int c = 0; c < VEC; c++) acc[c] = S::comb(acc[c], shfl_xor_t(acc[c], (int)m));
+      }
     }
     __syncthreads();
     if (rl == 0) {
@@ -787,8 +790,11 @@ void launch_dim(bool rows, int lpr, int vec, dim3 grid, hipStream_t stream, cons
     if (vec == 4) hipLaunchKernelGGL((reduce_cols_short<KIND, ARG, 4>), grid, block, 0, stream, P);
     else hipLaunchKernelGGL((reduce_cols_short<KIND, ARG, 1>), grid, block, 0, stream, P);
   } else {
-    if (vec == 4) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 4>), grid, block, 0, stream, P);
-    else hipLaunchKernelGGL((reduce_cols<KIND, ARG, 1>), grid, block, 0, stream, P);
+    const bool narrow = P.ub_log2 < 6;
+    if (vec == 4 && narrow) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 4, true>), grid, block, 0, stream, P);
+    else if (vec == 4) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 4, false>), grid, block, 0, stream, P);
+    else if (narrow) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 1, true>), grid, block, 0, stream, P);
+    else hipLaunchKernelGGL((reduce_cols<KIND, ARG, 1, false>), grid, block, 0, stream, P);
   }
 }
 
