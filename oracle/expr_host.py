@@ -8,6 +8,14 @@ literals become fp32, the type an fp32-only OpenCL C device gives them.
 Expressions made of + - * / sqrt are correctly rounded on both sides and
 compare bit for bit; transcendental functions compare within the reference
 tests' own tolerance (src/test/unit_tensor.lua:73-93).
+
+Pinned by tests/test_oracle.py (no GPU needed): ``rewrite`` against the
+reference's substitutions on its own test strings in both spellings, names
+that contain x/y/z, and literal typing; ``evaluate`` against IEEE fp32
+arithmetic written one rounding at a time with numpy (two roundings told
+from a fused multiply-add, fp32 literals told from double ones, operand
+binding, the prelude functions) and the transcendental statements within one
+unit of the last place of fp64-then-round.
 """
 import ctypes as C
 import hashlib

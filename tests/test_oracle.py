@@ -365,3 +365,146 @@ def test_indexed_movement_hand_cases():
     assert cat.masked_select(a, m).tolist() == [2, 4, 5, 11]
     assert cat.masked_copy(a, m, [-1, -2, -3, -4, -5])[0].tolist() == [1, -1, 3, -2]
     assert cat.masked_copy(a, m, [-1, -2, -3, -4])[2].tolist() == [9, 10, -4, 12]
+
+
+# ------------------------------------------- expression evaluator (expr_host) ---
+# oracle/expr_host.py judges every apply/map/map2 string other than the two
+# configuration strings, so its text rewrite and its arithmetic are pinned here:
+# the rewrite against the substitutions the reference makes
+# (src/lib/THClTensorMathPointwise.cpp:79-146) on the strings of its own tests
+# (src/test/unit_tensor.lua:583-635), the arithmetic against IEEE fp32 operations
+# written out one rounding at a time with numpy.
+def test_expr_rewrite_reference_strings():
+    from oracle import expr_host as eh
+    # the pointer syntax passes through untouched, the x/y/z syntax turns into it
+    raw1 = "*out = sqrt(*out + 3) + exp(*out)"
+    raw2 = "*out = sqrt(*out * *out + *in1 * *in1 + 3 + exp(*in1))"
+    raw3 = "*out = sqrt(*out * *out + *in1 * *in1 + *in2 + 3 + exp(*in2))"
+    assert eh.rewrite(raw1, 1) == raw1 and eh.rewrite(raw2, 2) == raw2 and eh.rewrite(raw3, 3) == raw3
+    assert eh.rewrite("x = sqrt(x + 3) + exp(x)", 1) == "(*out) = sqrt((*out) + 3) + exp((*out))"
+    assert eh.rewrite("x = sqrt(x * x + y * y + 3 + exp(y))", 2) == \
+        "(*out) = sqrt((*out) * (*out) + (*in1) * (*in1) + 3 + exp((*in1)))"
+    assert eh.rewrite("x = sqrt(x * x + y * y + z + 3 + exp(z))", 3) == \
+        "(*out) = sqrt((*out) * (*out) + (*in1) * (*in1) + (*in2) + 3 + exp((*in2)))"
+    # a call with fewer tensors leaves the later letters alone (apply replaces x only, map x and y)
+    assert eh.rewrite("x = y + z", 1) == "(*out) = y + z"
+    assert eh.rewrite("x = y + z", 2) == "(*out) = (*in1) + z"
+    # names that merely contain x, y or z are not variables
+    assert eh.rewrite("x = max(x, y) + hypot(x, y) + copysign(x, z) + exp(y)", 3) == \
+        "(*out) = max((*out), (*in1)) + hypot((*out), (*in1)) + copysign((*out), (*in2)) + exp((*in1))"
+    assert eh.rewrite("x = xx + y_1 + zeta", 3) == "(*out) = xx + y_1 + zeta"
+
+
+def test_expr_rewrite_literals():
+    from oracle import expr_host as eh
+    assert eh.rewrite("x = 1000*x + 0.5 + 1e-3 + 2. + .25 + 3.5f + 7", 1) == \
+        "(*out) = 1000*(*out) + 0.5f + 1e-3f + 2.f + .25f + 3.5f + 7"
+    assert eh.rewrite("x = 1.5e+2*x - 10/4", 1) == "(*out) = 1.5e+2f*(*out) - 10/4"
+    assert eh.rewrite("x = y2 + 3.25F", 1) == "(*out) = y2 + 3.25F"
+
+
+def _ulps(a, b):
+    """Distance in units of the last place between two finite fp32 arrays."""
+    def key(v):
+        i = np.ascontiguousarray(v, dtype=F).view(np.int32).astype(np.int64)
+        return np.where(i < 0, -(i & 0x7FFFFFFF), i)
+    return np.abs(key(a) - key(b))
+
+
+def test_expr_evaluate_exact_strings_are_ieee_fp32():
+    from oracle import expr_host as eh
+    n = 4096
+    x, y, z = (oracle.uniform(40 + i, n, -0.5, 0.5) for i in range(3))
+    k1000, k10, half, milli, quarter, two = F(1000), F(10), F(0.5), F(1e-3), F(0.25), F(2)
+
+    # 1000*x*x + y*10 + z*z associates left to right: ((1000*x)*x + y*10) + z*z, then one correctly rounded sqrt
+    with np.errstate(invalid="ignore"):
+        want = np.sqrt(((k1000 * x) * x + y * k10) + z * z)
+    assert want.dtype == F
+    assert np.array_equal(bits(eh.evaluate("x = sqrt(1000*x*x + y*10 + z*z)", x, y, z)), bits(want))
+
+    # two roundings, not one: the fused form differs on some elements and must not be what the evaluator gives
+    two_roundings = k1000 * x + y * k10
+    fused = (k1000.astype(np.float64) * x.astype(np.float64) + (y * k10).astype(np.float64)).astype(F)
+    assert np.any(bits(two_roundings) != bits(fused)), "inputs do not separate fused from unfused"
+    got = eh.evaluate("x = 1000*x + y*10", x, y)
+    assert np.array_equal(bits(got), bits(two_roundings))
+    assert np.array_equal(bits(eh.evaluate("*out = 1000 * *out + *in1 * 10", x, y)), bits(two_roundings))
+
+    # literals are fp32: 1e-3 as a double would round differently
+    want = x * half + milli
+    as_double = (x.astype(np.float64) * 0.5 + 1e-3).astype(F)
+    assert np.any(bits(want) != bits(as_double))
+    assert np.array_equal(bits(eh.evaluate("x = x * 0.5 + 1e-3", x)), bits(want))
+
+    assert np.array_equal(bits(eh.evaluate("x = (x > 0.25) ? x : 2*x", x)), bits(np.where(x > quarter, x, two * x)))
+    assert np.array_equal(bits(eh.evaluate("x = max(x, y) - min(x, y)", x, y)), bits(np.maximum(x, y) - np.minimum(x, y)))
+    # strings the GPU tests use on views
+    assert np.array_equal(bits(eh.evaluate("x = x*y + z", x, y, z)), bits(x * y + z))
+    assert np.array_equal(bits(eh.evaluate("x = x + 2*y - z", x, y, z)), bits((x + two * y) - z))
+    assert np.array_equal(bits(eh.evaluate("x = x*y + x", x, y)), bits(x * y + x))
+    assert np.array_equal(bits(eh.evaluate("x = x - y", x, y)), bits(x - y))
+
+
+def test_expr_evaluate_operand_binding():
+    from oracle import expr_host as eh
+    x = np.array([1.0, 2.0, 3.0], dtype=F)
+    y = np.array([10.0, 20.0, 30.0], dtype=F)
+    z = np.array([100.0, 200.0, 300.0], dtype=F)
+    # x is the tensor written, y the first source, z the second: an exchange of any two changes the answer
+    assert eh.evaluate("x = x + 2*y + 4*z", x, y, z).tolist() == [421.0, 842.0, 1263.0]
+    assert eh.evaluate("*out = *out + 2 * *in1 + 4 * *in2", x, y, z).tolist() == [421.0, 842.0, 1263.0]
+    assert eh.evaluate("x = y - x", x, y).tolist() == [9.0, 18.0, 27.0]
+    assert eh.evaluate("x = z", x, y, z).tolist() == [100.0, 200.0, 300.0]
+    # the inputs are left alone; only the returned array carries the result
+    assert x.tolist() == [1.0, 2.0, 3.0] and y.tolist() == [10.0, 20.0, 30.0]
+    # a statement may read the old x after naming it on the left
+    assert eh.evaluate("x = x * x", np.array([3.0, -4.0], dtype=F)).tolist() == [9.0, 16.0]
+    # integer literals promote to float as OpenCL C does: 10/4 stays an integer division, 10/4.0 does not
+    assert eh.evaluate("x = x + 10/4", np.zeros(1, dtype=F)).tolist() == [2.0]
+    assert eh.evaluate("x = x + 10/4.0", np.zeros(1, dtype=F)).tolist() == [2.5]
+
+
+def test_expr_evaluate_prelude_functions():
+    from oracle import expr_host as eh
+    v = np.array([-2.5, -0.0, 0.0, 0.75, 3.0], dtype=F)
+    assert eh.evaluate("x = sign(x)", v).tolist() == [-1.0, 0.0, 0.0, 1.0, 1.0]
+    assert eh.evaluate("x = clamp(x, -1.0, 1.0)", v).tolist() == [-1.0, -0.0, 0.0, 0.75, 1.0]
+    assert eh.evaluate("x = pown(x, 3)", v).tolist() == [-15.625, -0.0, 0.0, 0.421875, 27.0]
+    assert eh.evaluate("x = fabs(x) + floor(x) + ceil(x)", v).tolist() == [-2.5, 0.0, 0.0, 1.75, 9.0]
+    assert eh.evaluate("x = max(x, 1.0) + min(x, -1.0)", v).tolist() == [-1.5, 0.0, 0.0, 0.0, 2.0]
+
+
+def test_expr_evaluate_transcendental_strings_within_one_ulp():
+    from oracle import expr_host as eh
+    n = 3000
+    x, y, z = (oracle.uniform(50 + i, n, -0.5, 0.5) for i in range(3))
+    three = F(3)
+    e32 = lambda v: np.exp(v.astype(np.float64)).astype(F)       # exp in fp64, rounded once
+    # the function itself: within one unit of the correctly rounded value
+    assert _ulps(eh.evaluate("x = exp(x)", x), e32(x)).max() <= 1
+    # (the host C library documents 2 units for tanhf, 1 for the others)
+    for fn, ref, bound in (("log", np.log, 1), ("sin", np.sin, 1), ("cos", np.cos, 1), ("tanh", np.tanh, 2)):
+        arg = x + F(1.0)
+        assert _ulps(eh.evaluate(f"x = {fn}(x)", arg), ref(arg.astype(np.float64)).astype(F)).max() <= bound, fn
+    assert _ulps(eh.evaluate("x = pow(x, y)", x + F(1.0), y), np.power((x + F(1.0)).astype(np.float64), y.astype(np.float64)).astype(F)).max() <= 1
+    # the reference's three test statements, both spellings: fp32 steps with the exponential rounded from fp64.
+    # One unit of error in exp(.) (about 1) moves the sum under the root (about 4) by at most one of its units,
+    # and the root halves relative errors, so the result stays within one unit.
+    cases = [
+        ("x = sqrt(x + 3) + exp(x)", "*out = sqrt(*out + 3) + exp(*out)", (x,),
+         np.sqrt(x + three) + e32(x), np.sqrt(x.astype(np.float64) + 3) + np.exp(x.astype(np.float64))),
+        ("x = sqrt(x * x + y * y + 3 + exp(y))", "*out = sqrt(*out * *out + *in1 * *in1 + 3 + exp(*in1))", (x, y),
+         np.sqrt(((x * x + y * y) + three) + e32(y)),
+         np.sqrt(x.astype(np.float64) ** 2 + y.astype(np.float64) ** 2 + 3 + np.exp(y.astype(np.float64)))),
+        ("x = sqrt(x * x + y * y + z + 3 + exp(z))", "*out = sqrt(*out * *out + *in1 * *in1 + *in2 + 3 + exp(*in2))", (x, y, z),
+         np.sqrt((((x * x + y * y) + z) + three) + e32(z)),
+         np.sqrt(x.astype(np.float64) ** 2 + y.astype(np.float64) ** 2 + z.astype(np.float64) + 3 + np.exp(z.astype(np.float64)))),
+    ]
+    for xyz, raw, arrs, stepwise, exact64 in cases:
+        a = eh.evaluate(xyz, *arrs)
+        b = eh.evaluate(raw, *arrs)
+        assert np.array_equal(bits(a), bits(b)), xyz                    # the two spellings are one statement
+        assert stepwise.dtype == F
+        assert _ulps(a, stepwise).max() <= 1, xyz
+        assert _ulps(a, exact64.astype(F)).max() <= 2, xyz               # and close to the fp64 value of the whole statement
