@@ -105,53 +105,81 @@ def test_config3_reductions_along_each_dim_full_size(cl):
             assert np.array_equal(picked, wv)
 
 
+def _c4_chain(cl, A, ref):
+    """Config 4 on a device tensor and on its host copy with numpy fp32 arithmetic: the sum
+    stays on the device as a point tensor, A is divided by it, then 8 further in-place
+    operators run with no host synchronisation in between.  Returns the host result."""
+    s = cl.ClTensor()
+    s.sum(A)                                    # stays on the device
+    A.div(s)
+    A.mul(1.0001)
+    A.add(0.5)
+    A.cmul(A)
+    A.sqrt()
+    s2 = cl.ClTensor()
+    s2.max(A)
+    A.div(s2)
+    A.add(s2)
+    A.csub(0.25)
+    A.abs()
+    cl.synchronize()
+    sv, mx = F(s.s()), F(s2.s())
+    want_sum = oracle.sumall(View.contiguous(ref))
+    assert abs(float(sv) - want_sum) <= 1e-5 * want_sum
+    ref /= sv
+    ref *= F(1.0001)
+    ref += F(0.5)
+    ref *= ref
+    np.sqrt(ref, out=ref)
+    assert mx == ref.max()                      # max of the chain so far, exact
+    ref /= mx
+    ref += mx
+    ref += F(-0.25)
+    np.abs(ref, out=ref)
+    return ref
+
+
 def test_config4_point_tensor_chain_2p28(cl):
     n = 1 << 28
     a = oracle.uniform(7, n, 0.0, 1.0)
     A = cl.ClTensor(a)
-    s = cl.ClTensor()
-    s.sum(A)                                    # stays on the device
-    want_sum = oracle.sumall(View.contiguous(a))
-    sv = s.s()
-    assert abs(sv - want_sum) <= 1e-5 * want_sum
-    A.div(s)
-    first = A.narrow(1, 1, 1 << 20).float()
-    assert_bit_equal(first, a[:1 << 20] / F(sv), "div by the point tensor")
+    ref = _c4_chain(cl, A, a.copy())
+    got = A.float()
+    # every element, so the head, the middle (grid wrap at 2^27) and the tail of the launch are all covered
+    for lo, hi in ((0, 1 << 20), ((1 << 27) - (1 << 19), (1 << 27) + (1 << 19)), (n - (1 << 20), n)):
+        assert_bit_equal(got[lo:hi], ref[lo:hi], f"chained ops, elements {lo}..{hi}")
+    assert_bit_equal(got, ref, "chained ops, all 2^28 elements")
+    del got, ref
     # after normalisation the elements sum to 1 (to fp32 rounding of each quotient)
-    total = A.sum()
-    assert abs(total - 1.0) < 1e-5
-    # 8 further in-place ops, no host sync in between; mirrored on a slice with numpy fp32 arithmetic
-    ref = (a[:1 << 20] / F(sv)).astype(F)
-    A.mul(1.0001)
-    ref = ref * F(1.0001)
-    A.add(0.5)
-    ref = ref + F(0.5)
-    A.cmul(A)
-    ref = ref * ref
-    A.sqrt()
-    ref = np.sqrt(ref)
-    s2 = cl.ClTensor()
-    s2.max(A)
-    A.div(s2)
-    mx = F(s2.s())
-    ref = ref / mx
-    A.add(s2)
-    ref = ref + mx
-    A.csub(0.25)
-    ref = ref + F(-0.25)
-    A.abs()
-    ref = np.abs(ref)
-    cl.synchronize()
-    assert_bit_equal(A.narrow(1, 1, 1 << 20).float(), ref, "chained ops")
+    s = cl.ClTensor()
+    A.copy(cl.ClTensor(a))
+    s.sum(A)
+    A.div(s)
+    assert abs(A.sum() - 1.0) < 1e-5
     # closed forms at full size
     A.fill(1.0)
     assert A.sum() == float(n)
     A.fill(0.25)
     assert A.sum() == float(n) * 0.25 and A.max() == 0.25 and A.min() == 0.25
-    # idempotence of abs, and max/min bracket every element
+    # max/min bracket every element
     A.copy(cl.ClTensor(a))
     lo, hi = A.min(), A.max()
     assert lo == float(a.min()) and hi == float(a.max())
+
+
+def test_config4_chain_on_a_misaligned_view_of_2p28_minus_1(cl):
+    """The same chain on elements 2..2^28 of the storage: a dense view that starts 4 bytes
+    past a 16-byte boundary and whose length is odd, so the dword kernels and their tails run
+    at full size.  The element in front of the view must stay untouched."""
+    n = 1 << 28
+    a = oracle.uniform(7, n, 0.0, 1.0)
+    whole = cl.ClTensor(a)
+    V = whole.narrow(1, 2, n - 1)
+    assert V.storageOffset() == 2 and V.nElement() == n - 1
+    ref = _c4_chain(cl, V, a[1:].copy())
+    got = whole.float()
+    assert got[0] == a[0]
+    assert_bit_equal(got[1:], ref, "chained ops on the misaligned view")
 
 
 def test_config5_addmm_square_8192_sampled_and_skinny(cl):
@@ -167,6 +195,15 @@ def test_config5_addmm_square_8192_sampled_and_skinny(cl):
     want = oracle.addmm_f64_sampled(rows, cols, 0.5, View.contiguous(c), 1.0, View.contiguous(a), View.contiguous(b))
     scale = float(np.sqrt(np.mean(want ** 2)))
     assert np.max(np.abs(got[rows, cols] - want)) / scale < 1e-4
+    # whole 128x128 output tiles (the kernel's block tile), every entry against fp64 accumulation: the two corners,
+    # an interior tile, and the two tiles either side of the seam between the first and second of the eight runs
+    # of 512 blocks that the kernel's block renumbering hands to the XCDs (the row-major result is the kernel's
+    # column-major one transposed, so its tile (m 7, n 63) is rows 63*128.., columns 7*128.. here)
+    for tr, tc in ((0, 0), (63, 63), (29, 41), (63, 7), (0, 8)):
+        r0, c0 = tr * 128, tc * 128
+        wt = oracle.addmm_f64(0.5, View.contiguous(c[r0:r0 + 128, c0:c0 + 128].copy()), 1.0,
+                              View.contiguous(a[r0:r0 + 128].copy()), View.contiguous(b[:, c0:c0 + 128].copy()))
+        assert np.max(np.abs(got[r0:r0 + 128, c0:c0 + 128] - wt)) / scale < 1e-4, (tr, tc)
     # checksum of checksums: ones^T (A B) ones == (ones^T A)(B ones), in fp64 from the device result
     lhs = got.astype(np.float64).sum() - 0.5 * c.astype(np.float64).sum()
     rhs = float(a.astype(np.float64).sum(axis=0) @ b.astype(np.float64).sum(axis=1))
@@ -245,9 +282,8 @@ def test_released_blocks_are_reused_without_stalling_or_mixing_owners(cl):
 
 
 def test_pinned_host_arrays(cl):
-    """Page-locked host arrays: a round trip through a tensor is exact, views keep the allocation
-    alive, and the transfer runs faster than the pageable one."""
-    import time
+    """Page-locked host arrays: a round trip through a tensor is exact and views keep the allocation
+    alive.  (Transfer rates are a measurement, not a parity property: bench.py reports them.)"""
     n = 1 << 26
     p = cl.pinned_array((n,))
     p[:] = np.arange(n, dtype=F) % 1000
@@ -270,12 +306,5 @@ def test_pinned_host_arrays(cl):
     d2h(view)
     assert np.array_equal(view, p)
     pageable = np.zeros(n, dtype=F)
-    rates = {}
-    for name, arr in (("pinned", view), ("pageable", pageable)):
-        best = 0.0
-        for _ in range(3):
-            t0 = time.perf_counter()
-            d2h(arr)
-            best = max(best, 4 * n / (time.perf_counter() - t0) * 1e-9)
-        rates[name] = best
-    assert rates["pinned"] > 1.2 * rates["pageable"], rates
+    d2h(pageable)
+    assert np.array_equal(pageable, p)
