@@ -127,6 +127,9 @@ enum ThclReduce : int {
 void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out);
 void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *src, long dim);
 void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent = 0.f);
+// The variant for callers that cannot allocate: tickets and partials in a static device array.
+void thcl_reduce_all_noalloc(THClState *state, ThclReduce kind, THClTensor *src, float *out);
+void thcl_reduce_static_setup(int device);  // once per device, with that device current
 // along `dim`; `values` resized to size 1 along dim; idx outputs optional:
 // idx_f32 = fp32 device buffer of 1-based positions laid out like `values`,
 // idx_i64 = contiguous int64 device buffer.

@@ -540,6 +540,21 @@ void THClTensor_sumall_gpu(THClState *state, THClTensor *self, THClTensor *src) 
   reduce_all_to_point(state, RED_SUM, self, src);
   THCL_GUARD_END()
 }
+// The variant that allocates nothing.  It stays clear of the guard macros and of thcl_ctx, both of
+// which may create or destroy profiling events.
+void THClTensor_sumall_gpu_noalloc(THClState *state, THClTensor *self, THClTensor *src) {
+  thcl_clear_error();
+  try {
+    THCL_CHECK(state && self && src, "NULL argument");
+    thcl_check_same_device(state, 2, self, src);
+    THCL_CHECK(self != src, "result and source must be different tensors");
+    THCL_CHECK(self->nDimension == 0 && self->storage != nullptr && self->storage->wrapper != nullptr,
+               "the result must already be a point tensor that owns its storage: this entry point allocates nothing");
+    thcl_reduce_all_noalloc(state, RED_SUM, src, thcl_dptr(self));
+  } catch (const std::exception &e) {
+    thcl_report(e.what());
+  }
+}
 void THClTensor_prodall_gpu(THClState *state, THClTensor *self, THClTensor *src) {
   THCL_GUARD_BEGIN
   reduce_all_to_point(state, RED_PROD, self, src);

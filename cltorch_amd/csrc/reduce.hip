@@ -807,12 +807,54 @@ bool aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 }  // namespace
 
 // ----------------------------------------------------------------- reduce all
+// Tickets and partials of the entry point that allocates nothing live in this
+// array instead of the context's scratch block: 256 bytes of tickets, then
+// kStaticSlots 8-byte partials.  Every device the library runs on holds its own
+// copy, zero at load; the kernels leave the ticket at zero when they finish.
+constexpr size_t kStaticTicketBytes = 256;
+constexpr long kStaticSlots = 2048;
+constexpr size_t kStaticScratchBytes = kStaticTicketBytes + (size_t)kStaticSlots * sizeof(double);
+constexpr int kStaticMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+namespace {
+// the array's address on each device (hipGetSymbolAddress); in host code the name `scratch` is not one
+void *g_static_scratch[kStaticMaxDevices] = {nullptr};
+}  // namespace
+
+// Called once per device when its context is opened; makes that device current for the look-up.
+void thcl_reduce_static_setup(int device) {
+  THCL_CHECK(device >= 0 && device < kStaticMaxDevices, "device %d out of range", device);
+  if (g_static_scratch[device]) return;
+  int prev = -1;
+  hipError_t e = hipGetDevice(&prev);
+  if (e == hipSuccess && prev != device) e = hipSetDevice(device);  // each device holds its own copy at its own address
+  THCL_CHECK(e == hipSuccess, "making device %d current: %s", device, hipGetErrorString(e));
+  void *ptr = nullptr;
+  e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e == hipSuccess && ptr != nullptr) e = hipMemset(ptr, 0, kStaticScratchBytes);
+  if (prev >= 0 && prev != device) (void)hipSetDevice(prev);
+  THCL_CHECK(e == hipSuccess && ptr != nullptr, "static scratch of device %d (hipGetSymbolAddress / clearing it): %s", device,
+             hipGetErrorString(e));
+  g_static_scratch[device] = ptr;
+}
+
+namespace {
+// where one whole-tensor reduction keeps its tickets and partials
+struct ReduceAllScratch {
+  unsigned *ticket;
+  void *partials;
+  long slots;  // 8-byte partials
+};
+
+void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, float *out, float exponent,
+                       const ReduceAllScratch &S);
+}  // namespace
+
 void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent) {
   const long n = THClTensor_nElement(state, src);
   THCL_CHECK(src->nDimension <= THCL_MAX_DIMS, THCL_DIM_WARNING);
   int device = THClTensor_getDevice(state, src);
   thcl_rt *rt = thcl_ctx(state, device);
-  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   if (n == 0) {  // nothing to fold: the identity element
     thcl_fill_contig(rt, out, init_value(kind), 1);
     thcl_after_launch(state, rt);
@@ -820,13 +862,53 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
   }
   THCL_CHECK(src->storage && src->storage->wrapper, "tensor has no device storage");
   size_t sbytes = 0;
-  char *scratch = (char *)thcl_rt_scratch(rt, &sbytes);
+  char *block = (char *)thcl_rt_scratch(rt, &sbytes);
+  ReduceAllScratch S;
+  S.ticket = (unsigned *)(block + kTicketOff);
+  S.partials = block + kPartialOff;
+  S.slots = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
+  reduce_all_launch(rt, kind, src, n, out, exponent, S);
+  thcl_after_launch(state, rt);
+}
+
+// The same reduction with its tickets and partials in the static array: no device memory is
+// requested or released, no event is created, nothing is booked by the profiler.  The device's
+// context must already be open (opening one allocates).
+void thcl_reduce_all_noalloc(THClState *state, ThclReduce kind, THClTensor *src, float *out) {
+  const long n = THClTensor_nElement(state, src);
+  THCL_CHECK(src->nDimension <= THCL_MAX_DIMS, THCL_DIM_WARNING);
+  THCL_CHECK(n <= THCL_NOALLOC_MAX_ELEMENTS,
+             "this entry point takes at most %ld elements (the tensor has %ld): use the allocating form",
+             (long)THCL_NOALLOC_MAX_ELEMENTS, n);
+  const int device = THClTensor_getDevice(state, src);
+  THCL_CHECK(state && state->initialized && device >= 0 && device < state->allocatedDevices && device < kStaticMaxDevices &&
+                 state->clByDevice[device] != nullptr && g_static_scratch[device] != nullptr,
+             "device %d has not been opened yet, and opening it allocates: make any other call on it first", device);
+  thcl_rt *rt = state->clByDevice[device];
+  if (n == 0) {
+    thcl_fill_contig(rt, out, init_value(kind), 1);
+  } else {
+    THCL_CHECK(src->storage && src->storage->wrapper, "tensor has no device storage");
+    char *block = (char *)g_static_scratch[device];
+    ReduceAllScratch S;
+    S.ticket = (unsigned *)block;
+    S.partials = block + kStaticTicketBytes;
+    S.slots = kStaticSlots;
+    reduce_all_launch(rt, kind, src, n, out, 0.f, S);
+  }
+  if (state->addFinish) THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
+}
+
+namespace {
+void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, float *out, float exponent,
+                       const ReduceAllScratch &S) {
+  hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   ReduceAllParams P;
   memset(&P, 0, sizeof(P));
   P.in = thcl_dptr(src);
   P.n = (thcl_u64)n;
-  P.partials = scratch + kPartialOff;
-  P.ticket = (unsigned *)(scratch + kTicketOff);
+  P.partials = S.partials;
+  P.ticket = S.ticket;
   P.out = out;
   P.exponent = exponent;
   // The order in which elements are folded is free, so the view is walked in memory order: dims sorted
@@ -854,8 +936,7 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
   // dense: two resident blocks per CU keep HBM busy (fewer blocks, fewer tickets); strided walks read
   // 4 bytes per lane and need more of them in flight
   long cap = (long)cus * (dense ? 2 : 8);
-  const long max_partials = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
-  if (cap > max_partials) cap = max_partials;
+  if (cap > S.slots) cap = S.slots;
   unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));
   switch (kind) {
     case RED_SUM: launch_all<RED_SUM>(dense, grid, stream, P); break;
@@ -870,8 +951,8 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
     case RED_ANY: launch_all<RED_ANY>(dense, grid, stream, P); break;
   }
   check_launch("reduce-all");
-  thcl_after_launch(state, rt);
 }
+}  // namespace
 
 // out[0] = sum a[i] * b[i], both dense with n elements
 void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out) {

@@ -291,6 +291,7 @@ thcl_rt *thcl_ctx(THClState *state, int device) {
   if (!state->clByDevice[device]) {
     thcl_rt *rt = thcl_rt_get(device);
     THCL_CHECK(rt != nullptr, "cannot open device %d: %s", device, thcl_rt_error());
+    thcl_reduce_static_setup(device);
     state->clByDevice[device] = rt;
     state->deviceInfoByDevice[device] = (void *)thcl_rt_get_props(rt);
     auto *sp = (THClScratchSpace *)calloc(1, sizeof(THClScratchSpace));

@@ -470,6 +470,19 @@ void THClTensor_prodall_gpu(THClState *state, THClTensor *self, THClTensor *src)
 void THClTensor_maxall_gpu(THClState *state, THClTensor *self, THClTensor *src);
 void THClTensor_minall_gpu(THClState *state, THClTensor *self, THClTensor *src);
 float THClTensor_as_float(THClState *state, THClTensor *self);
+/* THClTensor_sumall_gpu for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it).  No counterpart in the reference.
+ * Requests and releases no device memory and creates no event: the kernel's arrival
+ * ticket and per-block partials live in a static device array of 16.25 KiB that every
+ * GPU the library runs on holds until the process ends, in place of the context's scratch
+ * block.  `self` must already be a point tensor that owns its storage (it is not
+ * resized), the device's context must already be open (any earlier call on that device
+ * opens it), and `src` may have any layout with at most THCL_NOALLOC_MAX_ELEMENTS
+ * elements; anything else is reported as an error and nothing is launched.  Same kernel,
+ * same grid and same result as THClTensor_sumall_gpu.  All calls on one GPU share its
+ * array: calls that overlap on one GPU (two host threads) race. */
+#define THCL_NOALLOC_MAX_ELEMENTS 2147483647L
+void THClTensor_sumall_gpu_noalloc(THClState *state, THClTensor *self, THClTensor *src);
 
 void THClTensor_sum(THClState *state, THClTensor *self, THClTensor *src, long dim);
 void THClTensor_prod(THClState *state, THClTensor *self, THClTensor *src, long dim);

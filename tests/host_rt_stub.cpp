@@ -117,6 +117,8 @@ void THClTensor_copy(THClState *, THClTensor *dst, THClTensor *src) {
 }
 }
 
+void thcl_reduce_static_setup(int) {}  // device-side set-up of the reduction kernels: nothing to do on the host
+
 void thcl_fill_contig(thcl_rt *, float *dst, float value, long n) {
   for (long i = 0; i < n; i++) dst[i] = value;
 }
