@@ -125,9 +125,14 @@ def main():
     ap.add_argument("--no-detail", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-log2n", type=int, default=27)
-    ap.add_argument("--pmc-workload", action="store_true",
-                    help="run each headline kernel twice plus a same-size copy (counter calibration) and exit; "
-                         "meant to run under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --kernel-trace`")
+    ap.add_argument("--pmc-configs", action="store_true",
+                    help="run every configuration's operations 1 + 3 times each behind marker launches and exit; meant to run "
+                         "under `rocprofv3 --kernel-trace [--pmc FETCH_SIZE | --pmc WRITE_SIZE]`; writes --manifest")
+    ap.add_argument("--manifest", default=os.path.join(ROOT, "gpurun_out", "pmc_configs_manifest.json"))
+    ap.add_argument("--summarise", nargs=3, metavar=("TRACE_DB", "FETCH_DB", "WRITE_DB"),
+                    help="print the text summary of three rocprofv3 runs of --pmc-configs (no GPU needed)")
+    ap.add_argument("--summarise-trace", metavar="TRACE_DB", help="print per-kernel totals of a --kernel-trace --stats run of this script")
+    ap.add_argument("--summarise-mfma", metavar="PMC_DB", help="print the matrix-core duty summary of a --pmc-gemm counter run")
     ap.add_argument("--pmc-gemm", action="store_true",
                     help="run the two addmm configurations a few times and exit; meant to run under "
                          "`rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE --kernel-trace`")
@@ -136,10 +141,25 @@ def main():
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.summarise:
+        r = "$R"
+        cmds = [f"rocprofv3 --kernel-trace --stats -d {r}/gpurun_out/cfg_trace -o t -- python3 {r}/bench.py --pmc-configs",
+                f"rocprofv3 --pmc FETCH_SIZE --kernel-trace -d {r}/gpurun_out/cfg_fetch -o f -- python3 {r}/bench.py --pmc-configs",
+                f"rocprofv3 --pmc WRITE_SIZE --kernel-trace -d {r}/gpurun_out/cfg_write -o w -- python3 {r}/bench.py --pmc-configs",
+                "python3 bench.py --summarise gpurun_out/cfg_trace/t_results.db gpurun_out/cfg_fetch/f_results.db "
+                "gpurun_out/cfg_write/w_results.db > " + PROFILE_SUMMARY]
+        sys.stdout.write(summarise(*args.summarise, args.manifest, cmds))
+        return
+    if args.summarise_trace:
+        sys.stdout.write(summarise_trace(args.summarise_trace))
+        return
+    if args.summarise_mfma:
+        sys.stdout.write(summarise_mfma(args.summarise_mfma))
+        return
     import cltorch_amd as cl
     import oracle
-    if args.pmc_workload:
-        return pmc_workload(cl, 1 << args.log2n)
+    if args.pmc_configs:
+        return pmc_configs(cl, oracle, 1 << args.log2n, args.manifest)
     if args.pmc_gemm:
         return pmc_gemm(cl, oracle)
     T = Timers(cl)
@@ -172,6 +192,8 @@ def main():
         k["frac_of_peak"] = round(k["achieved"] / HBM_PEAK_GBS, 4)
     value = 48.0 * n / (ms_per_step * 1e-3) * 1e-9
     dom = kernels["map2"]
+    prof = committed_profile()
+    map2_prof = prof.get("ops", {}).get("c1_map2") if prof.get("elements") == n else None
     out = {
         "metric": "effective HBM GB/s (% of peak) for apply/reduce; fp32 addmm TFLOP/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -184,9 +206,10 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "thcl_expr3_d6642be2_contig_v4 (the map2 expression, 3 operands)",
                      "achieved": dom["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom["achieved"] / HBM_PEAK_GBS, 4),
-                     # HBM bytes per launch from rocprofv3 FETCH_SIZE/WRITE_SIZE, calibrated on a copy kernel
-                     # (profiles/headline_kernels_2p28_pmc_traffic.txt): 15.999 bytes/element at 2^28 elements
-                     "traffic": int(round(15.999 * n)) if args.log2n == 28 else None,
+                     # HBM bytes per launch: rocprofv3 FETCH_SIZE + WRITE_SIZE scaled on a dense copy of known size, read
+                     # from the committed summary of the counter runs (null when that summary covers another size)
+                     "traffic": (map2_prof["read_bytes"] + map2_prof["written_bytes"]) if map2_prof else None,
+                     "traffic_source": (PROFILE_SUMMARY + " (operation c1_map2)") if map2_prof else None,
                      "algorithmic_bytes_per_launch": 16 * n, "avg_launch_ms": dom["avg_ms"]},
         "kernels": kernels,
     }
@@ -219,52 +242,161 @@ def pmc_gemm(cl, oracle):
     print(json.dumps({"pmc_gemm": "done"}))
 
 
-def pmc_workload(cl, n):
-    """Launches for hardware-counter runs: a copy between the two halves of one
-    storage (runs the library's dense copy kernel: reads 4n bytes, writes 4n
-    bytes -- the calibration point for FETCH_SIZE / WRITE_SIZE) and the five
-    kernels of the headline step, twice."""
-    rng = np.random.RandomState(0)
-    x = rng.uniform(-1, 1, n).astype(np.float32)
-    X, Y, Z = cl.ClTensor(x), cl.ClTensor(x[::-1].copy()), cl.ClTensor(np.abs(x))
-    W = cl.ClTensor(2 * n)
-    lo, hi = W.narrow(1, 1, n), W.narrow(1, n + 1, n)
-    lo.copy(X)
+def config_ops(cl, oracle, X, Y, Z, n):
+    """The operations of the other configurations and of the callers either side of the path, as a
+    generator of (name, fn, work, unit, reps, peak).  Tensors of a group are created when the
+    generator reaches it and released when it moves on; ``work`` is algorithmic bytes or flops."""
+    H, M = HBM_PEAK_GBS, FP32_MFMA_PEAK_TFLOPS
+    lg = int(np.log2(n))
+    # config 4: reduce-all into a point tensor, then pointwise ops fed by it, no host sync in between
     pt = cl.ClTensor()
-    for _ in range(2):
-        hi.copy(lo)
-        X.add(Y)
-        X.cmul(Y)
-        X.map2_on_gpu(Y, Z, EXPR)
-        pt.sum(X)
-        pt.max(X)
-    cl.synchronize()
-    print(json.dumps({"pmc_workload": "done", "elements": n}))
+    A = X
+    A.copy(cl.ClTensor(oracle.uniform(7, n, 0.0, 1.0)))
+    yield ("c4_sumall_gpu_2^%d" % lg, lambda: pt.sum(A), 4 * n, "GB/s", 20, H)
+    yield ("c4_div_point_tensor", lambda: A.div(pt) and pt.sum(A), 12 * n, "GB/s", 20, H)   # div (8 B) + the sum that feeds the next div (4 B)
+    yield ("c1_fill", lambda: A.fill(0.5), 4 * n, "GB/s", 20, H)
+
+    # config 2: strided views of a 512x512x256 tensor
+    m = 512 * 512 * 256
+    a = cl.ClTensor(oracle.uniform(4, m)).resize(512, 512, 256)
+    b = cl.ClTensor(oracle.uniform(5, m)).resize(512, 512, 256)
+    aT, bT = a.transpose(1, 3), b.transpose(1, 3)
+    yield ("c2_map_transposed_views", lambda: aT.map_on_gpu(bT, "x = 1000*x + y*10"), 12 * m, "GB/s", 20, H)
+    dst = cl.ClTensor(256, 512, 512)
+    yield ("c2_copy_transposed_to_dense", lambda: dst.copy(aT), 8 * m, "GB/s", 20, H)
+    aS = a.strided((512, 512, 128), (131072, 256, 2))
+    bS = b.strided((512, 512, 128), (131072, 256, 2))
+    yield ("c2_map_stride2_views", lambda: aS.map_on_gpu(bS, "x = 1000*x + y*10"), 12 * (m // 2), "GB/s", 20, H)
+    dS = cl.ClTensor(512, 512, 128)
+    yield ("c2_copy_stride2_to_dense", lambda: dS.copy(aS), 8 * (m // 2), "GB/s", 20, H)
+    aN, bN = a.narrow(3, 65, 128), b.narrow(3, 65, 128)
+    yield ("c2_map_narrow_views", lambda: aN.map_on_gpu(bN, "x = 1000*x + y*10"), 12 * (m // 2), "GB/s", 20, H)
+    del a, b, aT, bT, aS, bS, aN, bN, dst, dS
+
+    # config 3: reductions along each dim of 4096 x 16384; the Lua-style call returns new tensors, the
+    # `res:sum(src, dim)` form writes into tensors that exist
+    r, c = 4096, 16384
+    G = cl.ClTensor(oracle.normal(6, r * c)).resize(r, c)
+    rv, ri = cl.ClTensor(), cl.ClTensor()
+    for dim, nout in ((1, c), (2, r)):
+        yield (f"c3_sum_dim{dim}", lambda: G.sum(dim), 4 * r * c + 4 * nout, "GB/s", 20, H)
+        yield (f"c3_max_dim{dim}", lambda: G.max(dim), 4 * r * c + 8 * nout, "GB/s", 20, H)
+        yield (f"c3_min_dim{dim}", lambda: G.min(dim), 4 * r * c + 8 * nout, "GB/s", 20, H)
+        yield (f"c3_sum_dim{dim}_into_existing", lambda: rv.sum(G, dim), 4 * r * c + 4 * nout, "GB/s", 20, H)
+        yield (f"c3_max_dim{dim}_into_existing", lambda: rv.max(ri, G, dim), 4 * r * c + 8 * nout, "GB/s", 20, H)
+    del G, rv, ri
+
+    # config 5: addmm
+    k = 8192
+    sd = 1.0 / np.sqrt(k)
+    Am, Bm, Cm = (cl.ClTensor(oracle.normal(s, k * k, 0.0, sd)).resize(k, k) for s in (8, 9, 10))
+    yield ("c5_addmm_8192", lambda: Cm.addmm(0.5, 1.0, Am, Bm), 2.0 * k ** 3, "TFLOP/s", 10, M)
+    del Am, Bm, Cm
+    Ms, Ns, Ks = 64, 16384, 4096
+    At = cl.ClTensor(oracle.normal(11, Ks * Ms, 0.0, sd)).resize(Ks, Ms)
+    Bs = cl.ClTensor(oracle.normal(12, Ks * Ns, 0.0, sd)).resize(Ks, Ns)
+    Cs = cl.ClTensor(oracle.normal(13, Ms * Ns, 0.0, sd)).resize(Ms, Ns)
+    yield ("c5_addmm_skinny_64x16384x4096", lambda: Cs.addmm(0.5, 1.0, At.t(), Bs), 2.0 * Ms * Ns * Ks, "TFLOP/s", 20, M)
+    del At, Bs, Cs
+
+    # ---- the callers either side of the path: operator catalogue, scans, level-1/2, indexed movement
+    A.fill(0.75)
+    B = Y
+    yield ("w_clamp_2^%d" % lg, lambda: A.clamp(-0.5, 0.5), 8 * n, "GB/s", 20, H)
+    yield ("w_lt_tensor", lambda: Z.lt(A, B), 12 * n, "GB/s", 20, H)
+    yield ("w_norm2_to_host", lambda: A.norm(2.0), 4 * n, "GB/s", 20, H)
+    yield ("w_dot_to_host", lambda: A.dot(B), 8 * n, "GB/s", 20, H)
+    yield ("w_cumsum_1d", lambda: Z.cumsum(A, 1), 8 * n, "GB/s", 20, H)
+    G = cl.ClTensor(4096 * 16384).resize(4096, 16384)
+    G.fill(0.5)
+    R = cl.ClTensor(4096, 16384)
+    for dim in (1, 2):
+        yield (f"w_cumsum_4096x16384_dim{dim}", lambda: R.cumsum(G, dim), 8 * 4096 * 16384, "GB/s", 20, H)
+    del R, G
+    q = 16384
+    Mq = cl.ClTensor(q * q).resize(q, q)
+    Mq.fill(0.01)
+    v, y = cl.ClTensor(q), cl.ClTensor(q)
+    v.fill(1.0)
+    y.fill(0.0)
+    yield ("w_addmv_rowmajor_16384", lambda: y.addmv(0.0, 1.0, Mq, v), 4 * q * q, "GB/s", 20, H)
+    yield ("w_addmv_colmajor_16384", lambda: y.addmv(0.0, 1.0, Mq.t(), v), 4 * q * q, "GB/s", 20, H)
+    yield ("w_addr_16384", lambda: Mq.addr(1.0, 0.5, v, y), 8 * q * q, "GB/s", 20, H)
+    del Mq
+    rows, width, cnt = 100000, 1024, 65536
+    rs = np.random.RandomState(0)
+    tab = cl.ClTensor(rows * width).resize(rows, width)
+    tab.fill(1.0)
+    idx = cl.ClTensor(rs.randint(1, rows + 1, size=cnt).astype(np.float32))
+    sel = cl.ClTensor(cnt, width)
+    yield ("w_indexSelect_rows_65536x1024", lambda: sel.index(tab, 1, idx), 8 * cnt * width, "GB/s", 20, H)
+    yield ("w_indexCopy_rows_65536x1024", lambda: tab.indexCopy(1, idx, sel), 8 * cnt * width, "GB/s", 20, H)
+    del tab, sel
+    # shapes that leave a plain slice-per-block or element-order walk idle: few long slices, a handful of
+    # columns, a whole-tensor sum over a transposed view, a ragged product
+    few = cl.ClTensor(64 << 20).resize(64, 1 << 20)
+    few.fill(0.5)
+    res = cl.ClTensor()
+    yield ("w_sum_dim2_64x2^20", lambda: res.sum(few, 2), 4 * (64 << 20), "GB/s", 20, H)
+    yield ("w_max_dim2_64x2^20", lambda: few.max(2), 4 * (64 << 20), "GB/s", 20, H)
+    tall = few.resize(1 << 24, 4)
+    yield ("w_sum_dim1_2^24x4", lambda: res.sum(tall, 1), 4 * (64 << 20), "GB/s", 20, H)
+    sq = tall.resize(8192, 8192).t()
+    yield ("w_sumall_transposed_8192^2", lambda: res.sum(sq), 4 * (64 << 20), "GB/s", 20, H)
+    del few, tall, sq
+    ra, rb, rc = cl.ClTensor(3000, 7000), cl.ClTensor(7000, 5000), cl.ClTensor(3000, 5000)
+    ra.fill(0.01)
+    rb.fill(0.02)
+    rc.fill(0.0)
+    yield ("w_addmm_3000x5000x7000", lambda: rc.addmm(0.0, 1.0, ra, rb), 2.0 * 3000 * 5000 * 7000, "TFLOP/s", 6, M)
+    del ra, rb, rc
+    mask = cl.ClTensor((rs.rand(1 << 26) > 0.5).astype(np.float32))
+    src = cl.ClTensor(1 << 26)
+    src.fill(1.0)
+    packed = cl.ClTensor()
+    # algorithmic bytes: mask and source read once, half of the source written (the call also
+    # waits for the count, which sizes the result)
+    yield ("w_maskedSelect_2^26_half", lambda: packed.maskedSelect(src, mask), (4 + 4 + 2) * (1 << 26), "GB/s", 20, H)
 
 
 def detail(cl, oracle, T, X, Y, Z, n):
-    """The other benchmark configurations, a few launches each."""
+    """The other benchmark configurations, a few launches each.  Per operation: ``avg_ms`` etc. come from
+    one HIP-event pair per call (the pair's own packets sit between the calls); ``back_to_back_ms`` is one
+    pair around all the calls divided by their number, which is what a caller that just keeps calling
+    sees; ``kernel_only_ms`` is the sum of the call's kernel durations in the committed rocprofv3 trace."""
     d = {}
-    reps = 20
-
-    def measure(name, fn, work, unit="GB/s", reps=reps, peak=HBM_PEAK_GBS):
+    profiled = committed_profile()
+    for name, fn, work, unit, reps, peak in config_ops(cl, oracle, X, Y, Z, n):
         fn()
         cl.synchronize()
         for _ in range(reps):
             T.timed(name, fn)
         cl.synchronize()
         s = stats(T.collect()[name], work, unit)
+        T.timed(name, lambda: [fn() for _ in range(reps)])
+        cl.synchronize()
+        b2b = T.collect()[name][0] / reps
+        s["back_to_back_ms"] = round(b2b, 4)
+        s["achieved_back_to_back"] = round(work / (b2b * 1e-3) * (1e-9 if unit == "GB/s" else 1e-12), 1)
         s["frac_of_peak"] = round(s["achieved"] / peak, 4)
+        s["frac_of_peak_back_to_back"] = round(s["achieved_back_to_back"] / peak, 4)
+        p = profiled.get("ops", {}).get(name)
+        if p:
+            s["kernel_only_ms"] = round(p["kernel_us"] * 1e-3, 4)
+            s["frac_of_peak_kernel_only"] = round(work / (p["kernel_us"] * 1e-6) * (1e-9 if unit == "GB/s" else 1e-12) / peak, 4)
         d[name] = s
+    if profiled:
+        d["kernel_only_source"] = PROFILE_SUMMARY + " (rocprofv3 --kernel-trace of `bench.py --pmc-configs`, committed)"
+    sk = d["c5_addmm_skinny_64x16384x4096"]
+    sk["hbm_GBs"] = round(4.0 * (64 * 4096 + 4096 * 16384 + 2 * 64 * 16384) / (sk["avg_ms"] * 1e-3) * 1e-9, 1)
 
-    # config 4: reduce-all into a point tensor, then pointwise ops fed by it, no host sync in between
+    # config 4 as one chain: sumall_gpu + div_gpu + 8 in-place ops, one sync at the end
     pt = cl.ClTensor()
     A = X
     A.copy(cl.ClTensor(oracle.uniform(7, n, 0.0, 1.0)))
-    measure("c4_sumall_gpu_2^%d" % int(np.log2(n)), lambda: pt.sum(A), 4 * n)
-    measure("c4_div_point_tensor", lambda: A.div(pt) and pt.sum(A), 12 * n)   # div (8 B) + the sum that feeds the next div (4 B)
     chain = [lambda: A.mul(1.0001), lambda: A.add(0.5), lambda: A.cmul(A), lambda: A.sqrt(), lambda: A.add(pt),
              lambda: A.mul(pt), lambda: A.abs(), lambda: A.csub(0.25)]
+    [f() for f in chain[:1]]
     cl.synchronize()
     t0 = time.perf_counter()
     T.timed("c4_chain_10_launches", lambda: [pt.sum(A), A.div(pt)] + [f() for f in chain])
@@ -274,49 +406,6 @@ def detail(cl, oracle, T, X, Y, Z, n):
     d["c4_chain_10_launches"] = {"gpu_ms": round(ms[0], 3), "wall_ms": round(wall, 3),
                                  "achieved": round((4 + 8 * 9) * n / (ms[0] * 1e-3) * 1e-9, 1), "unit": "GB/s",
                                  "note": "sumall_gpu + div_gpu + 8 in-place ops, one sync at the end"}
-    measure("c1_fill", lambda: A.fill(0.5), 4 * n)
-
-    # config 2: strided views of a 512x512x256 tensor
-    m = 512 * 512 * 256
-    a = cl.ClTensor(oracle.uniform(4, m)).resize(512, 512, 256)
-    b = cl.ClTensor(oracle.uniform(5, m)).resize(512, 512, 256)
-    aT, bT = a.transpose(1, 3), b.transpose(1, 3)
-    measure("c2_map_transposed_views", lambda: aT.map_on_gpu(bT, "x = 1000*x + y*10"), 12 * m)
-    dst = cl.ClTensor(256, 512, 512)
-    measure("c2_copy_transposed_to_dense", lambda: dst.copy(aT), 8 * m)
-    aS = a.strided((512, 512, 128), (131072, 256, 2))
-    bS = b.strided((512, 512, 128), (131072, 256, 2))
-    measure("c2_map_stride2_views", lambda: aS.map_on_gpu(bS, "x = 1000*x + y*10"), 12 * (m // 2))
-    dS = cl.ClTensor(512, 512, 128)
-    measure("c2_copy_stride2_to_dense", lambda: dS.copy(aS), 8 * (m // 2))
-    aN, bN = a.narrow(3, 65, 128), b.narrow(3, 65, 128)
-    measure("c2_map_narrow_views", lambda: aN.map_on_gpu(bN, "x = 1000*x + y*10"), 12 * (m // 2))
-    del a, b, aT, bT, aS, bS, aN, bN, dst, dS
-
-    # config 3: reductions along each dim of 4096 x 16384
-    r, c = 4096, 16384
-    G = cl.ClTensor(oracle.normal(6, r * c)).resize(r, c)
-    for dim, nout in ((1, c), (2, r)):
-        measure(f"c3_sum_dim{dim}", lambda: G.sum(dim), 4 * r * c + 4 * nout)
-        measure(f"c3_max_dim{dim}", lambda: G.max(dim), 4 * r * c + 8 * nout)
-        measure(f"c3_min_dim{dim}", lambda: G.min(dim), 4 * r * c + 8 * nout)
-    del G
-
-    # config 5: addmm
-    k = 8192
-    sd = 1.0 / np.sqrt(k)
-    Am, Bm, Cm = (cl.ClTensor(oracle.normal(s, k * k, 0.0, sd)).resize(k, k) for s in (8, 9, 10))
-    measure("c5_addmm_8192", lambda: Cm.addmm(0.5, 1.0, Am, Bm), 2.0 * k ** 3, "TFLOP/s", reps=10, peak=FP32_MFMA_PEAK_TFLOPS)
-    del Am, Bm, Cm
-    M, N, K = 64, 16384, 4096
-    At = cl.ClTensor(oracle.normal(11, K * M, 0.0, sd)).resize(K, M)
-    Bs = cl.ClTensor(oracle.normal(12, K * N, 0.0, sd)).resize(K, N)
-    Cs = cl.ClTensor(oracle.normal(13, M * N, 0.0, sd)).resize(M, N)
-    measure("c5_addmm_skinny_64x16384x4096", lambda: Cs.addmm(0.5, 1.0, At.t(), Bs), 2.0 * M * N * K, "TFLOP/s",
-            peak=FP32_MFMA_PEAK_TFLOPS)
-    d["c5_addmm_skinny_64x16384x4096"]["hbm_GBs"] = round(
-        4.0 * (M * K + K * N + 2 * M * N) / (d["c5_addmm_skinny_64x16384x4096"]["avg_ms"] * 1e-3) * 1e-9, 1)
-    del At, Bs, Cs
 
     # the reference's own perf script times 900 calls of cmul / add / sum on 6400- and 64000-element
     # tensors (src/test/test-perf.lua:43-106): per-call cost where launches, not bytes, dominate
@@ -336,67 +425,232 @@ def detail(cl, oracle, T, X, Y, Z, n):
             lat[f"{name}_{m_small}"] = round((time.perf_counter() - t0) / 900 * 1e6, 2)
     d["small_tensor_us_per_call"] = dict(lat, note="900 calls through the Python mirror, one synchronisation at the end "
                                                    "(sum_to_host waits for every result)")
-
-    # ---- the callers either side of the path: operator catalogue, scans, level-1/2, indexed movement
-    A.fill(0.75)
-    B = Y
-    measure("w_clamp_2^%d" % int(np.log2(n)), lambda: A.clamp(-0.5, 0.5), 8 * n)
-    measure("w_lt_tensor", lambda: Z.lt(A, B), 12 * n)
-    measure("w_norm2_to_host", lambda: A.norm(2.0), 4 * n)
-    measure("w_dot_to_host", lambda: A.dot(B), 8 * n)
-    measure("w_cumsum_1d", lambda: Z.cumsum(A, 1), 8 * n)
-    G = cl.ClTensor(4096 * 16384).resize(4096, 16384)
-    G.fill(0.5)
-    R = cl.ClTensor(4096, 16384)
-    for dim in (1, 2):
-        measure(f"w_cumsum_4096x16384_dim{dim}", lambda: R.cumsum(G, dim), 8 * 4096 * 16384)
-    del R
-    q = 16384
-    Mq = cl.ClTensor(q * q).resize(q, q)
-    Mq.fill(0.01)
-    v, y = cl.ClTensor(q), cl.ClTensor(q)
-    v.fill(1.0)
-    y.fill(0.0)
-    measure("w_addmv_rowmajor_16384", lambda: y.addmv(0.0, 1.0, Mq, v), 4 * q * q)
-    measure("w_addmv_colmajor_16384", lambda: y.addmv(0.0, 1.0, Mq.t(), v), 4 * q * q)
-    measure("w_addr_16384", lambda: Mq.addr(1.0, 0.5, v, y), 8 * q * q)
-    del Mq
-    rows, width, cnt = 100000, 1024, 65536
-    rs = np.random.RandomState(0)
-    tab = cl.ClTensor(rows * width).resize(rows, width)
-    tab.fill(1.0)
-    idx = cl.ClTensor(rs.randint(1, rows + 1, size=cnt).astype(np.float32))
-    sel = cl.ClTensor(cnt, width)
-    measure("w_indexSelect_rows_65536x1024", lambda: sel.index(tab, 1, idx), 8 * cnt * width)
-    measure("w_indexCopy_rows_65536x1024", lambda: tab.indexCopy(1, idx, sel), 8 * cnt * width)
-    del tab, sel
-    # shapes that leave a plain slice-per-block or element-order walk idle: few long slices, a handful of
-    # columns, a whole-tensor sum over a transposed view, a ragged product
-    few = cl.ClTensor(64 << 20).resize(64, 1 << 20)
-    few.fill(0.5)
-    res = cl.ClTensor()
-    measure("w_sum_dim2_64x2^20", lambda: res.sum(few, 2), 4 * (64 << 20))
-    measure("w_max_dim2_64x2^20", lambda: few.max(2), 4 * (64 << 20))
-    tall = few.resize(1 << 24, 4)
-    measure("w_sum_dim1_2^24x4", lambda: res.sum(tall, 1), 4 * (64 << 20))
-    sq = tall.resize(8192, 8192).t()
-    measure("w_sumall_transposed_8192^2", lambda: res.sum(sq), 4 * (64 << 20))
-    del few, tall, sq
-    ra, rb, rc = cl.ClTensor(3000, 7000), cl.ClTensor(7000, 5000), cl.ClTensor(3000, 5000)
-    ra.fill(0.01)
-    rb.fill(0.02)
-    rc.fill(0.0)
-    measure("w_addmm_3000x5000x7000", lambda: rc.addmm(0.0, 1.0, ra, rb), 2.0 * 3000 * 5000 * 7000, "TFLOP/s", reps=6,
-            peak=FP32_MFMA_PEAK_TFLOPS)
-    del ra, rb, rc
-    mask = cl.ClTensor((rs.rand(1 << 26) > 0.5).astype(np.float32))
-    src = cl.ClTensor(1 << 26)
-    src.fill(1.0)
-    packed = cl.ClTensor()
-    # algorithmic bytes: mask and source read once, half of the source written (the call also
-    # waits for the count, which sizes the result)
-    measure("w_maskedSelect_2^26_half", lambda: packed.maskedSelect(src, mask), (4 + 4 + 2) * (1 << 26))
+    d["host_copy_GBs"] = host_copy_rates(cl)
     return d
+
+
+def host_copy_rates(cl, n=1 << 26):
+    """Device-to-host copies of 256 MiB into page-locked and into ordinary host memory (best of 3)."""
+    from cltorch_amd.tensor import _call
+    lib = cl.state().lib
+    t = cl.ClTensor(n)
+    t.fill(1.0)
+    rates = {}
+    for name, arr in (("pinned", cl.pinned_array((n,))), ("pageable", np.zeros(n, dtype=np.float32))):
+        sz = (C.c_long * 1)(arr.size)
+        ft = lib.THFloatTensor_newWithData(arr.ctypes.data_as(C.c_void_p), arr.size, 0, 1, sz, None)
+        best = 0.0
+        for _ in range(3):
+            t0 = time.perf_counter()
+            _call("THFloatTensor_copyCl", ft, t._h)
+            best = max(best, 4 * n / (time.perf_counter() - t0) * 1e-9)
+        lib.THFloatTensor_free(ft)
+        rates["d2h_" + name] = round(best, 1)
+    return rates
+
+
+# ------------------------------------------------------------------ profiles ---
+PROFILE_SUMMARY = "profiles/bench_pmc_configs_traffic_and_kernel_times.txt"
+
+
+def committed_profile():
+    """The machine-readable line of the committed counter summary (see --summarise), or {}."""
+    path = os.path.join(ROOT, PROFILE_SUMMARY)
+    if not os.path.exists(path):
+        return {}
+    for line in open(path):
+        if line.startswith("json: "):
+            return json.loads(line[6:])
+    return {}
+
+
+def pmc_configs(cl, oracle, n, manifest_path):
+    """Launches for hardware-counter and kernel-trace runs over every configuration: a marker (a fill of
+    7 elements) opens and closes each operation, which runs 1 + 3 times in between; the first call (it may
+    compile) is dropped by the summariser.  The first operation is a dense copy of known size, the calibration point
+    of FETCH_SIZE / WRITE_SIZE.  Writes the list of operations with their algorithmic work to
+    ``manifest_path``."""
+    X, Y, Z = (cl.ClTensor(oracle.uniform(s, n)) for s in (1, 2, 3))
+    W = cl.ClTensor(2 * n)
+    lo, hi = W.narrow(1, 1, n), W.narrow(1, n + 1, n)
+    lo.copy(X)
+    pt = cl.ClTensor()
+    mk = cl.ClTensor(7)
+    ops = [("calibration_copy_2^%d" % int(np.log2(n)), lambda: hi.copy(lo), 8 * n, "GB/s", 3, HBM_PEAK_GBS),
+           ("c1_add", lambda: X.add(Y), 12 * n, "GB/s", 3, HBM_PEAK_GBS),
+           ("c1_cmul", lambda: X.cmul(Y), 12 * n, "GB/s", 3, HBM_PEAK_GBS),
+           ("c1_map2", lambda: X.map2_on_gpu(Y, Z, EXPR), 16 * n, "GB/s", 3, HBM_PEAK_GBS),
+           ("c1_sum", lambda: pt.sum(X), 4 * n, "GB/s", 3, HBM_PEAK_GBS),
+           ("c1_max", lambda: pt.max(X), 4 * n, "GB/s", 3, HBM_PEAK_GBS)]
+    manifest = []
+
+    def run(op):
+        name, fn, work, unit, _, peak = op
+        mk.fill(0.0)
+        for _ in range(4):
+            fn()
+        mk.fill(0.0)              # closes the operation: what follows (the next one's set-up) is not part of it
+        cl.synchronize()
+        manifest.append({"name": name, "work": work, "unit": unit, "peak": peak})
+
+    for op in ops:
+        run(op)
+    del W, lo, hi
+    for op in config_ops(cl, oracle, X, Y, Z, n):
+        run(op)
+    with open(manifest_path, "w") as f:
+        json.dump({"elements": n, "calls_per_op": 4, "ops": manifest}, f)
+    print(json.dumps({"pmc_configs": "done", "ops": len(manifest), "manifest": manifest_path}))
+
+
+def _segments(db_path, want_counters):
+    """Dispatches of a rocprofv3 results database in order, per operation (between two one-block FILL markers)."""
+    import sqlite3
+    c = sqlite3.connect(db_path)
+    rows = {}
+    if want_counters:
+        q = "select dispatch_id, kernel_name, grid_size_x, counter_name, value, duration from counters_collection order by dispatch_id"
+        for did, name, gx, cn, v, dur in c.execute(q):
+            r = rows.setdefault(did, {"name": name, "gx": gx, "dur": dur, "c": {}})
+            r["c"][cn] = r["c"].get(cn, 0.0) + v
+    else:
+        for did, name, gx, dur in c.execute("select dispatch_id, name, grid_x, duration from kernels order by dispatch_id"):
+            rows[did] = {"name": name, "gx": gx, "dur": dur, "c": {}}
+    segs, cur = [], None
+    for did in sorted(rows):
+        r = rows[did]
+        if "FILL" in r["name"] and r["gx"] <= 1024:
+            cur = []
+            segs.append(cur)
+        elif cur is not None:
+            cur.append(r)
+    return segs[0::2]            # a marker opens and another closes every operation: odd segments are set-up in between
+
+
+def _short(name):
+    name = name.replace("void (anonymous namespace)::", "").replace("(anonymous namespace)::", "")
+    i = name.find("(")
+    return name[:i] if i > 0 else name
+
+
+def summarise(trace_db, fetch_db, write_db, manifest_path, commands):
+    """Text summary of three rocprofv3 runs of ``--pmc-configs`` (kernel trace; FETCH_SIZE; WRITE_SIZE)."""
+    man = json.load(open(manifest_path))
+    ops, calls = man["ops"], man["calls_per_op"]
+    tr, fe, wr = _segments(trace_db, False), _segments(fetch_db, True), _segments(write_db, True)
+    assert len(tr) == len(fe) == len(wr) == len(ops), (len(tr), len(fe), len(wr), len(ops))
+    out = ["commands (each run from /tmp with TMPDIR=/tmp; $R is the repository root on the GPU box):"]
+    out += ["  " + c for c in commands]
+    out += ["workload: every operation runs 1 + 3 times behind a marker launch; the first call is dropped, the figures are means",
+            "  of the other three.  Durations come from the --kernel-trace run (no counters), KiB from the two counter runs.", ""]
+
+    def per_call(seg):
+        assert len(seg) % calls == 0, (len(seg), calls)
+        k = len(seg) // calls
+        return k, seg[k:]          # drop the first call
+
+    # calibration on the dense copy: reads and writes 4 bytes per element
+    k, cal_f = per_call(fe[0])
+    _, cal_w = per_call(wr[0])
+    n = man["elements"]
+    want_kib = 4.0 * n / 1024
+    f_read = sum(r["c"].get("FETCH_SIZE", 0.0) for r in cal_f) / (len(cal_f) / k)
+    w_read = sum(r["c"].get("WRITE_SIZE", 0.0) for r in cal_w) / (len(cal_w) / k)
+    fs, ws = want_kib / f_read, want_kib / w_read
+    out += [f"calibration: {_short(cal_f[0]['name'])} on 2^{int(np.log2(n))} elements reads {want_kib:.0f} KiB and writes {want_kib:.0f} KiB;",
+            f"  FETCH_SIZE reports {f_read:.1f} KiB -> scale {fs:.4f}; WRITE_SIZE reports {w_read:.1f} KiB -> scale {ws:.4f}", ""]
+    hdr = "%-34s %-44s %3s %9s %11s %11s %9s %9s %7s %7s" % ("operation", "kernel", "x", "dur_us", "FETCH_KiB", "WRITE_KiB", "read_MiB",
+                                                               "wrote_MiB", "traf/alg", "frac")
+    out += [hdr, "-" * len(hdr)]
+    js = {"elements": n, "fetch_scale": round(fs, 4), "write_scale": round(ws, 4), "ops": {}}
+    for op, st, sf, sw in zip(ops, tr, fe, wr):
+        k, t = per_call(st)
+        _, f = per_call(sf)
+        _, w = per_call(sw)
+        ncalls = len(t) // k if k else 0
+        if not k:
+            out.append("%-34s (no device kernel)" % op["name"])
+            continue
+        tot_us = tot_rd = tot_wr = 0.0
+        lines = []
+        for j in range(k):         # j-th kernel of each call
+            us = np.mean([t[i * k + j]["dur"] for i in range(ncalls)]) / 1e3
+            fk = np.mean([f[i * k + j]["c"].get("FETCH_SIZE", 0.0) for i in range(ncalls)])
+            wk = np.mean([w[i * k + j]["c"].get("WRITE_SIZE", 0.0) for i in range(ncalls)])
+            tot_us += us
+            tot_rd += fk * fs * 1024
+            tot_wr += wk * ws * 1024
+            lines.append((_short(t[j]["name"])[:44], us, fk, wk))
+        is_bw = op["unit"] == "GB/s"
+        ratio = (tot_rd + tot_wr) / op["work"] if is_bw else None
+        frac = op["work"] / (tot_us * 1e-6) * (1e-9 if is_bw else 1e-12) / op["peak"]
+        for j, (kn, us, fk, wk) in enumerate(lines):
+            first = j == 0
+            out.append("%-34s %-44s %3s %9.1f %11.1f %11.1f %9s %9s %7s %7s" % (
+                op["name"][:34] if first else "", kn, "", us, fk, wk,
+                "%.1f" % (tot_rd / 2 ** 20) if first else "", "%.1f" % (tot_wr / 2 ** 20) if first else "",
+                ("%.3f" % ratio if ratio is not None else "-") if first else "", "%.3f" % frac if first else ""))
+        js["ops"][op["name"]] = {"kernel_us": round(tot_us, 2), "read_bytes": int(tot_rd), "written_bytes": int(tot_wr),
+                                 "work": op["work"], "unit": op["unit"], "frac": round(frac, 4)}
+    out += ["", "columns: dur_us = mean kernel duration; FETCH/WRITE_KiB = counter values per dispatch; read/wrote_MiB = scaled HBM bytes of one call;",
+            "  traf/alg = (read + written) / algorithmic bytes of the call; frac = algorithmic work / kernel time / peak (8000 GB/s or 157.3 TFLOP/s).",
+            "json: " + json.dumps(js)]
+    return "\n".join(out) + "\n"
+
+
+def summarise_trace(db_path):
+    """Per-kernel totals of a `rocprofv3 --kernel-trace --stats -- python3 bench.py` run."""
+    import sqlite3
+    c = sqlite3.connect(db_path)
+    rows = list(c.execute("select name, total_calls, total_duration, average, percentage from top_kernels"))
+    extra = {}
+    for name, mn, mx, vg, lds in c.execute("select name, min(duration), max(duration), max(vgpr_count), max(lds_size) from kernels group by name"):
+        extra[name] = (mn, mx, vg, lds)
+    out = ["command (run from /tmp with TMPDIR=/tmp; $R is the repository root on the GPU box):",
+           "  rocprofv3 --kernel-trace --stats -d $R/gpurun_out/bench_trace -o b -- python3 $R/bench.py --no-cpu",
+           "  python3 bench.py --summarise-trace gpurun_out/bench_trace/b_results.db > profiles/bench_all_configs_kernel_trace.txt",
+           "source: view top_kernels of the results database; durations in microseconds", "",
+           "%-84s %6s %12s %10s %10s %10s %6s %6s %7s" % ("kernel", "calls", "total_us", "avg_us", "min_us", "max_us", "pct", "vgpr", "lds")]
+    for name, calls, tot, avg, pct in rows:
+        mn, mx, vg, lds = extra.get(name, (0, 0, 0, 0))
+        out.append("%-84s %6d %12.1f %10.1f %10.1f %10.1f %6.2f %6s %7s" % (_short(name)[:84], calls, tot, avg, mn / 1e3, mx / 1e3, pct, vg, lds))
+    return "\n".join(out) + "\n"
+
+
+def summarise_mfma(db_path):
+    """Matrix-core duty of the addmm launches of ``--pmc-gemm`` from one counter run."""
+    import sqlite3
+    c = sqlite3.connect(db_path)
+    rows = {}
+    q = "select dispatch_id, kernel_name, grid_size_x, grid_size_y, counter_name, value, duration from counters_collection order by dispatch_id"
+    for did, name, gx, gy, cn, v, dur in c.execute(q):
+        r = rows.setdefault(did, {"name": name, "gx": gx, "gy": gy, "dur": dur, "c": {}})
+        r["c"][cn] = r["c"].get(cn, 0.0) + v
+    out = ["command (run from /tmp with TMPDIR=/tmp; $R is the repository root on the GPU box):",
+           "  rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE --kernel-trace -d $R/gpurun_out/pmc_gemm -o g -- python3 $R/bench.py --pmc-gemm",
+           "  python3 bench.py --summarise-mfma gpurun_out/pmc_gemm/g_results.db > profiles/addmm_8192_and_skinny_pmc_mfma_duty.txt",
+           "workload: addmm 8192^3 five times, then addmm 64x16384x4096 (A given transposed) thirty times; fp32, random normal operands", "",
+           "how to read it: every v_mfma_f32_32x32x2_f32 books 64 busy cycles on its SIMD, so flops = busy / 64 * 4096;",
+           "  duty = SQ_VALU_MFMA_BUSY_CYCLES / (1024 SIMDs * GRBM_GUI_ACTIVE / 8 XCDs); clock = GRBM_GUI_ACTIVE / 8 / duration.",
+           "  For kernels shorter than ~0.2 ms GRBM_GUI_ACTIVE also covers some time around the launch, so their clock reads a little",
+           "  high and their duty a little low.  Of the thirty skinny launches every fifth is listed.", "",
+           "%-52s %10s %8s %14s %14s %8s %10s %8s" % ("kernel", "grid", "dur_us", "MFMA_BUSY", "GRBM_ACTIVE", "duty", "clock_GHz", "TFLOP/s")]
+    seen = {}
+    for did in sorted(rows):
+        r = rows[did]
+        if "gemm" not in r["name"]:
+            continue
+        key = _short(r["name"])
+        seen[key] = seen.get(key, 0) + 1
+        big = r["dur"] > 2e6
+        if not big and seen[key] % 5:
+            continue
+        busy, act = r["c"].get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0), max(r["c"].get("GRBM_GUI_ACTIVE", 1.0), 1.0)
+        flops = busy / 64.0 * 4096.0
+        out.append("%-52s %10s %8.1f %14.4g %14.4g %8.3f %10.2f %8.1f" % (
+            key[:52], "%dx%d" % (r["gx"] // 256, r["gy"]), r["dur"] / 1e3, busy, act, busy / 1024.0 / (act / 8.0), act / 8.0 / r["dur"],
+            flops / r["dur"] / 1e3))
+    return "\n".join(out) + "\n"
 
 
 if __name__ == "__main__":

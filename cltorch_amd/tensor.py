@@ -892,6 +892,10 @@ class ClTensor:
             values, indices = ClTensor(), ClTensor()
             _call(f"THClTensor_{name}", values._h, indices._h, self._h, C.c_long(args[0] - 1))
             return values, indices
+        if len(args) == 3 and isinstance(args[0], ClTensor) and isinstance(args[1], ClTensor):
+            # values:max(indices, src, dim): both results into tensors that exist (src/TensorMath.lua:975-988)
+            _call(f"THClTensor_{name}", self._h, args[0]._h, args[1]._h, C.c_long(args[2] - 1))
+            return self, args[0]
         return self._reduce(name, args)
 
     def max(self, *args):
