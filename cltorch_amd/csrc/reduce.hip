@@ -501,16 +501,18 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
 // slices; UB = 64 unless the slices are fewer, then the wave's other lanes take
 // further rows), the 4 waves of a block interleave over the reduced dim and meet in
 // LDS; blockIdx.y splits long reductions, leaving partials for the finisher.
-template <int KIND, bool ARG, int VEC, bool NARROW>
+// GEOM 6 fixes the wave's geometry at compile time (64 units x 1 row); 0 reads it from the launch.
+template <int KIND, bool ARG, int VEC, int GEOM>
 __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
   typedef Slot<KIND, ARG> S;
   typedef typename S::T T;
   constexpr int WAVES = kThreads / kWave;
+  constexpr bool NARROW = GEOM != 6;   // several rows across the wave
   __shared__ T lds[WAVES][kWave * VEC];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  // units and rows across a wave; constants in the common case of 64 units or more
-  const thcl_u32 UB = NARROW ? (1u << P.ub_log2) : (thcl_u32)kWave, RL = NARROW ? ((thcl_u32)kWave >> P.ub_log2) : 1u;
-  const thcl_u32 ul = NARROW ? (lane & (UB - 1)) : (thcl_u32)lane, rl = NARROW ? ((thcl_u32)lane >> P.ub_log2) : 0u;
+  const thcl_u32 ubl = GEOM ? (thcl_u32)GEOM : P.ub_log2;
+  const thcl_u32 UB = 1u << ubl, RL = (thcl_u32)kWave >> ubl;
+  const thcl_u32 ul = lane & (UB - 1), rl = (thcl_u32)lane >> ubl;
   const thcl_u32 ntiles = (P.nunits + UB - 1) / UB;
   const thcl_u32 r_begin = blockIdx.y * P.rows_per_split;
   thcl_u32 r_end = r_begin + P.rows_per_split;
@@ -790,11 +792,17 @@ void launch_dim(bool rows, int lpr, int vec, dim3 grid, hipStream_t stream, cons
     if (vec == 4) hipLaunchKernelGGL((reduce_cols_short<KIND, ARG, 4>), grid, block, 0, stream, P);
     else hipLaunchKernelGGL((reduce_cols_short<KIND, ARG, 1>), grid, block, 0, stream, P);
   } else {
-    const bool narrow = P.ub_log2 < 6;
-    if (vec == 4 && narrow) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 4, true>), grid, block, 0, stream, P);
-    else if (vec == 4) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 4, false>), grid, block, 0, stream, P);
-    else if (narrow) hipLaunchKernelGGL((reduce_cols<KIND, ARG, 1, true>), grid, block, 0, stream, P);
-    else hipLaunchKernelGGL((reduce_cols<KIND, ARG, 1, false>), grid, block, 0, stream, P);
+    // fewer than 64 units across the wave: the geometry is read from the launch (fixing 32 or 16 units at compile
+    // time measured the same or 5 % slower)
+#define COLS_CASE(V, G) hipLaunchKernelGGL((reduce_cols<KIND, ARG, V, G>), grid, block, 0, stream, P)
+    if (vec == 4) {
+      if (P.ub_log2 == 6) COLS_CASE(4, 6);
+      else COLS_CASE(4, 0);
+    } else {
+      if (P.ub_log2 == 6) COLS_CASE(1, 6);
+      else COLS_CASE(1, 0);
+    }
+#undef COLS_CASE
   }
 }
 
@@ -1098,15 +1106,25 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
       const long blocks = ((long)P.nunits + kThreads - 1) / kThreads;
       grid.x = (unsigned)(blocks > (1l << 22) ? (1l << 22) : blocks);
     } else {
-    // fewer units than lanes: the wave's spare lanes take further rows
+    // Geometry of a wave: 2^ub_log2 units side by side, 64 >> ub_log2 rows.  Fewer units than lanes: the spare lanes
+    // take further rows.  Otherwise the widest tile that still gives every CU a block without splitting the reduced
+    // dim, down to 16 units (256 bytes of each row): partials and their fold cost more than the narrower runs
+    // (4096x16384 along dim 1: 64 units and 16 splits 46.5 us, 16 units and no split 39.9; 4096x8192: 26.5 -> 22.8),
+    // as long as a lane still walks 16 rows or more.  With 4-byte units a narrower tile would read less than
+    // 256 bytes of a row, so those keep the full wave.
     unsigned ub_log2 = 6;
     while (ub_log2 > 0 && (1u << (ub_log2 - 1)) >= P.nunits) ub_log2--;
+    if (vec == 4) {
+      while (ub_log2 > 4 && ((long)P.nunits + (1l << ub_log2) - 1) >> ub_log2 < (long)cus &&
+             R / ((kThreads / kWave) * (long)(kWave >> (ub_log2 - 1))) >= 16)
+        ub_log2--;
+    }
     P.ub_log2 = ub_log2;
     const long ub = 1l << ub_log2, row_lanes = kWave >> ub_log2;
     const long tiles = (P.nunits + ub - 1) / ub;
-    // enough blocks to fill the chip: split the reduced dim when slices are few
+    // a block per CU: split the reduced dim when the tiles are fewer (every extra split is another partial per slice)
     long split = 1;
-    const long target = (long)cus * 4;
+    const long target = (long)cus;
     if (tiles < target) {
       split = (target + tiles - 1) / tiles;
       const long max_by_rows = (R + 32 * row_lanes - 1) / (32 * row_lanes);  // at least 32 rows per lane
