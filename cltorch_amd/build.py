@@ -21,7 +21,7 @@ LIB = os.path.join(HERE, "libthcl_hip.so")
 
 ARCH = "gfx950"
 SOURCES = ["rt.cpp", "state.cpp", "tensor.cpp", "layout.cpp", "expr.cpp", "math.cpp", "host_copy.cpp", "catalogue.cpp", "user_kernel.cpp", "blas.cpp",
-           "apply.hip", "reduce.hip", "scan.hip", "index.hip", "blas12.hip", "gemm.hip"]
+           "apply.hip", "apply_catalogue.hip", "reduce.hip", "scan.hip", "index.hip", "blas12.hip", "gemm.hip"]
 
 COMMON = ["-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function", "-Wno-unused-const-variable",
           "-I", os.path.join(ROOT, "include"), "-I", CSRC]

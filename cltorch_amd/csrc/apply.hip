@@ -10,7 +10,7 @@
 
 #include <cstring>
 
-#include "apply_device.h"
+#include "apply_kernels.h"
 #include "internal.h"
 
 namespace {
@@ -251,17 +251,7 @@ bool make_plan(THClState *state, const ApplyCall &call, ApplyPlan &plan, bool dr
 }
 
 // ---------------------------------------------------------- fixed kernels ---
-#define X(name, nt, stmt)                                                                             \
-  struct Op_##name {                                                                                  \
-    static constexpr int NT = nt;                                                                     \
-    static __device__ __forceinline__ void run(float &o, float a, float b, float v1, float v2, float p1, \
-                                               float p2) {                                            \
-      (void)a; (void)b; (void)v1; (void)v2; (void)p1; (void)p2;                                        \
-      stmt;                                                                                           \
-    }                                                                                                 \
-  };
-THCL_FIXED_OPS(X)
-#undef X
+THCL_FIXED_OPS(THCL_DEFINE_OP_STRUCT)
 }  // namespace
 
 #define X(name, nt, stmt) THCL_DEFINE_APPLY_KERNELS(thcl_k_##name, Op_##name, nt)
@@ -269,21 +259,11 @@ THCL_FIXED_OPS(X)
 #undef X
 
 namespace {
-struct KernelSet {
-  int nt;
-  void (*contig_v4)(ThclContigParams);
-  void (*contig_s)(ThclContigParams);
-  void (*joint_v4)(ThclJointParams);
-  void (*joint_s)(ThclJointParams);
-  void (*generic)(ThclGenericParams);
-  void (*tiled)(ThclTileParams);
-};
-const KernelSet kFixed[OP_COUNT] = {
-#define X(name, nt, stmt) \
-  {nt, thcl_k_##name##_contig_v4, thcl_k_##name##_contig_s, thcl_k_##name##_joint_v4, thcl_k_##name##_joint_s, thcl_k_##name##_generic, thcl_k_##name##_tiled},
-    THCL_FIXED_OPS(X)
-#undef X
-};
+typedef ThclKernelSet KernelSet;
+const KernelSet kFixed[OP_FIXED_COUNT] = {THCL_FIXED_OPS(THCL_KERNEL_SET_ENTRY)};
+const KernelSet &kernel_set(ThclOp op) {
+  return op < OP_FIXED_COUNT ? kFixed[op] : thcl_catalogue_kernel_sets()[op - OP_FIXED_COUNT];
+}
 
 void launch_fixed(const KernelSet &ks, ApplyPlan &plan) {
   hipStream_t stream = (hipStream_t)thcl_rt_stream(plan.rt);
@@ -372,7 +352,7 @@ std::string thcl_apply_config_defines() {
 
 void thcl_apply_fixed(THClState *state, ThclOp op, ApplyCall &call) {
   THCL_CHECK(op >= 0 && op < OP_COUNT, "unknown operator %d", (int)op);
-  const KernelSet &ks = kFixed[op];
+  const KernelSet &ks = kernel_set(op);
   THCL_CHECK(ks.nt == call.n, "operator %d takes %d tensors, got %d", (int)op, ks.nt, call.n);
   with_overlap_fixup(state, call, [&](ApplyCall &c) {
     ApplyPlan plan;

@@ -104,6 +104,15 @@ struct ThclGenericParams {
   ThclGenericOperand op[3];
 };
 
+// OpenCL's pown(x, n): x to an integer power by repeated squaring (what the reference's pow uses
+// for integral exponents, src/lib/THClTensorMath2.cpp:22-61); user expressions reach it as pown().
+__device__ __forceinline__ float thcl_pown(float x, int n) {
+  float r = 1.0f, b = x;
+  unsigned e = n < 0 ? (unsigned)(-(long long)n) : (unsigned)n;
+  while (e) { if (e & 1u) r *= b; b *= b; e >>= 1; }
+  return n < 0 ? 1.0f / r : r;
+}
+
 template <class Op>
 __device__ __forceinline__ void thcl_apply_one(float &o, float a, float b, float v1, float v2, float p1, float p2) {
   Op::run(o, a, b, v1, v2, p1, p2);

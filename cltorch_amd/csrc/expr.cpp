@@ -22,12 +22,6 @@ const char kSkeleton[] =
 // OpenCL C built-ins an expression may use that HIP spells differently.
 // Everything is fp32; nothing here is a fast-math variant.
 const char kPrelude[] = R"PRELUDE(
-__device__ __forceinline__ float thcl_pown(float x, int n) {
-  float r = 1.0f, b = x;
-  unsigned e = n < 0 ? (unsigned)(-(long long)n) : (unsigned)n;
-  while (e) { if (e & 1u) r *= b; b *= b; e >>= 1; }
-  return n < 0 ? 1.0f / r : r;
-}
 #define pown(x, n) thcl_pown((x), (int)(n))
 #define powr(x, y) powf((x), (y))
 #define rootn(x, n) powf((x), 1.0f / (float)(n))
