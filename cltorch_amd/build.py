@@ -23,7 +23,7 @@ ARCH = "gfx950"
 SOURCES = ["rt.cpp", "state.cpp", "tensor.cpp", "layout.cpp", "expr.cpp", "math.cpp", "host_copy.cpp", "catalogue.cpp", "user_kernel.cpp", "blas.cpp",
            "apply.hip", "apply_catalogue.hip", "reduce.hip", "scan.hip", "index.hip", "blas12.hip", "gemm.hip"]
 
-COMMON = ["-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function", "-Wno-unused-const-variable",
+COMMON = ["-O3", "-fPIC", "-fvisibility=hidden", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function", "-Wno-unused-const-variable",
           "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 # packed fp32 instructions stay out of the generated code
 DEVICE = [f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -77,7 +77,13 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
             if verbose and warn:
                 print(f"--- {name}\n{warn}", file=sys.stderr)
     objs = [os.path.join(OBJ, s + ".o") for s in SOURCES]
-    cmd = [hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB] + objs + ["-lhiprtc"]
+    # the dynamic symbol table is exactly what the two public headers declare
+    from cltorch_amd import _lib
+    names = sorted(_lib.declared_symbols())
+    vmap = os.path.join(OBJ, "exports.map")
+    with open(vmap, "w") as f:
+        f.write("{\n  global:\n" + "".join(f"    {n};\n" for n in names) + "  local:\n    *;\n};\n")
+    cmd = [hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", f"-Wl,--version-script={vmap}", "-o", LIB] + objs + ["-lhiprtc"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"linking failed:\n{r.stdout}\n{r.stderr}")

@@ -390,44 +390,18 @@ void thcl_fill_contig(thcl_rt *rt, float *dst, float value, long n) {
   launch_fixed(kFixed[OP_FILL], plan);
 }
 
-// ------------------------------------------------------------ test hooks ---
-// Host-only helpers so the layout logic can be checked without a device.
-extern "C" {
-// Which kernel family a call with these views would launch, and its grid:
-// 0 dense 128-bit, 1 dense scalar, 2 joint 128-bit, 3 joint scalar, 4 generic,
-// 5 tiled, 6 nothing to do, -1 rejected.  Views are rows of [n][25] arrays;
-// misalign[i] = bytes by which operand i's storage misses a 16-byte boundary.
-int thcl_dbg_plan_kind(int n, const int *nd, long *sizes, long *strides, const long *offsets, const int *misalign,
-                       unsigned *grid) {
-  THClTensor hdr[3];
-  THClStorage st[3];
-  ApplyCall call;
-  call.n = n;
-  for (int i = 0; i < n; i++) {
-    hdr[i] = THClTensor{};
-    st[i] = THClStorage{};
-    st[i].wrapper = (void *)(uintptr_t)(0x10000000ull * (i + 1) + (unsigned)misalign[i]);
-    st[i].size = 1l << 40;
-    hdr[i].size = sizes + i * THCL_MAX_DIMS;
-    hdr[i].stride = strides + i * THCL_MAX_DIMS;
-    hdr[i].nDimension = nd[i];
-    hdr[i].storageOffset = offsets[i];
-    hdr[i].storage = &st[i];
-    call.t[i] = &hdr[i];
-  }
-  try {
-    ApplyPlan plan;
-    if (!make_plan(nullptr, call, plan, true)) return 6;
-    if (grid) *grid = plan.grid;
-    return (int)plan.kind;
-  } catch (const std::exception &) {
-    return -1;
-  }
-}
-
-unsigned thcl_dbg_divide(unsigned n, long d) {
-  ThclDivisor dv = thcl_make_divisor(d);
+// n / d by the multiply-and-shift the kernels use for their index arithmetic
+unsigned thcl_host_divide(unsigned n, long d) {
+  const ThclDivisor dv = thcl_make_divisor(d);
   return (unsigned)((((unsigned long long)n * dv.magic) >> 32) + n) >> dv.shift;
 }
 
+// Which kernel family a call would launch and with what grid, without opening a device or
+// launching anything: 0 dense 128-bit, 1 dense scalar, 2 joint 128-bit, 3 joint scalar,
+// 4 generic, 5 tiled, 6 nothing to do.
+int thcl_apply_classify(const ApplyCall &call, unsigned *grid) {
+  ApplyPlan plan;
+  if (!make_plan(nullptr, call, plan, true)) return 6;
+  if (grid) *grid = plan.grid;
+  return (int)plan.kind;
 }

@@ -141,29 +141,3 @@ std::string thcl_expr_source(const std::string &rewritten, int ntensors, int fam
          ", ThclUserOp, " + std::to_string(ntensors) + ")\n";
   return src;
 }
-
-extern "C" {
-// Host-side hooks (no device needed): the rewritten text, and a compile of the
-// generated source for a named architecture.
-int thcl_dbg_rewrite_expr(const char *expr, int ntensors, char *buf, size_t buflen) {
-  try {
-    std::string r = thcl_rewrite_expr(expr, ntensors);
-    if (r.size() + 1 > buflen) return -1;
-    memcpy(buf, r.c_str(), r.size() + 1);
-    return (int)r.size();
-  } catch (const std::exception &) {
-    return -1;
-  }
-}
-int thcl_dbg_compile_expr_family(const char *expr, int ntensors, int family, const char *arch, size_t *code_bytes) {
-  try {
-    std::string src = thcl_expr_source(thcl_rewrite_expr(expr, ntensors), ntensors, family);
-    return thcl_rt_compile_check(src.c_str(), arch, code_bytes);
-  } catch (const std::exception &) {
-    return -2;
-  }
-}
-int thcl_dbg_compile_expr(const char *expr, int ntensors, const char *arch, size_t *code_bytes) {
-  return thcl_dbg_compile_expr_family(expr, ntensors, -1, arch, code_bytes);
-}
-}

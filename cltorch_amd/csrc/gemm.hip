@@ -347,12 +347,11 @@ static void choose_ksplit(long tiles, long k, int cus, int &ksplit, int &kchunk)
     kchunk = (int)chunk;
   }
 }
-// host-only hooks for tests: the tile and the K slicing a product of this shape would use
-extern "C" void thcl_dbg_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk) {
+// the block tile and the K slicing a product of this shape gets on a chip with `cus` compute units
+void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk) {
   choose_tile(m, n, cus, *bm, *bn);
   choose_ksplit(((m + *bm - 1) / *bm) * ((n + *bn - 1) / *bn), k, cus, *ksplit, *kchunk);
 }
-extern "C" void thcl_dbg_gemm_tile(long m, long n, int cus, int *bm, int *bn) { choose_tile(m, n, cus, *bm, *bn); }
 
 void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m, long n, long k, float alpha,
                 const float *a, long lda, const float *b, long ldb, float beta, float *c, long ldc) {

@@ -113,6 +113,10 @@ std::string thcl_rewrite_expr(const char *expr, int ntensors);
 std::string thcl_expr_source(const std::string &rewritten, int ntensors, int family);
 std::string thcl_expr_tag(const std::string &rewritten, int ntensors);
 std::string thcl_apply_config_defines();
+// Planning only (no device): the kernel family a call would launch (0 dense 128-bit, 1 dense scalar,
+// 2 joint 128-bit, 3 joint scalar, 4 generic, 5 tiled, 6 nothing to do) and its grid.
+int thcl_apply_classify(const ApplyCall &call, unsigned *grid);
+unsigned thcl_host_divide(unsigned n, long d);  // n / d by the kernels' multiply-and-shift
 
 // ------------------------------------------------------------- reductions ---
 // The first four also run along a dimension with positions (max, min).  The
@@ -140,6 +144,9 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
 // column-major C[m x n] = alpha * op(A) * op(B) + beta * C on device pointers
 void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m, long n, long k, float alpha,
                 const float *a, long lda, const float *b, long ldb, float beta, float *c, long ldc);
+
+// the block tile and the K slicing a product of this shape gets on a chip with `cus` compute units
+void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk);
 
 // ------------------------------------------------------------------ misc ---
 // contiguous device fill / copy kernels used by storage-level calls

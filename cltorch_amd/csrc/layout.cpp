@@ -122,45 +122,3 @@ JointLayout thcl_joint_collapse(int n, THClTensor *const *t) {
 }
 
 // ------------------------------------------------------------ test hooks ---
-// Host-only entry points so the layout rules can be checked without a device.
-extern "C" {
-static void dbg_header(THClTensor &h, int nd, long *sz, long *st, long off) {
-  h = THClTensor{};
-  h.size = sz;
-  h.stride = st;
-  h.nDimension = nd;
-  h.storageOffset = off;
-}
-int thcl_dbg_collapse(int nd, long *sizes, long *strides, int reduce_dim, long *out_sizes, long *out_strides) {
-  THClTensor h;
-  dbg_header(h, nd, sizes, strides, 0);
-  Layout L = thcl_collapse(&h, reduce_dim);
-  for (int d = 0; d < L.dims; d++) {
-    out_sizes[d] = L.sizes[d];
-    out_strides[d] = L.strides[d];
-  }
-  return L.dims;
-}
-int thcl_dbg_overlapping(int nd, long *sizes, long *strides) {
-  THClTensor h;
-  dbg_header(h, nd, sizes, strides, 0);
-  return thcl_overlapping(&h) ? 1 : 0;
-}
-// n operands, each with `nd[i]` dims stored at row i of the [n][25] arrays;
-// returns the joint dim count (-1: shapes differ) and the joint sizes/strides.
-int thcl_dbg_joint_collapse(int n, const int *nd, long *sizes, long *strides, long *out_sizes, long *out_strides) {
-  THClTensor h[3];
-  THClTensor *tp[3];
-  for (int i = 0; i < n; i++) {
-    dbg_header(h[i], nd[i], sizes + i * THCL_MAX_DIMS, strides + i * THCL_MAX_DIMS, 0);
-    tp[i] = &h[i];
-  }
-  JointLayout J = thcl_joint_collapse(n, tp);
-  if (!J.valid) return -1;
-  for (int d = 0; d < J.dims; d++) {
-    out_sizes[d] = J.sizes[d];
-    for (int i = 0; i < n; i++) out_strides[i * THCL_MAX_DIMS + d] = J.strides[i][d];
-  }
-  return J.dims;
-}
-}

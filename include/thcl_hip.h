@@ -20,6 +20,8 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the library is built with hidden visibility: what is declared here is what it exports */
+#pragma GCC visibility push(default)
 
 /* ------------------------------------------------------------------------- */
 /* Torch7 `TH` stand-ins.  Field order matches TH's own structs, so objects   */
@@ -590,6 +592,7 @@ void THClKernel_run(THClState *state, THClKernel *kernel, const int *ints, const
                     THClTensor *const *tensors, long numWorkgroups, long workgroupSize);
 int THClKernel_compileCheck(THClKernel *kernel, const char *arch, size_t *code_bytes);
 
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

@@ -20,6 +20,8 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the library is built with hidden visibility: what is declared here is what it exports */
+#pragma GCC visibility push(default)
 
 typedef struct thcl_rt thcl_rt;
 typedef struct thcl_rt_kernel thcl_rt_kernel;
@@ -98,6 +100,7 @@ int thcl_rt_timer_stop(thcl_rt_timer *t);
 float thcl_rt_timer_ms(thcl_rt_timer *t); /* waits for the stop event */
 void thcl_rt_timer_free(thcl_rt_timer *t);
 
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

@@ -17,8 +17,11 @@ MAXD = 25
 
 
 @pytest.fixture(scope="module")
-def lib():
-    L = _lib.load()
+def lib(hooks_lib):
+    L = hooks_lib                       # the library's objects plus the test-only entry points
+    for name, (res, args) in _lib.declared_symbols().items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
     L.thcl_dbg_divide.restype = C.c_uint
     L.thcl_dbg_divide.argtypes = [C.c_uint, C.c_long]
     L.thcl_dbg_rewrite_expr.restype = C.c_int
@@ -39,6 +42,18 @@ def test_library_exports_every_declared_symbol():
                  "THClTensor_maxall", "THClTensor_minall", "THClTensor_sum", "THClTensor_max", "THClTensor_min",
                  "THClTensor_addmm", "THClBlas_gemm", "THClTensor_as_float", "thcl_rt_kernel_get", "thcl_rt_launch"):
         assert must in decls, must
+
+
+def test_library_exports_only_what_the_headers_declare():
+    """Built with hidden visibility: the dynamic symbol table holds the declared entry points and no test hook,
+    internal C++ function or kernel stub."""
+    import subprocess
+    decls = set(_lib.declared_symbols())
+    out = subprocess.check_output(["nm", "-D", "--defined-only", _lib.LIB_PATH], text=True)
+    exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    extra = sorted(n for n in exported - decls if not n.startswith(("_init", "_fini", "__bss", "_edata", "_end", "__hip_")))
+    assert not extra, extra[:20]
+    assert not any("dbg" in n for n in exported)
 
 
 def test_product_never_touches_the_oracle():
@@ -283,8 +298,8 @@ def test_user_kernel_renders_and_compiles_for_gfx950(lib):
 def test_gemm_tile_choice(lib):
     """128x128 tiles unless that leaves fewer than 4 tiles per CU; ragged or small dims use 64-wide tiles."""
     def tile(m, n, cus=256):
-        bm, bn = C.c_int(0), C.c_int(0)
-        lib.thcl_dbg_gemm_tile(C.c_long(m), C.c_long(n), C.c_int(cus), C.byref(bm), C.byref(bn))
+        bm, bn, ks, kc = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
+        lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(1), C.c_int(cus), C.byref(bm), C.byref(bn), C.byref(ks), C.byref(kc))
         return bm.value, bn.value
     assert tile(8192, 8192) == (128, 128) and tile(4096, 4096) == (128, 128)
     assert tile(3072, 3072) == (128, 64) and tile(2048, 2048) == (64, 64) and tile(1024, 1024) == (64, 64)
