@@ -11,7 +11,9 @@
 // The indexed tensor is taken as dense [O][N][I] around the dimension; one
 // thread moves one unit (4 adjacent floats along I where alignment allows), so
 // accesses coalesce along I and the index vector is read from cache.  An index
-// outside 1..N moves nothing (the reference reads or writes out of bounds).
+// outside 1..N (or NaN) moves nothing and raises a pinned flag word that the
+// host reports as "index out of range" at its next wait for the stream (the
+// reference reads or writes out of bounds; Torch's CPU path raises at once).
 // All of it is bound by HBM.
 #include <hip/hip_runtime.h>
 
@@ -29,6 +31,7 @@ struct IndexParams {
   float *b;            // the other one: [O][M][I]
   const float *index;  // [M] (select / copy / fill) or [O][M][I] (gather / scatter)
   int *winner;         // indexCopy: for every target slice, the last position of the index vector naming it
+  unsigned *fault;     // pinned word the host looks at after its next wait: set when an index is out of range
   ThclDivisor units_i, m;  // units along I, entries along the dim
   thcl_u32 total;      // units in [O][M][I]
   thcl_u32 N, M, I;
@@ -44,6 +47,7 @@ __global__ __launch_bounds__(kThreads) void index_winner(IndexParams P) {
   if (i >= P.M) return;
   const long j = (long)P.index[i] - 1;
   if (j >= 0 && j < (long)P.N) atomicMax(P.winner + j, (int)i);
+  else *P.fault = 1u;
 }
 
 template <int MODE, int VEC>
@@ -63,7 +67,10 @@ __global__ __launch_bounds__(kThreads) void index_move(IndexParams P) {
 #pragma unroll
     for (int c = 0; c < VEC; c++) {
       const long j = (long)P.index[boff + c] - 1;
-      if (j < 0 || j >= (long)P.N) continue;
+      if (j < 0 || j >= (long)P.N) {
+        *P.fault = 1u;
+        continue;
+      }
       const thcl_u64 aoff = ((thcl_u64)o * P.N + (thcl_u64)j) * P.I + k + c;
       if (MODE == GATHER) P.b[boff + c] = P.a[aoff];
       else if (MODE == SCATTER) P.a[aoff] = P.b[boff + c];
@@ -72,7 +79,10 @@ __global__ __launch_bounds__(kThreads) void index_move(IndexParams P) {
     return;
   }
   const long j = (long)P.index[i] - 1;
-  if (j < 0 || j >= (long)P.N) return;
+  if (j < 0 || j >= (long)P.N) {
+    if (ku == 0 && o == 0) *P.fault = 1u;  // once per bad entry, not once per unit of its slice
+    return;
+  }
   if (MODE == COPY && P.winner[j] != (int)i) return;
   const thcl_u64 aoff = ((thcl_u64)o * P.N + (thcl_u64)j) * P.I + k;
   if (VEC == 4) {
@@ -410,6 +420,7 @@ void THClTensor_indexSelect(THClState *state, THClTensor *res_, THClTensor *src,
   thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, src));
   IndexParams P;
   memset(&P, 0, sizeof(P));
+  P.fault = thcl_rt_fault_word_device(rt);
   P.a = thcl_dptr(s.t);
   P.b = thcl_dptr(r.t);
   P.index = thcl_dptr(ix.t);
@@ -445,6 +456,7 @@ void THClTensor_indexCopy(THClState *state, THClTensor *res_, int dim, THClTenso
   hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   IndexParams P;
   memset(&P, 0, sizeof(P));
+  P.fault = thcl_rt_fault_word_device(rt);
   P.a = thcl_dptr(r.t);
   P.b = thcl_dptr(s.t);
   P.index = thcl_dptr(ix.t);
@@ -482,6 +494,7 @@ void THClTensor_indexFill(THClState *state, THClTensor *res_, int dim, THClTenso
   thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, res_));
   IndexParams P;
   memset(&P, 0, sizeof(P));
+  P.fault = thcl_rt_fault_word_device(rt);
   P.a = thcl_dptr(r.t);
   P.index = thcl_dptr(ix.t);
   P.N = (thcl_u32)N;
@@ -551,6 +564,7 @@ static void run_gather_scatter(THClState *state, int mode, THClTensor *full, THC
   hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   IndexParams P;
   memset(&P, 0, sizeof(P));
+  P.fault = thcl_rt_fault_word_device(rt);
   P.a = thcl_dptr(full);
   P.b = other ? thcl_dptr(other) : nullptr;
   P.index = thcl_dptr(index);
@@ -610,10 +624,12 @@ void THClTensor_scatterFill(THClState *state, THClTensor *self, long dim, THClTe
 }
 
 // ------------------------------------------------------------- masked ---
+// per-chunk counts, group offsets and the grand total are 32-bit words
+constexpr long kMaskMaxElements = 1l << 32;
 static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long n) {
   hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   const long nb = (n + kChunk - 1) / kChunk;
-  THCL_CHECK(nb < (1l << 31) - 1, THCL_DIM_WARNING);
+  THCL_CHECK(n < kMaskMaxElements, THCL_DIM_WARNING);
   P.n = (thcl_u64)n;
   P.nblocks = (thcl_u32)nb;
   // the bit words first (8-byte aligned), then the counts and the group totals
@@ -650,6 +666,7 @@ void THClTensor_maskedSelect(THClState *state, THClTensor *tensor, THClTensor *s
   thcl_check_same_device(state, 3, tensor, src, mask);
   const long n = THClTensor_nElement(state, mask);
   THCL_ARGCHECK(n == THClTensor_nElement(state, src), 2, "sizes do not match");
+  THCL_CHECK(n < kMaskMaxElements, "maskedSelect takes at most 2^32 - 1 elements (the mask has %ld): its offsets are 32-bit", n);
   THCL_CHECK(tensor != src && tensor != mask, "result cannot alias the source or the mask");
   const int device = THClTensor_getDevice(state, src);
   if (tensor->nDimension < 0 && !tensor->storage) tensor->device = device;
@@ -690,6 +707,7 @@ void THClTensor_maskedCopy(THClState *state, THClTensor *tensor, THClTensor *mas
   thcl_check_same_device(state, 3, tensor, src, mask);
   const long n = THClTensor_nElement(state, mask);
   THCL_ARGCHECK(n == THClTensor_nElement(state, tensor), 2, "mask and tensor must have the same number of elements");
+  THCL_CHECK(n < kMaskMaxElements, "maskedCopy takes at most 2^32 - 1 elements (the mask has %ld): its offsets are 32-bit", n);
   THCL_CHECK(tensor != src && tensor != mask, "tensor cannot alias the source or the mask");
   if (n == 0) return;
   Dense s(state, src, true, false), m(state, mask, true, false), r(state, tensor, true, true);

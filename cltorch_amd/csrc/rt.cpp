@@ -263,12 +263,24 @@ int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
   return 0;
 }
 
+// Word of the pinned block that kernels raise when they meet something the host should hear about
+// (an index outside its range).  Looked at whenever the host has waited for the stream.
+constexpr int kFaultWord = 32;
+static int check_fault(thcl_rt *rt) {
+  volatile unsigned *w = (volatile unsigned *)(rt->host_word + kFaultWord);
+  if (*w == 0u) return 0;
+  *w = 0u;
+  g_err = "index out of range: an indexing kernel met an index outside 1..size of the indexed dimension "
+          "(that entry moved nothing; reported at the first wait after the launch)";
+  return -3;
+}
+
 int thcl_rt_memcpy_d2h(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
   if (!bytes) return 0;
   DeviceGuard g(rt->device);
   RT_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, rt->stream));
   RT_CHECK(hipStreamSynchronize(rt->stream));
-  return 0;
+  return check_fault(rt);
 }
 
 int thcl_rt_memcpy_d2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
@@ -283,8 +295,10 @@ void *thcl_rt_stream(thcl_rt *rt) { return (void *)rt->stream; }
 int thcl_rt_sync(thcl_rt *rt) {
   DeviceGuard g(rt->device);
   RT_CHECK(hipStreamSynchronize(rt->stream));
-  return 0;
+  return check_fault(rt);
 }
+
+unsigned *thcl_rt_fault_word_device(thcl_rt *rt) { return (unsigned *)(rt->host_word_dev + kFaultWord); }
 
 void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes) {
   if (bytes) *bytes = rt->scratch_bytes;

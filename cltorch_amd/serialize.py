@@ -81,6 +81,8 @@ def decode_tensor(raw: bytes):
     r = _Reader(raw)
     tclass = r.header(TENSOR_CLASSES, 1)
     (nd,) = r.take("=i")
+    if nd == -1:
+        nd = 0          # the reference writes its header field as is, and its empty header holds -1
     if nd < 0 or nd > 64:
         raise ValueError("bad dimension count")
     sizes = list(r.take("=%dq" % nd)) if nd else []
@@ -102,7 +104,7 @@ def save(path: str, tensor) -> None:
     """``torch.save(path, clTensor)``: header plus the whole storage the tensor views."""
     from .tensor import _call
     nd = tensor.nDimension()
-    if nd <= 0 and tensor.nElement() == 0:
+    if nd < 0 or (nd > 0 and tensor.nElement() == 0):          # empty; a point tensor has 0 dimensions and a storage
         raw = encode_tensor([], [], 0, None)
     else:
         st = _call("THClTensor_storage", tensor._h)
@@ -118,8 +120,16 @@ def load(path: str):
     from .tensor import ClTensor
     with open(path, "rb") as f:
         sizes, strides, offset0, storage, _, _ = decode_tensor(f.read())
-    if storage is None or not sizes:
+    if storage is None:
         return ClTensor()
+    if not sizes:
+        # no dimensions but a storage: a point tensor, whose one value sits at the offset.  It is
+        # rebuilt as the sum of that one element (exact: one fp64 addend, one rounding back).
+        if not 0 <= offset0 < storage.size:
+            return ClTensor()
+        point = ClTensor()
+        point.sum(ClTensor(storage[offset0:offset0 + 1]))
+        return point
     need = offset0 + sum((s - 1) * t for s, t in zip(sizes, strides)) + 1
     if any(s <= 0 for s in sizes) or any(t < 0 for t in strides) or offset0 < 0 or need > storage.size:
         raise ValueError("tensor header points outside its storage")

@@ -73,6 +73,11 @@ float *thcl_rt_host_word(thcl_rt *rt);
  * directly, and the host reads it after thcl_rt_sync (no copy in between) */
 float *thcl_rt_host_word_device(thcl_rt *rt);
 
+/* A pinned word, at the address kernels use, that a kernel sets to non-zero when it meets input
+ * the host must hear about (an index outside its range).  thcl_rt_sync and thcl_rt_memcpy_d2h
+ * look at it after they have waited: if it is set they clear it and return -3 with a message. */
+unsigned *thcl_rt_fault_word_device(thcl_rt *rt);
+
 /* Page-locked host memory for callers that stage their own transfers: copies between a
  * tensor and such a buffer run at the link's rate (57 GB/s measured on MI355X, against
  * 30 GB/s in and 17 GB/s out for pageable memory).  The reference keeps its host mirrors

@@ -94,6 +94,7 @@ void *thcl_rt_host_alloc(size_t bytes) { return malloc(bytes ? bytes : 1); }
 int thcl_rt_host_free(void *ptr) { free(ptr); return 0; }
 float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
 float *thcl_rt_host_word_device(thcl_rt *rt) { return rt->host_word; }
+unsigned *thcl_rt_fault_word_device(thcl_rt *rt) { return (unsigned *)rt->host_word + 32; }
 thcl_rt_timer *thcl_rt_timer_new(thcl_rt *) { return new thcl_rt_timer(); }
 int thcl_rt_timer_start(thcl_rt_timer *) { return 0; }
 int thcl_rt_timer_stop(thcl_rt_timer *) { return 0; }

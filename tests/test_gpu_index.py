@@ -61,12 +61,29 @@ def test_index_ops_on_views_and_bad_arguments(cl):
     assert_bit_equal(dst.dev.float(), cat.index_copy(np.zeros((30, 40), dtype=F), 0, idx, src), "copy into a transposed view")
     dst.dev.indexFill(2, [1, 40], 9.0)
     assert np.all(dst.dev.float()[:, [0, 39]] == 9.0)
-    # an index outside the dimension moves nothing
+    # an index outside the dimension moves nothing and is reported as an error at the next wait for the device
+    # (Torch's CPU path raises at once; the reference's kernels read or write out of bounds)
     Y = cl.ClTensor(x)
-    out = Y.index(1, cl.ClTensor(np.array([1, 41, 0, 40], dtype=F))).float()
-    assert_bit_equal(out[[0, 3]], x[[0, 39]], "valid rows")
+    sel = Y.index(1, cl.ClTensor(np.array([1, 41, 0, 40], dtype=F)))
+    with pytest.raises(cl.ClError, match="index out of range"):
+        cl.synchronize()
+    assert_bit_equal(sel.float()[[0, 3]], x[[0, 39]], "valid rows")           # the report is made once; the library goes on
     Y.indexFill(1, cl.ClTensor(np.array([0, 41, -3], dtype=F)), 5.0)
+    with pytest.raises(cl.ClError, match="index out of range"):
+        Y.float()                                                              # a read-back waits too
     assert_bit_equal(Y.float(), x, "out-of-range fill is a no-op")
+    gi = np.ones((1, 30), dtype=F)
+    gi[0, 7] = 99.0
+    g = cl.ClTensor(x).gather(1, cl.ClTensor(gi))
+    with pytest.raises(cl.ClError, match="index out of range"):
+        cl.synchronize()
+    del g
+    Z = cl.ClTensor(x)
+    Z.indexCopy(1, cl.ClTensor(np.array([2, float("nan")], dtype=F)), cl.ClTensor(x[:2] * 0 + 1))
+    with pytest.raises(cl.ClError, match="index out of range"):
+        cl.synchronize()
+    assert np.all(Z.float()[1] == 1.0) and np.array_equal(Z.float()[[0, 2]], x[[0, 2]])
+    cl.synchronize()                                                           # nothing pending any more
     with pytest.raises(cl.ClError):
         Y.index(3, [1])
     with pytest.raises(cl.ClError):
@@ -337,4 +354,23 @@ def test_save_and_load(cl, tmp_path):
     assert (w.size(), w.stride(), w.storageOffset()) == (v.size(), v.stride(), v.storageOffset())
     assert np.array_equal(w.float(), v.float())
     cl.save(path, cl.ClTensor())
+    e = cl.load(path)
+    assert e.nElement() == 0 and e.nDimension() == cl.ClTensor().nDimension()
+    # a point tensor keeps its value (and stays a point tensor); NaN and infinities included
+    for value in (2.5, float("inf"), float("nan")):
+        src = cl.ClTensor(np.array([1.0, value], dtype=F))
+        p = cl.ClTensor()
+        p.sum(src.narrow(1, 2, 1))
+        assert p.nDimension() == 0
+        cl.save(path, p)
+        q = cl.load(path)
+        assert q.nDimension() == 0
+        assert np.array([q.s()], dtype=F).view(np.uint32)[0] == np.array([value], dtype=F).view(np.uint32)[0] or (value != value and q.s() != q.s())
+    # an empty header as the reference itself would write it (dimension count -1, no storage)
+    import struct
+    from cltorch_amd import serialize
+    raw = serialize.encode_tensor([], [], 0, None)
+    at = raw.index(struct.pack("=i", 0), raw.index(b"torch.ClTensor") + len(b"torch.ClTensor"))
+    with open(path, "wb") as f:
+        f.write(raw[:at] + struct.pack("=i", -1) + raw[at + 4:])
     assert cl.load(path).nElement() == 0

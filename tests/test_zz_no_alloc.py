@@ -89,6 +89,10 @@ def test_what_it_refuses(cl):
     out = _point(cl)
     with pytest.raises(cl.ClError, match="at most"):
         _call("THClTensor_sumall_gpu_noalloc", out._h, huge._h)
+    # maskedSelect / maskedCopy keep 32-bit offsets: 2^32 elements or more are refused before anything is allocated
+    wide = a.strided((1 << 16, 1 << 16), (0, 0))
+    with pytest.raises(cl.ClError, match="at most 2\\^32 - 1 elements"):
+        cl.ClTensor().maskedSelect(wide, wide)
     # an empty source gives the identity element, and the library goes on working
     _call("THClTensor_sumall_gpu_noalloc", out._h, empty._h)
     assert out.s() == 0.0
