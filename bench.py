@@ -82,7 +82,8 @@ def cpu_baseline(n_sample, seed_base=1, min_seconds=12.0):
     x, y, z = (oracle.uniform(seed_base + i, n_sample) for i in range(3))
     vx = oracle.View.contiguous(x)
     p = lambda a: a.ctypes.data_as(C.c_void_p)
-    steps, first = 0, None
+    steps, first, first_clean = 0, None, None
+    x0 = x.copy()
     t0 = time.perf_counter()
     while True:
         L.th_pointwise_contig_omp(C.c_int(oracle.OPS["cadd"]), C.c_float(1.0), p(vx.storage), p(vx.storage), p(y), C.c_long(n_sample))
@@ -93,6 +94,14 @@ def cpu_baseline(n_sample, seed_base=1, min_seconds=12.0):
         steps += 1
         if first is None:
             first = (s, m)
+            t_pause = time.perf_counter()
+            # the configuration's own sqrt of negative arguments leaves NaNs, so sum and max of a step are NaN on
+            # both sides; the same two reductions with the NaNs set to zero give numbers that can be compared
+            clean = np.where(np.isnan(vx.storage), np.float32(0), vx.storage)
+            vc = oracle.View.contiguous(clean)
+            first_clean = (oracle.sumall(vc), oracle.maxall(vc), int(np.isnan(vx.storage).sum()))
+            del clean, vc
+            t0 += time.perf_counter() - t_pause          # not part of the timed work
         dt = time.perf_counter() - t0
         if dt >= min_seconds or steps >= 200:
             break
@@ -112,6 +121,8 @@ def cpu_baseline(n_sample, seed_base=1, min_seconds=12.0):
                       f"OpenMP loops on {oracle.num_threads()} threads, sum (fp64 accumulator) and max serial in element order "
                       f"(max stops at the first NaN, as TH does); Torch7's own map2 calls a Lua closure per element and is far slower",
             "seconds": round(dt, 3), "steps": steps, "first_step_sum_max": [fmt(first[0]), fmt(first[1])],
+            "first_step_nan_free": {"sum": float(np.float32(first_clean[0])), "max": float(first_clean[1]), "nans": first_clean[2]},
+            "_inputs": (x0, y, z),
             "addmm_cpu": {"value": round(gemm_tflops, 3), "unit": "TFLOP/s", "kind": "torch.addmm on CPU tensors, fp32, 2048^3",
                           "threads": torch.get_num_threads()}}
 
@@ -217,7 +228,20 @@ def main():
     if not args.no_detail:
         out["detail"] = detail(cl, oracle, T, X, Y, Z, n)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(1 << args.cpu_log2n)
+        del X, Y, Z
+        base = cpu_baseline(1 << args.cpu_log2n)
+        # the GPU on the baseline's own sample: one step, NaNs set to zero on the device, same two reductions
+        x0, y0, z0 = base.pop("_inputs")
+        Xs, Ys, Zs = cl.ClTensor(x0), cl.ClTensor(y0), cl.ClTensor(z0)
+        Xs.add(Ys).cmul(Ys).map2_on_gpu(Ys, Zs, EXPR)
+        nans = Xs.ne(Xs).sum()                      # a count returned as fp32: exact up to 2^24, rounded once beyond
+        Xs.apply_on_gpu("x = (x != x) ? 0.0 : x")
+        gs, gm = Xs.sum(), Xs.max()
+        want = base["first_step_nan_free"]
+        base["gpu_on_same_sample"] = {"sum": gs, "max": gm, "nans": nans,
+                                      "sum_rel_diff": abs(gs - want["sum"]) / max(abs(want["sum"]), 1e-30),
+                                      "max_equal": gm == want["max"], "nans_equal": nans == float(np.float32(want["nans"]))}
+        out["cpu_baseline"] = base
     print(json.dumps(out))
 
 
