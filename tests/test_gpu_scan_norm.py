@@ -146,3 +146,28 @@ def test_all_any(cl):
     assert pt.s() == 0.0
     s = Pair.dense(cl, x2.reshape(1024, 1024)).transpose(0, 1).narrow(1, 0, 1000)   # drops row 1023 with the 0.5
     assert s.dev.all() is bool(cat.truth(s.view.gather()).all())
+
+
+def test_scan_of_rows_longer_than_a_window(cl):
+    """Cut rows of more than 128 MiB in total go through in windows (totals pass and scan pass per window), and a
+    segment's carry-in comes partly from the previous window's last block, partly from the window's own totals:
+    rows that begin, end and straddle a window boundary, checked on ones (every prefix is a count) and on a ramp
+    of small integers (every prefix exact in fp64), plus run-to-run equality on random data."""
+    for rows, length in ((1, (1 << 26) + 12288 + 4), (3, (1 << 25) + 20480), (64, 1 << 20), (5, 9 * (1 << 20) + 4096)):
+        ones = cl.ClTensor(rows * length).fill(1.0).resize(rows, length)
+        got = ones.cumsum(2).float()
+        want = np.arange(1, length + 1, dtype=np.float64).astype(F)
+        for r in range(rows):
+            assert np.array_equal(got[r], want), (rows, length, r)
+        del ones, got
+    n = (1 << 26) + 4096 * 3
+    ramp = (np.arange(n, dtype=np.int64) % 7).astype(F)
+    got = cl.ClTensor(ramp).cumsum().float()
+    assert np.array_equal(got, np.cumsum(ramp.astype(np.float64)).astype(F))
+    x = oracle.uniform(68, n)
+    X = cl.ClTensor(x)
+    first = X.cumsum().float()
+    _scan_close(first, cat.cumulate(x, 0), "cumsum across windows")
+    assert_bit_equal(X.cumsum().float(), first, "repeat of the same scan")
+    y = oracle.uniform(69, n, 0.9999999, 1.0000001)
+    _scan_close(cl.ClTensor(y).cumprod().float(), cat.cumulate(y, 0, prod=True), "cumprod across windows")
