@@ -131,6 +131,8 @@ struct MaskParams {
   thcl_u64 n;
   thcl_u32 nblocks;
   thcl_u64 src_len;   // copy: elements available in src
+  unsigned *ticket;   // arrival counter of the group blocks, zero between launches
+  unsigned *host_total;  // pinned host word (device address) that receives the grand total
 };
 
 template <bool VEC>
@@ -174,10 +176,15 @@ __global__ __launch_bounds__(kThreads) void mask_count(MaskParams P) {
   }
 }
 
-// Block counts -> exclusive offsets in two levels.  mask_scan_groups: a block of 1024
+// Block counts -> exclusive offsets in two levels, one launch.  A block of 1024
 // threads turns 4096 adjacent counts into offsets within the group (4 per thread, one
-// 16-byte access) and leaves the group's total.  mask_scan_totals: one block turns
-// the group totals into group offsets and leaves the grand total behind them.
+// 16-byte access) and publishes the group's total; the block that arrives last turns
+// the group totals into group offsets, leaves the grand total behind them and hands it
+// to the host through a pinned word (the host only has to wait for the stream).
+// The hand-over between the group blocks is the one of the column reductions: totals
+// stored with device-scope stores (written through to where all XCDs meet), the storing
+// wave waits for their acknowledgement, then takes a ticket; the last arrival reads with
+// loads that bypass the caches.
 constexpr int kGroup = 4096;
 
 __device__ __forceinline__ unsigned block1024_exclusive(unsigned v, unsigned *lds, unsigned *total) {
@@ -214,21 +221,29 @@ __global__ __launch_bounds__(1024) void mask_scan_groups(MaskParams P) {
     if (i0 + k < P.nblocks) P.counts[i0 + k] = run;
     run += v[k];
   }
-  if (threadIdx.x == 0) P.groups[blockIdx.x] = total;
-}
-
-__global__ __launch_bounds__(1024) void mask_scan_totals(MaskParams P) {
-  __shared__ unsigned lds[1024 / 64];
+  __shared__ unsigned s_last;
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(P.groups + blockIdx.x, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned t = atomicAdd(P.ticket, 1u);
+    s_last = (t == gridDim.x - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!s_last) return;
   unsigned carry = 0;
   for (thcl_u32 g0 = 0; g0 < P.ngroups; g0 += 1024) {
     const thcl_u32 g = g0 + threadIdx.x;
-    const unsigned v = g < P.ngroups ? P.groups[g] : 0u;
-    unsigned total;
-    const unsigned excl = block1024_exclusive(v, lds, &total);
+    const unsigned v = g < P.ngroups ? __atomic_load_n(P.groups + g, __ATOMIC_RELAXED) : 0u;
+    unsigned gtotal;
+    const unsigned excl = block1024_exclusive(v, lds, &gtotal);
     if (g < P.ngroups) P.groups[g] = carry + excl;
-    carry += total;
+    carry += gtotal;
   }
-  if (threadIdx.x == 0) P.groups[P.ngroups] = carry;
+  if (threadIdx.x == 0) {
+    P.groups[P.ngroups] = carry;
+    *P.host_total = carry;
+    *P.ticket = 0u;
+  }
 }
 
 // COPY false: dst[rank] = src[i] for selected i.  COPY true: dst[i] = src[rank].
@@ -626,6 +641,8 @@ void THClTensor_scatterFill(THClState *state, THClTensor *self, long dim, THClTe
 // ------------------------------------------------------------- masked ---
 // per-chunk counts, group offsets and the grand total are 32-bit words
 constexpr long kMaskMaxElements = 1l << 32;
+constexpr int kMaskTicket = 8;     // word of the context's scratch block (words 1..63 are free for such counters)
+constexpr int kMaskHostWord = 2;   // word of the context's pinned block that receives the count
 static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long n) {
   hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   const long nb = (n + kChunk - 1) / kChunk;
@@ -644,18 +661,19 @@ static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long 
   if (aligned16(P.mask)) hipLaunchKernelGGL(mask_count<true>, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
   else hipLaunchKernelGGL(mask_count<false>, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
   check("mask count");
+  P.ticket = (unsigned *)thcl_rt_scratch(rt, nullptr) + kMaskTicket;
+  P.host_total = (unsigned *)(thcl_rt_host_word_device(rt) + kMaskHostWord);
   hipLaunchKernelGGL(mask_scan_groups, dim3((unsigned)ng), dim3(1024), 0, stream, P);
-  hipLaunchKernelGGL(mask_scan_totals, dim3(1), dim3(1024), 0, stream, P);
   check("mask offsets");
   (void)state;
   return P.counts;
 }
 
-static long read_total(thcl_rt *rt, const MaskParams &P) {
-  float *hw = thcl_rt_host_word(rt);  // a pinned 4-byte word: carries the count's bits
-  THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, P.groups + P.ngroups, sizeof(unsigned)) == 0, "%s", thcl_rt_error());
+static long read_total(thcl_rt *rt, const MaskParams &) {
+  // the last group block left the count in a pinned word: waiting for the stream is all it takes
+  THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
   unsigned total;
-  memcpy(&total, hw, sizeof(total));
+  memcpy(&total, thcl_rt_host_word(rt) + kMaskHostWord, sizeof(total));
   return (long)total;
 }
 
