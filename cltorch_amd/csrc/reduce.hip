@@ -994,13 +994,13 @@ void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *
     return;
   }
   size_t sbytes = 0;
-  char *scratch = (char *)thcl_rt_scratch(rt, &sbytes);
+  char *sblock = (char *)thcl_rt_scratch(rt, &sbytes);
   ReduceAllParams P;
   memset(&P, 0, sizeof(P));
   P.in = a;
   P.n = (thcl_u64)n;
-  P.partials = scratch + kPartialOff;
-  P.ticket = (unsigned *)(scratch + kTicketOff);
+  P.partials = sblock + kPartialOff;
+  P.ticket = (unsigned *)(sblock + kTicketOff);
   P.out = out;
   const bool vec = aligned16(a) && aligned16(b);
   const long want = vec ? (n / 4 + kThreads * 4 - 1) / (kThreads * 4) : (n + kThreads - 1) / kThreads;
@@ -1083,9 +1083,9 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   fill_operand(P.L, L);
 
   size_t sbytes = 0;
-  char *scratch = (char *)thcl_rt_scratch(rt, &sbytes);
-  P.partials = scratch + kPartialOff;
-  P.ticket = (unsigned *)(scratch + kTicketOff) + kColTicket0;
+  char *sblock = (char *)thcl_rt_scratch(rt, &sbytes);
+  P.partials = sblock + kPartialOff;
+  P.ticket = (unsigned *)(sblock + kTicketOff) + kColTicket0;
   const long partial_cap = (long)((sbytes - kPartialOff - kResultSlot) / 8);  // 8-byte entries
   const int cus = thcl_rt_get_props(rt)->compute_units;
 
