@@ -32,8 +32,10 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWave = 64;
 // Rows that are cut into segments go through in windows of this many input bytes: totals pass and scan pass of a
-// window run back to back, so the second read is served by the memory-side cache (256 MiB on this chip).
-constexpr unsigned long long kScanWindowBytes = 128ull << 20;
+// window run back to back, so the second read is served by the memory-side cache (256 MiB on this chip; windows of
+// 128, 192 and 256 MiB measured within 4 % of each other, 64 MiB 12 % slower).
+constexpr unsigned long long kScanWindowBytes = 256ull << 20;
+constexpr int kScanSegment = 8192;
 
 struct ScanParams {
   const float *in;
@@ -491,10 +493,11 @@ void run_scan(hipStream_t stream, ScanParams &P, bool rows, bool vec) {
     const thcl_u64 blocks = P.O * P.S;
     if (P.S > 1) {
       // Cut rows are read twice (totals, then the scan with each segment's carry-in).  The input goes through
-      // in windows of about 128 MiB, totals pass and scan pass back to back per window, so the second read comes
-      // out of the memory-side cache instead of HBM (measured: a 128 MiB window re-read in 35 us against 50 us
-      // cold; 2^28 elements 570 -> 480 us).  A segment's carry-in is folded from the totals by its own block,
-      // which saves a launch per window.
+      // in windows of 256 MiB, totals pass and scan pass back to back per window, so the second read comes out of
+      // the memory-side cache instead of HBM (measured on plain kernels: a 128 MiB window re-read and copied in
+      // 35 us after an ordinary read of it, 50 us cold; nothing gained after a nontemporal read).  2^28 elements:
+      // 570 us in three chip-wide passes, 498 us this way.  A segment's carry-in is folded from the totals by
+      // its own block, which saves a launch per window.
       thcl_u64 per_window = (kScanWindowBytes / sizeof(float) + P.seg - 1) / P.seg;
       if (per_window < 1) per_window = 1;
       P.own_carry = 1;
@@ -619,12 +622,11 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     if (S < 1) S = 1;
     thcl_u64 seg = (P.R + S - 1) / S;
     if (rows) seg = (seg + 4095) / 4096 * 4096;  // whole steps, so vector accesses stay aligned
-    // cut rows longer than a window go through window by window: every window must fill the chip by itself
-    // (4 blocks per CU), which makes the segments shorter than the whole input alone would
-    if (rows && S > 1 && total * sizeof(float) > kScanWindowBytes) {
-      thcl_u64 wseg = (kScanWindowBytes / sizeof(float) / ((thcl_u64)cus * 4) + 4095) / 4096 * 4096;
-      if (wseg < 4096) wseg = 4096;
-      if (wseg < seg) seg = wseg;
+    // Cut rows take segments of 8192 elements (two steps of a block) when that still leaves several blocks per CU:
+    // measured best for the windowed passes (2^28 elements: 8192 -> 497 us, 16384 -> 514, 32768 -> 520, 4096 -> 605),
+    // whatever the window.
+    if (rows && S > 1 && seg > (thcl_u64)kScanSegment && total >= (thcl_u64)cus * 8 * kScanSegment) {
+      seg = (thcl_u64)kScanSegment;
     }
     S = (P.R + seg - 1) / seg;
     P.S = S;
