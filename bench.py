@@ -15,8 +15,16 @@ three-operand expression kernel).  ``detail`` carries the other configurations
 (strided map/copy, reductions along a dim, the point-tensor chain, addmm) and,
 under ``w_`` names, the operators either side of the path (catalogue ops,
 scans, level-1/2 contractions, indexed movement), each with its own effective
-GB/s or TFLOP/s.  The CPU baseline is the TH-semantics
-restatement (oracle/) on the host's cores over a bounded sample.
+GB/s or TFLOP/s (timed back to back, see ``detail``).  The CPU baseline is the
+TH-semantics restatement (oracle/) on the host's cores over a bounded sample;
+that leg also runs one step of the same sample on the GPU and compares sum and
+max with the NaNs set to zero.  ``roofline.traffic`` and the ``kernel_only_ms``
+fields are read from the committed summary of the counter runs
+(``profiles/``), which this script also produces:
+
+    rocprofv3 --kernel-trace --stats ... -- python3 bench.py --pmc-configs      (and --pmc FETCH_SIZE / WRITE_SIZE)
+    python3 bench.py --summarise TRACE_DB FETCH_DB WRITE_DB > profiles/...txt
+    python3 bench.py --pmc-gemm / --summarise-mfma, --summarise-trace
 
 Prints ONE JSON line.
 """
@@ -384,30 +392,32 @@ def config_ops(cl, oracle, X, Y, Z, n):
 
 
 def detail(cl, oracle, T, X, Y, Z, n):
-    """The other benchmark configurations, a few launches each.  Per operation: ``avg_ms`` etc. come from
-    one HIP-event pair per call (the pair's own packets sit between the calls); ``back_to_back_ms`` is one
-    pair around all the calls divided by their number, which is what a caller that just keeps calling
-    sees; ``kernel_only_ms`` is the sum of the call's kernel durations in the committed rocprofv3 trace."""
+    """The other benchmark configurations, a few launches each.  Per operation: ``avg_ms`` is one HIP-event pair
+    around ``reps`` calls in a row divided by their number -- what a caller that just keeps calling sees, launch
+    gaps and result allocation included -- and ``achieved`` / ``frac_of_peak`` follow from it.  ``event_pair_*``
+    come from one event pair per call (the pairs' own packets then sit between the calls, which costs a short
+    kernel 2-3 us); ``kernel_only_ms`` is the sum of the call's kernel durations in the committed rocprofv3 trace."""
     d = {}
     profiled = committed_profile()
     for name, fn, work, unit, reps, peak in config_ops(cl, oracle, X, Y, Z, n):
+        scale = 1e-9 if unit == "GB/s" else 1e-12
         fn()
         cl.synchronize()
         for _ in range(reps):
             T.timed(name, fn)
         cl.synchronize()
-        s = stats(T.collect()[name], work, unit)
+        pairs = np.array(T.collect()[name], dtype=np.float64)
         T.timed(name, lambda: [fn() for _ in range(reps)])
         cl.synchronize()
         b2b = T.collect()[name][0] / reps
-        s["back_to_back_ms"] = round(b2b, 4)
-        s["achieved_back_to_back"] = round(work / (b2b * 1e-3) * (1e-9 if unit == "GB/s" else 1e-12), 1)
-        s["frac_of_peak"] = round(s["achieved"] / peak, 4)
-        s["frac_of_peak_back_to_back"] = round(s["achieved_back_to_back"] / peak, 4)
+        s = {"avg_ms": round(b2b, 4), "achieved": round(work / (b2b * 1e-3) * scale, 1), "unit": unit,
+             "frac_of_peak": round(work / (b2b * 1e-3) * scale / peak, 4), "calls": reps,
+             "event_pair_avg_ms": round(float(pairs.mean()), 4), "event_pair_min_ms": round(float(pairs.min()), 4),
+             "frac_of_peak_event_pair": round(work / (float(pairs.mean()) * 1e-3) * scale / peak, 4)}
         p = profiled.get("ops", {}).get(name)
         if p:
             s["kernel_only_ms"] = round(p["kernel_us"] * 1e-3, 4)
-            s["frac_of_peak_kernel_only"] = round(work / (p["kernel_us"] * 1e-6) * (1e-9 if unit == "GB/s" else 1e-12) / peak, 4)
+            s["frac_of_peak_kernel_only"] = round(work / (p["kernel_us"] * 1e-6) * scale / peak, 4)
         d[name] = s
     if profiled:
         d["kernel_only_source"] = PROFILE_SUMMARY + " (rocprofv3 --kernel-trace of `bench.py --pmc-configs`, committed)"
