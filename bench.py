@@ -147,7 +147,8 @@ def main():
     ap.add_argument("--pmc-configs", action="store_true",
                     help="run every configuration's operations 1 + 3 times each behind marker launches and exit; meant to run "
                          "under `rocprofv3 --kernel-trace [--pmc FETCH_SIZE | --pmc WRITE_SIZE]`; writes --manifest")
-    ap.add_argument("--manifest", default=os.path.join(ROOT, "gpurun_out", "pmc_configs_manifest.json"))
+    ap.add_argument("--manifest", default="pmc_configs_manifest.json",
+                    help="where --pmc-configs writes (and --summarise reads) the list of operations")
     ap.add_argument("--summarise", nargs=3, metavar=("TRACE_DB", "FETCH_DB", "WRITE_DB"),
                     help="print the text summary of three rocprofv3 runs of --pmc-configs (no GPU needed)")
     ap.add_argument("--summarise-trace", metavar="TRACE_DB", help="print per-kernel totals of a --kernel-trace --stats run of this script")
@@ -161,12 +162,12 @@ def main():
         sys.exit(2)
 
     if args.summarise:
-        r = "$R"
-        cmds = [f"rocprofv3 --kernel-trace --stats -d {r}/gpurun_out/cfg_trace -o t -- python3 {r}/bench.py --pmc-configs",
-                f"rocprofv3 --pmc FETCH_SIZE --kernel-trace -d {r}/gpurun_out/cfg_fetch -o f -- python3 {r}/bench.py --pmc-configs",
-                f"rocprofv3 --pmc WRITE_SIZE --kernel-trace -d {r}/gpurun_out/cfg_write -o w -- python3 {r}/bench.py --pmc-configs",
-                "python3 bench.py --summarise gpurun_out/cfg_trace/t_results.db gpurun_out/cfg_fetch/f_results.db "
-                "gpurun_out/cfg_write/w_results.db > " + PROFILE_SUMMARY]
+        w = "python3 $R/bench.py --pmc-configs --manifest $OUT/pmc_configs_manifest.json"
+        cmds = [f"rocprofv3 --kernel-trace --stats -d $OUT/cfg_trace -o t -- {w}",
+                f"rocprofv3 --pmc FETCH_SIZE --kernel-trace -d $OUT/cfg_fetch -o f -- {w}",
+                f"rocprofv3 --pmc WRITE_SIZE --kernel-trace -d $OUT/cfg_write -o w -- {w}",
+                "python3 bench.py --manifest $OUT/pmc_configs_manifest.json --summarise $OUT/cfg_trace/t_results.db "
+                "$OUT/cfg_fetch/f_results.db $OUT/cfg_write/w_results.db > " + PROFILE_SUMMARY]
         sys.stdout.write(summarise(*args.summarise, args.manifest, cmds))
         return
     if args.summarise_trace:
@@ -573,7 +574,7 @@ def summarise(trace_db, fetch_db, write_db, manifest_path, commands):
     ops, calls = man["ops"], man["calls_per_op"]
     tr, fe, wr = _segments(trace_db, False), _segments(fetch_db, True), _segments(write_db, True)
     assert len(tr) == len(fe) == len(wr) == len(ops), (len(tr), len(fe), len(wr), len(ops))
-    out = ["commands (each run from /tmp with TMPDIR=/tmp; $R is the repository root on the GPU box):"]
+    out = ["commands (each run from /tmp with TMPDIR=/tmp; $R is the repository root, $OUT a scratch directory):"]
     out += ["  " + c for c in commands]
     out += ["workload: every operation runs 1 + 3 times behind a marker launch; the first call is dropped, the figures are means",
             "  of the other three.  Durations come from the --kernel-trace run (no counters), KiB from the two counter runs.", ""]
@@ -640,9 +641,9 @@ def summarise_trace(db_path):
     extra = {}
     for name, mn, mx, vg, lds in c.execute("select name, min(duration), max(duration), max(vgpr_count), max(lds_size) from kernels group by name"):
         extra[name] = (mn, mx, vg, lds)
-    out = ["command (run from /tmp with TMPDIR=/tmp; $R is the repository root on the GPU box):",
-           "  rocprofv3 --kernel-trace --stats -d $R/gpurun_out/bench_trace -o b -- python3 $R/bench.py --no-cpu",
-           "  python3 bench.py --summarise-trace gpurun_out/bench_trace/b_results.db > profiles/bench_all_configs_kernel_trace.txt",
+    out = ["command (run from /tmp with TMPDIR=/tmp; $R is the repository root, $OUT a scratch directory):",
+           "  rocprofv3 --kernel-trace --stats -d $OUT/bench_trace -o b -- python3 $R/bench.py --no-cpu",
+           "  python3 bench.py --summarise-trace $OUT/bench_trace/b_results.db > profiles/bench_all_configs_kernel_trace.txt",
            "source: view top_kernels of the results database; durations in microseconds", "",
            "%-84s %6s %12s %10s %10s %10s %6s %6s %7s" % ("kernel", "calls", "total_us", "avg_us", "min_us", "max_us", "pct", "vgpr", "lds")]
     for name, calls, tot, avg, pct in rows:
@@ -660,9 +661,9 @@ def summarise_mfma(db_path):
     for did, name, gx, gy, cn, v, dur in c.execute(q):
         r = rows.setdefault(did, {"name": name, "gx": gx, "gy": gy, "dur": dur, "c": {}})
         r["c"][cn] = r["c"].get(cn, 0.0) + v
-    out = ["command (run from /tmp with TMPDIR=/tmp; $R is the repository root on the GPU box):",
-           "  rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE --kernel-trace -d $R/gpurun_out/pmc_gemm -o g -- python3 $R/bench.py --pmc-gemm",
-           "  python3 bench.py --summarise-mfma gpurun_out/pmc_gemm/g_results.db > profiles/addmm_8192_and_skinny_pmc_mfma_duty.txt",
+    out = ["command (run from /tmp with TMPDIR=/tmp; $R is the repository root, $OUT a scratch directory):",
+           "  rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE --kernel-trace -d $OUT/pmc_gemm -o g -- python3 $R/bench.py --pmc-gemm",
+           "  python3 bench.py --summarise-mfma $OUT/pmc_gemm/g_results.db > profiles/addmm_8192_and_skinny_pmc_mfma_duty.txt",
            "workload: addmm 8192^3 five times, then addmm 64x16384x4096 (A given transposed) thirty times; fp32, random normal operands", "",
            "how to read it: every v_mfma_f32_32x32x2_f32 books 64 busy cycles on its SIMD, so flops = busy / 64 * 4096;",
            "  duty = SQ_VALU_MFMA_BUSY_CYCLES / (1024 SIMDs * GRBM_GUI_ACTIVE / 8 XCDs); clock = GRBM_GUI_ACTIVE / 8 / duration.",

@@ -632,7 +632,9 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     P.S = S;
     P.seg = seg;
     THCL_CHECK(P.O * P.S < (1ull << 31) && (P.O * P.S * P.I + kThreads - 1) / kThreads < (1ull << 31), THCL_DIM_WARNING);
-    const thcl_u64 windows = rows && S > 1 ? (total * sizeof(float) + kScanWindowBytes - 1) / kScanWindowBytes + 2 : 0;
+    // one hand-over slot per window and one more (run_scan walks the same windows)
+    const thcl_u64 per_window = (kScanWindowBytes / sizeof(float) + seg - 1) / seg;
+    const thcl_u64 windows = rows && S > 1 ? (P.O * S + per_window - 1) / per_window + 1 : 0;
     if (S > 1) P.totals = (double *)thcl_rt_workspace(rt, (size_t)(P.O * P.S * P.I + windows) * sizeof(double));
     THCL_CHECK(S == 1 || P.totals != nullptr, "%s", thcl_rt_error());
     const bool vec = (rows || shortrows) && (P.R % 4 == 0) && aligned;
