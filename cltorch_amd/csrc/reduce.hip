@@ -514,6 +514,57 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
   }
 }
 
+// Reduced dim dense and short (at most 2048 elements, a multiple of 4, 16-byte aligned slices): 2^lpr_log2 lanes
+// share a slice, PER float4 each, and FLY = 8 / PER passes of the block's slices are requested before any is
+// consumed, so a lane has 8 loads in flight whatever the slice length.  reduce_rows keeps one pass in flight, which
+// leaves short slices waiting on memory (2^22 x 16 along dim 2: 71 us, bound 39).
+template <int KIND, bool ARG, int LPRL2, int PER>
+__global__ __launch_bounds__(kThreads) void reduce_rows_short(ReduceDimParams P) {
+  typedef Slot<KIND, ARG> S;
+  typedef typename S::T T;
+  constexpr int FLY = 8 / PER;
+  constexpr thcl_u32 lpr = 1u << LPRL2, rows = (thcl_u32)kThreads >> LPRL2;  // lanes per slice, slices per pass
+  const thcl_u32 sub = threadIdx.x & (lpr - 1), rib = threadIdx.x >> LPRL2;
+  const thcl_u32 r4 = P.R >> 2;
+  const thcl_u32 npass = (P.nslices + rows - 1) / rows;
+  for (thcl_u32 p0 = blockIdx.x * FLY; p0 < npass; p0 += gridDim.x * FLY) {
+    thcl_f4 v[FLY][PER];
+#pragma unroll
+    for (int f = 0; f < FLY; f++) {
+      // every load is issued: slices and lanes past the end read the last slice / the slice's last float4 again
+      // (a branch around a load makes the compiler wait for the loads before it)
+      thcl_u32 s = (p0 + f) * rows + rib;
+      if (s >= P.nslices) s = P.nslices - 1;
+      const thcl_f4 *row4 = (const thcl_f4 *)(P.in + thcl_generic_offset(s, P.L));
+#pragma unroll
+      for (int k = 0; k < PER; k++) {
+        thcl_u32 i = sub + (thcl_u32)k * lpr;
+        if (i >= r4) i = r4 - 1;
+        v[f][k] = __builtin_nontemporal_load(row4 + i);
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < FLY; f++) {
+      const thcl_u32 s = (p0 + f) * rows + rib;
+      const bool in = p0 + f < npass && s < P.nslices;
+      T acc = S::init();
+      if (in) {
+#pragma unroll
+        for (int k = 0; k < PER; k++) {
+          const thcl_u32 i = sub + (thcl_u32)k * lpr;
+          if (i < r4) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc = S::take(acc, v[f][k][c], (int)(i * 4 + c), P.exponent);
+          }
+        }
+        acc = S::seal(acc, (int)(sub * 4), sub < r4);
+      }
+      acc = S::reduce(acc, (int)lpr);
+      if (in && sub == 0) S::store(P, s, acc);
+    }
+  }
+}
+
 // Reduced dim is strided: lanes lie along the slices (UB lanes x VEC adjacent
 // slices; UB = 64 unless the slices are fewer, then the wave's other lanes take
 // further rows), the 4 waves of a block interleave over the reduced dim and meet in
@@ -805,7 +856,17 @@ void launch_all(bool dense, unsigned grid, hipStream_t stream, const ReduceAllPa
 template <int KIND, bool ARG>
 void launch_dim(bool rows, int lpr, int vec, dim3 grid, hipStream_t stream, const ReduceDimParams &P) {
   dim3 block(kThreads);
-  if (rows) {
+  if (rows && lpr == -2) {  // short dense slices: vec carries the float4 per lane
+#define SHORT_CASE(L2, PER) hipLaunchKernelGGL((reduce_rows_short<KIND, ARG, L2, PER>), grid, block, 0, stream, P)
+    if (P.ub_log2 == 0) SHORT_CASE(0, 1);
+    else if (P.ub_log2 == 2) SHORT_CASE(2, 1);
+    else if (P.ub_log2 == 4) SHORT_CASE(4, 1);
+    else if (vec == 1) SHORT_CASE(6, 1);
+    else if (vec == 2) SHORT_CASE(6, 2);
+    else if (vec == 4) SHORT_CASE(6, 4);
+    else SHORT_CASE(6, 8);
+#undef SHORT_CASE
+  } else if (rows) {
 #define ROWS_CASE(L, V) \
   if (lpr == L && vec == V) { hipLaunchKernelGGL((reduce_rows<KIND, ARG, L, V>), grid, block, 0, stream, P); return; }
     ROWS_CASE(1, 1) ROWS_CASE(1, 4) ROWS_CASE(8, 1) ROWS_CASE(8, 4) ROWS_CASE(64, 1) ROWS_CASE(64, 4) ROWS_CASE(256, 1) ROWS_CASE(256, 4)
@@ -1098,6 +1159,20 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     bool v4 = (R % 4 == 0) && aligned16(P.in);
     for (int d = 0; d < L.dims && v4; d++) v4 = (L.strides[d] % 4 == 0) || L.sizes[d] == 1;
     vec = v4 ? 4 : 1;
+    if (v4 && R <= 2048 && R > 1) {
+      // short dense slices: enough lanes for one float4 each up to 256 elements, then 2, 4 or 8 float4 per lane
+      const long r4 = R / 4;
+      unsigned l2 = 0;
+      while ((1l << l2) < r4 && l2 < 6) l2 += 2;   // 1, 4, 16 or 64 lanes
+      int per = 1;
+      while ((long)per * 64 < r4) per *= 2;
+      P.ub_log2 = l2;
+      lpr = -2;
+      vec = per;
+      const long slices_per_pass = kThreads >> l2, passes = (nslices + slices_per_pass - 1) / slices_per_pass;
+      const long fly = 8 / per, blocks = (passes + fly - 1) / fly;
+      grid.x = (unsigned)(blocks > (1l << 22) ? (1l << 22) : blocks);
+    } else {
     const long groups = (nslices + (kThreads / lpr) - 1) / (kThreads / lpr);
     grid.x = (unsigned)(groups > (1l << 22) ? (1l << 22) : groups);
     // few long slices: cut them into pieces of at least 8192 elements until the chip is full
@@ -1115,6 +1190,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
           grid.y = (unsigned)split;
         }
       }
+    }
     }
   } else {
     const int last = L.dims - 1;

@@ -272,3 +272,41 @@ def test_profiling_books_launches_under_their_entry_points(cl):
     assert 0.001 < rows["THClTensor_cadd"][2] < 5.0      # milliseconds per launch: microseconds, not seconds
     assert total == 6.0 * (1 << 20)
     assert cl.dumpProfiling().strip().count("\n") == 0    # records were cleared
+
+
+@pytest.mark.parametrize("R", [4, 8, 12, 16, 20, 60, 64, 100, 252, 256, 260, 512, 1000, 1024, 2044, 2048])
+def test_short_dense_slices_of_every_lane_grouping(cl, R):
+    """Dense slices of 4 to 2048 elements (a multiple of 4) take the kernel that shares a slice among 1, 4, 16 or 64
+    lanes with one to eight 16-byte loads each and keeps eight passes in flight: slice counts that leave passes and
+    blocks ragged, values with ties, NaNs, infinities and slices made of the start value only, outer dims that are
+    views (slices start at multiples of 4 elements but are not adjacent), and the value-only kinds."""
+    rs = np.random.RandomState(R)
+    for n in (1, 3, 257, 5000 if R <= 256 else 700):
+        x = rs.randint(-4, 5, size=(n, R)).astype(F)                    # many ties
+        x[rs.randint(n), rs.randint(R)] = np.nan
+        if n > 2:
+            x[1] = -np.inf                                               # a slice made of max's start value
+            x[2] = np.inf
+            x[2, R - 1] = -np.inf
+        p = Pair.dense(cl, x)
+        for kind in ("max", "min"):
+            wv, wi = oracle.reduce_dim(kind, p.view, 1)
+            gv, gi = getattr(p.dev, kind)(2)
+            assert_bit_equal(gv.float(), wv, f"{kind} of {n} slices of {R}")
+            assert np.array_equal(gi.long(), wi), f"positions of {kind}, {n} slices of {R}"
+        y = rs.standard_normal((n, R)).astype(F)
+        Y = cl.ClTensor(y)
+        close_sum(Y.sum(2).float(), y.astype(np.float64).sum(axis=1, keepdims=True))
+        got = Y.prod(2).float() if R <= 64 else None
+        if got is not None:
+            want = y.astype(np.float64).prod(axis=1, keepdims=True)
+            assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-30)
+        assert np.allclose(Y.norm(2.0, 2).float(), np.sqrt((y.astype(np.float64) ** 2).sum(axis=1, keepdims=True)), rtol=1e-5)
+    # slices that are not adjacent: a narrowed outer dim and a 3-d tensor whose middle dim is narrowed
+    z = rs.standard_normal((6, 9, R)).astype(F)
+    pz = Pair.dense(cl, z).narrow(1, 2, 5).narrow(0, 1, 4)
+    wv, wi = oracle.reduce_dim("max", pz.view, 2)
+    gv, gi = pz.dev.max(3)
+    assert_bit_equal(gv.float(), wv, "max over the last dim of a narrowed 3-d view")
+    assert np.array_equal(gi.long(), wi)
+    close_sum(pz.dev.sum(3).float(), z[1:5, 2:7].astype(np.float64).sum(axis=2, keepdims=True))
