@@ -275,44 +275,76 @@ __device__ __forceinline__ void finish_all(typename Acc<KIND>::T blockval, const
   }
 }
 
+// One of a thread's running values over a dense stream of float4 loads.
+template <int KIND>
+struct Chain {
+  typedef typename Acc<KIND>::T T;
+  T acc = Acc<KIND>::init();
+  __device__ __forceinline__ void take4(thcl_f4 v, float e) {
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(v[c], e));
+  }
+  __device__ __forceinline__ T value() const { return acc; }
+};
+// Max and min: the extremum of the numbers with the three-operand instruction
+// (it skips quiet NaNs), and whether a NaN went by with one unordered compare
+// per two elements, folded in scalar registers.  One vector instruction per
+// element where Acc's rule takes three.  The instruction is written out
+// because fmaxf() puts a canonicalising v_max in front of every loaded operand.
+template <bool MAX>
+struct ChainExtremum {
+  typedef float T;
+  float acc = MAX ? -INFINITY : INFINITY;
+  bool nan = false;
+  static __device__ __forceinline__ float three(float a, float b, float c) {
+    float r;
+    if (MAX) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    else asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+  }
+  __device__ __forceinline__ void take4(thcl_f4 v, float) {
+    acc = three(acc, v[0], v[1]);
+    acc = three(acc, v[2], v[3]);
+    nan |= __builtin_isunordered(v[0], v[1]) | __builtin_isunordered(v[2], v[3]);
+  }
+  __device__ __forceinline__ T value() const { return nan ? __builtin_nanf("") : acc; }
+};
+template <>
+struct Chain<RED_MAX> : ChainExtremum<true> {};
+template <>
+struct Chain<RED_MIN> : ChainExtremum<false> {};
+
 template <int KIND>
 __global__ __launch_bounds__(kThreads) void reduce_all_dense(ReduceAllParams P) {
   typedef typename Acc<KIND>::T T;
   __shared__ T lds[kThreads / kWave];
   constexpr int U = 4;
-  T acc[U];
-#pragma unroll
-  for (int k = 0; k < U; k++) acc[k] = Acc<KIND>::init();
+  Chain<KIND> chain[U];
   // 16-byte aligned body as float4, unaligned head/tail as scalars
   const uintptr_t addr = (uintptr_t)P.in;
   thcl_u64 head = ((16 - (addr & 15)) & 15) / 4;
   if (head > P.n) head = P.n;
   const thcl_u64 n4 = (P.n - head) >> 2;
   const thcl_f4 *in4 = (const thcl_f4 *)(P.in + head);
-  const thcl_u64 tile = (thcl_u64)kThreads * U;
-  for (thcl_u64 base = (thcl_u64)blockIdx.x * tile + threadIdx.x; base < n4; base += (thcl_u64)gridDim.x * tile) {
+  const thcl_u64 tile = (thcl_u64)kThreads * U, all = (thcl_u64)gridDim.x * tile;
+  thcl_u64 base = (thcl_u64)blockIdx.x * tile + threadIdx.x;
+  // whole tiles: U loads issued back to back with nothing conditional between them
+  for (; base + (U - 1) * kThreads < n4; base += all) {
     thcl_f4 v[U];
 #pragma unroll
-    for (int k = 0; k < U; k++) {
-      const thcl_u64 i = base + (thcl_u64)k * kThreads;
-      if (i < n4) v[k] = __builtin_nontemporal_load(in4 + i);
-    }
+    for (int k = 0; k < U; k++) v[k] = __builtin_nontemporal_load(in4 + base + (thcl_u64)k * kThreads);
 #pragma unroll
-    for (int k = 0; k < U; k++) {
-      const thcl_u64 i = base + (thcl_u64)k * kThreads;
-      if (i < n4) {
-#pragma unroll
-        for (int c = 0; c < 4; c++) acc[k] = Acc<KIND>::comb(acc[k], Acc<KIND>::lift(v[k][c], P.exponent));
-      }
-    }
+    for (int k = 0; k < U; k++) chain[k].take4(v[k], P.exponent);
   }
+  for (; base < n4; base += kThreads) chain[0].take4(in4[base], P.exponent);  // the one ragged tile
+  T acc0 = chain[0].value();
   if (blockIdx.x == 0) {
     const thcl_u64 tail0 = head + (n4 << 2);
-    for (thcl_u64 i = threadIdx.x; i < head; i += kThreads) acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i], P.exponent));
+    for (thcl_u64 i = threadIdx.x; i < head; i += kThreads) acc0 = Acc<KIND>::comb(acc0, Acc<KIND>::lift(P.in[i], P.exponent));
     for (thcl_u64 i = tail0 + threadIdx.x; i < P.n; i += kThreads)
-      acc[0] = Acc<KIND>::comb(acc[0], Acc<KIND>::lift(P.in[i], P.exponent));
+      acc0 = Acc<KIND>::comb(acc0, Acc<KIND>::lift(P.in[i], P.exponent));
   }
-  T v = Acc<KIND>::comb(Acc<KIND>::comb(acc[0], acc[1]), Acc<KIND>::comb(acc[2], acc[3]));
+  T v = Acc<KIND>::comb(Acc<KIND>::comb(acc0, chain[1].value()), Acc<KIND>::comb(chain[2].value(), chain[3].value()));
   v = block_reduce<KIND, T>(v, lds);
   finish_all<KIND>(v, P, lds);
 }

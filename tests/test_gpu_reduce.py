@@ -89,6 +89,21 @@ def test_reduce_all_special_values(cl):
     y[4321] = -3.0
     assert cl.ClTensor(y).max() == -3.0 and cl.ClTensor(y).min() == -np.inf
     assert cl.ClTensor(np.array([-0.0, 0.0], dtype=F)).sum() == 0.0
+    # a NaN anywhere in a stream of whole and ragged tiles (quiet or signalling), infinities among numbers
+    for n in (1, 5, 1023, 4099, (1 << 20) + 7):
+        a = oracle.uniform(15 + n, n)
+        A = cl.ClTensor(a)
+        assert A.max() == a.max() and A.min() == a.min()
+        for pos in {0, n // 2, n - 1}:
+            for bits in (0x7fc00000, 0x7f800001, 0xffc00000):
+                b = a.copy()
+                b.view(np.uint32)[pos] = bits
+                B = cl.ClTensor(b)
+                assert np.isnan(B.max()) and np.isnan(B.min()), (n, pos, hex(bits))
+        if n >= 4:
+            b = a.copy()
+            b[n // 3], b[n // 2] = np.inf, -np.inf
+            assert cl.ClTensor(b).max() == np.inf and cl.ClTensor(b).min() == -np.inf
 
 
 def test_reduce_all_on_views(cl):
