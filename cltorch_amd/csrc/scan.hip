@@ -294,8 +294,8 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
 // adjacent columns (one 16-byte access per row; the TC threads that share a row read 16 * TC
 // contiguous bytes), so 256 / TC rows per column are combined side by side: thread totals, a
 // shuffle scan over the row groups of a wave, the 4 waves' totals through LDS, then the rows are
-// finished from the registers.  One barrier a step; the next step's rows are requested before
-// this step's work.  TC = 8 for wide tensors; with 4 to 28 columns TC = 1, 2, 4 or 8 covers the whole
+// finished from the registers.  One barrier a step; the rows of the next two steps are requested before
+// this step's work (two steps ahead instead of one: 108 -> 103 us on 4096 x 16384).  TC = 8 for wide tensors; with 4 to 28 columns TC = 1, 2, 4 or 8 covers the whole
 // width and consecutive rows are adjacent in memory, so a step reads one contiguous run.  PHASE 0 leaves the segment's
 // totals, PHASE 1 scans (from the segment's carry when the lines are cut into segments).
 template <bool PROD, int TC, int PHASE>
@@ -329,12 +329,8 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
   double carry[4];
 #pragma unroll
   for (int c = 0; c < 4; c++) carry[c] = (PHASE == 1 && P.S > 1) ? tot[c] : Op<PROD>::identity();
-  thcl_f4 x[K], xn[K];
-  fetch(x, rbegin);
-  int buf = 0;
-  for (thcl_u64 r0 = rbegin; r0 < rend; r0 += ROWS, buf ^= 1) {
-    fetch(xn, r0 + ROWS);
-    __builtin_amdgcn_sched_barrier(0);
+  // one step: the 256 / TC * K rows from r0, held in x
+  auto step = [&](thcl_f4 (&x)[K], thcl_u64 r0, int buf) {
 #pragma unroll
     for (int k = 0; k < K; k++)
       if (r0 + (thcl_u64)tr * K + k >= rend) x[k] = thcl_f4{fill, fill, fill, fill};
@@ -383,8 +379,44 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
         if (live && r < rend) __builtin_nontemporal_store(v, (thcl_f4 *)(dst + r * P.I));
       }
     }
-#pragma unroll
-    for (int k = 0; k < K; k++) x[k] = xn[k];
+  };
+  // three sets of registers take turns: while one step is worked on, the rows of the next two are on their way
+  // (six steps a round: the register sets come round every three, the two LDS buffers every two)
+  thcl_f4 xa[K], xb[K], xc[K];
+  fetch(xa, rbegin);
+  fetch(xb, rbegin + ROWS);
+  thcl_u64 r0 = rbegin;
+  for (;;) {
+    fetch(xc, r0 + 2 * ROWS);
+    __builtin_amdgcn_sched_barrier(0);
+    step(xa, r0, 0);
+    r0 += ROWS;
+    if (r0 >= rend) break;
+    fetch(xa, r0 + 2 * ROWS);
+    __builtin_amdgcn_sched_barrier(0);
+    step(xb, r0, 1);
+    r0 += ROWS;
+    if (r0 >= rend) break;
+    fetch(xb, r0 + 2 * ROWS);
+    __builtin_amdgcn_sched_barrier(0);
+    step(xc, r0, 0);
+    r0 += ROWS;
+    if (r0 >= rend) break;
+    fetch(xc, r0 + 2 * ROWS);
+    __builtin_amdgcn_sched_barrier(0);
+    step(xa, r0, 1);
+    r0 += ROWS;
+    if (r0 >= rend) break;
+    fetch(xa, r0 + 2 * ROWS);
+    __builtin_amdgcn_sched_barrier(0);
+    step(xb, r0, 0);
+    r0 += ROWS;
+    if (r0 >= rend) break;
+    fetch(xb, r0 + 2 * ROWS);
+    __builtin_amdgcn_sched_barrier(0);
+    step(xc, r0, 1);
+    r0 += ROWS;
+    if (r0 >= rend) break;
   }
   if (PHASE == 0 && tr == 0 && live) {
 #pragma unroll
@@ -592,11 +624,6 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     // 0.8 -> 2.0, 1.7 -> 2.1, 2.5 -> 3.0 TB/s.
     int strip_tc = 8;
     bool narrow = false;
-    if (!strip && few_lines && P.I <= 28 && P.R >= 16384) {
-      strip_tc = P.I <= 4 ? 1 : (P.I <= 8 ? 2 : (P.I <= 16 ? 4 : 8));
-      strips = P.O;
-      strip = narrow = true;
-    }
     thcl_u64 S = 1;
     if (narrow) {
       const thcl_u64 want = (thcl_u64)cus * 8;  // blocks
