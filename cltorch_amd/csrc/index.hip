@@ -141,14 +141,19 @@ __global__ __launch_bounds__(kThreads) void mask_count(MaskParams P) {
   const thcl_u64 chunk0 = (thcl_u64)blockIdx.x * kChunk;
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   float m[kMaskSteps][kMaskPer];
+  if (VEC && chunk0 + kChunk <= P.n) {
+    // a whole chunk (the same for every thread of the block): the loads go out together, nothing between them
 #pragma unroll
-  for (int step = 0; step < kMaskSteps; step++) {
-    const thcl_u64 first = chunk0 + (thcl_u64)step * kMaskStep + (thcl_u64)threadIdx.x * kMaskPer;
-    if (VEC && first + kMaskPer <= P.n) {
+    for (int step = 0; step < kMaskSteps; step++) {
+      const thcl_u64 first = chunk0 + (thcl_u64)step * kMaskStep + (thcl_u64)threadIdx.x * kMaskPer;
       const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(P.mask + first));
 #pragma unroll
       for (int e = 0; e < kMaskPer; e++) m[step][e] = v[e];
-    } else {
+    }
+  } else {
+#pragma unroll
+    for (int step = 0; step < kMaskSteps; step++) {
+      const thcl_u64 first = chunk0 + (thcl_u64)step * kMaskStep + (thcl_u64)threadIdx.x * kMaskPer;
 #pragma unroll
       for (int e = 0; e < kMaskPer; e++) m[step][e] = (first + e < P.n) ? P.mask[first + e] : 0.0f;
     }
