@@ -379,24 +379,24 @@ __global__ __launch_bounds__(kThreads) void dot_dense(ReduceAllParams P, const f
   if (VEC) {
     const thcl_u64 n4 = P.n >> 2, tile = (thcl_u64)kThreads * U;
     const thcl_f4 *a4 = (const thcl_f4 *)P.in, *b4 = (const thcl_f4 *)other;
-    for (thcl_u64 base = (thcl_u64)blockIdx.x * tile + threadIdx.x; base < n4; base += (thcl_u64)gridDim.x * tile) {
+    thcl_u64 base = (thcl_u64)blockIdx.x * tile + threadIdx.x;
+    // whole tiles: 2 * U loads issued back to back with nothing conditional between them
+    for (; base + (U - 1) * kThreads < n4; base += (thcl_u64)gridDim.x * tile) {
       thcl_f4 x[U], y[U];
 #pragma unroll
       for (int k = 0; k < U; k++) {
-        const thcl_u64 i = base + (thcl_u64)k * kThreads;
-        if (i < n4) {
-          x[k] = __builtin_nontemporal_load(a4 + i);
-          y[k] = __builtin_nontemporal_load(b4 + i);
-        }
+        x[k] = __builtin_nontemporal_load(a4 + base + (thcl_u64)k * kThreads);
+        y[k] = __builtin_nontemporal_load(b4 + base + (thcl_u64)k * kThreads);
       }
 #pragma unroll
-      for (int k = 0; k < U; k++) {
-        const thcl_u64 i = base + (thcl_u64)k * kThreads;
-        if (i < n4) {
+      for (int k = 0; k < U; k++)
 #pragma unroll
-          for (int c = 0; c < 4; c++) acc[k] += (double)x[k][c] * (double)y[k][c];
-        }
-      }
+        for (int c = 0; c < 4; c++) acc[k] += (double)x[k][c] * (double)y[k][c];
+    }
+    for (; base < n4; base += kThreads) {  // the one ragged tile
+      const thcl_f4 x = a4[base], y = b4[base];
+#pragma unroll
+      for (int c = 0; c < 4; c++) acc[0] += (double)x[c] * (double)y[c];
     }
     if (blockIdx.x == 0)
       for (thcl_u64 i = (n4 << 2) + threadIdx.x; i < P.n; i += kThreads) acc[0] += (double)P.in[i] * (double)other[i];
