@@ -36,9 +36,15 @@
 // keep 256-thread blocks because a grid of one-wave blocks outruns the dispatcher.
 #define THCL_CONTIG_W_FOR(NT) ((NT) >= 3 ? 2 : 4)
 #define THCL_CONTIG_THREADS_FOR(NT) ((NT) >= 2 ? 64 : 256)
+#ifndef THCL_JOINT_V4_UNROLL
 #define THCL_JOINT_V4_UNROLL 1
-#define THCL_JOINT_S_UNROLL 4
+#endif
+#ifndef THCL_JOINT_S_UNROLL
+#define THCL_JOINT_S_UNROLL 8
+#endif
+#ifndef THCL_GENERIC_UNROLL
 #define THCL_GENERIC_UNROLL 4
+#endif
 #define THCL_JOINT_MAX_DIMS 8
 #define THCL_GENERIC_MAX_DIMS 25
 
@@ -232,14 +238,15 @@ __device__ __forceinline__ void thcl_apply_contig_s(const ThclContigParams &P) {
   for (thcl_u64 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
     const thcl_u64 base = tile * (THCL_APPLY_THREADS * THCL_CONTIG_S_UNROLL) + threadIdx.x;
     float o[THCL_CONTIG_S_UNROLL], a[THCL_CONTIG_S_UNROLL], b[THCL_CONTIG_S_UNROLL];
+    // Every load is issued: lanes past the end read the last element again and store nothing.  (A test
+    // around the loads makes the compiler wait for each group before it issues the next.)
 #pragma unroll
     for (int k = 0; k < THCL_CONTIG_S_UNROLL; k++) {
-      const thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
-      if (i < P.n) {
-        o[k] = thcl_ld(P.p[0] + i);
-        if (NT > 1) a[k] = thcl_ld(P.p[1] + i);
-        if (NT > 2) b[k] = thcl_ld(P.p[2] + i);
-      }
+      thcl_u64 i = base + (thcl_u64)k * THCL_APPLY_THREADS;
+      if (i >= P.n) i = P.n - 1;
+      o[k] = thcl_ld(P.p[0] + i);
+      if (NT > 1) a[k] = thcl_ld(P.p[1] + i);
+      if (NT > 2) b[k] = thcl_ld(P.p[2] + i);
     }
 #pragma unroll
     for (int k = 0; k < THCL_CONTIG_S_UNROLL; k++) {
@@ -268,6 +275,7 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
 #pragma unroll
     for (int k = 0; k < U; k++) {
       thcl_u32 u = base + k * THCL_APPLY_THREADS;
+      if (u >= P.nunits) u = P.nunits - 1;  // lanes past the end read the last unit again and store nothing
       thcl_u64 o0 = 0, o1 = 0, o2 = 0;
       for (int d = P.dims - 1; d > 0; d--) {
         const thcl_u32 q = thcl_div(u, P.size[d]);
@@ -288,12 +296,10 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
       const bool same1 = NT > 1 && P.stride[1][P.dims - 1] == 0, same2 = NT > 2 && P.stride[2][P.dims - 1] == 0;
       thcl_f4 o[U], a[U], b[U];
 #pragma unroll
-      for (int k = 0; k < U; k++) {
-        if (base + k * THCL_APPLY_THREADS < P.nunits) {
-          o[k] = thcl_ld((const thcl_f4 *)(P.p[0] + off[k][0]));
-          if (NT > 1) a[k] = thcl_ld_unit<thcl_f4>(P.p[1] + off[k][1], same1);
-          if (NT > 2) b[k] = thcl_ld_unit<thcl_f4>(P.p[2] + off[k][2], same2);
-        }
+      for (int k = 0; k < U; k++) {  // all loads issued, no test between them
+        o[k] = thcl_ld((const thcl_f4 *)(P.p[0] + off[k][0]));
+        if (NT > 1) a[k] = thcl_ld_unit<thcl_f4>(P.p[1] + off[k][1], same1);
+        if (NT > 2) b[k] = thcl_ld_unit<thcl_f4>(P.p[2] + off[k][2], same2);
       }
 #pragma unroll
       for (int k = 0; k < U; k++) {
@@ -315,12 +321,10 @@ __device__ __forceinline__ void thcl_apply_joint(const ThclJointParams &P) {
       const bool stream0 = P.stride[0][P.dims - 1] == 1;
       float o[U], a[U], b[U];
 #pragma unroll
-      for (int k = 0; k < U; k++) {
-        if (base + k * THCL_APPLY_THREADS < P.nunits) {
-          o[k] = stream0 ? thcl_ld(P.p[0] + off[k][0]) : P.p[0][off[k][0]];
-          if (NT > 1) a[k] = thcl_ld(P.p[1] + off[k][1]);
-          if (NT > 2) b[k] = thcl_ld(P.p[2] + off[k][2]);
-        }
+      for (int k = 0; k < U; k++) {  // all loads issued, no test between them
+        o[k] = stream0 ? thcl_ld(P.p[0] + off[k][0]) : P.p[0][off[k][0]];
+        if (NT > 1) a[k] = thcl_ld(P.p[1] + off[k][1]);
+        if (NT > 2) b[k] = thcl_ld(P.p[2] + off[k][2]);
       }
 #pragma unroll
       for (int k = 0; k < U; k++) {
@@ -357,18 +361,25 @@ __device__ __forceinline__ void thcl_apply_generic(const ThclGenericParams &P) {
   const float v1 = P.val[0], v2 = P.val[1];
   for (thcl_u32 tile = blockIdx.x; tile < P.ntiles; tile += gridDim.x) {
     const thcl_u32 base = tile * (THCL_APPLY_THREADS * THCL_GENERIC_UNROLL) + threadIdx.x;
+    // all of the tile's loads first (lanes past the end read the last element again and store nothing),
+    // then the arithmetic, then the stores: a store between two loads would hold the second load back,
+    // since the operands may share memory
+    thcl_u64 o0[THCL_GENERIC_UNROLL];
+    float oo[THCL_GENERIC_UNROLL], a[THCL_GENERIC_UNROLL], b[THCL_GENERIC_UNROLL];
 #pragma unroll
     for (int k = 0; k < THCL_GENERIC_UNROLL; k++) {
-      const thcl_u32 i = base + k * THCL_APPLY_THREADS;
-      if (i < P.n) {
-        const thcl_u64 o0 = thcl_generic_offset(i, P.op[0]);
-        float oo = P.p[0][o0];
-        float a = 0.f, b = 0.f;
-        if (NT > 1) a = P.p[1][thcl_generic_offset(i, P.op[1])];
-        if (NT > 2) b = P.p[2][thcl_generic_offset(i, P.op[2])];
-        thcl_apply_one<Op>(oo, a, b, v1, v2, p1, p2);
-        P.p[0][o0] = oo;
-      }
+      thcl_u32 i = base + k * THCL_APPLY_THREADS;
+      if (i >= P.n) i = P.n - 1;
+      o0[k] = thcl_generic_offset(i, P.op[0]);
+      oo[k] = P.p[0][o0[k]];
+      a[k] = b[k] = 0.f;
+      if (NT > 1) a[k] = P.p[1][thcl_generic_offset(i, P.op[1])];
+      if (NT > 2) b[k] = P.p[2][thcl_generic_offset(i, P.op[2])];
+    }
+#pragma unroll
+    for (int k = 0; k < THCL_GENERIC_UNROLL; k++) {
+      thcl_apply_one<Op>(oo[k], a[k], b[k], v1, v2, p1, p2);
+      if (base + k * THCL_APPLY_THREADS < P.n) P.p[0][o0[k]] = oo[k];
     }
   }
 }
