@@ -39,7 +39,7 @@ struct GemmParams {
   int ksplit;   // blockIdx.y slices of K; > 1: raw partial products go to `work`
   int kchunk;   // K per slice (multiple of BK)
   float *work;  // [ksplit][n][m] dense partials
-  // edge kernels: the operand's 16-byte groups along its contiguous dim are whole and aligned
+  // the operand's 16-byte groups along its contiguous dim are whole and aligned (a and b: picks the edge kernel)
   int vec_a, vec_b, vec_c;
 };
 
@@ -49,24 +49,29 @@ struct TileLds {
   static constexpr int FLOATS = KC ? BMN * KPITCH : BK * BMN;
 };
 
-// global -> registers: each thread carries BMN*BK/256/4 float4
-template <int BMN, bool KC, bool EDGE>
+// global -> registers: each thread carries BMN*BK/256/4 float4.  EDGE 0: the tile is whole and aligned.  EDGE 1: a
+// 16-byte group of the operand is either inside it or outside, and aligned; every load is issued (from the operand's
+// first element when the group is outside) and groups outside become zeros, so there is no branch around a load.
+// EDGE 2: any pitch and alignment, one element at a time.  The choice is made at compile time: a run-time branch
+// between the two edge forms made the compiler wait for all loads at every slab (aligned 4096^3 through the edge
+// kernel: 101 TFLOP/s with the branch against 138 through the whole-tile kernel).
+template <int BMN, bool KC, int EDGE>
 struct TileLoader {
   static constexpr int NV = BMN * BK / 256 / 4;
   f4 r[NV];
 
   // g: operand base; ld: leading dim; mn0: first row/col of the tile; k0: first k; lim_mn/lim_k: extents
   // vec (edge kernels): a 16-byte group is either inside the operand or outside, and aligned
-  __device__ __forceinline__ void load(const float *g, int ld, int mn0, int k0, int lim_mn, int lim_k, bool vec) {
+  __device__ __forceinline__ void load(const float *g, int ld, int mn0, int k0, int lim_mn, int lim_k) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = threadIdx.x + 256 * p;
       if (KC) {
         const int mn = f / (BK / 4), kq = f % (BK / 4);
         const float *src = g + (size_t)(mn0 + mn) * ld + k0 + kq * 4;
-        if (!EDGE) {
+        if (EDGE == 0) {
           r[p] = *(const f4 *)src;
-        } else if (vec) {
+        } else if (EDGE == 1) {
           const bool in = mn0 + mn < lim_mn && k0 + kq * 4 < lim_k;
           const f4 v = *(const f4 *)(in ? src : g);
           r[p] = in ? v : f4{0.f, 0.f, 0.f, 0.f};
@@ -78,9 +83,9 @@ struct TileLoader {
       } else {
         const int kk = f / (BMN / 4), q = f % (BMN / 4);
         const float *src = g + (size_t)(k0 + kk) * ld + mn0 + q * 4;
-        if (!EDGE) {
+        if (EDGE == 0) {
           r[p] = *(const f4 *)src;
-        } else if (vec) {
+        } else if (EDGE == 1) {
           const bool in = k0 + kk < lim_k && mn0 + q * 4 < lim_mn;
           const f4 v = *(const f4 *)(in ? src : g);
           r[p] = in ? v : f4{0.f, 0.f, 0.f, 0.f};
@@ -126,7 +131,7 @@ __device__ __forceinline__ void read_frags(const float *lds, int mn_wave0, int k
 }
 
 // TA: op(A) = A^T (A stored k-contiguous); TB: op(B) = B^T (B stored n-contiguous)
-template <int BM, int BN, bool TA, bool TB, bool EDGE>
+template <int BM, int BN, bool TA, bool TB, int EDGE>
 __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   constexpr bool AKC = TA;    // 'n': a[i + l*lda] (m-contiguous); 't': a[l + i*lda] (k-contiguous)
   constexpr bool BKC = !TB;   // 'n': b[l + j*ldb] (k-contiguous); 't': b[j + l*ldb] (n-contiguous)
@@ -181,11 +186,10 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   TileLoader<BN, BKC, EDGE> lb1;
   const int last = KT > 0 ? KT - 1 : 0;
   auto slab_k = [&](int kt) { return k_begin + (kt < last ? kt : last) * BK; };
-  const bool va = P.vec_a != 0, vb = P.vec_b != 0;
-  la.load(P.a, P.lda, m0, slab_k(0), P.m, k_end, va);
-  lb.load(P.b, P.ldb, n0, slab_k(0), P.n, k_end, vb);
-  la1.load(P.a, P.lda, m0, slab_k(1), P.m, k_end, va);
-  lb1.load(P.b, P.ldb, n0, slab_k(1), P.n, k_end, vb);
+  la.load(P.a, P.lda, m0, slab_k(0), P.m, k_end);
+  lb.load(P.b, P.ldb, n0, slab_k(0), P.n, k_end);
+  la1.load(P.a, P.lda, m0, slab_k(1), P.m, k_end);
+  lb1.load(P.b, P.ldb, n0, slab_k(1), P.n, k_end);
   la.store(lds);
   lb.store(lds + AF);
   __syncthreads();
@@ -193,8 +197,8 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   auto step = [&](int kt, int cur, auto &issue_a, auto &issue_b, auto &keep_a, auto &keep_b) {
     float *As = lds + cur * (AF + BF);
     float *Bs = As + AF;
-    issue_a.load(P.a, P.lda, m0, slab_k(kt + 2), P.m, k_end, va);
-    issue_b.load(P.b, P.ldb, n0, slab_k(kt + 2), P.n, k_end, vb);
+    issue_a.load(P.a, P.lda, m0, slab_k(kt + 2), P.m, k_end);
+    issue_b.load(P.b, P.ldb, n0, slab_k(kt + 2), P.n, k_end);
     __builtin_amdgcn_sched_barrier(0);   // keep the loads at the top of the step
     {
 #pragma unroll
@@ -301,7 +305,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(GemmParams P) {
   }
 }
 
-template <int BM, int BN, bool EDGE>
+template <int BM, int BN, int EDGE>
 void launch_tt(bool ta, bool tb, dim3 grid, hipStream_t s, const GemmParams &P) {
   dim3 block(256);
   if (!ta && !tb) hipLaunchKernelGGL((sgemm_mfma<BM, BN, false, false, EDGE>), grid, block, 0, s, P);
@@ -313,20 +317,6 @@ void launch_tt(bool ta, bool tb, dim3 grid, hipStream_t s, const GemmParams &P) 
 bool al16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 }  // namespace
 
-// tile choice: 128x128 by default; 64-wide tiles when a dimension is small
-static void choose_tile(long m, long n, int cus, int &bm, int &bn) {
-  bm = (m >= 128 && (m % 128 == 0 || m >= 1024)) ? 128 : 64;
-  bn = (n >= 128 && (n % 128 == 0 || n >= 1024)) ? 128 : 64;
-  // With fewer than 4 tiles of 128x128 per CU the chip is partly idle in the last
-  // round of blocks: halve the tile until there are that many.  Measured in
-  // steady state with random operands: 3072^3 98 -> 112 TFLOP/s, 3584^3 100 -> 110,
-  // 2560^3 101 -> 104, 1024^3 62 -> 66; from 4096^3 on 128x128 wins (130).
-  const long cus4 = 4L * cus;
-  if (bm == 128 && bn == 128 && (m / 128) * (n / 128) < cus4) {
-    bn = 64;
-    if ((m / 128) * (n / 64) < cus4) bm = 64;
-  }
-}
 // Few tiles and a long K: slice K over blockIdx.y so every CU has work; the slices'
 // partial products are summed in slice order by a second kernel.  Below one tile per
 // CU any K from 1024 up is sliced; between one and two tiles per CU only K >= 2048
@@ -347,9 +337,47 @@ static void choose_ksplit(long tiles, long k, int cus, int &ksplit, int &kchunk)
     kchunk = (int)chunk;
   }
 }
+// Tile choice by a small model of the launch, fitted to measurements on 256 CUs (cubes of 1024 to 6144 and ragged
+// shapes, predicted within a few percent):
+//   rate     what the tile's kernel sustains on a large product, in TFLOP/s: whole tiles / tiles with edges
+//   balance  a CU works through whole tiles, so the launch takes ceil(tiles / CUs) tile times
+//   useful   the part of the tiles' area that lies inside the matrix
+//   fill     one or two blocks on a CU do not keep its matrix pipes busy
+//   start    a block's first loads and its epilogue cost about as much as 8 of its K slabs
+// Products with few tiles are sliced along K as well (choose_ksplit), which fills the chip at the price of a
+// second pass over the result.
+static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, int &bn) {
+  struct Cand {
+    int bm, bn;
+    double whole, edge;
+    int resident;  // blocks a CU holds
+  };
+  static const Cand cands[4] = {{128, 128, 138., 128., 3}, {128, 64, 133., 124., 5}, {64, 128, 126., 118., 5}, {64, 64, 123., 110., 8}};
+  double best = -1.;
+  bm = bn = 64;
+  for (const Cand &c : cands) {
+    if ((c.bm == 128 && m < 128) || (c.bn == 128 && n < 128)) continue;
+    const long tm = (m + c.bm - 1) / c.bm, tn = (n + c.bn - 1) / c.bn, tiles = tm * tn;
+    const bool whole = aligned && m % c.bm == 0 && n % c.bn == 0;
+    int ks, kc;
+    choose_ksplit(tiles, k, cus, ks, kc);
+    const long blocks = tiles * ks, rounds = (blocks + cus - 1) / cus;
+    const double balance = (double)blocks / (double)(rounds * cus);
+    const double useful = ((double)m * (double)n) / ((double)(tm * c.bm) * (double)(tn * c.bn));
+    const long held = rounds < c.resident ? rounds : c.resident;
+    const double fill = held >= 3 ? 1.0 : held == 2 ? 0.9 : 0.75;
+    const double slabs = (double)((kc + BK - 1) / BK), start = slabs / (slabs + 8.);
+    const double score = (whole ? c.whole : c.edge) * balance * useful * fill * start * (ks > 1 ? 0.93 : 1.0);
+    if (score > best) {
+      best = score;
+      bm = c.bm;
+      bn = c.bn;
+    }
+  }
+}
 // the block tile and the K slicing a product of this shape gets on a chip with `cus` compute units
 void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk) {
-  choose_tile(m, n, cus, *bm, *bn);
+  choose_tile(m, n, k, cus, k % BK == 0, *bm, *bn);
   choose_ksplit(((m + *bm - 1) / *bm) * ((n + *bn - 1) / *bn), k, cus, *ksplit, *kchunk);
 }
 
@@ -376,11 +404,10 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   P.ldc = (int)ldc;
   P.alpha = alpha;
   P.beta = beta;
-  // tile choice: 128x128 by default; 64-wide tiles when a dimension is small
   int bm, bn;
-  choose_tile(m, n, thcl_rt_get_props(rt)->compute_units, bm, bn);
-  const bool fast = (m % bm == 0) && (n % bn == 0) && (k % BK == 0) && k > 0 && (lda % 4 == 0) && (ldb % 4 == 0) &&
-                    (ldc % 4 == 0) && al16(a) && al16(b) && al16(c);
+  const bool aligned = (k % BK == 0) && k > 0 && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && al16(a) && al16(b) && al16(c);
+  choose_tile(m, n, k, thcl_rt_get_props(rt)->compute_units, aligned, bm, bn);
+  const bool fast = aligned && (m % bm == 0) && (n % bn == 0);
   // an operand's contiguous dim is m for a 'n', k for a 't'; n for b 't', k for b 'n'
   const long a_run = ta ? k : m, b_run = tb ? n : k;
   P.vec_a = (lda % 4 == 0 && a_run % 4 == 0 && al16(a)) ? 1 : 0;
@@ -396,8 +423,9 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   }
   dim3 grid((unsigned)(P.tiles_m * P.tiles_n), (unsigned)P.ksplit);
 #define GO(BM_, BN_)                                                   \
-  if (fast) launch_tt<BM_, BN_, false>(ta, tb, grid, stream, P);        \
-  else launch_tt<BM_, BN_, true>(ta, tb, grid, stream, P);
+  if (fast) launch_tt<BM_, BN_, 0>(ta, tb, grid, stream, P);                        \
+  else if (P.vec_a && P.vec_b) launch_tt<BM_, BN_, 1>(ta, tb, grid, stream, P);     \
+  else launch_tt<BM_, BN_, 2>(ta, tb, grid, stream, P);
   if (bm == 128 && bn == 128) { GO(128, 128) }
   else if (bm == 128 && bn == 64) { GO(128, 64) }
   else if (bm == 64 && bn == 128) { GO(64, 128) }

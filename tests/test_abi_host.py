@@ -296,16 +296,22 @@ def test_user_kernel_renders_and_compiles_for_gfx950(lib):
 
 
 def test_gemm_tile_choice(lib):
-    """128x128 tiles unless that leaves fewer than 4 tiles per CU; ragged or small dims use 64-wide tiles."""
-    def tile(m, n, cus=256):
+    """The tile comes from a model of the launch: the kernel's rate, whole rounds of tiles per CU, the tiles' area
+    outside the matrix, blocks per CU, K slicing.  Known outcomes on 256 CUs, each confirmed by measurement."""
+    def tile(m, n, k, cus=256):
         bm, bn, ks, kc = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
-        lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(1), C.c_int(cus), C.byref(bm), C.byref(bn), C.byref(ks), C.byref(kc))
+        lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(k), C.c_int(cus), C.byref(bm), C.byref(bn), C.byref(ks), C.byref(kc))
         return bm.value, bn.value
-    assert tile(8192, 8192) == (128, 128) and tile(4096, 4096) == (128, 128)
-    assert tile(3072, 3072) == (128, 64) and tile(2048, 2048) == (64, 64) and tile(1024, 1024) == (64, 64)
-    assert tile(16384, 64) == (128, 64)          # the skinny configuration after the row-major swap
-    assert tile(100, 100) == (64, 64) and tile(200, 4096) == (64, 128)
-
+    assert tile(8192, 8192, 8192) == (128, 128) and tile(4096, 4096, 4096) == (128, 128) and tile(6144, 6144, 6144) == (128, 128)
+    assert tile(16384, 64, 4096) == (128, 64)    # the skinny configuration after the row-major swap
+    assert tile(4608, 4608, 4608) == (128, 64) and tile(5120, 5120, 5120) == (128, 64)   # 6 and 7 rounds of 128x128 tiles leave CUs idle
+    assert tile(3072, 3072, 3072) == (64, 64) and tile(2560, 2560, 2560) == (64, 64)     # 9 and 7 whole rounds of 64x64 tiles
+    assert tile(2048, 2048, 2048) == (64, 64) and tile(1024, 1024, 1024) == (64, 64)
+    assert tile(100, 100, 100) == (64, 64)
+    # ragged sizes: every tile shape has edges, the larger tiles' edge kernels keep the higher rate
+    assert tile(3000, 5000, 7000) == (128, 128) and tile(6000, 6000, 2000) == (128, 128)
+    # 63 x 64 rows and columns: whole 64-wide tiles (123 x 0.97 for the last round) lose to 128-wide ones with edges (128 x 0.97 of area)
+    assert tile(4032, 4032, 4096) == (128, 128)
 
 
 def test_gemm_k_slicing(lib):
@@ -318,7 +324,7 @@ def test_gemm_k_slicing(lib):
         return bm.value, bn.value, ks.value, kc.value
     assert plan(8192, 8192, 8192) == (128, 128, 1, 8192)
     assert plan(16384, 64, 4096) == (128, 64, 4, 1024)           # skinny: 128 tiles on 256 CUs
-    assert plan(2048, 512, 4096) == (64, 64, 2, 2048)            # 256 tiles: one per CU, long K
+    assert plan(2048, 512, 4096) == (128, 64, 4, 1024)           # 128 tiles, long K: the same 512 blocks as 256 tiles in 2 slices, at the larger tile's rate
     assert plan(1024, 1024, 1024) == (64, 64, 1, 1024)           # 256 tiles but K too short to pay for a second pass
     assert plan(64, 64, 100000)[2] == 368                        # one tile: as many slices of at least 256 as fit
     assert plan(32, 32, 1 << 20)[2] == 512                       # capped

@@ -152,6 +152,25 @@ def test_large_square_sampled(cl):
     assert np.array_equal(two, 2 * one)                      # scaling by 2 is exact
 
 
+@pytest.mark.parametrize("M,N,K", [(3000, 5000, 208), (1500, 7000, 120), (10000, 2000, 64), (4000, 4000, 104), (3000, 2900, 1000),
+                                   (2999, 5001, 77), (6016, 1000, 48)])
+def test_ragged_mid_size_shapes(cl, M, N, K):
+    """Sizes that are no multiple of the tiles, large enough for the 128-wide edge kernels (whole 16-byte groups, and
+    with the odd sizes one element at a time): the whole result against an fp64 product, row- and column-major A."""
+    rng = np.random.RandomState(M + N + K)
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
+    b = rng.standard_normal((K, N)).astype(F)
+    c = rng.standard_normal((M, N)).astype(F)
+    want = 0.5 * c.astype(np.float64) + 1.5 * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = float(np.sqrt(np.mean(want ** 2)))
+    B = cl.ClTensor(b)
+    got = cl.ClTensor(c).addmm(0.5, 1.5, cl.ClTensor(a), B).float()
+    assert np.max(np.abs(got - want)) / scale < RTOL
+    At = cl.ClTensor(np.ascontiguousarray(a.T)).t()
+    got = cl.ClTensor(c).addmm(0.5, 1.5, At, B).float()
+    assert np.max(np.abs(got - want)) / scale < RTOL
+
+
 def test_sliced_products_repeat_bit_exactly(cl):
     """K-sliced products sum their slices in slice order: every repetition gives the same
     bits, also with other reductions in between, with ragged shapes, with beta = 0 over
