@@ -163,12 +163,16 @@ def test_ragged_mid_size_shapes(cl, M, N, K):
     c = rng.standard_normal((M, N)).astype(F)
     want = 0.5 * c.astype(np.float64) + 1.5 * (a.astype(np.float64) @ b.astype(np.float64))
     scale = float(np.sqrt(np.mean(want ** 2)))
-    B = cl.ClTensor(b)
-    got = cl.ClTensor(c).addmm(0.5, 1.5, cl.ClTensor(a), B).float()
-    assert np.max(np.abs(got - want)) / scale < RTOL
-    At = cl.ClTensor(np.ascontiguousarray(a.T)).t()
-    got = cl.ClTensor(c).addmm(0.5, 1.5, At, B).float()
-    assert np.max(np.abs(got - want)) / scale < RTOL
+    As = (cl.ClTensor(a), cl.ClTensor(np.ascontiguousarray(a.T)).t())
+    Bs = (cl.ClTensor(b), cl.ClTensor(np.ascontiguousarray(b.T)).t())
+    for A in As:
+        for B in Bs:
+            got = cl.ClTensor(c).addmm(0.5, 1.5, A, B).float()
+            assert np.max(np.abs(got - want)) / scale < RTOL, (A.stride(), B.stride())
+    # a column-major result (the product's operands swap roles inside)
+    Ct = cl.ClTensor(np.ascontiguousarray(c.T)).t()
+    Ct.addmm(0.5, 1.5, As[0], Bs[1])
+    assert np.max(np.abs(Ct.float() - want)) / scale < RTOL
 
 
 def test_sliced_products_repeat_bit_exactly(cl):
