@@ -474,9 +474,10 @@ float THClTensor_dot(THClState *state, THClTensor *self, THClTensor *src) {
   const bool in_place = J.valid && J.dims == 1 && J.strides[0][0] == 1 && J.strides[1][0] == 1;
   ThclTemp a(state, in_place ? nullptr : THClTensor_newContiguous(state, self));
   ThclTemp b(state, in_place ? nullptr : THClTensor_newContiguous(state, src));
-  thcl_dot_dense(state, rt, thcl_dptr(in_place ? self : a.t), thcl_dptr(in_place ? src : b.t), n, thcl_rt_host_word_device(rt));
-  THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
-  const float result = thcl_rt_host_word(rt)[0];
+  const unsigned tag = thcl_rt_next_tag(rt);
+  thcl_dot_dense(state, rt, thcl_dptr(in_place ? self : a.t), thcl_dptr(in_place ? src : b.t), n, thcl_rt_tagged_word_device(rt), tag);
+  float result = 0.f;
+  THCL_CHECK(thcl_rt_await_tagged(rt, tag, &result) == 0, "%s", thcl_rt_error());
   return result;
   THCL_GUARD_END(0.f)
 }

@@ -132,7 +132,8 @@ struct MaskParams {
   thcl_u32 nblocks;
   thcl_u64 src_len;   // copy: elements available in src
   unsigned *ticket;   // arrival counter of the group blocks, zero between launches
-  unsigned *host_total;  // pinned host word (device address) that receives the grand total
+  unsigned long long *host_total;  // pinned host word pair (device address) that receives {grand total, tag} in one store
+  unsigned host_tag;
 };
 
 template <bool VEC>
@@ -246,7 +247,8 @@ __global__ __launch_bounds__(1024) void mask_scan_groups(MaskParams P) {
   }
   if (threadIdx.x == 0) {
     P.groups[P.ngroups] = carry;
-    *P.host_total = carry;
+    __hip_atomic_store(P.host_total, (unsigned long long)carry | ((unsigned long long)P.host_tag << 32), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
     *P.ticket = 0u;
   }
 }
@@ -647,7 +649,6 @@ void THClTensor_scatterFill(THClState *state, THClTensor *self, long dim, THClTe
 // per-chunk counts, group offsets and the grand total are 32-bit words
 constexpr long kMaskMaxElements = 1l << 32;
 constexpr int kMaskTicket = 8;     // word of the context's scratch block (words 1..63 are free for such counters)
-constexpr int kMaskHostWord = 2;   // word of the context's pinned block that receives the count
 static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long n) {
   hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   const long nb = (n + kChunk - 1) / kChunk;
@@ -667,18 +668,20 @@ static unsigned *mask_prefix(THClState *state, thcl_rt *rt, MaskParams &P, long 
   else hipLaunchKernelGGL(mask_count<false>, dim3((unsigned)nb), dim3(kThreads), 0, stream, P);
   check("mask count");
   P.ticket = (unsigned *)thcl_rt_scratch(rt, nullptr) + kMaskTicket;
-  P.host_total = (unsigned *)(thcl_rt_host_word_device(rt) + kMaskHostWord);
+  P.host_total = (unsigned long long *)thcl_rt_tagged_word_device(rt);
+  P.host_tag = thcl_rt_next_tag(rt);
   hipLaunchKernelGGL(mask_scan_groups, dim3((unsigned)ng), dim3(1024), 0, stream, P);
   check("mask offsets");
   (void)state;
   return P.counts;
 }
 
-static long read_total(thcl_rt *rt, const MaskParams &) {
-  // the last group block left the count in a pinned word: waiting for the stream is all it takes
-  THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
+static long read_total(thcl_rt *rt, const MaskParams &P) {
+  // the last group block left {count, tag} in the pinned pair: the host picks it up as soon as it lands
+  float as_float = 0.f;
+  THCL_CHECK(thcl_rt_await_tagged(rt, P.host_tag, &as_float) == 0, "%s", thcl_rt_error());
   unsigned total;
-  memcpy(&total, thcl_rt_host_word(rt) + kMaskHostWord, sizeof(total));
+  memcpy(&total, &as_float, sizeof(total));
   return (long)total;
 }
 

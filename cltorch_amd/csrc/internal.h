@@ -128,9 +128,12 @@ enum ThclReduce : int {
   RED_SUM_NE0 = 4, RED_SUM_ABS = 5, RED_SUM_SQ = 6, RED_SUM_POW = 7, RED_ALL = 8, RED_ANY = 9
 };
 // whole tensor -> one float at device address `out`
-void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out);
+void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out, unsigned host_tag = 0);
+// queues a launch that hands the device scalar at `src` to the host through the tagged word pair
+void thcl_scalar_to_host(THClState *state, thcl_rt *rt, const float *src, unsigned host_tag);
 void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *src, long dim);
-void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent = 0.f);
+// host_tag != 0: `out` is the pinned word pair of thcl_rt_tagged_word_device, which receives {result, tag} in one store
+void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent = 0.f, unsigned host_tag = 0);
 // The variant for callers that cannot allocate: tickets and partials in a static device array.
 void thcl_reduce_all_noalloc(THClState *state, ThclReduce kind, THClTensor *src, float *out);
 void thcl_reduce_static_setup(int device);  // once per device, with that device current

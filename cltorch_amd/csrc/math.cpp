@@ -503,9 +503,17 @@ static float reduce_all_to_host(THClState *state, ThclReduce kind, THClTensor *s
   // the last block stores the scalar straight into pinned host memory; waiting
   // for the stream is the only synchronising step, no copy follows
   // (the reference: blocking read-back of the scratch buffer, src/lib/THClTensorMath.cpp:346-368)
-  thcl_reduce_all(state, kind, self, thcl_rt_host_word_device(rt), exponent);
-  THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
-  return thcl_rt_host_word(rt)[0];
+  if (THClTensor_nElement(state, self) == 0) {
+    thcl_reduce_all(state, kind, self, thcl_rt_host_word_device(rt), exponent);
+    THCL_CHECK(thcl_rt_sync(rt) == 0, "%s", thcl_rt_error());
+    return thcl_rt_host_word(rt)[0];
+  }
+  // the kernel stores {result, tag} in one piece; the host picks it up as soon as it lands
+  const unsigned tag = thcl_rt_next_tag(rt);
+  thcl_reduce_all(state, kind, self, thcl_rt_tagged_word_device(rt), exponent, tag);
+  float value = 0.f;
+  THCL_CHECK(thcl_rt_await_tagged(rt, tag, &value) == 0, "%s", thcl_rt_error());
+  return value;
 }
 static void reduce_all_to_point(THClState *state, ThclReduce kind, THClTensor *self, THClTensor *src) {
   thcl_check_same_device(state, 2, self, src);
@@ -576,9 +584,13 @@ float THClTensor_as_float(THClState *state, THClTensor *self) {
   THCL_ARGCHECK(self->nDimension == 0, 1, "tensor must be point tensor, zero dimensions");
   THCL_ARGCHECK(self->storage != nullptr && self->storage->wrapper != nullptr, 1, "tensor must have allocated storage");
   thcl_rt *rt = thcl_ctx(state, self->storage->device);
-  float *hw = thcl_rt_host_word(rt);
-  THCL_CHECK(thcl_rt_memcpy_d2h(rt, hw, thcl_dptr(self), sizeof(float)) == 0, "%s", thcl_rt_error());
-  return hw[0];
+  // a one-thread launch hands the scalar over through the pinned {value, tag} pair: quicker than a copy
+  // followed by a wait for the stream
+  const unsigned tag = thcl_rt_next_tag(rt);
+  thcl_scalar_to_host(state, rt, thcl_dptr(self), tag);
+  float value = 0.f;
+  THCL_CHECK(thcl_rt_await_tagged(rt, tag, &value) == 0, "%s", thcl_rt_error());
+  return value;
   THCL_GUARD_END(0.f)
 }
 

@@ -214,6 +214,7 @@ struct ReduceAllParams {
   unsigned *ticket;
   float *out;
   float exponent;        // p of the |x|^p sum
+  unsigned host_tag;     // non-zero: `out` is a pinned host word pair that receives {result, tag} in one 8-byte store
   ThclGenericOperand L;  // strided input only
 };
 
@@ -270,7 +271,14 @@ __device__ __forceinline__ void finish_all(typename Acc<KIND>::T blockval, const
     v = Acc<KIND>::comb(v, load_fresh(&partials[i]));
   v = block_reduce<KIND, T>(v, lds);
   if (threadIdx.x == 0) {
-    P.out[0] = Acc<KIND>::lower(v);
+    const float r = Acc<KIND>::lower(v);
+    if (P.host_tag) {
+      // result and tag travel together, so a host that polls the pair sees both or neither
+      const unsigned long long pair = (unsigned long long)__float_as_uint(r) | ((unsigned long long)P.host_tag << 32);
+      __hip_atomic_store((unsigned long long *)P.out, pair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    } else {
+      P.out[0] = r;
+    }
     *P.ticket = 0u;
   }
 }
@@ -971,10 +979,10 @@ struct ReduceAllScratch {
 };
 
 void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, float *out, float exponent,
-                       const ReduceAllScratch &S);
+                       const ReduceAllScratch &S, unsigned host_tag = 0);
 }  // namespace
 
-void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent) {
+void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent, unsigned host_tag) {
   const long n = THClTensor_nElement(state, src);
   THCL_CHECK(src->nDimension <= THCL_MAX_DIMS, THCL_DIM_WARNING);
   int device = THClTensor_getDevice(state, src);
@@ -991,7 +999,7 @@ void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *
   S.ticket = (unsigned *)(block + kTicketOff);
   S.partials = block + kPartialOff;
   S.slots = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
-  reduce_all_launch(rt, kind, src, n, out, exponent, S);
+  reduce_all_launch(rt, kind, src, n, out, exponent, S, host_tag);
   thcl_after_launch(state, rt);
 }
 
@@ -1025,7 +1033,7 @@ void thcl_reduce_all_noalloc(THClState *state, ThclReduce kind, THClTensor *src,
 
 namespace {
 void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, float *out, float exponent,
-                       const ReduceAllScratch &S) {
+                       const ReduceAllScratch &S, unsigned host_tag) {
   hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   ReduceAllParams P;
   memset(&P, 0, sizeof(P));
@@ -1035,6 +1043,7 @@ void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, fl
   P.ticket = S.ticket;
   P.out = out;
   P.exponent = exponent;
+  P.host_tag = host_tag;
   // The order in which elements are folded is free, so the view is walked in memory order: dims sorted
   // by stride and merged.  A transposed or permuted view of a whole block of memory becomes dense.
   Layout walk;
@@ -1078,8 +1087,20 @@ void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, fl
 }
 }  // namespace
 
+// One device scalar to the pinned {value, tag} pair the host polls.
+__global__ void scalar_to_host(const float *src, unsigned long long *pair, unsigned tag) {
+  const unsigned long long w = (unsigned long long)__float_as_uint(*src) | ((unsigned long long)tag << 32);
+  __hip_atomic_store(pair, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+void thcl_scalar_to_host(THClState *state, thcl_rt *rt, const float *src, unsigned host_tag) {
+  hipLaunchKernelGGL(scalar_to_host, dim3(1), dim3(1), 0, (hipStream_t)thcl_rt_stream(rt), src,
+                     (unsigned long long *)thcl_rt_tagged_word_device(rt), host_tag);
+  check_launch("scalar to host");
+  thcl_after_launch(state, rt);
+}
+
 // out[0] = sum a[i] * b[i], both dense with n elements
-void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out) {
+void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out, unsigned host_tag) {
   hipStream_t stream = (hipStream_t)thcl_rt_stream(rt);
   if (n == 0) {
     thcl_fill_contig(rt, out, 0.f, 1);
@@ -1095,6 +1116,7 @@ void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *
   P.partials = sblock + kPartialOff;
   P.ticket = (unsigned *)(sblock + kTicketOff);
   P.out = out;
+  P.host_tag = host_tag;
   const bool vec = aligned16(a) && aligned16(b);
   const long want = vec ? (n / 4 + kThreads * 4 - 1) / (kThreads * 4) : (n + kThreads - 1) / kThreads;
   long cap = (long)thcl_rt_get_props(rt)->compute_units * 2;

@@ -8,6 +8,7 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <chrono>
 #include <cstring>
 #include <map>
 #include <unordered_map>
@@ -32,6 +33,7 @@ struct thcl_rt {
   size_t scratch_bytes = 0;
   float *host_word = nullptr;
   float *host_word_dev = nullptr;  // the same words as the device addresses them
+  unsigned tag = 0;                // last tag handed out for the tagged word pair
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
   thcl_rt_props props{};
@@ -299,6 +301,40 @@ int thcl_rt_sync(thcl_rt *rt) {
 }
 
 unsigned *thcl_rt_fault_word_device(thcl_rt *rt) { return (unsigned *)(rt->host_word_dev + kFaultWord); }
+
+// A pinned pair of words {value, tag} that a kernel fills with one 8-byte store, so the host can pick a
+// scalar up as soon as it lands instead of waiting for the stream's completion signal.
+constexpr int kTaggedWord = 40;  // 8-byte aligned
+float *thcl_rt_tagged_word_device(thcl_rt *rt) { return rt->host_word_dev + kTaggedWord; }
+unsigned thcl_rt_next_tag(thcl_rt *rt) {
+  if (++rt->tag == 0u) ++rt->tag;
+  return rt->tag;
+}
+int thcl_rt_await_tagged(thcl_rt *rt, unsigned tag, float *value) {
+  volatile unsigned long long *w = (volatile unsigned long long *)(rt->host_word + kTaggedWord);
+  // poll for up to 2 ms (a reduction of 2^28 elements takes 0.15 ms), then wait for the stream the ordinary way
+  const auto t0 = std::chrono::steady_clock::now();
+  for (;;) {
+    for (int i = 0; i < 64; i++) {
+      const unsigned long long pair = *w;
+      if ((unsigned)(pair >> 32) == tag) {
+        const unsigned bits = (unsigned)pair;
+        memcpy(value, &bits, sizeof(bits));
+        return check_fault(rt);
+      }
+    }
+    if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(2000)) break;
+  }
+  const int rc = thcl_rt_sync(rt);
+  const unsigned long long pair = *w;
+  const unsigned bits = (unsigned)pair;
+  memcpy(value, &bits, sizeof(bits));
+  if (rc == 0 && (unsigned)(pair >> 32) != tag) {
+    g_err = "the kernel that was to hand a scalar to the host did not leave it";
+    return -4;
+  }
+  return rc;
+}
 
 void *thcl_rt_scratch(thcl_rt *rt, size_t *bytes) {
   if (bytes) *bytes = rt->scratch_bytes;

@@ -78,6 +78,16 @@ float *thcl_rt_host_word_device(thcl_rt *rt);
  * look at it after they have waited: if it is set they clear it and return -3 with a message. */
 unsigned *thcl_rt_fault_word_device(thcl_rt *rt);
 
+/* A scalar handed to the host without waiting for the stream's completion signal: a kernel that is given
+ * thcl_rt_tagged_word_device() and a tag from thcl_rt_next_tag() writes {value, tag} there in one 8-byte store when
+ * it has the value; thcl_rt_await_tagged() polls the pair for up to 2 ms and then falls back to
+ * thcl_rt_sync().  Returns what thcl_rt_sync would (also -3 when the fault word is set).  Work queued behind the
+ * kernel is unaffected: the stream stays in order.  The reference reads such scalars back with a blocking copy
+ * (src/lib/THClTensorMath.cpp:346-368). */
+float *thcl_rt_tagged_word_device(thcl_rt *rt);
+unsigned thcl_rt_next_tag(thcl_rt *rt);
+int thcl_rt_await_tagged(thcl_rt *rt, unsigned tag, float *value);
+
 /* Page-locked host memory for callers that stage their own transfers: copies between a
  * tensor and such a buffer run at the link's rate (57 GB/s measured on MI355X, against
  * 30 GB/s in and 17 GB/s out for pageable memory).  The reference keeps its host mirrors

@@ -106,6 +106,25 @@ def test_reduce_all_special_values(cl):
             assert cl.ClTensor(b).max() == np.inf and cl.ClTensor(b).min() == -np.inf
 
 
+def test_scalars_handed_to_the_host_in_a_row(cl):
+    """Scalar results reach the host through one pinned word pair with a tag per call: many calls in a row,
+    of different kinds and sizes, must each return their own value (no stale one from the call before)."""
+    sizes = (1, 7, 1000, 4097, 1 << 16, (1 << 20) + 3)
+    tensors = [(n, cl.ClTensor(np.full(n, 1.0 + i, dtype=F))) for i, n in enumerate(sizes)]
+    pt = cl.ClTensor()
+    for rep in range(300):
+        i = rep % len(tensors)
+        n, t = tensors[i]
+        v = 1.0 + i
+        assert t.sum() == F(n) * F(v)
+        assert t.max() == v and t.min() == v
+        assert t.dot(t) == float(F(n * v * v))
+        pt.sum(t)
+        assert pt.s() == F(n) * F(v)
+    big = cl.ClTensor(np.ones(1 << 26, dtype=F))              # a reduction long enough to outlast a short poll
+    assert big.sum() == float(1 << 26) and tensors[0][1].sum() == 1.0 and big.sum() == float(1 << 26)
+
+
 def test_reduce_all_on_views(cl):
     base = oracle.uniform(15, 40 * 30 * 20).reshape(40, 30, 20)
     p = Pair.dense(cl, base)
