@@ -13,6 +13,8 @@
 //     time with a block-wide fp64 prefix in each step.
 //   * scan_short_rows: I == 1 and many short rows; 1 to 64 lanes share a row
 //     and adjacent lane groups take adjacent rows.
+//   * scan_wave_rows: I == 1 and many aligned rows of 1024 to 8191 elements; a
+//     wave per row with the next 1024 elements requested ahead.
 //   * scan_strip: I > 1 with fewer columns than the chip has threads; a block
 //     walks 32 columns, 256 rows a step.
 // When O * I alone cannot fill the chip, R is cut into S segments and the scan
@@ -480,6 +482,66 @@ __global__ __launch_bounds__(kThreads) void scan_short_rows(ScanParams P) {
   }
 }
 
+// I == 1, many rows of 1024 elements or more, 16-byte aligned: a wave per row, no LDS and no barrier.  A batch is
+// 4 steps of 256 elements (4 consecutive ones per lane); the next batch is requested before the current one is
+// worked on, so a wave always has 4 KiB on its way.  The running value crosses steps through a shuffle.
+template <bool PROD>
+__global__ __launch_bounds__(kThreads) void scan_wave_rows(ScanParams P) {
+  constexpr int PER = 4, UNR = 4, STEP = kWave * PER, BATCH = STEP * UNR;
+  const int lane = threadIdx.x % kWave;
+  const thcl_u64 o = (thcl_u64)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
+  if (o >= P.O) return;  // whole waves
+  const float *row = P.in + o * P.R + (thcl_u64)lane * PER;
+  float *orow = P.out + o * P.R + (thcl_u64)lane * PER;
+  double carry = Op<PROD>::identity();
+  auto fetch = [&](thcl_f4 (&x)[UNR], thcl_u64 base) {
+#pragma unroll
+    for (int u = 0; u < UNR; u++) x[u] = __builtin_nontemporal_load((const thcl_f4 *)(row + base + (thcl_u64)u * STEP));
+  };
+  // one step: 256 elements from `base`, this lane's four in x
+  auto step = [&](const thcl_f4 &x, thcl_u64 base) {
+    double a[PER];
+    a[0] = (double)x[0];
+#pragma unroll
+    for (int c = 1; c < PER; c++) a[c] = Op<PROD>::comb(a[c - 1], (double)x[c]);
+    const double incl = wave_inclusive<PROD>(a[PER - 1]);
+    double before = carry;
+    const double prev = __shfl_up(incl, 1, kWave);
+    if (lane > 0) before = Op<PROD>::comb(before, prev);
+    carry = Op<PROD>::comb(carry, __shfl(incl, kWave - 1, kWave));
+    thcl_f4 v;
+#pragma unroll
+    for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[c]);
+    return v;
+  };
+  thcl_u64 base = 0;
+  if (BATCH <= P.R) {
+    thcl_f4 x[UNR], xn[UNR];
+    fetch(x, 0);
+    for (; base + 2 * BATCH <= P.R; base += BATCH) {
+      fetch(xn, base + BATCH);
+#pragma unroll
+      for (int u = 0; u < UNR; u++)
+        __builtin_nontemporal_store(step(x[u], base + (thcl_u64)u * STEP), (thcl_f4 *)(orow + base + (thcl_u64)u * STEP));
+#pragma unroll
+      for (int u = 0; u < UNR; u++) x[u] = xn[u];
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; u++)
+      __builtin_nontemporal_store(step(x[u], base + (thcl_u64)u * STEP), (thcl_f4 *)(orow + base + (thcl_u64)u * STEP));
+    base += BATCH;
+  }
+  // what is left of the row (R is a multiple of 4: a lane's four elements are inside or outside together)
+  const float fill = PROD ? 1.0f : 0.0f;
+  for (; base < P.R; base += STEP) {
+    const bool in = base + (thcl_u64)lane * PER < P.R;
+    thcl_f4 x = {fill, fill, fill, fill};
+    if (in) x = *(const thcl_f4 *)(row + base);
+    const thcl_f4 v = step(x, base);
+    if (in) *(thcl_f4 *)(orow + base) = v;
+  }
+}
+
 template <bool PROD, int G>
 void launch_short(hipStream_t stream, const ScanParams &P, bool vec) {
   const dim3 grid((unsigned)((P.O + kThreads / G - 1) / (kThreads / G))), block(kThreads);
@@ -606,16 +668,20 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     const long cus = thcl_rt_get_props(rt)->compute_units;
     // innermost scans: long rows (or few of them) take a block per row segment,
     // many short rows take a lane group per row
-    const bool shortrows = P.I == 1 && P.R > 1 && (P.R < 1024 || (P.R < 8192 && P.O >= (thcl_u64)cus * 16));
-    const bool rows = (P.I == 1 && P.R >= 1024) && !shortrows;
+    const bool aligned = ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
+    // enough aligned rows of 1024 to 8191 elements for a wave each (16 per CU).  Measured against the lane-group kernel
+    // without prefetch: 65536 x 1024 85 -> 82 us, 4096 x 4100 34 -> 27 us; on longer rows a block per row wins
+    // (4096 x 16384: 95 us against 105).
+    const bool waverows = P.I == 1 && P.R >= 1024 && P.R < 8192 && P.R % 4 == 0 && aligned && P.O >= (thcl_u64)cus * 16;
+    const bool shortrows = !waverows && P.I == 1 && P.R > 1 && (P.R < 1024 || (P.R < 8192 && P.O >= (thcl_u64)cus * 16));
+    const bool rows = (P.I == 1 && P.R >= 1024) && !shortrows && !waverows;
     // cut R into segments until the launch fills the chip; a segment keeps
     // enough elements to amortise the extra pass
     // Outer scans with too few columns for a thread each: strips of 32 columns in one pass, when there
     // is a strip for every other CU and the lines are long enough to amortise a block's start.  On 256
     // CUs, 2^26 elements: 16384 columns 4.9 TB/s against 3.7 in three passes, 8192 columns 5.2,
     // 4096 columns (128 strips) 4.2 against 3.8, 2048 columns 2.5 against 3.7.
-    const bool aligned = ((((uintptr_t)P.in) | ((uintptr_t)P.out)) & 15u) == 0;
-    const bool few_lines = !rows && !shortrows && P.I % 4 == 0 && aligned && P.O * P.I < (thcl_u64)cus * 512;
+    const bool few_lines = !rows && !shortrows && !waverows && P.I % 4 == 0 && aligned && P.O * P.I < (thcl_u64)cus * 512;
     thcl_u64 strips = P.O * ((P.I / 4 + 7) / 8);
     bool strip = few_lines && P.R >= 1024 && strips * 2 >= (thcl_u64)cus && strips < (1ull << 31);
     // A handful of columns (4 to 28): the thread-per-column kernel would read 16 to 112 bytes per row
@@ -630,7 +696,7 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
       if (P.O < want) S = (want + P.O - 1) / P.O;
       const thcl_u64 most = P.R / 4096;  // a few steps of the block at least
       if (S > most) S = most;
-    } else if (shortrows || strip) {
+    } else if (shortrows || waverows || strip) {
       S = 1;
     } else if (rows) {
       // Segments cost a second read of the input (12 bytes an element instead of 8), which pays
@@ -665,7 +731,13 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     if (S > 1) P.totals = (double *)thcl_rt_workspace(rt, (size_t)(P.O * P.S * P.I + windows) * sizeof(double));
     THCL_CHECK(S == 1 || P.totals != nullptr, "%s", thcl_rt_error());
     const bool vec = (rows || shortrows) && (P.R % 4 == 0) && aligned;
-    if (shortrows) {
+    if (waverows) {
+      const thcl_u64 blocks = (P.O + kThreads / kWave - 1) / (kThreads / kWave);
+      THCL_CHECK(blocks < (1ull << 31), THCL_DIM_WARNING);
+      if (prod) hipLaunchKernelGGL(scan_wave_rows<true>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, P);
+      else hipLaunchKernelGGL(scan_wave_rows<false>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, P);
+      check("scan");
+    } else if (shortrows) {
       THCL_CHECK(P.O < (1ull << 31), THCL_DIM_WARNING);
       if (prod) run_short<true>(stream, P, vec);
       else run_short<false>(stream, P, vec);

@@ -148,6 +148,22 @@ def test_all_any(cl):
     assert s.dev.all() is bool(cat.truth(s.view.gather()).all())
 
 
+@pytest.mark.parametrize("rows,length", [(4200, 1028), (4100, 2048), (4096, 3000), (5000, 1024), (4300, 8188)])
+def test_many_rows_of_a_thousand_to_eight_thousand_elements(cl, rows, length):
+    """Enough aligned rows for a wave each: whole batches of 1024 elements plus a ragged rest, out of place, in
+    place, and as products."""
+    x = oracle.uniform(91 + length, rows * length).reshape(rows, length)
+    X = cl.ClTensor(x)
+    _scan_close(X.cumsum(2).float(), cat.cumulate(x, 1), f"cumsum {rows} x {length}")
+    Y = cl.ClTensor(x)
+    Y.cumsum(Y, 2)
+    _scan_close(Y.float(), cat.cumulate(x, 1), "in place")
+    y = (1.0 + 0.001 * x).astype(F)
+    _scan_close(cl.ClTensor(y).cumprod(2).float(), cat.cumulate(y, 1, prod=True), "cumprod")
+    ones = cl.ClTensor(np.ones((rows, length), dtype=F))
+    assert np.array_equal(ones.cumsum(2).float()[rows - 1], np.arange(1, length + 1, dtype=F))
+
+
 def test_scan_of_rows_longer_than_a_window(cl):
     """Cut rows of more than 128 MiB in total go through in windows (totals pass and scan pass per window), and a
     segment's carry-in comes partly from the previous window's last block, partly from the window's own totals:
