@@ -357,23 +357,43 @@ __global__ __launch_bounds__(kThreads) void reduce_all_dense(ReduceAllParams P) 
   finish_all<KIND>(v, P, lds);
 }
 
-template <int KIND>
+// VEC 4: the view's innermost run is dense, a multiple of 4 long and 16-byte aligned in every row, so it is
+// walked in units of four elements (P.n and P.L count units; one index decomposition and one load per unit).
+template <int KIND, int VEC>
 __global__ __launch_bounds__(kThreads) void reduce_all_strided(ReduceAllParams P) {
   typedef typename Acc<KIND>::T T;
   __shared__ T lds[kThreads / kWave];
-  T acc = Acc<KIND>::init();
   const thcl_u64 all = (thcl_u64)gridDim.x * kThreads;
   thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x;
-  constexpr int FLY = 8;  // independent loads per thread and turn
-  for (; i + (FLY - 1) * all < P.n; i += FLY * all) {
-    float v[FLY];
+  T acc;
+  if (VEC == 4) {
+    constexpr int FLY = 8;
+    Chain<KIND> chain[FLY];
+    for (; i + (FLY - 1) * all < P.n; i += FLY * all) {
+      thcl_f4 v[FLY];
 #pragma unroll
-    for (int k = 0; k < FLY; k++) v[k] = P.in[thcl_generic_offset((thcl_u32)(i + k * all), P.L)];
+      for (int k = 0; k < FLY; k++)
+        v[k] = __builtin_nontemporal_load((const thcl_f4 *)(P.in + thcl_generic_offset((thcl_u32)(i + k * all), P.L)));
 #pragma unroll
-    for (int k = 0; k < FLY; k++) acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(v[k], P.exponent));
+      for (int k = 0; k < FLY; k++) chain[k].take4(v[k], P.exponent);
+    }
+    for (; i < P.n; i += all) chain[0].take4(*(const thcl_f4 *)(P.in + thcl_generic_offset((thcl_u32)i, P.L)), P.exponent);
+    acc = chain[0].value();
+#pragma unroll
+    for (int k = 1; k < FLY; k++) acc = Acc<KIND>::comb(acc, chain[k].value());
+  } else {
+    acc = Acc<KIND>::init();
+    constexpr int FLY = 8;  // independent loads per thread and turn
+    for (; i + (FLY - 1) * all < P.n; i += FLY * all) {
+      float v[FLY];
+#pragma unroll
+      for (int k = 0; k < FLY; k++) v[k] = P.in[thcl_generic_offset((thcl_u32)(i + k * all), P.L)];
+#pragma unroll
+      for (int k = 0; k < FLY; k++) acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(v[k], P.exponent));
+    }
+    for (; i < P.n; i += all)
+      acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(P.in[thcl_generic_offset((thcl_u32)i, P.L)], P.exponent));
   }
-  for (; i < P.n; i += all)
-    acc = Acc<KIND>::comb(acc, Acc<KIND>::lift(P.in[thcl_generic_offset((thcl_u32)i, P.L)], P.exponent));
   acc = block_reduce<KIND, T>(acc, lds);
   finish_all<KIND>(acc, P, lds);
 }
@@ -887,10 +907,12 @@ void check_launch(const char *what) {
   THCL_CHECK(e == hipSuccess, "%s launch failed: %s", what, hipGetErrorString(e));
 }
 
+// walk: 0 dense, 1 strided one element at a time, 4 strided in units of four
 template <int KIND>
-void launch_all(bool dense, unsigned grid, hipStream_t stream, const ReduceAllParams &P) {
-  if (dense) hipLaunchKernelGGL(reduce_all_dense<KIND>, dim3(grid), dim3(kThreads), 0, stream, P);
-  else hipLaunchKernelGGL(reduce_all_strided<KIND>, dim3(grid), dim3(kThreads), 0, stream, P);
+void launch_all(int walk, unsigned grid, hipStream_t stream, const ReduceAllParams &P) {
+  if (walk == 0) hipLaunchKernelGGL(reduce_all_dense<KIND>, dim3(grid), dim3(kThreads), 0, stream, P);
+  else if (walk == 4) hipLaunchKernelGGL((reduce_all_strided<KIND, 4>), dim3(grid), dim3(kThreads), 0, stream, P);
+  else hipLaunchKernelGGL((reduce_all_strided<KIND, 1>), dim3(grid), dim3(kThreads), 0, stream, P);
 }
 
 template <int KIND, bool ARG>
@@ -1059,29 +1081,44 @@ void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, fl
   const bool dense = walk.contiguous();
   const int cus = thcl_rt_get_props(rt)->compute_units;
   long want;
+  int how = 0;
   if (dense) {
     want = (n / 4 + kThreads * 4 - 1) / (kThreads * 4);
   } else {
     THCL_CHECK(n < (1l << 31), THCL_DIM_WARNING);
+    // units of four when every row of the innermost dim is a dense, 16-byte aligned run of a multiple of 4
+    const int last = walk.dims - 1;
+    bool vec4 = walk.dims >= 1 && walk.strides[last] == 1 && walk.sizes[last] % 4 == 0 && aligned16(P.in);
+    for (int d = 0; d < last && vec4; d++) vec4 = walk.strides[d] % 4 == 0;
+    if (vec4) {
+      walk.sizes[last] /= 4;
+      walk.strides[last] = 4;
+      P.n = (thcl_u64)(n / 4);
+      how = 4;
+    } else {
+      how = 1;
+    }
     fill_operand(P.L, walk);
-    want = (n + kThreads * 8 - 1) / (kThreads * 8);
+    want = ((long)P.n + kThreads * 8 - 1) / (kThreads * 8);
   }
-  // dense: two resident blocks per CU keep HBM busy (fewer blocks, fewer tickets); strided walks read
-  // 4 bytes per lane and need more of them in flight
-  long cap = (long)cus * (dense ? 2 : 8);
+  // Every block costs about 10 ns at the end (its partial and its ticket go through one point of the memory
+  // system), so the grid is as small as keeps HBM busy: two blocks per CU from 128 MiB up, one below (2^22
+  // elements: 10.5 -> 7.1 us), two for walks in units of four, four for walks one element at a time
+  // (measured with 1 to 12 blocks per CU: the half rows of an 8192^2 matrix 39 -> 27 us with 2 instead of 8).
+  long cap = (long)cus * (dense ? ((size_t)n * sizeof(float) >= (size_t)cus * 2 * 262144 ? 2 : 1) : (how == 4 ? 2 : 4));
   if (cap > S.slots) cap = S.slots;
   unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));
   switch (kind) {
-    case RED_SUM: launch_all<RED_SUM>(dense, grid, stream, P); break;
-    case RED_PROD: launch_all<RED_PROD>(dense, grid, stream, P); break;
-    case RED_MAX: launch_all<RED_MAX>(dense, grid, stream, P); break;
-    case RED_MIN: launch_all<RED_MIN>(dense, grid, stream, P); break;
-    case RED_SUM_NE0: launch_all<RED_SUM_NE0>(dense, grid, stream, P); break;
-    case RED_SUM_ABS: launch_all<RED_SUM_ABS>(dense, grid, stream, P); break;
-    case RED_SUM_SQ: launch_all<RED_SUM_SQ>(dense, grid, stream, P); break;
-    case RED_SUM_POW: launch_all<RED_SUM_POW>(dense, grid, stream, P); break;
-    case RED_ALL: launch_all<RED_ALL>(dense, grid, stream, P); break;
-    case RED_ANY: launch_all<RED_ANY>(dense, grid, stream, P); break;
+    case RED_SUM: launch_all<RED_SUM>(how, grid, stream, P); break;
+    case RED_PROD: launch_all<RED_PROD>(how, grid, stream, P); break;
+    case RED_MAX: launch_all<RED_MAX>(how, grid, stream, P); break;
+    case RED_MIN: launch_all<RED_MIN>(how, grid, stream, P); break;
+    case RED_SUM_NE0: launch_all<RED_SUM_NE0>(how, grid, stream, P); break;
+    case RED_SUM_ABS: launch_all<RED_SUM_ABS>(how, grid, stream, P); break;
+    case RED_SUM_SQ: launch_all<RED_SUM_SQ>(how, grid, stream, P); break;
+    case RED_SUM_POW: launch_all<RED_SUM_POW>(how, grid, stream, P); break;
+    case RED_ALL: launch_all<RED_ALL>(how, grid, stream, P); break;
+    case RED_ANY: launch_all<RED_ANY>(how, grid, stream, P); break;
   }
   check_launch("reduce-all");
 }
@@ -1119,7 +1156,9 @@ void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *
   P.host_tag = host_tag;
   const bool vec = aligned16(a) && aligned16(b);
   const long want = vec ? (n / 4 + kThreads * 4 - 1) / (kThreads * 4) : (n + kThreads - 1) / kThreads;
-  long cap = (long)thcl_rt_get_props(rt)->compute_units * 2;
+  // one block per CU below 128 MiB of operands, two above (every block costs about 10 ns at the end)
+  const long cus = thcl_rt_get_props(rt)->compute_units;
+  long cap = cus * ((size_t)n * 2 * sizeof(float) >= (size_t)cus * 2 * 262144 ? 2 : 1);
   const long max_partials = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
   if (cap > max_partials) cap = max_partials;
   const unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));

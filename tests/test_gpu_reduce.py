@@ -106,6 +106,26 @@ def test_reduce_all_special_values(cl):
             assert cl.ClTensor(b).max() == np.inf and cl.ClTensor(b).min() == -np.inf
 
 
+def test_reduce_all_on_views_walked_in_units_of_four(cl):
+    """Views whose innermost run is dense, a multiple of 4 long and 16-byte aligned in every row are walked four
+    elements at a time; neighbours that miss one of the conditions take the one-element walk.  Both against the oracle."""
+    base = oracle.uniform(16, 96 * 64 * 72).reshape(96, 64, 72)
+    p = Pair.dense(cl, base)
+    views = (p.narrow(2, 4, 32), p.narrow(2, 8, 64).narrow(1, 3, 40), p.narrow(0, 5, 80).narrow(2, 0, 36),     # aligned runs
+             p.narrow(2, 3, 32), p.narrow(2, 4, 30), p.transpose(0, 1).narrow(2, 12, 48), p.step(1, 2).narrow(2, 16, 40))
+    for q in views:
+        close_sum(q.dev.sum(), oracle.sumall(q.view))
+        assert q.dev.max() == oracle.maxall(q.view) and q.dev.min() == oracle.minall(q.view)
+    big = oracle.uniform(17, 2048 * 4096).reshape(2048, 4096)
+    b = Pair.dense(cl, big)
+    for q in (b.narrow(1, 0, 2048), b.narrow(1, 4, 4088), b.step(0, 2)):
+        close_sum(q.dev.sum(), oracle.sumall(q.view))
+        assert q.dev.max() == oracle.maxall(q.view)
+    x = big.copy()
+    x[1000, 77] = np.nan
+    assert np.isnan(Pair.dense(cl, x).narrow(1, 0, 2048).dev.max()) and not np.isnan(Pair.dense(cl, x).narrow(1, 2048, 2048).dev.max())
+
+
 def test_scalars_handed_to_the_host_in_a_row(cl):
     """Scalar results reach the host through one pinned word pair with a tag per call: many calls in a row,
     of different kinds and sizes, must each return their own value (no stale one from the call before)."""
