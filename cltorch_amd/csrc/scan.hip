@@ -300,19 +300,22 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
 // this step's work (two steps ahead instead of one: 108 -> 103 us on 4096 x 16384).  TC = 8 for wide tensors; with 4 to 28 columns TC = 1, 2, 4 or 8 covers the whole
 // width and consecutive rows are adjacent in memory, so a step reads one contiguous run.  PHASE 0 leaves the segment's
 // totals, PHASE 1 scans (from the segment's carry when the lines are cut into segments).
-template <bool PROD, int TC, int PHASE>
+// ANY: the width need not be a multiple of 4 nor the rows 16-byte aligned (narrow tensors only): a thread's up to 4
+// columns are read and written one element each, columns past the width are dead.
+template <bool PROD, int TC, int PHASE, bool ANY = false>
 __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
   // rows per thread: 8; 2 on the narrowest strips, where a thread's 8 rows would be 128 or 256 contiguous
   // bytes read 16 at a time (measured 0.6 TB/s on 4 columns against 2.0 with 2 rows)
-  constexpr int K = TC >= 4 ? 8 : 2;
+  constexpr int K = (TC >= 4 && !ANY) ? 8 : 2;  // element-wise strips: lanes that share an instruction stay 2 rows apart
   constexpr int WAVES = kThreads / kWave, ROWS = kThreads / TC * K, CW = TC * 4;
   __shared__ double wave_tot[2][WAVES][CW];
-  const thcl_u64 strips = (P.I / 4 + TC - 1) / TC;
+  const thcl_u64 strips = ((P.I + 3) / 4 + TC - 1) / TC;
   const thcl_u64 strip = blockIdx.x % strips, seg_id = (blockIdx.x / strips) % P.S, o = blockIdx.x / (strips * P.S);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int tc = threadIdx.x % TC, tr = threadIdx.x / TC;
   const thcl_u64 col = (strip * TC + tc) * 4;
   const bool live = col < P.I;
+  const int ncols = !ANY ? 4 : (!live ? 0 : (P.I - col < 4 ? (int)(P.I - col) : 4));  // this thread's columns inside the width
   const thcl_u64 first = o * P.R * P.I + (live ? col : 0);
   const float *src = P.in + first;
   float *dst = P.out + first;
@@ -324,13 +327,23 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
 #pragma unroll
     for (int k = 0; k < K; k++) {
       const thcl_u64 r = r0 + (thcl_u64)tr * K + k;
-      x[k] = __builtin_nontemporal_load((const thcl_f4 *)(src + (r < rend ? r : rend - 1) * P.I));
+      const float *at = src + (r < rend ? r : rend - 1) * P.I;
+      if (!ANY) {
+        x[k] = __builtin_nontemporal_load((const thcl_f4 *)at);
+      } else {
+        // dead columns read the thread's first column again (an address inside the tensor) and become the identity
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const float v = at[c < ncols ? c : 0];
+          x[k][c] = c < ncols ? v : fill;
+        }
+      }
     }
   };
   double *tot = P.totals + (o * P.S + seg_id) * P.I + (live ? col : 0);
   double carry[4];
 #pragma unroll
-  for (int c = 0; c < 4; c++) carry[c] = (PHASE == 1 && P.S > 1) ? tot[c] : Op<PROD>::identity();
+  for (int c = 0; c < 4; c++) carry[c] = (PHASE == 1 && P.S > 1 && c < ncols) ? tot[c] : Op<PROD>::identity();
   // one step: the 256 / TC * K rows from r0, held in x
   auto step = [&](thcl_f4 (&x)[K], thcl_u64 r0, int buf) {
 #pragma unroll
@@ -378,7 +391,13 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
           v[c] = (float)incl[c];
         }
         const thcl_u64 r = r0 + (thcl_u64)tr * K + k;
-        if (live && r < rend) __builtin_nontemporal_store(v, (thcl_f4 *)(dst + r * P.I));
+        if (!ANY) {
+          if (live && r < rend) __builtin_nontemporal_store(v, (thcl_f4 *)(dst + r * P.I));
+        } else if (r < rend) {
+#pragma unroll
+          for (int c = 0; c < 4; c++)
+            if (c < ncols) dst[r * P.I + c] = v[c];
+        }
       }
     }
   };
@@ -422,7 +441,8 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
   }
   if (PHASE == 0 && tr == 0 && live) {
 #pragma unroll
-    for (int c = 0; c < 4; c++) tot[c] = carry[c];
+    for (int c = 0; c < 4; c++)
+      if (c < ncols) tot[c] = carry[c];
   }
 }
 
@@ -688,13 +708,27 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     // and line segment.  Strips as wide as the tensor read whole runs of rows instead; the lines are
     // cut into segments (three passes) to fill the chip.  2^26 elements in rows of 4 / 8 / 16 columns:
     // 0.8 -> 2.0, 1.7 -> 2.1, 2.5 -> 3.0 TB/s.
+    // Widths that are no multiple of 4, or rows that are not 16-byte aligned, take the same strips one element
+    // at a time (2^20 x 3: 106 us with a thread per column, 30 us this way; 2^18 x 27: 37 us).
     int strip_tc = 8;
-    bool narrow = false;
+    bool narrow = false, narrow_any = false;
+    // (from 1.5 million elements per tensor slice up: below that the three launches of the strips cost more than the
+    // thread-per-column walk, 20000 x 8: 42 us against 10)
+    const bool few_narrow = !rows && !shortrows && !waverows && P.I > 1 && P.I <= 28 && P.R >= 16384 && P.R * P.I >= (3ull << 19) &&
+                            P.O * P.I < (thcl_u64)cus * 512;
+    if (!strip && few_narrow) {
+      const thcl_u64 quads = (P.I + 3) / 4;
+      strip_tc = quads <= 1 ? 1 : (quads <= 2 ? 2 : (quads <= 4 ? 4 : 8));
+      strips = P.O;
+      strip = narrow = true;
+      narrow_any = !(P.I % 4 == 0 && aligned);
+    }
     thcl_u64 S = 1;
     if (narrow) {
       const thcl_u64 want = (thcl_u64)cus * 8;  // blocks
       if (P.O < want) S = (want + P.O - 1) / P.O;
-      const thcl_u64 most = P.R / 4096;  // a few steps of the block at least
+      // a few steps of the block at least (a step of the element-wise strips is 2 rows per thread)
+      const thcl_u64 most = narrow_any ? P.R / (thcl_u64)(kThreads / strip_tc * 2 * 8) : P.R / 4096;
       if (S > most) S = most;
     } else if (shortrows || waverows || strip) {
       S = 1;
@@ -744,16 +778,19 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
       check("scan");
     } else if (strip) {
       const dim3 grid((unsigned)(strips * P.S)), block(kThreads);
+#define STRIP_CASE(PR, TC_, PH)                                                                               \
+  if (narrow_any) hipLaunchKernelGGL((scan_strip<PR, TC_, PH, true>), grid, block, 0, stream, P);              \
+  else hipLaunchKernelGGL((scan_strip<PR, TC_, PH, false>), grid, block, 0, stream, P);
 #define STRIP_PHASE(PH)                                                                                        \
   switch (strip_tc * 2 + (prod ? 1 : 0)) {                                                                     \
-    case 2: hipLaunchKernelGGL((scan_strip<false, 1, PH>), grid, block, 0, stream, P); break;                  \
-    case 3: hipLaunchKernelGGL((scan_strip<true, 1, PH>), grid, block, 0, stream, P); break;                   \
-    case 4: hipLaunchKernelGGL((scan_strip<false, 2, PH>), grid, block, 0, stream, P); break;                  \
-    case 5: hipLaunchKernelGGL((scan_strip<true, 2, PH>), grid, block, 0, stream, P); break;                   \
-    case 8: hipLaunchKernelGGL((scan_strip<false, 4, PH>), grid, block, 0, stream, P); break;                  \
-    case 9: hipLaunchKernelGGL((scan_strip<true, 4, PH>), grid, block, 0, stream, P); break;                   \
-    case 16: hipLaunchKernelGGL((scan_strip<false, 8, PH>), grid, block, 0, stream, P); break;                 \
-    default: hipLaunchKernelGGL((scan_strip<true, 8, PH>), grid, block, 0, stream, P); break;                  \
+    case 2: STRIP_CASE(false, 1, PH) break;                                                                    \
+    case 3: STRIP_CASE(true, 1, PH) break;                                                                     \
+    case 4: STRIP_CASE(false, 2, PH) break;                                                                    \
+    case 5: STRIP_CASE(true, 2, PH) break;                                                                     \
+    case 8: STRIP_CASE(false, 4, PH) break;                                                                    \
+    case 9: STRIP_CASE(true, 4, PH) break;                                                                     \
+    case 16: STRIP_CASE(false, 8, PH) break;                                                                   \
+    default: STRIP_CASE(true, 8, PH) break;                                                                    \
   }
       if (P.S > 1) {
         STRIP_PHASE(0)
@@ -763,6 +800,7 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
       }
       STRIP_PHASE(1)
 #undef STRIP_PHASE
+#undef STRIP_CASE
       check("scan");
     } else if (prod) {
       run_scan<true>(stream, P, rows, vec);

@@ -148,6 +148,25 @@ def test_all_any(cl):
     assert s.dev.all() is bool(cat.truth(s.view.gather()).all())
 
 
+@pytest.mark.parametrize("rows,cols,skip", [(600000, 3, 0), (300000, 7, 0), (200000, 10, 0), (70000, 27, 0), (300000, 6, 1), (250000, 8, 1),
+                                            (400000, 4, 0), (20000, 5, 0)])
+def test_scans_down_a_few_columns(cl, rows, cols, skip):
+    """Long scans down 3 to 27 columns: strips as wide as the tensor, with whole 16-byte groups where the width and
+    the rows' alignment allow (skip = rows dropped in front, which shifts the alignment), one element at a time
+    otherwise; short tensors take the thread-per-column walk."""
+    x = oracle.uniform(200 + cols, (rows + skip) * cols).reshape(rows + skip, cols)
+    X = cl.ClTensor(x)
+    V = X.narrow(1, skip + 1, rows) if skip else X
+    xv = x[skip:]
+    _scan_close(V.cumsum(1).float(), cat.cumulate(xv, 0), f"cumsum {rows} x {cols}")
+    y = (1.0 + 1e-5 * xv).astype(F)
+    Y = cl.ClTensor(y)
+    Y.cumprod(Y, 1)
+    _scan_close(Y.float(), cat.cumulate(y, 0, prod=True), "cumprod in place")
+    ones = cl.ClTensor(np.ones((rows, cols), dtype=F))
+    assert np.array_equal(ones.cumsum(1).float()[:, cols - 1], np.arange(1, rows + 1, dtype=F))
+
+
 @pytest.mark.parametrize("rows,length", [(4200, 1028), (4100, 2048), (4096, 3000), (5000, 1024), (4300, 8188)])
 def test_many_rows_of_a_thousand_to_eight_thousand_elements(cl, rows, length):
     """Enough aligned rows for a wave each: whole batches of 1024 elements plus a ragged rest, out of place, in
