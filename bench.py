@@ -383,6 +383,11 @@ def config_ops(cl, oracle, X, Y, Z, n):
     rc.fill(0.0)
     yield ("w_addmm_3000x5000x7000", lambda: rc.addmm(0.0, 1.0, ra, rb), 2.0 * 3000 * 5000 * 7000, "TFLOP/s", 6, M)
     del ra, rb, rc
+    # cubes between the two config-5 shapes: the block tile is picked per shape (whole rounds of tiles per CU)
+    for side in (3072, 4608):
+        qa, qb, qc = (cl.ClTensor((rs.standard_normal((side, side)) / np.sqrt(side)).astype(np.float32)) for _ in range(3))
+        yield ("w_addmm_%d^3" % side, lambda: qc.addmm(0.0, 1.0, qa, qb), 2.0 * side ** 3, "TFLOP/s", 10, M)
+        del qa, qb, qc
     mask = cl.ClTensor((rs.rand(1 << 26) > 0.5).astype(np.float32))
     src = cl.ClTensor(1 << 26)
     src.fill(1.0)
