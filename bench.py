@@ -402,7 +402,9 @@ def detail(cl, oracle, T, X, Y, Z, n):
     around ``reps`` calls in a row divided by their number -- what a caller that just keeps calling sees, launch
     gaps and result allocation included -- and ``achieved`` / ``frac_of_peak`` follow from it.  ``event_pair_*``
     come from one event pair per call (the pairs' own packets then sit between the calls, which costs a short
-    kernel 2-3 us); ``kernel_only_ms`` is the sum of the call's kernel durations in the committed rocprofv3 trace."""
+    kernel 2-3 us); ``kernel_only_ms`` is the sum of the call's kernel durations in the committed rocprofv3 trace.
+    Matrix products get ``reps`` untimed calls directly in front of the timed ones (the clock settles over the first
+    ~10 ms of such work after an idle period)."""
     d = {}
     profiled = committed_profile()
     for name, fn, work, unit, reps, peak in config_ops(cl, oracle, X, Y, Z, n):
@@ -413,6 +415,8 @@ def detail(cl, oracle, T, X, Y, Z, n):
             T.timed(name, fn)
         cl.synchronize()
         pairs = np.array(T.collect()[name], dtype=np.float64)
+        if unit == "TFLOP/s":
+            [fn() for _ in range(reps)]   # matrix products: the clock takes ~10 ms of such work to settle after a wait
         T.timed(name, lambda: [fn() for _ in range(reps)])
         cl.synchronize()
         b2b = T.collect()[name][0] / reps
