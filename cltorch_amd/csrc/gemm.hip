@@ -5,7 +5,8 @@
 // src/lib/THClBlas.cpp:381-449), whose arithmetic lives in clBLAS.
 //
 // Shape of the kernel: 256 threads = 4 waves in a 2x2 arrangement over a
-// BM x BN block tile; K advances in slabs of 16 staged through double-buffered
+// BM x BN block tile (4x1 or 1x4 over the 128x32 and 32x128 tiles that serve
+// products with one side of at most 32); K advances in slabs of 16 staged through double-buffered
 // LDS (one barrier per slab), the next slab's global loads are issued before
 // the current slab's MFMAs.  Operands that are contiguous along m/n in memory
 // sit in LDS as [k][mn] and are read one dword per MFMA; operands contiguous
@@ -49,7 +50,8 @@ struct TileLds {
   static constexpr int FLOATS = KC ? BMN * KPITCH : BK * BMN;
 };
 
-// global -> registers: each thread carries BMN*BK/256/4 float4.  EDGE 0: the tile is whole and aligned.  EDGE 1: a
+// global -> registers: each thread carries BMN*BK/256/4 float4 (a 32-wide tile has 128 of them: the upper half of the
+// block loads the same groups again and does not store them).  EDGE 0: the tile is whole and aligned.  EDGE 1: a
 // 16-byte group of the operand is either inside it or outside, and aligned; every load is issued (from the operand's
 // first element when the group is outside) and groups outside become zeros, so there is no branch around a load.
 // EDGE 2: any pitch and alignment, one element at a time.  The choice is made at compile time: a run-time branch
@@ -57,7 +59,9 @@ struct TileLds {
 // kernel: 101 TFLOP/s with the branch against 138 through the whole-tile kernel).
 template <int BMN, bool KC, int EDGE>
 struct TileLoader {
-  static constexpr int NV = BMN * BK / 256 / 4;
+  static constexpr int GROUPS = BMN * BK / 4;
+  static constexpr int NV = GROUPS >= 256 ? GROUPS / 256 : 1;
+  static constexpr bool PART = GROUPS < 256;
   f4 r[NV];
 
   // g: operand base; ld: leading dim; mn0: first row/col of the tile; k0: first k; lim_mn/lim_k: extents
@@ -65,7 +69,7 @@ struct TileLoader {
   __device__ __forceinline__ void load(const float *g, int ld, int mn0, int k0, int lim_mn, int lim_k) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
-      const int f = threadIdx.x + 256 * p;
+      const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
       if (KC) {
         const int mn = f / (BK / 4), kq = f % (BK / 4);
         const float *src = g + (size_t)(mn0 + mn) * ld + k0 + kq * 4;
@@ -98,6 +102,7 @@ struct TileLoader {
     }
   }
   __device__ __forceinline__ void store(float *lds) const {
+    if (PART && threadIdx.x >= GROUPS) return;
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = threadIdx.x + 256 * p;
@@ -135,7 +140,8 @@ template <int BM, int BN, bool TA, bool TB, int EDGE>
 __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   constexpr bool AKC = TA;    // 'n': a[i + l*lda] (m-contiguous); 't': a[l + i*lda] (k-contiguous)
   constexpr bool BKC = !TB;   // 'n': b[l + j*ldb] (k-contiguous); 't': b[j + l*ldb] (n-contiguous)
-  constexpr int WM = BM / 2, WN = BN / 2;   // wave tile
+  constexpr int WAVES_M = BN == 32 ? 4 : BM == 32 ? 1 : 2, WAVES_N = 4 / WAVES_M;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // wave tile
   constexpr int MT = WM / 32, NT = WN / 32; // 32x32 MFMA tiles per wave
   constexpr int AF = TileLds<BM, AKC>::FLOATS, BF = TileLds<BN, BKC>::FLOATS;
   __shared__ __attribute__((aligned(16))) float lds[2 * (AF + BF)];
@@ -161,7 +167,7 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int wave = threadIdx.x >> 6;
-  const int wm0 = (wave & 1) * WM, wn0 = (wave >> 1) * WN;
+  const int wm0 = (wave % WAVES_M) * WM, wn0 = (wave / WAVES_M) * WN;
 
   f16v acc[MT][NT];
 #pragma unroll
@@ -352,11 +358,14 @@ static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, 
     double whole, edge;
     int resident;  // blocks a CU holds
   };
-  static const Cand cands[4] = {{128, 128, 138., 128., 3}, {128, 64, 133., 124., 5}, {64, 128, 126., 118., 5}, {64, 64, 123., 110., 8}};
+  // the two thin tiles only stand for products with a side of at most 32, where they halve the padding
+  static const Cand cands[6] = {{128, 128, 138., 128., 3}, {128, 64, 133., 124., 5}, {64, 128, 126., 118., 5},
+                                {64, 64, 123., 110., 8},   {128, 32, 115., 105., 8}, {32, 128, 115., 105., 8}};
   double best = -1.;
   bm = bn = 64;
   for (const Cand &c : cands) {
     if ((c.bm == 128 && m < 128) || (c.bn == 128 && n < 128)) continue;
+    if ((c.bn == 32 && n > 32) || (c.bm == 32 && m > 32)) continue;
     const long tm = (m + c.bm - 1) / c.bm, tn = (n + c.bn - 1) / c.bn, tiles = tm * tn;
     const bool whole = aligned && m % c.bm == 0 && n % c.bn == 0;
     int ks, kc;
@@ -429,6 +438,8 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   if (bm == 128 && bn == 128) { GO(128, 128) }
   else if (bm == 128 && bn == 64) { GO(128, 64) }
   else if (bm == 64 && bn == 128) { GO(64, 128) }
+  else if (bm == 128 && bn == 32) { GO(128, 32) }
+  else if (bm == 32 && bn == 128) { GO(32, 128) }
   else { GO(64, 64) }
 #undef GO
   if (P.ksplit > 1) {

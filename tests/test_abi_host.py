@@ -312,6 +312,10 @@ def test_gemm_tile_choice(lib):
     assert tile(3000, 5000, 7000) == (128, 128) and tile(6000, 6000, 2000) == (128, 128)
     # 63 x 64 rows and columns: whole 64-wide tiles (123 x 0.97 for the last round) lose to 128-wide ones with edges (128 x 0.97 of area)
     assert tile(4032, 4032, 4096) == (128, 128)
+    # a side of at most 32: thin tiles halve the padding of a 64-wide tile; they never stand for wider products
+    assert tile(16384, 16, 16384) == (128, 32) and tile(32, 4096, 1024) == (32, 128) and tile(4096, 32, 4096) == (128, 32)
+    assert tile(16384, 33, 4096)[1] == 64 and tile(40, 4096, 4096)[0] == 64
+    assert tile(20, 20, 64) == (64, 64)
 
 
 def test_gemm_k_slicing(lib):

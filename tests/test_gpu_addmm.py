@@ -175,6 +175,25 @@ def test_ragged_mid_size_shapes(cl, M, N, K):
     assert np.max(np.abs(Ct.float() - want)) / scale < RTOL
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 300, 128), (300, 16, 128), (32, 256, 64), (256, 32, 64), (1, 1000, 50), (1000, 1, 50),
+                                   (7, 129, 33), (129, 7, 33), (32, 4096, 1024), (4096, 24, 2048), (20, 640, 17)])
+def test_products_with_a_side_of_at_most_32(cl, M, N, K):
+    """A result with at most 32 rows or columns is covered by 128x32 (or 32x128) tiles, four waves side by side along
+    the long side: all eight layouts of A, B and the result, whole and ragged sizes, with and without K slicing."""
+    rng = np.random.RandomState(M * 7 + N * 3 + K)
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
+    b = rng.standard_normal((K, N)).astype(F)
+    c = rng.standard_normal((M, N)).astype(F)
+    want = 0.5 * c.astype(np.float64) + 2.0 * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = max(1.0, float(np.sqrt(np.mean(want ** 2))))
+    for lay in range(8):
+        A = cl.ClTensor(np.ascontiguousarray(a.T)).t() if lay & 1 else cl.ClTensor(a)
+        B = cl.ClTensor(np.ascontiguousarray(b.T)).t() if lay & 2 else cl.ClTensor(b)
+        Cd = cl.ClTensor(np.ascontiguousarray(c.T)).t() if lay & 4 else cl.ClTensor(c)
+        Cd.addmm(0.5, 2.0, A, B)
+        assert np.max(np.abs(Cd.float() - want)) / scale < RTOL, lay
+
+
 def test_sliced_products_repeat_bit_exactly(cl):
     """K-sliced products sum their slices in slice order: every repetition gives the same
     bits, also with other reductions in between, with ragged shapes, with beta = 0 over
