@@ -18,6 +18,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <type_traits>
 
 #include "internal.h"
 
@@ -50,10 +51,39 @@ struct TileLds {
   static constexpr int FLOATS = KC ? BMN * KPITCH : BK * BMN;
 };
 
+// EDGE 1: what a lane's loads of one operand keep from slab to slab.  at[p] is the lane's 16-byte group in k row 0
+// (operands contiguous along m/n) or the start of its row (operands contiguous along k), moved to the operand's last
+// group or row when it lies beyond the m/n extent; in[p] tells which.  Worked out once per tile: with the extent
+// tests and the 64-bit products redone at every slab a tile on the rim took 1.6 times as long as a whole one.
+template <int BMN, bool KC>
+struct EdgeLanes {
+  static constexpr int GROUPS = BMN * BK / 4;
+  static constexpr int NV = GROUPS >= 256 ? GROUPS / 256 : 1;
+  static constexpr bool PART = GROUPS < 256;
+  const float *at[NV];
+  bool in[NV];
+  __device__ __forceinline__ void set(const float *g, int ld, int mn0, int lim_mn) {
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
+      if (KC) {
+        const int mn = mn0 + f / (BK / 4);
+        in[p] = mn < lim_mn;
+        at[p] = g + (size_t)(in[p] ? mn : lim_mn - 1) * ld;
+      } else {
+        const int mq = mn0 + (f % (BMN / 4)) * 4;
+        in[p] = mq < lim_mn;
+        at[p] = g + (in[p] ? mq : lim_mn - 4);
+      }
+    }
+  }
+};
+
 // global -> registers: each thread carries BMN*BK/256/4 float4 (a 32-wide tile has 128 of them: the upper half of the
 // block loads the same groups again and does not store them).  EDGE 0: the tile is whole and aligned.  EDGE 1: a
 // 16-byte group of the operand is either inside it or outside, and aligned; every load is issued (from the operand's
-// first element when the group is outside) and groups outside become zeros, so there is no branch around a load.
+// last row or group when the lane's own lies outside) and groups outside become zeros, so there is no branch around
+// a load.
 // EDGE 2: any pitch and alignment, one element at a time.  The choice is made at compile time: a run-time branch
 // between the two edge forms made the compiler wait for all loads at every slab (aligned 4096^3 through the edge
 // kernel: 101 TFLOP/s with the branch against 138 through the whole-tile kernel).
@@ -63,6 +93,8 @@ struct TileLoader {
   static constexpr int NV = GROUPS >= 256 ? GROUPS / 256 : 1;
   static constexpr bool PART = GROUPS < 256;
   f4 r[NV];
+  bool keep[NV];   // EDGE 1: the group lies inside the operand; looked at when the registers go to LDS, so that nothing
+                   // has to wait for the load before then
 
   // g: operand base; ld: leading dim; mn0: first row/col of the tile; k0: first k; lim_mn/lim_k: extents
   // vec (edge kernels): a 16-byte group is either inside the operand or outside, and aligned
@@ -75,10 +107,6 @@ struct TileLoader {
         const float *src = g + (size_t)(mn0 + mn) * ld + k0 + kq * 4;
         if (EDGE == 0) {
           r[p] = *(const f4 *)src;
-        } else if (EDGE == 1) {
-          const bool in = mn0 + mn < lim_mn && k0 + kq * 4 < lim_k;
-          const f4 v = *(const f4 *)(in ? src : g);
-          r[p] = in ? v : f4{0.f, 0.f, 0.f, 0.f};
         } else {
 #pragma unroll
           for (int c = 0; c < 4; c++)
@@ -89,10 +117,6 @@ struct TileLoader {
         const float *src = g + (size_t)(k0 + kk) * ld + mn0 + q * 4;
         if (EDGE == 0) {
           r[p] = *(const f4 *)src;
-        } else if (EDGE == 1) {
-          const bool in = k0 + kk < lim_k && mn0 + q * 4 < lim_mn;
-          const f4 v = *(const f4 *)(in ? src : g);
-          r[p] = in ? v : f4{0.f, 0.f, 0.f, 0.f};
         } else {
 #pragma unroll
           for (int c = 0; c < 4; c++)
@@ -101,17 +125,52 @@ struct TileLoader {
       }
     }
   }
+  // EDGE 1: every load is issued, from an address inside the operand, and groups outside it become zeros
+  __device__ __forceinline__ void load_edge(const EdgeLanes<BMN, KC> &e, int ld, int k0, int lim_k) {
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
+      bool ok;
+      if (KC) {
+        const int kc = k0 + (f % (BK / 4)) * 4;
+        ok = kc < lim_k;
+        r[p] = *(const f4 *)(e.at[p] + (ok ? kc : lim_k - 4));
+      } else {
+        const int kr = k0 + f / (BMN / 4);
+        ok = kr < lim_k;
+        r[p] = *(const f4 *)(e.at[p] + (size_t)(ok ? kr : lim_k - 1) * ld);
+      }
+      keep[p] = ok && e.in[p];
+    }
+  }
+  // the whole-tile form of load(), for tiles and slabs that the caller knows to lie inside the operand (EDGE 1:
+  // aligned as well)
+  __device__ __forceinline__ void load_whole(const float *g, int ld, int mn0, int k0) {
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
+      if (KC) {
+        const int mn = f / (BK / 4), kq = f % (BK / 4);
+        r[p] = *(const f4 *)(g + (size_t)(mn0 + mn) * ld + k0 + kq * 4);
+      } else {
+        const int kk = f / (BMN / 4), q = f % (BMN / 4);
+        r[p] = *(const f4 *)(g + (size_t)(k0 + kk) * ld + mn0 + q * 4);
+      }
+      keep[p] = true;
+    }
+  }
   __device__ __forceinline__ void store(float *lds) const {
     if (PART && threadIdx.x >= GROUPS) return;
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = threadIdx.x + 256 * p;
+      const f4 v = (EDGE != 1 || keep[p]) ? r[p] : f4{0.f, 0.f, 0.f, 0.f};
       if (KC) {
         const int mn = f / (BK / 4), kq = f % (BK / 4);
-        *(f4 *)(lds + mn * KPITCH + kq * 4) = r[p];
+        *(f4 *)(lds + mn * KPITCH + kq * 4) = v;
       } else {
         const int kk = f / (BMN / 4), q = f % (BMN / 4);
-        *(f4 *)(lds + kk * BMN + q * 4) = r[p];
+        *(f4 *)(lds + kk * BMN + q * 4) = v;
       }
     }
   }
@@ -192,19 +251,36 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   TileLoader<BN, BKC, EDGE> lb1;
   const int last = KT > 0 ? KT - 1 : 0;
   auto slab_k = [&](int kt) { return k_begin + (kt < last ? kt : last) * BK; };
-  la.load(P.a, P.lda, m0, slab_k(0), P.m, k_end);
-  lb.load(P.b, P.ldb, n0, slab_k(0), P.n, k_end);
-  la1.load(P.a, P.lda, m0, slab_k(1), P.m, k_end);
-  lb1.load(P.b, P.ldb, n0, slab_k(1), P.n, k_end);
+  EdgeLanes<BM, AKC> ea;
+  EdgeLanes<BN, BKC> eb;
+  if (EDGE == 1) {
+    ea.set(P.a, P.lda, m0, P.m);
+    eb.set(P.b, P.ldb, n0, P.n);
+  }
+  auto fetch = [&](auto &to_a, auto &to_b, int k0) {
+    if constexpr (EDGE == 1) {
+      to_a.load_edge(ea, P.lda, k0, k_end);
+      to_b.load_edge(eb, P.ldb, k0, k_end);
+    } else {
+      to_a.load(P.a, P.lda, m0, k0, P.m, k_end);
+      to_b.load(P.b, P.ldb, n0, k0, P.n, k_end);
+    }
+  };
+  fetch(la, lb, slab_k(0));
+  fetch(la1, lb1, slab_k(1));
   la.store(lds);
   lb.store(lds + AF);
   __syncthreads();
 
-  auto step = [&](int kt, int cur, auto &issue_a, auto &issue_b, auto &keep_a, auto &keep_b) {
+  auto step = [&](auto inside, int kt, int cur, auto &issue_a, auto &issue_b, auto &keep_a, auto &keep_b) {
     float *As = lds + cur * (AF + BF);
     float *Bs = As + AF;
-    issue_a.load(P.a, P.lda, m0, slab_k(kt + 2), P.m, k_end);
-    issue_b.load(P.b, P.ldb, n0, slab_k(kt + 2), P.n, k_end);
+    if constexpr (decltype(inside)::value) {
+      issue_a.load_whole(P.a, P.lda, m0, slab_k(kt + 2));
+      issue_b.load_whole(P.b, P.ldb, n0, slab_k(kt + 2));
+    } else {
+      fetch(issue_a, issue_b, slab_k(kt + 2));
+    }
     __builtin_amdgcn_sched_barrier(0);   // keep the loads at the top of the step
     {
 #pragma unroll
@@ -227,11 +303,23 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
     __syncthreads();
   };
   int kt = 0;
-  for (; kt + 1 < KT; kt += 2) {
-    step(kt, 0, la, lb, la1, lb1);
-    step(kt + 1, 1, la1, lb1, la, lb);
+  constexpr std::true_type whole_slab{};
+  constexpr std::false_type any_slab{};
+  if (EDGE == 1 && m0 + BM <= P.m && n0 + BN <= P.n) {
+    // a tile inside the matrix (the same for the whole block): its slabs are whole except the last ones, so the
+    // steps that request a whole slab (kt + 2 and kt + 3 below KF) use the plain loads, and the edge form is left
+    // to the tiles on the rim and to the end of K
+    const int KF = (k_end - k_begin) / BK;
+    for (; kt + 3 < KF; kt += 2) {
+      step(whole_slab, kt, 0, la, lb, la1, lb1);
+      step(whole_slab, kt + 1, 1, la1, lb1, la, lb);
+    }
   }
-  if (kt < KT) step(kt, 0, la, lb, la1, lb1);
+  for (; kt + 1 < KT; kt += 2) {
+    step(any_slab, kt, 0, la, lb, la1, lb1);
+    step(any_slab, kt + 1, 1, la1, lb1, la, lb);
+  }
+  if (kt < KT) step(any_slab, kt, 0, la, lb, la1, lb1);
 
   // epilogue: lane holds rows 8*(r/4) + 4*(lane/32) + (r%4) of column lane%32
   const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
@@ -311,6 +399,16 @@ __global__ __launch_bounds__(256) void splitk_reduce(GemmParams P) {
   }
 }
 
+// K = 0: the product is empty and the operands may not exist
+__global__ __launch_bounds__(256) void scale_result(GemmParams P) {
+  const size_t total = (size_t)P.m * P.n;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
+    const size_t col = e / P.m, row = e - col * P.m;
+    float *cp = P.c + col * P.ldc + row;
+    *cp = P.beta != 0.f ? P.beta * *cp : 0.f;
+  }
+}
+
 template <int BM, int BN, int EDGE>
 void launch_tt(bool ta, bool tb, dim3 grid, hipStream_t s, const GemmParams &P) {
   dim3 block(256);
@@ -359,13 +457,14 @@ static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, 
     int resident;  // blocks a CU holds
   };
   // the two thin tiles only stand for products with a side of at most 32, where they halve the padding
-  static const Cand cands[6] = {{128, 128, 138., 128., 3}, {128, 64, 133., 124., 5}, {64, 128, 126., 118., 5},
-                                {64, 64, 123., 110., 8},   {128, 32, 115., 105., 8}, {32, 128, 115., 105., 8}};
+  static const Cand cands[6] = {{128, 128, 138., 134., 3}, {128, 64, 133., 129., 5}, {64, 128, 126., 116., 5},
+                                {64, 64, 123., 119., 8},   {128, 32, 115., 110., 8}, {32, 128, 115., 110., 8}};
   double best = -1.;
   bm = bn = 64;
   for (const Cand &c : cands) {
     if ((c.bm == 128 && m < 128) || (c.bn == 128 && n < 128)) continue;
     if ((c.bn == 32 && n > 32) || (c.bm == 32 && m > 32)) continue;
+    if ((n <= 32 && m >= 1024 && c.bn != 32) || (m <= 32 && n >= 1024 && c.bm != 32)) continue;   // measured: the thin tile wins there
     const long tm = (m + c.bm - 1) / c.bm, tn = (n + c.bn - 1) / c.bn, tiles = tm * tn;
     const bool whole = aligned && m % c.bm == 0 && n % c.bn == 0;
     int ks, kc;
@@ -413,6 +512,14 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   P.ldc = (int)ldc;
   P.alpha = alpha;
   P.beta = beta;
+  if (P.k == 0) {
+    const size_t total = (size_t)m * n;
+    hipLaunchKernelGGL(scale_result, dim3((unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256)), dim3(256), 0, stream, P);
+    hipError_t e0 = hipGetLastError();
+    THCL_CHECK(e0 == hipSuccess, "gemm launch failed: %s", hipGetErrorString(e0));
+    thcl_after_launch(state, rt);
+    return;
+  }
   int bm, bn;
   const bool aligned = (k % BK == 0) && k > 0 && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && al16(a) && al16(b) && al16(c);
   choose_tile(m, n, k, thcl_rt_get_props(rt)->compute_units, aligned, bm, bn);

@@ -119,6 +119,26 @@ def test_gemm_entry_point_column_major(cl):
     assert rel_err(tC.float().T, want) < RTOL
 
 
+def test_gemm_with_an_empty_inner_dimension(cl):
+    """K = 0 through the BLAS entry point: the result is beta * C (zeros for beta = 0, whatever C held) and the
+    operands, which have no elements, are not read."""
+    m, n = 70, 45
+    Cm = oracle.normal(16, m * n).reshape(n, m)
+    Cm[3, 5] = np.nan
+    st = cl.state()
+    dummy = cl.ClTensor(4)
+    for beta in (0.5, 0.0):
+        tC = cl.ClTensor(Cm)
+        st.lib.THClBlas_gemm(st.ptr, C.c_char(b"n"), C.c_char(b"t"), m, n, 0, C.c_float(2.0), dummy._h, m, dummy._h, n,
+                             C.c_float(beta), tC._h, m)
+        st.check()
+        got = tC.float()
+        if beta == 0.0:
+            assert np.array_equal(got, np.zeros((n, m), np.float32))
+        else:
+            assert np.array_equal(got, np.float32(beta) * Cm, equal_nan=True)
+
+
 def test_skinny_config_shape_reduced(cl):
     # M=64, A given as the transpose of a dense (K x M) array, as in the benchmark configuration
     M, N, K = 64, 2048, 512
