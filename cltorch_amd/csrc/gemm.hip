@@ -51,29 +51,41 @@ struct TileLds {
   static constexpr int FLOATS = KC ? BMN * KPITCH : BK * BMN;
 };
 
-// EDGE 1: what a lane's loads of one operand keep from slab to slab.  at[p] is the lane's 16-byte group in k row 0
-// (operands contiguous along m/n) or the start of its row (operands contiguous along k), moved to the operand's last
-// group or row when it lies beyond the m/n extent; in[p] tells which.  Worked out once per tile: with the extent
-// tests and the 64-bit products redone at every slab a tile on the rim took 1.6 times as long as a whole one.
-template <int BMN, bool KC>
+// Edge kernels: what a lane's loads of one operand keep from slab to slab, worked out once per tile (with the extent
+// tests and the 64-bit products redone at every slab a tile on the rim took 1.6 times as long as a whole one).
+// EDGE 1: at[p] is the lane's 16-byte group in k row 0 (operands contiguous along m/n) or the start of its row
+// (operands contiguous along k), moved to the operand's last group or row when it lies beyond the m/n extent; in[p]
+// is 15 when it lies inside.  EDGE 2: the same per element: for operands contiguous along m/n at[p] is the operand's
+// base, mo[p][c] the element's offset along m/n (the last one when it lies beyond), in[p] one bit per element.
+template <int BMN, bool KC, int EDGE>
 struct EdgeLanes {
   static constexpr int GROUPS = BMN * BK / 4;
   static constexpr int NV = GROUPS >= 256 ? GROUPS / 256 : 1;
   static constexpr bool PART = GROUPS < 256;
   const float *at[NV];
-  bool in[NV];
+  unsigned in[NV];
+  int mo[(EDGE == 2 && !KC) ? NV : 1][4];
   __device__ __forceinline__ void set(const float *g, int ld, int mn0, int lim_mn) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
       if (KC) {
         const int mn = mn0 + f / (BK / 4);
-        in[p] = mn < lim_mn;
-        at[p] = g + (size_t)(in[p] ? mn : lim_mn - 1) * ld;
+        in[p] = mn < lim_mn ? 15u : 0u;
+        at[p] = g + (size_t)(mn < lim_mn ? mn : lim_mn - 1) * ld;
+      } else if (EDGE == 1) {
+        const int mq = mn0 + (f % (BMN / 4)) * 4;
+        in[p] = mq < lim_mn ? 15u : 0u;
+        at[p] = g + (mq < lim_mn ? mq : lim_mn - 4);
       } else {
         const int mq = mn0 + (f % (BMN / 4)) * 4;
-        in[p] = mq < lim_mn;
-        at[p] = g + (in[p] ? mq : lim_mn - 4);
+        at[p] = g;
+        in[p] = 0u;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          in[p] |= (mq + c < lim_mn ? 1u : 0u) << c;
+          mo[p][c] = mq + c < lim_mn ? mq + c : lim_mn - 1;
+        }
       }
     }
   }
@@ -84,7 +96,8 @@ struct EdgeLanes {
 // 16-byte group of the operand is either inside it or outside, and aligned; every load is issued (from the operand's
 // last row or group when the lane's own lies outside) and groups outside become zeros, so there is no branch around
 // a load.
-// EDGE 2: any pitch and alignment, one element at a time.  The choice is made at compile time: a run-time branch
+// EDGE 2: any pitch and alignment, one element at a time, in the same way (every load issued from an address inside
+// the operand, elements outside zeroed on the way to LDS).  The choice is made at compile time: a run-time branch
 // between the two edge forms made the compiler wait for all loads at every slab (aligned 4096^3 through the edge
 // kernel: 101 TFLOP/s with the branch against 138 through the whole-tile kernel).
 template <int BMN, bool KC, int EDGE>
@@ -93,54 +106,39 @@ struct TileLoader {
   static constexpr int NV = GROUPS >= 256 ? GROUPS / 256 : 1;
   static constexpr bool PART = GROUPS < 256;
   f4 r[NV];
-  bool keep[NV];   // EDGE 1: the group lies inside the operand; looked at when the registers go to LDS, so that nothing
-                   // has to wait for the load before then
+  unsigned keep[NV];   // edge kernels: one bit per element that lies inside the operand; looked at when the registers
+                       // go to LDS, so that nothing has to wait for the load before then
 
-  // g: operand base; ld: leading dim; mn0: first row/col of the tile; k0: first k; lim_mn/lim_k: extents
-  // vec (edge kernels): a 16-byte group is either inside the operand or outside, and aligned
-  __device__ __forceinline__ void load(const float *g, int ld, int mn0, int k0, int lim_mn, int lim_k) {
+  // edge kernels: every load is issued, from an address inside the operand; what lies outside becomes zeros in store()
+  __device__ __forceinline__ void load_edge(const EdgeLanes<BMN, KC, EDGE> &e, int ld, int k0, int lim_k) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
-      if (KC) {
-        const int mn = f / (BK / 4), kq = f % (BK / 4);
-        const float *src = g + (size_t)(mn0 + mn) * ld + k0 + kq * 4;
-        if (EDGE == 0) {
-          r[p] = *(const f4 *)src;
-        } else {
-#pragma unroll
-          for (int c = 0; c < 4; c++)
-            r[p][c] = (mn0 + mn < lim_mn && k0 + kq * 4 + c < lim_k) ? src[c] : 0.f;
-        }
-      } else {
-        const int kk = f / (BMN / 4), q = f % (BMN / 4);
-        const float *src = g + (size_t)(k0 + kk) * ld + mn0 + q * 4;
-        if (EDGE == 0) {
-          r[p] = *(const f4 *)src;
-        } else {
-#pragma unroll
-          for (int c = 0; c < 4; c++)
-            r[p][c] = (k0 + kk < lim_k && mn0 + q * 4 + c < lim_mn) ? src[c] : 0.f;
-        }
-      }
-    }
-  }
-  // EDGE 1: every load is issued, from an address inside the operand, and groups outside it become zeros
-  __device__ __forceinline__ void load_edge(const EdgeLanes<BMN, KC> &e, int ld, int k0, int lim_k) {
-#pragma unroll
-    for (int p = 0; p < NV; p++) {
-      const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
-      bool ok;
       if (KC) {
         const int kc = k0 + (f % (BK / 4)) * 4;
-        ok = kc < lim_k;
-        r[p] = *(const f4 *)(e.at[p] + (ok ? kc : lim_k - 4));
+        if (EDGE == 1) {
+          r[p] = *(const f4 *)(e.at[p] + (kc < lim_k ? kc : lim_k - 4));
+          keep[p] = kc < lim_k ? e.in[p] : 0u;
+        } else {
+          unsigned ok = 0u;
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            r[p][c] = e.at[p][kc + c < lim_k ? kc + c : lim_k - 1];
+            ok |= (kc + c < lim_k ? 1u : 0u) << c;
+          }
+          keep[p] = e.in[p] & ok;
+        }
       } else {
         const int kr = k0 + f / (BMN / 4);
-        ok = kr < lim_k;
-        r[p] = *(const f4 *)(e.at[p] + (size_t)(ok ? kr : lim_k - 1) * ld);
+        const float *row = e.at[p] + (size_t)(kr < lim_k ? kr : lim_k - 1) * ld;
+        if (EDGE == 1) {
+          r[p] = *(const f4 *)row;
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; c++) r[p][c] = row[e.mo[p][c]];
+        }
+        keep[p] = kr < lim_k ? e.in[p] : 0u;
       }
-      keep[p] = ok && e.in[p];
     }
   }
   // the whole-tile form of load(), for tiles and slabs that the caller knows to lie inside the operand (EDGE 1:
@@ -156,7 +154,7 @@ struct TileLoader {
         const int kk = f / (BMN / 4), q = f % (BMN / 4);
         r[p] = *(const f4 *)(g + (size_t)(k0 + kk) * ld + mn0 + q * 4);
       }
-      keep[p] = true;
+      keep[p] = 15u;
     }
   }
   __device__ __forceinline__ void store(float *lds) const {
@@ -164,7 +162,12 @@ struct TileLoader {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = threadIdx.x + 256 * p;
-      const f4 v = (EDGE != 1 || keep[p]) ? r[p] : f4{0.f, 0.f, 0.f, 0.f};
+      f4 v = r[p];
+      if (EDGE == 1) v = keep[p] ? v : f4{0.f, 0.f, 0.f, 0.f};
+      if (EDGE == 2) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) v[c] = (keep[p] >> c & 1u) ? v[c] : 0.f;
+      }
       if (KC) {
         const int mn = f / (BK / 4), kq = f % (BK / 4);
         *(f4 *)(lds + mn * KPITCH + kq * 4) = v;
@@ -251,19 +254,19 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   TileLoader<BN, BKC, EDGE> lb1;
   const int last = KT > 0 ? KT - 1 : 0;
   auto slab_k = [&](int kt) { return k_begin + (kt < last ? kt : last) * BK; };
-  EdgeLanes<BM, AKC> ea;
-  EdgeLanes<BN, BKC> eb;
-  if (EDGE == 1) {
+  EdgeLanes<BM, AKC, EDGE> ea;
+  EdgeLanes<BN, BKC, EDGE> eb;
+  if (EDGE != 0) {
     ea.set(P.a, P.lda, m0, P.m);
     eb.set(P.b, P.ldb, n0, P.n);
   }
   auto fetch = [&](auto &to_a, auto &to_b, int k0) {
-    if constexpr (EDGE == 1) {
+    if constexpr (EDGE != 0) {
       to_a.load_edge(ea, P.lda, k0, k_end);
       to_b.load_edge(eb, P.ldb, k0, k_end);
     } else {
-      to_a.load(P.a, P.lda, m0, k0, P.m, k_end);
-      to_b.load(P.b, P.ldb, n0, k0, P.n, k_end);
+      to_a.load_whole(P.a, P.lda, m0, k0);
+      to_b.load_whole(P.b, P.ldb, n0, k0);
     }
   };
   fetch(la, lb, slab_k(0));
