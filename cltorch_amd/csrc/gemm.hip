@@ -26,6 +26,7 @@ namespace {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
+typedef f4 f4u __attribute__((aligned(4)));   // a 16-byte access that only needs the alignment of its elements
 
 constexpr int BK = 16;
 constexpr int KPITCH = BK + 4;  // [mn][k] rows: odd number of 16-byte chunks -> conflict-free 128-bit reads
@@ -55,8 +56,10 @@ struct TileLds {
 // tests and the 64-bit products redone at every slab a tile on the rim took 1.6 times as long as a whole one).
 // EDGE 1: at[p] is the lane's 16-byte group in k row 0 (operands contiguous along m/n) or the start of its row
 // (operands contiguous along k), moved to the operand's last group or row when it lies beyond the m/n extent; in[p]
-// is 15 when it lies inside.  EDGE 2: the same per element: for operands contiguous along m/n at[p] is the operand's
-// base, mo[p][c] the element's offset along m/n (the last one when it lies beyond), in[p] one bit per element.
+// is 15 when it lies inside.  EDGE 2: the same with groups that may straddle the extent: the 16-byte window is then
+// moved back to end at the extent and sh[p] tells by how many elements.  EDGE 3: per element: for operands
+// contiguous along m/n at[p] is the operand's base, mo[p][c] the element's offset along m/n (the last one when it
+// lies beyond), in[p] one bit per element.
 template <int BMN, bool KC, int EDGE>
 struct EdgeLanes {
   static constexpr int GROUPS = BMN * BK / 4;
@@ -64,19 +67,23 @@ struct EdgeLanes {
   static constexpr bool PART = GROUPS < 256;
   const float *at[NV];
   unsigned in[NV];
-  int mo[(EDGE == 2 && !KC) ? NV : 1][4];
+  unsigned sh[NV];
+  int mo[(EDGE == 3 && !KC) ? NV : 1][4];
   __device__ __forceinline__ void set(const float *g, int ld, int mn0, int lim_mn) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
+      sh[p] = 0u;
       if (KC) {
         const int mn = mn0 + f / (BK / 4);
         in[p] = mn < lim_mn ? 15u : 0u;
         at[p] = g + (size_t)(mn < lim_mn ? mn : lim_mn - 1) * ld;
-      } else if (EDGE == 1) {
+      } else if (EDGE == 1 || EDGE == 2) {
         const int mq = mn0 + (f % (BMN / 4)) * 4;
+        const int mw = mq + 4 <= lim_mn ? mq : lim_mn - 4;   // EDGE 1: extents are multiples of 4, so mw is mq or outside
         in[p] = mq < lim_mn ? 15u : 0u;
-        at[p] = g + (mq < lim_mn ? mq : lim_mn - 4);
+        sh[p] = mq < lim_mn ? (unsigned)(mq - mw) : 0u;
+        at[p] = g + mw;
       } else {
         const int mq = mn0 + (f % (BMN / 4)) * 4;
         at[p] = g;
@@ -96,18 +103,21 @@ struct EdgeLanes {
 // 16-byte group of the operand is either inside it or outside, and aligned; every load is issued (from the operand's
 // last row or group when the lane's own lies outside) and groups outside become zeros, so there is no branch around
 // a load.
-// EDGE 2: any pitch and alignment, one element at a time, in the same way (every load issued from an address inside
-// the operand, elements outside zeroed on the way to LDS).  The choice is made at compile time: a run-time branch
+// EDGE 2: any pitch and alignment, with 16-byte loads that need no alignment; a group that straddles the operand's
+// extent is read through a window moved back to end there and shifted into place on the way to LDS.  Needs at least
+// 4 elements along each operand's contiguous dimension.  EDGE 3: one element at a time, for what is left.  The choice is made at compile time: a run-time branch
 // between the two edge forms made the compiler wait for all loads at every slab (aligned 4096^3 through the edge
 // kernel: 101 TFLOP/s with the branch against 138 through the whole-tile kernel).
 template <int BMN, bool KC, int EDGE>
 struct TileLoader {
+  using LoadT = typename std::conditional<EDGE == 2, f4u, f4>::type;
   static constexpr int GROUPS = BMN * BK / 4;
   static constexpr int NV = GROUPS >= 256 ? GROUPS / 256 : 1;
   static constexpr bool PART = GROUPS < 256;
   f4 r[NV];
-  unsigned keep[NV];   // edge kernels: one bit per element that lies inside the operand; looked at when the registers
-                       // go to LDS, so that nothing has to wait for the load before then
+  unsigned keep[NV];   // edge kernels: one bit per element that lies inside the operand (and, from bit 4, how far the
+                       // window was moved back); looked at when the registers go to LDS, so that nothing has to
+                       // wait for the load before then
 
   // edge kernels: every load is issued, from an address inside the operand; what lies outside becomes zeros in store()
   __device__ __forceinline__ void load_edge(const EdgeLanes<BMN, KC, EDGE> &e, int ld, int k0, int lim_k) {
@@ -116,9 +126,10 @@ struct TileLoader {
       const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
       if (KC) {
         const int kc = k0 + (f % (BK / 4)) * 4;
-        if (EDGE == 1) {
-          r[p] = *(const f4 *)(e.at[p] + (kc < lim_k ? kc : lim_k - 4));
-          keep[p] = kc < lim_k ? e.in[p] : 0u;
+        if (EDGE == 1 || EDGE == 2) {
+          const int kw = kc + 4 <= lim_k ? kc : lim_k - 4;
+          r[p] = *(const LoadT *)(e.at[p] + kw);
+          keep[p] = kc < lim_k ? (e.in[p] | (unsigned)(kc - kw) << 4) : 0u;
         } else {
           unsigned ok = 0u;
 #pragma unroll
@@ -131,13 +142,14 @@ struct TileLoader {
       } else {
         const int kr = k0 + f / (BMN / 4);
         const float *row = e.at[p] + (size_t)(kr < lim_k ? kr : lim_k - 1) * ld;
-        if (EDGE == 1) {
-          r[p] = *(const f4 *)row;
+        if (EDGE == 1 || EDGE == 2) {
+          r[p] = *(const LoadT *)row;
+          keep[p] = kr < lim_k ? (e.in[p] | e.sh[p] << 4) : 0u;
         } else {
 #pragma unroll
           for (int c = 0; c < 4; c++) r[p][c] = row[e.mo[p][c]];
+          keep[p] = kr < lim_k ? e.in[p] : 0u;
         }
-        keep[p] = kr < lim_k ? e.in[p] : 0u;
       }
     }
   }
@@ -149,10 +161,10 @@ struct TileLoader {
       const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
       if (KC) {
         const int mn = f / (BK / 4), kq = f % (BK / 4);
-        r[p] = *(const f4 *)(g + (size_t)(mn0 + mn) * ld + k0 + kq * 4);
+        r[p] = *(const LoadT *)(g + (size_t)(mn0 + mn) * ld + k0 + kq * 4);
       } else {
         const int kk = f / (BMN / 4), q = f % (BMN / 4);
-        r[p] = *(const f4 *)(g + (size_t)(k0 + kk) * ld + mn0 + q * 4);
+        r[p] = *(const LoadT *)(g + (size_t)(k0 + kk) * ld + mn0 + q * 4);
       }
       keep[p] = 15u;
     }
@@ -164,7 +176,13 @@ struct TileLoader {
       const int f = threadIdx.x + 256 * p;
       f4 v = r[p];
       if (EDGE == 1) v = keep[p] ? v : f4{0.f, 0.f, 0.f, 0.f};
-      if (EDGE == 2) {
+      if (EDGE == 2) {   // element c of the group sits at c + (how far the window was moved back)
+        const unsigned back = keep[p] >> 4;
+        const f4 w = r[p];
+        v = back == 0u ? w : back == 1u ? f4{w[1], w[2], w[3], 0.f} : back == 2u ? f4{w[2], w[3], 0.f, 0.f} : f4{w[3], 0.f, 0.f, 0.f};
+        v = (keep[p] & 15u) ? v : f4{0.f, 0.f, 0.f, 0.f};
+      }
+      if (EDGE == 3) {
 #pragma unroll
         for (int c = 0; c < 4; c++) v[c] = (keep[p] >> c & 1u) ? v[c] : 0.f;
       }
@@ -308,7 +326,7 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   int kt = 0;
   constexpr std::true_type whole_slab{};
   constexpr std::false_type any_slab{};
-  if (EDGE == 1 && m0 + BM <= P.m && n0 + BN <= P.n) {
+  if ((EDGE == 1 || EDGE == 2) && m0 + BM <= P.m && n0 + BN <= P.n) {
     // a tile inside the matrix (the same for the whole block): its slabs are whole except the last ones, so the
     // steps that request a whole slab (kt + 2 and kt + 3 below KF) use the plain loads, and the edge form is left
     // to the tiles on the rim and to the end of K
@@ -526,9 +544,12 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   int bm, bn;
   const bool aligned = (k % BK == 0) && k > 0 && (lda % 4 == 0) && (ldb % 4 == 0) && (ldc % 4 == 0) && al16(a) && al16(b) && al16(c);
   choose_tile(m, n, k, thcl_rt_get_props(rt)->compute_units, aligned, bm, bn);
-  const bool fast = aligned && (m % bm == 0) && (n % bn == 0);
   // an operand's contiguous dim is m for a 'n', k for a 't'; n for b 't', k for b 'n'
   const long a_run = ta ? k : m, b_run = tb ? n : k;
+  // fewer than 4 elements along an operand's contiguous dim and no alignment to rely on: one element at a time, one tile shape
+  const bool by_element = !(lda % 4 == 0 && a_run % 4 == 0 && al16(a) && ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) && (a_run < 4 || b_run < 4);
+  if (by_element) bm = bn = 64;
+  const bool fast = aligned && (m % bm == 0) && (n % bn == 0);
   P.vec_a = (lda % 4 == 0 && a_run % 4 == 0 && al16(a)) ? 1 : 0;
   P.vec_b = (ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) ? 1 : 0;
   P.vec_c = (ldc % 4 == 0 && m % 4 == 0 && al16(c)) ? 1 : 0;
@@ -545,7 +566,8 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   if (fast) launch_tt<BM_, BN_, 0>(ta, tb, grid, stream, P);                        \
   else if (P.vec_a && P.vec_b) launch_tt<BM_, BN_, 1>(ta, tb, grid, stream, P);     \
   else launch_tt<BM_, BN_, 2>(ta, tb, grid, stream, P);
-  if (bm == 128 && bn == 128) { GO(128, 128) }
+  if (by_element) launch_tt<64, 64, 3>(ta, tb, grid, stream, P);
+  else if (bm == 128 && bn == 128) { GO(128, 128) }
   else if (bm == 128 && bn == 64) { GO(128, 64) }
   else if (bm == 64 && bn == 128) { GO(64, 128) }
   else if (bm == 128 && bn == 32) { GO(128, 32) }

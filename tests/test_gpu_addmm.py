@@ -214,6 +214,33 @@ def test_products_with_a_side_of_at_most_32(cl, M, N, K):
         assert np.max(np.abs(Cd.float() - want)) / scale < RTOL, lay
 
 
+def _odd_pitch(cl, arr, transposed):
+    """device tensor equal to arr (2-D), its rows 3 elements apart from dense so that nothing is 16-byte aligned,
+    optionally stored transposed"""
+    a = np.ascontiguousarray(arr.T if transposed else arr)
+    big = np.zeros((a.shape[0], a.shape[1] + 3), F)
+    big[:, :a.shape[1]] = a
+    t = cl.ClTensor(big).narrow(2, 1, a.shape[1])
+    return t.t() if transposed else t
+
+
+@pytest.mark.parametrize("M,N,K", [(50, 3, 37), (3, 50, 37), (50, 40, 3), (2, 2, 2), (70, 3, 3), (1, 300, 2), (301, 299, 5),
+                                   (129, 131, 67), (1001, 515, 130)])
+def test_unaligned_operands_of_any_extent(cl, M, N, K):
+    """Operands whose rows start at odd element offsets: 16-byte loads that need no alignment, a window moved back
+    at the end of a row, and, with fewer than four elements along a row, one element at a time.  All eight layouts."""
+    rng = np.random.RandomState(M * 5 + N * 11 + K)
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
+    b = rng.standard_normal((K, N)).astype(F)
+    c = rng.standard_normal((M, N)).astype(F)
+    want = -0.5 * c.astype(np.float64) + 1.25 * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = max(1.0, float(np.sqrt(np.mean(want ** 2))))
+    for lay in range(8):
+        A, B, Cd = _odd_pitch(cl, a, lay & 1), _odd_pitch(cl, b, lay & 2), _odd_pitch(cl, c, lay & 4)
+        Cd.addmm(-0.5, 1.25, A, B)
+        assert np.max(np.abs(Cd.float() - want)) / scale < RTOL, lay
+
+
 def test_sliced_products_repeat_bit_exactly(cl):
     """K-sliced products sum their slices in slice order: every repetition gives the same
     bits, also with other reductions in between, with ragged shapes, with beta = 0 over
