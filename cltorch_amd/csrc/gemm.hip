@@ -43,7 +43,7 @@ struct GemmParams {
   int kchunk;   // K per slice (multiple of BK)
   float *work;  // [ksplit][n][m] dense partials
   // the operand's 16-byte groups along its contiguous dim are whole and aligned (a and b: picks the edge kernel)
-  int vec_a, vec_b, vec_c;
+  int vec_a, vec_b;
 };
 
 // One operand tile in LDS.  KC: contiguous along k in global memory.
@@ -342,7 +342,10 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   }
   if (kt < KT) step(any_slab, kt, 0, la, lb, la1, lb1);
 
-  // epilogue: lane holds rows 8*(r/4) + 4*(lane/32) + (r%4) of column lane%32
+  // epilogue: lane holds rows 8*(r/4) + 4*(lane/32) + (r%4) of column lane%32.  The edge kernels use 16-byte accesses
+  // that need no alignment wherever the four rows lie inside the result, and single elements for the group that
+  // straddles its last row.
+  using CT = typename std::conditional<EDGE == 0, f4, f4u>::type;
   const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
   if (P.ksplit > 1) {
     // raw partial product of this K slice, dense [n][m]; scaled and summed by splitk_reduce
@@ -356,11 +359,11 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
         for (int rq = 0; rq < 4; rq++) {
           const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
           float *wp = w + (size_t)col * P.m + row;
-          if (!EDGE || (P.m % 4 == 0 && col < P.n && row < P.m)) {  // the partials are dense: pitch m, 16-byte aligned base
+          if (!EDGE || (col < P.n && row + 3 < P.m)) {  // edge kernels: a 16-byte store that needs no alignment
             f4 v;
 #pragma unroll
             for (int c = 0; c < 4; c++) v[c] = acc[i][j][rq * 4 + c];
-            *(f4 *)wp = v;
+            *(CT *)wp = v;
           } else if (col < P.n) {
 #pragma unroll
             for (int c = 0; c < 4; c++)
@@ -379,16 +382,16 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
       for (int rq = 0; rq < 4; rq++) {
         const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
         float *cp = P.c + (size_t)col * P.ldc + row;
-        if (!EDGE || (P.vec_c && col < P.n && row < P.m)) {
+        if (!EDGE || (col < P.n && row + 3 < P.m)) {
           f4 v;
 #pragma unroll
           for (int c = 0; c < 4; c++) v[c] = P.alpha * acc[i][j][rq * 4 + c];
           if (P.beta != 0.f) {
-            const f4 old = *(const f4 *)cp;
+            const f4 old = *(const CT *)cp;
 #pragma unroll
             for (int c = 0; c < 4; c++) v[c] += P.beta * old[c];
           }
-          *(f4 *)cp = v;
+          *(CT *)cp = v;
         } else {
           if (col < P.n) {
 #pragma unroll
@@ -552,7 +555,6 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   const bool fast = aligned && (m % bm == 0) && (n % bn == 0);
   P.vec_a = (lda % 4 == 0 && a_run % 4 == 0 && al16(a)) ? 1 : 0;
   P.vec_b = (ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) ? 1 : 0;
-  P.vec_c = (ldc % 4 == 0 && m % 4 == 0 && al16(c)) ? 1 : 0;
   P.tiles_m = (int)((m + bm - 1) / bm);
   P.tiles_n = (int)((n + bn - 1) / bn);
   P.group_m = P.tiles_m < 8 ? P.tiles_m : 8;
