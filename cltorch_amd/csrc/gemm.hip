@@ -409,15 +409,29 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   }
 }
 
-// C = alpha * (sum over K slices, in slice order) + beta * C
+// C = alpha * (sum over K slices, in slice order) + beta * C.  VEC: four rows of a column per thread (m a multiple
+// of 4, the result 16-byte aligned).  Four slices are requested before the first is added.
+template <bool VEC>
 __global__ __launch_bounds__(256) void splitk_reduce(GemmParams P) {
-  const size_t total = (size_t)P.m * P.n;
+  typedef typename std::conditional<VEC, f4, float>::type T;
+  constexpr int W = VEC ? 4 : 1;
+  const size_t total = (size_t)P.m * P.n / W;   // in units of T
+  const T *work = (const T *)P.work;
   for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
-    float s = P.work[e];
-    for (int k = 1; k < P.ksplit; k++) s += P.work[(size_t)k * total + e];
-    const size_t col = e / P.m, row = e - col * P.m;
-    float *cp = P.c + col * P.ldc + row;
-    float v = P.alpha * s;
+    T s = work[e];
+    int k = 1;
+    for (; k + 3 < P.ksplit; k += 4) {
+      const T a = work[(size_t)k * total + e], b = work[(size_t)(k + 1) * total + e], c = work[(size_t)(k + 2) * total + e],
+              d = work[(size_t)(k + 3) * total + e];
+      s += a;
+      s += b;
+      s += c;
+      s += d;
+    }
+    for (; k < P.ksplit; k++) s += work[(size_t)k * total + e];
+    const size_t col = e * W / P.m, row = e * W - col * P.m;
+    T *cp = (T *)(P.c + col * P.ldc + row);
+    T v = P.alpha * s;
     if (P.beta != 0.f) v += P.beta * *cp;
     *cp = v;
   }
@@ -577,9 +591,11 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   else { GO(64, 64) }
 #undef GO
   if (P.ksplit > 1) {
-    const size_t total = (size_t)m * n;
+    const bool vec = m % 4 == 0 && ldc % 4 == 0 && al16(c);
+    const size_t total = (size_t)m * n / (vec ? 4 : 1);
     unsigned rg = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
-    hipLaunchKernelGGL(splitk_reduce, dim3(rg), dim3(256), 0, stream, P);
+    if (vec) hipLaunchKernelGGL(splitk_reduce<true>, dim3(rg), dim3(256), 0, stream, P);
+    else hipLaunchKernelGGL(splitk_reduce<false>, dim3(rg), dim3(256), 0, stream, P);
   }
   hipError_t e = hipGetLastError();
   THCL_CHECK(e == hipSuccess, "gemm launch failed: %s", hipGetErrorString(e));
