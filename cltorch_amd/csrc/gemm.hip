@@ -461,14 +461,15 @@ bool al16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
 
 // Few tiles and a long K: slice K over blockIdx.y so every CU has work; the slices'
 // partial products are summed in slice order by a second kernel.  Below one tile per
-// CU any K from 1024 up is sliced; between one and two tiles per CU only K >= 2048
-// (512x2048x4096: 96 -> 108 TFLOP/s, while 1024^3 loses 10 % when sliced).
+// CU any K from 1024 up is sliced (from 512 up below half a tile per CU); between one and two tiles per CU only
+// K >= 2048 (512x2048x4096: 96 -> 108 TFLOP/s, while 1024^3 loses 10 % when sliced).
 static void choose_ksplit(long tiles, long k, int cus, int &ksplit, int &kchunk) {
   ksplit = 1;
   kchunk = (int)(k > 0 ? k : 0);
-  if (!((tiles < cus && k >= 1024) || (tiles < 2L * cus && k >= 2048))) return;
+  if (!((tiles < cus && k >= 1024) || (tiles < 2L * cus && k >= 2048) || (2 * tiles <= cus && k >= 512))) return;
   long want = (2L * cus + tiles - 1) / tiles;
-  const long max_by_k = k / 256;  // at least 16 slabs per slice
+  long max_by_k = k / 256;  // at least 16 slabs per slice,
+  if (tiles * max_by_k < cus) max_by_k = k / 128;  // 8 when that leaves CUs without a block (512^3: 13.2 -> 10.1 us)
   if (want > max_by_k) want = max_by_k;
   if (want > 512) want = 512;  // want * tiles stays near 2 * cus, so the partials stay near 2 * cus tiles
   if (want <= 1) return;

@@ -320,7 +320,8 @@ def test_gemm_tile_choice(lib):
 
 def test_gemm_k_slicing(lib):
     """K is sliced when there are too few tiles for the chip: below one tile per CU from K = 1024 up, below
-    two tiles per CU from K = 2048 up; slices are multiples of the K slab (16) and at least 256 long."""
+    two tiles per CU from K = 2048 up, below half a tile per CU from K = 512 up; slices are multiples of the K slab (16)
+    and at least 256 long, or 128 where slices of 256 would leave CUs without a block."""
     def plan(m, n, k, cus=256):
         bm, bn, ks, kc = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
         lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(k), C.c_int(cus), C.byref(bm), C.byref(bn),
@@ -332,11 +333,13 @@ def test_gemm_k_slicing(lib):
     assert plan(1024, 1024, 1024) == (64, 64, 1, 1024)           # 256 tiles but K too short to pay for a second pass
     assert plan(64, 64, 100000)[2] == 368                        # one tile: as many slices of at least 256 as fit
     assert plan(32, 32, 1 << 20)[2] == 512                       # capped
-    bm, bn, ks, kc = plan(128, 128, 1000)
-    assert ks == 1 and kc == 1000
+    assert plan(128, 128, 400)[2:] == (1, 400)                   # K below 512 is never sliced
+    assert plan(128, 128, 1000)[2:] == (7, 144)                  # very few tiles: slices down to 128 (23 -> 9.6 us)
+    assert plan(512, 512, 512)[2:] == (4, 128)                   # 64 tiles: 13.2 -> 10.6 us
+    assert plan(256, 1024, 1024)[2:] == (4, 256)                 # 64 tiles, and slices of 256 already give every CU a block
     for k in (1024, 1040, 3000, 5555):
         _, _, ks, kc = plan(64, 64, k)
-        assert kc % 16 == 0 and (ks - 1) * kc < k <= ks * kc and (ks == 1 or kc >= 256)
+        assert kc % 16 == 0 and (ks - 1) * kc < k <= ks * kc and (ks == 1 or kc >= 128)
 
 
 def test_torch7_file_framing_known_bytes():
