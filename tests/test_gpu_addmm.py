@@ -219,8 +219,8 @@ def _odd_pitch(cl, arr, transposed):
     optionally stored transposed"""
     a = np.ascontiguousarray(arr.T if transposed else arr)
     big = np.zeros((a.shape[0], a.shape[1] + 3), F)
-    big[:, :a.shape[1]] = a
-    t = cl.ClTensor(big).narrow(2, 1, a.shape[1])
+    big[:, 1:1 + a.shape[1]] = a
+    t = cl.ClTensor(big).narrow(2, 2, a.shape[1])      # the first element sits 4 bytes into the storage
     return t.t() if transposed else t
 
 
