@@ -18,6 +18,10 @@
 
 namespace {
 
+// a 16-byte read that only needs the alignment of its elements (columns of a view start anywhere)
+typedef thcl_f4 rd_f4 __attribute__((aligned(4)));
+
+
 constexpr int kThreads = 256;
 constexpr int kWave = 64;
 
@@ -45,7 +49,8 @@ __device__ __forceinline__ void store_result(const GemvParams &P, thcl_u32 i, do
 // trans = 't': y[j] = alpha * dot(A[:, j], x) + beta * y[j].  Column j is m
 // contiguous floats; LPR lanes walk it (1, 8, 64 or a whole block).  blockIdx.y cuts
 // long columns into pieces of per_split elements (a multiple of 4) that leave partials.
-template <int LPR, bool VEC>
+// VEC 0: one element at a time (incx != 1); 1: units of four, m a multiple of 4; 2: units of four and the last m % 4
+template <int LPR, int VEC>
 __global__ __launch_bounds__(kThreads) void gemv_t(GemvParams P) {
   constexpr int COLS = kThreads / LPR;
   __shared__ double lds[kThreads / kWave];
@@ -56,8 +61,8 @@ __global__ __launch_bounds__(kThreads) void gemv_t(GemvParams P) {
   double acc = 0.0;
   if (j < P.n) {
     const float *col = P.a + (thcl_u64)j * P.lda + i0;
-    if (VEC) {  // m % 4 == 0, 16-byte aligned columns, incx == 1
-      const thcl_f4 *c4 = (const thcl_f4 *)col, *x4 = (const thcl_f4 *)(P.x + i0);
+    if (VEC) {  // incx == 1
+      const rd_f4 *c4 = (const rd_f4 *)col, *x4 = (const rd_f4 *)(P.x + i0);
       const thcl_u32 m4 = len >> 2;
       constexpr int FLY = 4;
       thcl_u32 i = sub;
@@ -95,6 +100,8 @@ __global__ __launch_bounds__(kThreads) void gemv_t(GemvParams P) {
 #pragma unroll
         for (int c = 0; c < 4; c++) acc += (double)v[c] * (double)w[c];
       }
+      if (VEC == 2)
+        for (thcl_u32 e = (m4 << 2) + sub; e < len; e += LPR) acc += (double)col[e] * (double)P.x[i0 + e];   // the last len % 4
     } else {
       for (thcl_u32 i = sub; i < len; i += LPR) acc += (double)col[i] * (double)P.x[(long)(i0 + i) * P.incx];
     }
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
         thcl_f4 v[FLY];
 #pragma unroll
         for (int f = 0; f < FLY; f++) {
-          v[f] = __builtin_nontemporal_load((const thcl_f4 *)ptr);
+          v[f] = __builtin_nontemporal_load((const rd_f4 *)ptr);
           xs[f] = P.x[(long)(j + f * JSTEP) * P.incx];
           ptr += step;
         }
@@ -174,7 +181,7 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
     for (; j < j1; j += JSTEP) {
       const double xj = (double)P.x[(long)j * P.incx];
       if (VEC == 4) {
-        const thcl_f4 v = *(const thcl_f4 *)ptr;
+        const thcl_f4 v = *(const rd_f4 *)ptr;
 #pragma unroll
         for (int c = 0; c < 4; c++) acc[c] += (double)v[c] * xj;
       } else {
@@ -342,9 +349,9 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
   P.per_split = (thcl_u32)(t ? m : n);
   P.outputs = (thcl_u32)outputs;
   const long cus = thcl_rt_get_props(rt)->compute_units;
-  const bool rows_aligned = aligned16(P.a) && (lda % 4 == 0) && (m % 4 == 0);
+  const bool rows_aligned = (m % 4 == 0);   // units of four rows; their 16-byte reads need no alignment
   if (t) {
-    const bool vec = rows_aligned && incx == 1 && aligned16(P.x);
+    const bool vec = incx == 1;
     // few long columns: cut them into pieces of at least 8192 elements until the chip is full
     if (m >= 2048 && n < cus * 4) {
       long split = (cus * 8 + n - 1) / n;
@@ -364,8 +371,9 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
 #define GEMV_T(L)                                                                                        \
   {                                                                                                      \
     const dim3 grid((unsigned)((n + (kThreads / L) - 1) / (kThreads / L)), P.split);                     \
-    if (vec) hipLaunchKernelGGL((gemv_t<L, true>), grid, dim3(kThreads), 0, stream, P);                  \
-    else hipLaunchKernelGGL((gemv_t<L, false>), grid, dim3(kThreads), 0, stream, P);                     \
+    if (vec && rows_aligned) hipLaunchKernelGGL((gemv_t<L, 1>), grid, dim3(kThreads), 0, stream, P);     \
+    else if (vec) hipLaunchKernelGGL((gemv_t<L, 2>), grid, dim3(kThreads), 0, stream, P);                \
+    else hipLaunchKernelGGL((gemv_t<L, 0>), grid, dim3(kThreads), 0, stream, P);                         \
   }
     // a whole block per column only while columns are few: with 2048 columns or more a wave per column
     // measured 3-5 % faster on columns of 4096 to 65536 elements (no barrier, no exchange through LDS)

@@ -22,6 +22,10 @@
 
 namespace {
 
+// a 16-byte read that only needs the alignment of its elements (rows of a view start anywhere)
+typedef thcl_f4 rd_f4 __attribute__((aligned(4)));
+
+
 constexpr int kThreads = 256;
 constexpr int kWave = 64;
 
@@ -373,11 +377,11 @@ __global__ __launch_bounds__(kThreads) void reduce_all_strided(ReduceAllParams P
       thcl_f4 v[FLY];
 #pragma unroll
       for (int k = 0; k < FLY; k++)
-        v[k] = __builtin_nontemporal_load((const thcl_f4 *)(P.in + thcl_generic_offset((thcl_u32)(i + k * all), P.L)));
+        v[k] = __builtin_nontemporal_load((const rd_f4 *)(P.in + thcl_generic_offset((thcl_u32)(i + k * all), P.L)));
 #pragma unroll
       for (int k = 0; k < FLY; k++) chain[k].take4(v[k], P.exponent);
     }
-    for (; i < P.n; i += all) chain[0].take4(*(const thcl_f4 *)(P.in + thcl_generic_offset((thcl_u32)i, P.L)), P.exponent);
+    for (; i < P.n; i += all) chain[0].take4(*(const rd_f4 *)(P.in + thcl_generic_offset((thcl_u32)i, P.L)), P.exponent);
     acc = chain[0].value();
 #pragma unroll
     for (int k = 1; k < FLY; k++) acc = Acc<KIND>::comb(acc, chain[k].value());
@@ -519,7 +523,7 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
     if (s < P.nslices) {
       const float *row = P.in + thcl_generic_offset(s, P.L) + r0;
       if (VEC == 4) {
-        const thcl_f4 *row4 = (const thcl_f4 *)row;
+        const rd_f4 *row4 = (const rd_f4 *)row;
         const thcl_u32 r4 = len >> 2;
         constexpr int FLY = 4;  // independent loads issued before any is consumed
         thcl_u32 i = sub;
@@ -595,7 +599,7 @@ __global__ __launch_bounds__(kThreads) void reduce_rows_short(ReduceDimParams P)
       // (a branch around a load makes the compiler wait for the loads before it)
       thcl_u32 s = (p0 + f) * rows + rib;
       if (s >= P.nslices) s = P.nslices - 1;
-      const thcl_f4 *row4 = (const thcl_f4 *)(P.in + thcl_generic_offset(s, P.L));
+      const rd_f4 *row4 = (const rd_f4 *)(P.in + thcl_generic_offset(s, P.L));
 #pragma unroll
       for (int k = 0; k < PER; k++) {
         thcl_u32 i = sub + (thcl_u32)k * lpr;
@@ -679,7 +683,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
           auto fetch = [&](thcl_f4 (&x)[FLY]) {
 #pragma unroll
             for (int f = 0; f < FLY; f++) {
-              x[f] = __builtin_nontemporal_load((const thcl_f4 *)ptr);
+              x[f] = __builtin_nontemporal_load((const rd_f4 *)ptr);
               ptr += step;
             }
           };
@@ -720,7 +724,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
       }
       for (; r < r_end; r += RSTEP) {
         if (VEC == 4) {
-          const thcl_f4 v0 = *(const thcl_f4 *)ptr;
+          const thcl_f4 v0 = *(const rd_f4 *)ptr;
 #pragma unroll
           for (int c = 0; c < 4; c++) acc[c] = S::take(acc[c], v0[c], (int)r, P.exponent);
         } else {
@@ -828,7 +832,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_short(ReduceDimParams P)
 #pragma unroll
       for (int f = 0; f < FLY; f++) {
         if (VEC == 4) {
-          const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(ptr + (thcl_u64)(r + f) * P.rstride));
+          const thcl_f4 v = __builtin_nontemporal_load((const rd_f4 *)(ptr + (thcl_u64)(r + f) * P.rstride));
 #pragma unroll
           for (int c = 0; c < VEC; c++) x[f][c] = v[c];
         } else {
@@ -842,7 +846,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_short(ReduceDimParams P)
     }
     for (; r < P.R; r++) {
       if (VEC == 4) {
-        const thcl_f4 v = *(const thcl_f4 *)(ptr + (thcl_u64)r * P.rstride);
+        const thcl_f4 v = *(const rd_f4 *)(ptr + (thcl_u64)r * P.rstride);
 #pragma unroll
         for (int c = 0; c < VEC; c++) acc[c] = S::take(acc[c], v[c], (int)r, P.exponent);
       } else {
@@ -1088,8 +1092,7 @@ void reduce_all_launch(thcl_rt *rt, ThclReduce kind, THClTensor *src, long n, fl
     THCL_CHECK(n < (1l << 31), THCL_DIM_WARNING);
     // units of four when every row of the innermost dim is a dense, 16-byte aligned run of a multiple of 4
     const int last = walk.dims - 1;
-    bool vec4 = walk.dims >= 1 && walk.strides[last] == 1 && walk.sizes[last] % 4 == 0 && aligned16(P.in);
-    for (int d = 0; d < last && vec4; d++) vec4 = walk.strides[d] % 4 == 0;
+    const bool vec4 = walk.dims >= 1 && walk.strides[last] == 1 && walk.sizes[last] % 4 == 0;   // the units' 16-byte reads need no alignment
     if (vec4) {
       walk.sizes[last] /= 4;
       walk.strides[last] = 4;
@@ -1257,8 +1260,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   if (rows) {
     // lanes per slice: a whole block for long slices, a thread for the shortest ones
     lpr = R >= 2048 ? 256 : (R >= 128 ? 64 : (R > 16 ? 8 : 1));
-    bool v4 = (R % 4 == 0) && aligned16(P.in);
-    for (int d = 0; d < L.dims && v4; d++) v4 = (L.strides[d] % 4 == 0) || L.sizes[d] == 1;
+    const bool v4 = (R % 4 == 0);   // 16-byte reads that need no alignment: a slice may start at any element
     vec = v4 ? 4 : 1;
     if (v4 && R <= 2048 && R > 1) {
       // short dense slices: enough lanes for one float4 each up to 256 elements, then 2, 4 or 8 float4 per lane
@@ -1295,8 +1297,7 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     }
   } else {
     const int last = L.dims - 1;
-    bool v4 = L.strides[last] == 1 && (L.sizes[last] % 4 == 0) && (src->stride[dim] % 4 == 0) && aligned16(P.in);
-    for (int d = 0; d < last && v4; d++) v4 = (L.strides[d] % 4 == 0);
+    const bool v4 = L.strides[last] == 1 && (L.sizes[last] % 4 == 0);   // units of 4 columns, read without alignment
     vec = v4 ? 4 : 1;
     if (v4) P.L.size[last] = thcl_make_divisor(L.sizes[last] / 4);
     P.nunits = (thcl_u32)(nslices / vec);
@@ -1314,7 +1315,9 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     // 256 bytes of a row, so those keep the full wave.
     unsigned ub_log2 = 6;
     while (ub_log2 > 0 && (1u << (ub_log2 - 1)) >= P.nunits) ub_log2--;
-    if (vec == 4) {
+    // (a run of 256 or 512 bytes that does not start on a 128-byte line touches one line more than it fills:
+    // rows whose pitch is no multiple of 128 bytes keep the full kibibyte)
+    if (vec == 4 && src->stride[dim] % 32 == 0 && aligned16(P.in)) {
       while (ub_log2 > 4 && ((long)P.nunits + (1l << ub_log2) - 1) >> ub_log2 < (long)cus &&
              R / ((kThreads / kWave) * (long)(kWave >> (ub_log2 - 1))) >= 16)
         ub_log2--;

@@ -107,6 +107,21 @@ def test_addmv_layouts(cl, rows, cols):
         _close(rr.dev.float(), cat.addmv(0.0, np.zeros(rows), 1.0, m, vv.view.gather()))
 
 
+@pytest.mark.parametrize("rows,cols,pitch,first", [(300, 256, 259, 1), (300, 255, 259, 2), (64, 4100, 4101, 1), (64, 4099, 4101, 0),
+                                                   (2000, 64, 67, 3), (2000, 61, 67, 3), (16, 30001, 30004, 1)])
+def test_addmv_on_rows_that_start_at_odd_elements(cl, rows, cols, pitch, first):
+    """A block cut out of a wider matrix, row- and column-major: lines that start at any element, of any length (units
+    of four read without alignment, then the last elements one by one)."""
+    big = oracle.normal(88, rows * pitch).reshape(rows, pitch)
+    m = big[:, first:first + cols]
+    v, t = oracle.normal(89, cols), oracle.normal(90, rows)
+    M = cl.ClTensor(big).narrow(2, first + 1, cols)
+    V, T = cl.ClTensor(v), cl.ClTensor(t)
+    _close(cl.ClTensor().addmv(0.5, T, 2.0, M, V).float(), cat.addmv(0.5, t, 2.0, m, v))
+    # the transposed product walks the same memory along the other dim
+    _close(cl.ClTensor().addmv(0.5, V, 2.0, M.t(), T).float(), cat.addmv(0.5, v, 2.0, np.ascontiguousarray(m.T), t))
+
+
 def test_addmv_beta_zero_ignores_old_contents_and_checks_shapes(cl):
     m = oracle.normal(78, 40 * 30).reshape(40, 30)
     v = oracle.normal(79, 30)

@@ -201,6 +201,21 @@ def test_reduce_dim_on_views_like_the_reference_tests(cl):
             _check_dim(cl, q, d)
 
 
+@pytest.mark.parametrize("rows,cols,pitch,first", [(300, 256, 259, 1), (300, 256, 260, 0), (257, 1024, 1027, 2), (64, 4100, 4101, 1),
+                                                   (2000, 64, 67, 3), (40, 20000, 20003, 1), (5000, 8, 11, 1)])
+def test_reduce_dim_on_rows_that_start_at_odd_elements(cl, rows, cols, pitch, first):
+    """A block cut out of a wider matrix: a multiple of 4 columns, but rows that start at element offsets which are no
+    multiple of 4, so the units of four are read with 16-byte loads that need no alignment.  Both dims, values and
+    positions, against the oracle."""
+    x = oracle.normal(19, rows * pitch).reshape(rows, pitch)
+    p = Pair.dense(cl, x).narrow(1, first, cols)
+    for d in (0, 1):
+        _check_dim(cl, p, d)
+    assert_bit_equal(np.float32(p.dev.max()), np.float32(p.view.gather().max()))
+    got, want = p.dev.sum(), float(p.view.gather().astype(np.float64).sum())
+    assert abs(got - want) <= 1e-5 * abs(want) + 1e-3
+
+
 def test_positions_ties_and_nans(cl):
     row = np.array([[1, 5, 5, 2, 5], [3, 3, 3, 3, 3]], dtype=F)
     R = cl.ClTensor(row)
