@@ -403,14 +403,13 @@ __global__ __launch_bounds__(kThreads) void reduce_all_strided(ReduceAllParams P
 }
 
 // sum of a[i] * b[i] over two dense arrays: products and the running sum in fp64
-template <bool VEC>
 __global__ __launch_bounds__(kThreads) void dot_dense(ReduceAllParams P, const float *other) {
   __shared__ double lds[kThreads / kWave];
   constexpr int U = 4;
   double acc[U] = {0.0, 0.0, 0.0, 0.0};
-  if (VEC) {
+  {
     const thcl_u64 n4 = P.n >> 2, tile = (thcl_u64)kThreads * U;
-    const thcl_f4 *a4 = (const thcl_f4 *)P.in, *b4 = (const thcl_f4 *)other;
+    const rd_f4 *a4 = (const rd_f4 *)P.in, *b4 = (const rd_f4 *)other;   // dense arrays that may start at any element
     thcl_u64 base = (thcl_u64)blockIdx.x * tile + threadIdx.x;
     // whole tiles: 2 * U loads issued back to back with nothing conditional between them
     for (; base + (U - 1) * kThreads < n4; base += (thcl_u64)gridDim.x * tile) {
@@ -432,9 +431,6 @@ __global__ __launch_bounds__(kThreads) void dot_dense(ReduceAllParams P, const f
     }
     if (blockIdx.x == 0)
       for (thcl_u64 i = (n4 << 2) + threadIdx.x; i < P.n; i += kThreads) acc[0] += (double)P.in[i] * (double)other[i];
-  } else {
-    for (thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x; i < P.n; i += (thcl_u64)gridDim.x * kThreads)
-      acc[0] += (double)P.in[i] * (double)other[i];
   }
   double v = (acc[0] + acc[1]) + (acc[2] + acc[3]);
   v = block_reduce<RED_SUM, double>(v, lds);
@@ -1157,16 +1153,15 @@ void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *
   P.ticket = (unsigned *)(sblock + kTicketOff);
   P.out = out;
   P.host_tag = host_tag;
-  const bool vec = aligned16(a) && aligned16(b);
-  const long want = vec ? (n / 4 + kThreads * 4 - 1) / (kThreads * 4) : (n + kThreads - 1) / kThreads;
+  // units of four, read with 16-byte loads that need no alignment (vectors starting at odd elements: 2.1 -> 6.5 TB/s)
+  const long want = (n / 4 + kThreads * 4 - 1) / (kThreads * 4);
   // one block per CU below 128 MiB of operands, two above (every block costs about 10 ns at the end)
   const long cus = thcl_rt_get_props(rt)->compute_units;
   long cap = cus * ((size_t)n * 2 * sizeof(float) >= (size_t)cus * 2 * 262144 ? 2 : 1);
   const long max_partials = (long)((sbytes - kPartialOff - kResultSlot) / sizeof(double));
   if (cap > max_partials) cap = max_partials;
   const unsigned grid = (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));
-  if (vec) hipLaunchKernelGGL(dot_dense<true>, dim3(grid), dim3(kThreads), 0, stream, P, b);
-  else hipLaunchKernelGGL(dot_dense<false>, dim3(grid), dim3(kThreads), 0, stream, P, b);
+  hipLaunchKernelGGL(dot_dense, dim3(grid), dim3(kThreads), 0, stream, P, b);
   check_launch("dot");
   thcl_after_launch(state, rt);
 }
