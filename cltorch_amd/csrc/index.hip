@@ -100,6 +100,76 @@ __global__ __launch_bounds__(kThreads) void index_move(IndexParams P) {
   }
 }
 
+// The same movement one element per lane (inner sizes that are no multiple of 4, or unaligned tensors), eight
+// elements per thread: the index entries, then the elements are all requested before the first is stored, since a
+// thread's chain of index, element and store would otherwise leave too little in flight (8192 x 8191 rows selected:
+// 2.4 TB/s with one element per thread).  Lanes past the end repeat the last element and store nothing.
+template <int MODE>
+__global__ __launch_bounds__(kThreads) void index_move_by_element(IndexParams P) {
+  constexpr int U = 8;
+  const thcl_u32 base = blockIdx.x * (kThreads * U) + threadIdx.x;
+  thcl_u64 aoff[U], boff[U];
+  bool ok[U];
+  long j[U];
+  thcl_u32 slice[U];
+  // a thread's elements are 256 apart, so most of them lie in the slice of the first: the position is split by
+  // division only where the inner index runs over
+  thcl_u32 ku_prev = 0, o_prev = 0, i_prev = 0;
+#pragma unroll
+  for (int k = 0; k < U; k++) {
+    const thcl_u32 e = base + k * kThreads, ec = e < P.total ? e : P.total - 1;
+    thcl_u32 ku, o, i;
+    if (k > 0 && e < P.total && ku_prev + kThreads < P.units_i.d) {
+      ku = ku_prev + kThreads;
+      o = o_prev;
+      i = i_prev;
+    } else {
+      const thcl_u32 q = thcl_div(ec, P.units_i);
+      ku = ec - q * P.units_i.d;
+      o = thcl_div(q, P.m);
+      i = q - o * P.m.d;
+    }
+    ku_prev = ku;
+    o_prev = o;
+    i_prev = i;
+    slice[k] = i;
+    j[k] = (long)P.index[i] - 1;
+    ok[k] = e < P.total;
+    boff[k] = ((thcl_u64)o * P.M + i) * P.I + ku;
+    aoff[k] = (thcl_u64)o * P.N * P.I + ku;   // the slice's part is added once its index is known
+    if (ku != 0 || o != 0) slice[k] |= 0x80000000u;   // only the first element of a slice reports a bad entry
+  }
+#pragma unroll
+  for (int k = 0; k < U; k++) {
+    const bool in = j[k] >= 0 && j[k] < (long)P.N;
+    if (!in && ok[k] && !(slice[k] & 0x80000000u)) *P.fault = 1u;
+    ok[k] = ok[k] && in;
+    aoff[k] += (thcl_u64)(in ? j[k] : 0) * P.I;
+  }
+  if (MODE == COPY) {
+    int w[U];
+#pragma unroll
+    for (int k = 0; k < U; k++) w[k] = P.winner[ok[k] ? j[k] : 0];
+#pragma unroll
+    for (int k = 0; k < U; k++) ok[k] = ok[k] && w[k] == (int)(slice[k] & 0x7fffffffu);
+  }
+  if (MODE == FILL) {
+#pragma unroll
+    for (int k = 0; k < U; k++)
+      if (ok[k]) P.a[aoff[k]] = P.value;
+    return;
+  }
+  float v[U];
+#pragma unroll
+  for (int k = 0; k < U; k++) v[k] = (MODE == SELECT) ? P.a[aoff[k]] : P.b[boff[k]];
+#pragma unroll
+  for (int k = 0; k < U; k++) {
+    if (!ok[k]) continue;
+    if (MODE == SELECT) P.b[boff[k]] = v[k];
+    else P.a[aoff[k]] = v[k];
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void fill_int(int *p, int v, thcl_u32 n) {
   const thcl_u32 i = blockIdx.x * kThreads + threadIdx.x;
   if (i < n) p[i] = v;
@@ -399,6 +469,8 @@ void launch_move(hipStream_t stream, IndexParams &P, bool vec_ok) {
   if (total == 0) return;
   const dim3 grid((unsigned)((total + kThreads - 1) / kThreads)), block(kThreads);
   if (vec) hipLaunchKernelGGL((index_move<MODE, 4>), grid, block, 0, stream, P);
+  else if constexpr (MODE == SELECT || MODE == COPY || MODE == FILL)
+    hipLaunchKernelGGL((index_move_by_element<MODE>), dim3((unsigned)((total + kThreads * 8 - 1) / (kThreads * 8))), block, 0, stream, P);
   else hipLaunchKernelGGL((index_move<MODE, 1>), grid, block, 0, stream, P);
   check("index kernel");
 }
