@@ -663,7 +663,10 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
           off += (thcl_u64)((d == P.L.dims - 1) ? r * VEC : r) * P.L.stride[d];
           i = q;
         }
-        off += (thcl_u64)((P.L.dims == 1) ? i * VEC : i) * P.L.stride[0];
+        // one inner dim of any length: the last unit is moved back to end with the dim, and gives some slices a
+        // second time, from the same rows in the same order
+        if (VEC > 1 && P.L.dims == 1 && i * VEC + VEC > P.nslices) off += (thcl_u64)(P.nslices - VEC) * P.L.stride[0];
+        else off += (thcl_u64)((P.L.dims == 1) ? i * VEC : i) * P.L.stride[0];
       }
       // this wave takes rows r_begin + wave, + WAVES, ...; FLY of them are loaded
       // before any is consumed, the address advances by a constant step
@@ -750,7 +753,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
       for (int c = 0; c < VEC; c++) {
         T r = lds[0][ul * VEC + c];
         for (int w = 1; w < WAVES; w++) r = S::comb(r, lds[w][ul * VEC + c]);
-        const thcl_u32 s = u * VEC + c;
+        const thcl_u32 s = ((VEC > 1 && P.L.dims == 1 && u * VEC + VEC > P.nslices) ? P.nslices - VEC : u * VEC) + c;
         if (P.split > 1) store_shared((T *)P.partials + (thcl_u64)blockIdx.y * P.nslices + s, r);
         else S::store(P, s, r);
       }
@@ -815,8 +818,10 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_short(ReduceDimParams P)
         off += (thcl_u64)((d == P.L.dims - 1) ? r * VEC : r) * P.L.stride[d];
         i = q;
       }
-      off += (thcl_u64)((P.L.dims == 1) ? i * VEC : i) * P.L.stride[0];
+      if (VEC > 1 && P.L.dims == 1 && i * VEC + VEC > P.nslices) off += (thcl_u64)(P.nslices - VEC) * P.L.stride[0];
+      else off += (thcl_u64)((P.L.dims == 1) ? i * VEC : i) * P.L.stride[0];
     }
+    const thcl_u32 s0 = (VEC > 1 && P.L.dims == 1 && u * VEC + VEC > P.nslices) ? P.nslices - VEC : u * VEC;
     const float *ptr = P.in + off;
     T acc[VEC];
 #pragma unroll
@@ -850,7 +855,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_short(ReduceDimParams P)
       }
     }
 #pragma unroll
-    for (int c = 0; c < VEC; c++) S::store(P, u * VEC + c, S::seal(acc[c], 0, P.R > 0));
+    for (int c = 0; c < VEC; c++) S::store(P, s0 + c, S::seal(acc[c], 0, P.R > 0));
   }
 }
 
@@ -1292,10 +1297,12 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     }
   } else {
     const int last = L.dims - 1;
-    const bool v4 = L.strides[last] == 1 && (L.sizes[last] % 4 == 0);   // units of 4 columns, read without alignment
+    // units of 4 columns, read without alignment; a single inner dim may have any length from 8 up (its last unit
+    // is moved back to end with it)
+    const bool v4 = L.strides[last] == 1 && (L.sizes[last] % 4 == 0 || (L.dims == 1 && L.sizes[last] >= 8));
     vec = v4 ? 4 : 1;
-    if (v4) P.L.size[last] = thcl_make_divisor(L.sizes[last] / 4);
-    P.nunits = (thcl_u32)(nslices / vec);
+    if (v4) P.L.size[last] = thcl_make_divisor((L.sizes[last] + 3) / 4);
+    P.nunits = (thcl_u32)((nslices + vec - 1) / vec);
     // a short reduced dim with enough slices to fill the chip: a thread per unit, no exchange
     if (R <= 32 && (long)P.nunits >= (long)cus * 1024) {
       lpr = -1;

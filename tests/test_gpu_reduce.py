@@ -216,6 +216,20 @@ def test_reduce_dim_on_rows_that_start_at_odd_elements(cl, rows, cols, pitch, fi
     assert abs(got - want) <= 1e-5 * abs(want) + 1e-3
 
 
+@pytest.mark.parametrize("shape", [(300, 9), (300, 13), (5000, 8191 // 7), (64, 4099), (2049, 255), (31, 70001), (20, 11), (40000, 10)])
+def test_reduce_dim_over_widths_that_are_no_multiple_of_four(cl, shape):
+    """Along dim 1 of a matrix whose width is no multiple of 4 the units of four columns still apply: the last unit is
+    moved back to end with the row and repeats up to three columns, bit for bit.  Values and positions, planted
+    ties in the repeated columns included."""
+    x = oracle.normal(23, int(np.prod(shape))).reshape(shape)
+    x[3, -2] = x[1, -2] = x[:, -2].max() + 1.0          # a tie in a column that two units cover
+    x[2, -1] = x[0, -1] = x[:, -1].min() - 1.0
+    p = Pair.dense(cl, x)
+    for d in (0, 1):
+        _check_dim(cl, p, d)
+    _check_dim(cl, p.narrow(1, 1, shape[1] - 2), 0)     # the same inside a wider matrix
+
+
 def test_positions_ties_and_nans(cl):
     row = np.array([[1, 5, 5, 2, 5], [3, 3, 3, 3, 3]], dtype=F)
     R = cl.ClTensor(row)
