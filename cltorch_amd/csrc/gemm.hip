@@ -105,9 +105,10 @@ struct EdgeLanes {
 // a load.
 // EDGE 2: any pitch and alignment, with 16-byte loads that need no alignment; a group that straddles the operand's
 // extent is read through a window moved back to end there and shifted into place on the way to LDS.  Needs at least
-// 4 elements along each operand's contiguous dimension.  EDGE 3: one element at a time, for what is left.  The choice is made at compile time: a run-time branch
-// between the two edge forms made the compiler wait for all loads at every slab (aligned 4096^3 through the edge
-// kernel: 101 TFLOP/s with the branch against 138 through the whole-tile kernel).
+// 4 elements along each operand's contiguous dimension.  EDGE 3: one element at a time, for what is left.
+// The choice is made at compile time: a run-time branch between two edge forms made the compiler wait for all loads
+// at every slab (aligned 4096^3 through the edge kernel: 101 TFLOP/s with the branch against 138 through the
+// whole-tile kernel).
 template <int BMN, bool KC, int EDGE>
 struct TileLoader {
   using LoadT = typename std::conditional<EDGE == 2, f4u, f4>::type;
@@ -153,8 +154,7 @@ struct TileLoader {
       }
     }
   }
-  // the whole-tile form of load(), for tiles and slabs that the caller knows to lie inside the operand (EDGE 1:
-  // aligned as well)
+  // plain loads, for tiles and slabs that the caller knows to lie inside the operand (EDGE 0 and 1: aligned as well)
   __device__ __forceinline__ void load_whole(const float *g, int ld, int mn0, int k0) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
