@@ -144,13 +144,16 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
   const thcl_u32 j0 = blockIdx.y * P.per_split;
   thcl_u32 j1 = j0 + P.per_split;
   if (j1 > P.n) j1 = P.n;
+  // m no multiple of VEC: the last unit is moved back to end with the column; it computes some rows a second time and
+  // stores only its own
+  const thcl_u32 row0 = (VEC > 1 && u * VEC + VEC > P.m) ? P.m - VEC : u * VEC;
   double acc[VEC];
 #pragma unroll
   for (int c = 0; c < VEC; c++) acc[c] = 0.0;
   if (u < units) {
     constexpr int FLY = 4;
     thcl_u32 j = j0 + wave * RL + rl;
-    const float *ptr = P.a + (thcl_u64)j * P.lda + (thcl_u64)u * VEC;
+    const float *ptr = P.a + (thcl_u64)j * P.lda + (thcl_u64)row0;
     const thcl_u64 step = (thcl_u64)JSTEP * P.lda;
     for (; j + (FLY - 1) * JSTEP < j1; j += FLY * JSTEP) {
       float xs[FLY];
@@ -205,8 +208,8 @@ __global__ __launch_bounds__(kThreads) void gemv_n(GemvParams P) {
     for (int c = 0; c < VEC; c++) {
       double r = lds[0][ul * VEC + c];
       for (int w = 1; w < WAVES; w++) r += lds[w][ul * VEC + c];
-      const thcl_u32 i = u * VEC + c;
-      if (i < P.m) {
+      const thcl_u32 i = row0 + c;
+      if (i >= u * VEC) {
         if (P.split > 1) P.partials[(thcl_u64)blockIdx.y * P.m + i] = r;
         else store_result(P, i, r);
       }
@@ -385,7 +388,7 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
       check("gemv finish");
     }
   } else {
-    const int vecw = rows_aligned ? 4 : 1;
+    const int vecw = m >= 4 ? 4 : 1;   // units of four rows, the last one moved back when m is no multiple of 4
     const long units = (m + vecw - 1) / vecw;
     // fewer units than lanes: the wave's spare lanes take further columns
     unsigned ub_log2 = 6;
