@@ -537,6 +537,8 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
 #pragma unroll
           for (int c = 0; c < 4; c++) acc = S::take(acc, v[c], (int)(r0 + i * 4 + c), P.exponent);
         }
+        if (len & 3u)   // the last one to three elements of a slice whose length is no multiple of 4
+          for (thcl_u32 e = (r4 << 2) + sub; e < len; e += LPR) acc = S::take(acc, row[e], (int)(r0 + e), P.exponent);
       } else {
         constexpr int FLY = 4;
         thcl_u32 i = sub;
@@ -550,7 +552,12 @@ __global__ __launch_bounds__(kThreads) void reduce_rows(ReduceDimParams P) {
         for (; i < len; i += LPR) acc = S::take(acc, row[i], (int)(r0 + i), P.exponent);
       }
       // the first position this thread met
-      acc = S::seal(acc, (int)(r0 + (VEC == 4 ? sub * 4 : sub)), (VEC == 4 ? (thcl_u32)sub < (len >> 2) : (thcl_u32)sub < len));
+      if (VEC == 4) {
+        const thcl_u32 r4 = len >> 2;
+        acc = S::seal(acc, (int)(r0 + ((thcl_u32)sub < r4 ? (thcl_u32)sub * 4 : (r4 << 2) + sub)), (thcl_u32)sub < r4 || (r4 << 2) + sub < len);
+      } else {
+        acc = S::seal(acc, (int)(r0 + sub), (thcl_u32)sub < len);
+      }
     }
     if (LPR <= kWave) {
       acc = S::reduce(acc, LPR);
@@ -1260,9 +1267,11 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
   if (rows) {
     // lanes per slice: a whole block for long slices, a thread for the shortest ones
     lpr = R >= 2048 ? 256 : (R >= 128 ? 64 : (R > 16 ? 8 : 1));
-    const bool v4 = (R % 4 == 0);   // 16-byte reads that need no alignment: a slice may start at any element
+    // 16-byte reads that need no alignment: a slice may start at any element, and from 64 elements up it may have any
+    // length (the last one to three elements are taken singly)
+    const bool v4 = (R % 4 == 0) || R >= 64;
     vec = v4 ? 4 : 1;
-    if (v4 && R <= 2048 && R > 1) {
+    if (v4 && R % 4 == 0 && R <= 2048 && R > 1) {
       // short dense slices: enough lanes for one float4 each up to 256 elements, then 2, 4 or 8 float4 per lane
       const long r4 = R / 4;
       unsigned l2 = 0;

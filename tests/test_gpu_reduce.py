@@ -230,6 +230,21 @@ def test_reduce_dim_over_widths_that_are_no_multiple_of_four(cl, shape):
     _check_dim(cl, p.narrow(1, 1, shape[1] - 2), 0)     # the same inside a wider matrix
 
 
+@pytest.mark.parametrize("shape", [(40, 65), (300, 131), (33, 4099), (7, 70001), (2, 300003), (5000, 67), (64, 1023), (3, 8191)])
+def test_reduce_dim_over_slices_whose_length_is_no_multiple_of_four(cl, shape):
+    """Along the dense dim, slices of 64 elements or more are walked in units of four whatever their length; the last
+    one to three elements are taken singly.  Extremes planted in those last elements and ties between them and the
+    units; long slices are cut over blocks."""
+    x = oracle.normal(29, int(np.prod(shape))).reshape(shape)
+    x[0, -1] = x[0].max() + 1.0                       # the maximum is the very last element
+    x[1, -2] = x[1, 3] = x[1].min() - 1.0             # a tie between a unit and the tail: the first position wins
+    if shape[0] > 2:
+        x[2, :] = x[2, 0]                             # every element equal: position 1
+    p = Pair.dense(cl, x)
+    _check_dim(cl, p, 1)
+    _check_dim(cl, p.narrow(1, 1, shape[1] - 1), 1)   # slices that start at odd elements of a wider matrix
+
+
 def test_positions_ties_and_nans(cl):
     row = np.array([[1, 5, 5, 2, 5], [3, 3, 3, 3, 3]], dtype=F)
     R = cl.ClTensor(row)
