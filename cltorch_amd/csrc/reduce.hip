@@ -1338,12 +1338,15 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     const long tiles = (P.nunits + ub - 1) / ub;
     // a block per CU: split the reduced dim when the tiles are fewer (every extra split is another partial per slice)
     long split = 1;
-    const long target = (long)cus;
+    // (two per CU for very tall slices walked one element per lane, which keep less in flight per wave:
+    // 2^24 x 3 along dim 1 3.7 -> 5.2 TB/s; with 16-byte units a second block per CU costs 10 %)
+    const bool more = vec == 1 && R >= (1l << 22);
+    const long target = (long)cus * (more ? 2 : 1);
     if (tiles < target) {
       split = (target + tiles - 1) / tiles;
       const long max_by_rows = (R + 32 * row_lanes - 1) / (32 * row_lanes);  // at least 32 rows per lane
       if (split > max_by_rows) split = max_by_rows;
-      if (split > 256) split = 256;
+      if (split > (more ? 512 : 256)) split = more ? 512 : 256;
       if (split * nslices > partial_cap) split = partial_cap / nslices;
       if (split < 1) split = 1;
     }
