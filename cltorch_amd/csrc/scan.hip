@@ -31,6 +31,10 @@
 
 namespace {
 
+// a 16-byte access that only needs the alignment of its elements (rows of odd length start anywhere)
+typedef thcl_f4 sc_f4u __attribute__((aligned(4)));
+
+
 constexpr int kThreads = 256;
 constexpr int kWave = 64;
 // Rows that are cut into segments go through in windows of this many input bytes: totals pass and scan pass of a
@@ -164,8 +168,11 @@ __device__ __forceinline__ double wave_inclusive(double v) {
 // 1024 elements; in each run a thread holds 4 consecutive elements (one 16-byte
 // access), so every wave reads whole lines, and the UNR runs share one pair of
 // barriers and keep UNR loads in flight per thread.
+// VEC: rows are 16-byte aligned and a multiple of 4 long; otherwise whole groups of 4 still move as 16 bytes, through
+// accesses that need no alignment, and only a row's last group goes element by element
 template <bool PROD, int PHASE, bool VEC>
 __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
+  typedef typename std::conditional<VEC, thcl_f4, sc_f4u>::type LT;
   constexpr int WAVES = kThreads / kWave, PER = 4, RUN = kThreads * PER, UNR = 4, STEP = RUN * UNR;
   __shared__ double wave_tot[UNR][WAVES];
   const thcl_u64 bid = P.block0 + blockIdx.x;
@@ -229,11 +236,11 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
         const double prev = __shfl_up(incl[u], 1, kWave);
         if (lane > 0) before = Op<PROD>::comb(before, prev);
         const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
-        if (VEC && (FULL || j + PER <= r1)) {
+        if (FULL || j + PER <= r1) {
           thcl_f4 v;
 #pragma unroll
           for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[u][c]);
-          __builtin_nontemporal_store(v, (thcl_f4 *)(orow + j));
+          __builtin_nontemporal_store(v, (LT *)(orow + j));
         } else {
 #pragma unroll
           for (int c = 0; c < PER; c++)
@@ -243,7 +250,7 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
     }
   };
   thcl_u64 base = r0;
-  if (VEC && base + STEP <= r1) {
+  if (base + STEP <= r1) {
     // Whole steps: the next step's loads are issued before this step's work and carry
     // no bounds tests, so they stay in flight across the step's two barriers.
     auto fetch = [&](float (&x)[UNR][PER], thcl_u64 at) {
@@ -251,7 +258,7 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
       for (int u = 0; u < UNR; u++) {
         // the totals pass reads with ordinary loads, which leave the window in the memory-side cache for the
         // scan pass that follows it; the scan pass streams
-        const thcl_f4 *src = (const thcl_f4 *)(row + at + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER);
+        const LT *src = (const LT *)(row + at + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER);
         const thcl_f4 v = PHASE == 0 ? *src : __builtin_nontemporal_load(src);
 #pragma unroll
         for (int c = 0; c < PER; c++) x[u][c] = v[c];
@@ -275,8 +282,8 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
 #pragma unroll
     for (int u = 0; u < UNR; u++) {
       const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
-      if (VEC && j + PER <= r1) {
-        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
+      if (j + PER <= r1) {
+        const thcl_f4 v = __builtin_nontemporal_load((const LT *)(row + j));
 #pragma unroll
         for (int c = 0; c < PER; c++) x[u][c] = v[c];
       } else {
@@ -451,6 +458,7 @@ __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
 // the prefix over a row's lanes is a shuffle scan of width G.
 template <bool PROD, int G, bool VEC>
 __global__ __launch_bounds__(kThreads) void scan_short_rows(ScanParams P) {
+  typedef typename std::conditional<VEC, thcl_f4, sc_f4u>::type LT;
   constexpr int PER = 4, ROWS = kThreads / G;
   const int sub = threadIdx.x % G;
   const thcl_u64 o = (thcl_u64)blockIdx.x * ROWS + threadIdx.x / G;
@@ -461,8 +469,8 @@ __global__ __launch_bounds__(kThreads) void scan_short_rows(ScanParams P) {
   for (thcl_u64 base = 0; base < P.R; base += G * PER) {
     const thcl_u64 j = base + (thcl_u64)sub * PER;
     float x[PER];
-    if (VEC && live && j + PER <= P.R) {
-      const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(row + j));
+    if (live && j + PER <= P.R) {
+      const thcl_f4 v = __builtin_nontemporal_load((const LT *)(row + j));
 #pragma unroll
       for (int c = 0; c < PER; c++) x[c] = v[c];
     } else {
@@ -488,11 +496,11 @@ __global__ __launch_bounds__(kThreads) void scan_short_rows(ScanParams P) {
       carry = Op<PROD>::comb(carry, incl);
     }
     if (live) {
-      if (VEC && j + PER <= P.R) {
+      if (j + PER <= P.R) {
         thcl_f4 v;
 #pragma unroll
         for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[c]);
-        __builtin_nontemporal_store(v, (thcl_f4 *)(orow + j));
+        __builtin_nontemporal_store(v, (LT *)(orow + j));
       } else {
 #pragma unroll
         for (int c = 0; c < PER; c++)
