@@ -432,8 +432,13 @@ def detail(cl, oracle, T, X, Y, Z, n):
         if unit == "TFLOP/s":
             # matrix products: clocks take some tens of ms of such work to settle after a wait or after work of another
             # kind (64x16384x4096 in a row: 96, 112, 94 us per call over the first 30 ms, 85 us from then on)
-            [fn() for _ in range(max(reps, min(1000, int(40.0 / max(float(pairs.mean()), 1e-3)))))]
-        T.timed(name, lambda: [fn() for _ in range(reps)])
+            for _ in range(max(reps, min(1000, int(40.0 / max(float(pairs.mean()), 1e-3))))):
+                fn()
+
+        def in_a_row():          # every result is dropped before the next call, as a caller's loop would
+            for _ in range(reps):
+                fn()
+        T.timed(name, in_a_row)
         cl.synchronize()
         b2b = T.collect()[name][0] / reps
         s = {"avg_ms": round(b2b, 4), "achieved": round(work / (b2b * 1e-3) * scale, 1), "unit": unit,
