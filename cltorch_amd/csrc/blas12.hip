@@ -352,7 +352,7 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
   P.per_split = (thcl_u32)(t ? m : n);
   P.outputs = (thcl_u32)outputs;
   const long cus = thcl_rt_get_props(rt)->compute_units;
-  const bool rows_aligned = (m % 4 == 0);   // units of four rows; their 16-byte reads need no alignment
+  const bool whole_units = (m % 4 == 0);   // units of four rows; their 16-byte reads need no alignment
   if (t) {
     const bool vec = incx == 1;
     // few long columns: cut them into pieces of at least 8192 elements until the chip is full
@@ -374,7 +374,7 @@ void THClBlas_gemv(THClState *state, char trans, long m, long n, float alpha, TH
 #define GEMV_T(L)                                                                                        \
   {                                                                                                      \
     const dim3 grid((unsigned)((n + (kThreads / L) - 1) / (kThreads / L)), P.split);                     \
-    if (vec && rows_aligned) hipLaunchKernelGGL((gemv_t<L, 1>), grid, dim3(kThreads), 0, stream, P);     \
+    if (vec && whole_units) hipLaunchKernelGGL((gemv_t<L, 1>), grid, dim3(kThreads), 0, stream, P);     \
     else if (vec) hipLaunchKernelGGL((gemv_t<L, 2>), grid, dim3(kThreads), 0, stream, P);                \
     else hipLaunchKernelGGL((gemv_t<L, 0>), grid, dim3(kThreads), 0, stream, P);                         \
   }
