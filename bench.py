@@ -391,11 +391,18 @@ def config_ops(cl, oracle, X, Y, Z, n):
     sq = tall.resize(8192, 8192).t()
     yield ("w_sumall_transposed_8192^2", lambda: res.sum(sq), 4 * (64 << 20), "GB/s", 20, H)
     del few, tall, sq
-    ra, rb, rc = cl.ClTensor(3000, 7000), cl.ClTensor(7000, 5000), cl.ClTensor(3000, 5000)
-    ra.fill(0.01)
-    rb.fill(0.02)
-    rc.fill(0.0)
+    # matrix products outside the configuration: random normal operands like config 5 (constant operands run faster)
+    def normal(r, c, k):
+        return cl.ClTensor((rs.standard_normal((r, c)) / np.sqrt(k)).astype(np.float32))
+    ra, rb, rc = normal(3000, 7000, 7000), normal(7000, 5000, 1), normal(3000, 5000, 1)
     yield ("w_addmm_3000x5000x7000", lambda: rc.addmm(0.0, 1.0, ra, rb), 2.0 * 3000 * 5000 * 7000, "TFLOP/s", 6, M)
+    del ra, rb, rc
+    # sizes that are no multiple of 4 (16-byte loads without alignment), and a result of 32 rows (128x32 tiles)
+    ra, rb, rc = normal(4095, 4095, 4095), normal(4095, 4095, 1), normal(4095, 4095, 1)
+    yield ("w_addmm_4095^3", lambda: rc.addmm(0.0, 1.0, ra, rb), 2.0 * 4095 ** 3, "TFLOP/s", 8, M)
+    del ra, rb, rc
+    ra, rb, rc = normal(32, 4096, 4096), normal(4096, 16384, 1), normal(32, 16384, 1)
+    yield ("w_addmm_32x16384x4096", lambda: rc.addmm(0.0, 1.0, ra, rb), 2.0 * 32 * 16384 * 4096, "TFLOP/s", 50, M)
     del ra, rb, rc
     # cubes between the two config-5 shapes: the block tile is picked per shape (whole rounds of tiles per CU)
     for side in (3072, 4608):
