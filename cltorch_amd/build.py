@@ -83,7 +83,7 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     vmap = os.path.join(OBJ, "exports.map")
     with open(vmap, "w") as f:
         f.write("{\n  global:\n" + "".join(f"    {n};\n" for n in names) + "  local:\n    *;\n};\n")
-    cmd = [hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", f"-Wl,--version-script={vmap}", "-o", LIB] + objs + ["-lhiprtc"]
+    cmd = [hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", f"-Wl,--version-script={vmap}", "-o", LIB] + objs + ["-lhiprtc", "-pthread"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"linking failed:\n{r.stdout}\n{r.stderr}")

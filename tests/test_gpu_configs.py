@@ -281,6 +281,39 @@ def test_released_blocks_are_reused_without_stalling_or_mixing_owners(cl):
     assert x.sum() == 2.0 * n
 
 
+@pytest.mark.parametrize("n", [(128 << 8) - 1, 128 << 8, (1 << 18) + 3, (2 << 18) + 1, (9 << 18) - 5, (33 << 18) + 12, (64 << 18), (70 << 18) + 7])
+def test_ordinary_host_memory_in_pieces(cl, n):
+    """From 128 KiB up, copies from and to ordinary host memory travel in pieces through page-locked buffers with host
+    threads copying beside the DMA: lengths on both sides of every piece boundary, both directions, into a fresh array
+    and into one that already holds something, float and double hosts, with kernels queued before and after."""
+    rng = np.random.RandomState(n % 1000)
+    a = rng.standard_normal(n).astype(F)
+    t = cl.ClTensor(a)                       # host -> device
+    t.mul(2.0)                               # queued behind the upload, ahead of the download
+    back = t.float()                         # device -> a new host array
+    assert_bit_equal(back, a * F(2.0))
+    into = np.full(n, -7.0, dtype=F)
+    import ctypes as C
+    from cltorch_amd.tensor import _call
+    lib = cl.state().lib
+    sz = (C.c_long * 1)(n)
+    ft = lib.THFloatTensor_newWithData(into.ctypes.data_as(C.c_void_p), n, 0, 1, sz, None)
+    try:
+        _call("THFloatTensor_copyCl", ft, t._h)
+        assert_bit_equal(into, a * F(2.0))
+        into[:] = (np.arange(n) % 977).astype(F)
+        _call("THClTensor_copyFloat", t._h, ft)          # and back up from the same array
+    finally:
+        lib.THFloatTensor_free(ft)
+    assert t.sum() == float(np.float32(float((np.arange(n) % 977).sum())))
+    if n <= (9 << 18):
+        d = rng.standard_normal(n)                       # a double host array goes through a float copy first
+        s = cl.ClStorage(n)
+        s.copy(d)
+        assert_bit_equal(s.to_host(), d.astype(F))
+        assert np.array_equal(s.to_host(np.float64), d.astype(F).astype(np.float64))
+
+
 def test_pinned_host_arrays(cl):
     """Page-locked host arrays: a round trip through a tensor is exact and views keep the allocation
     alive.  (Transfer rates are a measurement, not a parity property: bench.py reports them.)"""
