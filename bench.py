@@ -504,7 +504,7 @@ def detail(cl, oracle, T, X, Y, Z, n):
 
 
 def host_copy_rates(cl, n=1 << 26):
-    """Device-to-host copies of 256 MiB into page-locked and into ordinary host memory (best of 3)."""
+    """Copies of 256 MiB between a tensor and page-locked or ordinary host memory, both directions (best of 3)."""
     from cltorch_amd.tensor import _call
     lib = cl.state().lib
     t = cl.ClTensor(n)
@@ -518,8 +518,14 @@ def host_copy_rates(cl, n=1 << 26):
             t0 = time.perf_counter()
             _call("THFloatTensor_copyCl", ft, t._h)
             best = max(best, 4 * n / (time.perf_counter() - t0) * 1e-9)
-        lib.THFloatTensor_free(ft)
         rates["d2h_" + name] = round(best, 1)
+        best = 0.0
+        for _ in range(3):
+            t0 = time.perf_counter()
+            _call("THClTensor_copyFloat", t._h, ft)
+            best = max(best, 4 * n / (time.perf_counter() - t0) * 1e-9)
+        rates["h2d_" + name] = round(best, 1)
+        lib.THFloatTensor_free(ft)
     return rates
 
 
