@@ -45,6 +45,27 @@ long host_count(const HostTensor<T> *t) {
   return n;
 }
 
+template <class T> struct RtKind;
+template <> struct RtKind<unsigned char> { static constexpr int value = THCL_RT_U8; };
+template <> struct RtKind<char> { static constexpr int value = THCL_RT_I8; };
+template <> struct RtKind<short> { static constexpr int value = THCL_RT_I16; };
+template <> struct RtKind<int> { static constexpr int value = THCL_RT_I32; };
+template <> struct RtKind<long> { static constexpr int value = THCL_RT_I64; };
+template <> struct RtKind<double> { static constexpr int value = THCL_RT_F64; };
+
+// dense in logical order: large tensors of this kind are converted by the runtime's host threads on their way
+// through its page-locked buffers (2^26 doubles: 80 ms with the element-by-element walk below, one thread)
+constexpr long kConvertedFrom = 1l << 16;
+template <class T>
+bool host_dense(const HostTensor<T> *t) {
+  long z = 1;
+  for (int d = t->nDimension - 1; d >= 0; d--) {
+    if (t->size[d] != 1 && t->stride[d] != z) return false;
+    z *= t->size[d];
+  }
+  return true;
+}
+
 // calls f(i, offset) for every element in logical order
 template <class T, class F>
 void host_walk(const HostTensor<T> *t, long n, F f) {
@@ -69,6 +90,12 @@ void to_device(THClState *state, THClTensor *self, const void *src_) {
   const long n = THClTensor_nElement(state, self);
   THCL_ARGCHECK(n == host_count(src), 2, "sizes do not match");
   if (n == 0) return;
+  if (n >= kConvertedFrom && host_dense(src) && THClTensor_isContiguous(state, self)) {
+    thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, self));
+    THCL_CHECK(thcl_rt_copy_converted(rt, thcl_dptr(self), src->storage->data + src->storageOffset, (size_t)n, RtKind<T>::value, 1) == 0,
+               "%s", thcl_rt_error());
+    return;
+  }
   std::vector<float> f((size_t)n);
   host_walk(src, n, [&](long i, long off) { f[(size_t)i] = (float)src->storage->data[off]; });
   long sz[1] = {n};
@@ -89,6 +116,12 @@ void to_host(THClState *state, void *self_, THClTensor *src) {
   const long n = THClTensor_nElement(state, src);
   THCL_ARGCHECK(host_count(self) == n, 2, "sizes do not match");
   if (n == 0) return;
+  if (n >= kConvertedFrom && host_dense(self) && THClTensor_isContiguous(state, src)) {
+    thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, src));
+    THCL_CHECK(thcl_rt_copy_converted(rt, thcl_dptr(src), self->storage->data + self->storageOffset, (size_t)n, RtKind<T>::value, 0) == 0,
+               "%s", thcl_rt_error());
+    return;
+  }
   std::vector<float> f((size_t)n);
   long sz[1] = {n};
   THFloatTensor *ft = THFloatTensor_newWithData(f.data(), n, 0, 1, sz, nullptr);
@@ -179,6 +212,11 @@ THCL_HOST_TYPE(Double, double)
   void THClStorage_copy##Name(THClState *state, THClStorage *self, TH##Name##Storage *src) {               \
     THCL_GUARD_BEGIN                                                                                         \
     THCL_ARGCHECK(self->size == src->size, 2, "size does not match");                                        \
+    if (src->size >= kConvertedFrom) {                                                                       \
+      THCL_CHECK(thcl_rt_copy_converted(self->cl, self->wrapper, src->data, (size_t)src->size, RtKind<T>::value, 1) == 0, "%s", \
+                 thcl_rt_error());                                                                           \
+      return;                                                                                                \
+    }                                                                                                        \
     std::vector<float> f((size_t)src->size);                                                                 \
     for (long i = 0; i < src->size; i++) f[(size_t)i] = (float)src->data[i];                                 \
     if (src->size > 0) THClStorage_rawCopy(state, self, f.data());                                           \
@@ -187,6 +225,11 @@ THCL_HOST_TYPE(Double, double)
   void TH##Name##Storage_copyCl(THClState *state, TH##Name##Storage *self, THClStorage *src) {             \
     THCL_GUARD_BEGIN                                                                                         \
     THCL_ARGCHECK(self->size == src->size, 2, "size does not match");                                        \
+    if (src->size >= kConvertedFrom) {                                                                       \
+      THCL_CHECK(thcl_rt_copy_converted(src->cl, src->wrapper, self->data, (size_t)src->size, RtKind<T>::value, 0) == 0, "%s", \
+                 thcl_rt_error());                                                                           \
+      return;                                                                                                \
+    }                                                                                                        \
     std::vector<float> f((size_t)src->size);                                                                 \
     THFloatStorage fs;                                                                                       \
     memset(&fs, 0, sizeof(fs));                                                                              \

@@ -392,12 +392,30 @@ void THClTensor_copyFloat(THClState *state, THClTensor *self, THFloatTensor *src
   THCL_GUARD_END()
 }
 
+// a host LongTensor whose elements lie dense in logical order
+static constexpr long kLongConvertedFrom = 1l << 16;
+static bool long_dense(const THLongTensor *t) {
+  long z = 1;
+  for (int d = t->nDimension - 1; d >= 0; d--) {
+    if (t->size[d] != 1 && t->stride[d] != z) return false;
+    z *= t->size[d];
+  }
+  return true;
+}
+
 void THClTensor_copyLong(THClState *state, THClTensor *self, THLongTensor *src) {
   // everything comes down to a copy from floats (src/lib/THClTensorCopy.cpp:38-66)
   THCL_GUARD_BEGIN
   const long n = THClTensor_nElement(state, self);
   THCL_ARGCHECK(n == THLongTensor_nElement(src), 2, "sizes do not match");
   if (n == 0) return;
+  if (n >= kLongConvertedFrom && long_dense(src) && THClTensor_isContiguous(state, self)) {
+    // large and dense on both sides: converted by the runtime's host threads on the way through its buffers
+    thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, self));
+    THCL_CHECK(thcl_rt_copy_converted(rt, thcl_dptr(self), src->storage->data + src->storageOffset, (size_t)n, THCL_RT_I64, 1) == 0, "%s",
+               thcl_rt_error());
+    return;
+  }
   std::vector<float> f((size_t)n);
   long idx[THCL_MAX_DIMS] = {0};
   long off = src->storageOffset;
@@ -469,6 +487,12 @@ void THLongTensor_copyCl(THClState *state, THLongTensor *self, THClTensor *src) 
   const long n = THClTensor_nElement(state, src);
   THCL_ARGCHECK(THLongTensor_nElement(self) == n, 2, "sizes do not match");
   if (n == 0) return;
+  if (n >= kLongConvertedFrom && long_dense(self) && THClTensor_isContiguous(state, src)) {
+    thcl_rt *rt = thcl_ctx(state, THClTensor_getDevice(state, src));
+    THCL_CHECK(thcl_rt_copy_converted(rt, thcl_dptr(src), self->storage->data + self->storageOffset, (size_t)n, THCL_RT_I64, 0) == 0, "%s",
+               thcl_rt_error());
+    return;
+  }
   std::vector<float> f((size_t)n);
   long sz[THCL_MAX_DIMS];
   for (int d = 0; d < src->nDimension; d++) sz[d] = src->size[d];

@@ -11,6 +11,7 @@
 #include <chrono>
 #include <cstring>
 #include <condition_variable>
+#include <functional>
 #include <map>
 #include <unordered_map>
 #include <mutex>
@@ -266,6 +267,8 @@ void thcl_rt_memory_stats(thcl_rt *rt, size_t *live_bytes, size_t *cached_bytes,
   if (cache_hits) *cache_hits = rt->cache_hits;
 }
 
+static int check_fault(thcl_rt *rt);
+
 // ---- large copies from and to ordinary (pageable) host memory -------------------------------------------
 // The driver moves such memory through a staging area of its own, one thread copying: 256 MiB come back at
 // 10-18 GB/s and go out at 30, against 57 GB/s both ways for page-locked memory, and its time for 256 KiB to 1 MiB
@@ -285,19 +288,26 @@ class HostCopiers {
     static HostCopiers *pool = new HostCopiers();   // never destroyed: its threads sleep until the process ends
     return *pool;
   }
-  void copy(void *dst, const void *src, size_t bytes) {
-    if (bytes < (1u << 20)) {   // not worth waking anybody
-      memcpy(dst, src, bytes);
+  // f(first, last) over [0, n) cut into one range per thread (multiples of 1024)
+  void run(size_t n, const std::function<void(size_t, size_t)> &f) {
+    if (n < (1u << 18)) {   // not worth waking anybody
+      f(0, n);
       return;
     }
     std::unique_lock<std::mutex> lock(mu_);
-    dst_ = (char *)dst;
-    src_ = (const char *)src;
-    bytes_ = bytes;
+    n_ = n;
+    f_ = &f;
     pending_ = (int)threads_.size();
     generation_++;
     wake_.notify_all();
     done_.wait(lock, [this] { return pending_ == 0; });
+  }
+  void copy(void *dst, const void *src, size_t bytes) {
+    if (bytes < (1u << 20)) {
+      memcpy(dst, src, bytes);
+      return;
+    }
+    run(bytes, [&](size_t a, size_t b) { memcpy((char *)dst + a, (const char *)src + a, b - a); });
   }
 
  private:
@@ -310,20 +320,18 @@ class HostCopiers {
   void work(unsigned me, unsigned n) {
     unsigned seen = 0;
     for (;;) {
-      char *dst;
-      const char *src;
-      size_t bytes;
+      size_t count;
+      const std::function<void(size_t, size_t)> *f;
       {
         std::unique_lock<std::mutex> lock(mu_);
         wake_.wait(lock, [&] { return generation_ != seen; });
         seen = generation_;
-        dst = dst_;
-        src = src_;
-        bytes = bytes_;
+        count = n_;
+        f = f_;
       }
-      const size_t per = ((bytes + n - 1) / n + 4095) / 4096 * 4096;   // whole pages per thread
+      const size_t per = ((count + n - 1) / n + 4095) / 4096 * 4096;   // whole pages (of bytes) per thread
       const size_t from = (size_t)me * per;
-      if (from < bytes) memcpy(dst + from, src + from, bytes - from < per ? bytes - from : per);
+      if (from < count) (*f)(from, count - from < per ? count : from + per);
       {
         std::lock_guard<std::mutex> lock(mu_);
         if (--pending_ == 0) done_.notify_one();
@@ -333,9 +341,8 @@ class HostCopiers {
   std::mutex mu_;
   std::condition_variable wake_, done_;
   std::vector<std::thread> threads_;
-  char *dst_ = nullptr;
-  const char *src_ = nullptr;
-  size_t bytes_ = 0;
+  size_t n_ = 0;
+  const std::function<void(size_t, size_t)> *f_ = nullptr;
   unsigned generation_ = 0;
   int pending_ = 0;
 };
@@ -398,7 +405,73 @@ int staged_copy(thcl_rt *rt, char *dev, char *host, size_t bytes, bool to_device
   }
   return 0;
 }
+// host elements of another type <-> device floats, converted by the host threads on the way through the buffers
+extern "C++" {
+template <class T>
+int staged_convert(thcl_rt *rt, float *dev, T *host, size_t count, bool to_device) {
+  if (stage_ready(rt) != 0) return -1;
+  HostCopiers &copiers = HostCopiers::get();
+  size_t piece = (count / 4 + (1u << 18) - 1) >> 18 << 18;   // in elements: a quarter of the copy, 512 Ki to 4 Mi
+  if (piece < (1u << 19)) piece = 1u << 19;
+  if (piece > kStageBytes / sizeof(float)) piece = kStageBytes / sizeof(float);
+  const size_t pieces = (count + piece - 1) / piece;
+  auto len = [&](size_t c) { return c + 1 < pieces ? piece : count - c * piece; };
+  if (to_device) {
+    for (size_t c = 0; c < pieces; c++) {
+      const int b = (int)(c % kStages);
+      if (c >= (size_t)kStages) RT_CHECK(hipEventSynchronize(rt->stage_done[b]));
+      float *st = (float *)rt->stage[b];
+      const T *from = host + c * piece;
+      copiers.run(len(c), [&](size_t i0, size_t i1) {
+        for (size_t i = i0; i < i1; i++) st[i] = (float)from[i];
+      });
+      RT_CHECK(hipMemcpyAsync(dev + c * piece, st, len(c) * sizeof(float), hipMemcpyHostToDevice, rt->stream));
+      RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
+    }
+    RT_CHECK(hipStreamSynchronize(rt->stream));
+    return 0;
+  }
+  for (size_t c = 0; c < pieces && c < (size_t)kStages; c++) {
+    RT_CHECK(hipMemcpyAsync(rt->stage[c], dev + c * piece, len(c) * sizeof(float), hipMemcpyDeviceToHost, rt->stream));
+    RT_CHECK(hipEventRecord(rt->stage_done[c], rt->stream));
+  }
+  for (size_t c = 0; c < pieces; c++) {
+    const int b = (int)(c % kStages);
+    RT_CHECK(hipEventSynchronize(rt->stage_done[b]));
+    const float *st = (const float *)rt->stage[b];
+    T *to = host + c * piece;
+    copiers.run(len(c), [&](size_t i0, size_t i1) {
+      for (size_t i = i0; i < i1; i++) to[i] = (T)st[i];
+    });
+    const size_t next = c + kStages;
+    if (next < pieces) {
+      RT_CHECK(hipMemcpyAsync(rt->stage[b], dev + next * piece, len(next) * sizeof(float), hipMemcpyDeviceToHost, rt->stream));
+      RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
+    }
+  }
+  return 0;
+}
+}  // extern "C++"
 }  // namespace
+
+int thcl_rt_copy_converted(thcl_rt *rt, void *dev, void *host, size_t count, int kind, int to_device) {
+  if (!count) return 0;
+  DeviceGuard g(rt->device);
+  int rc;
+  switch (kind) {
+    case THCL_RT_U8: rc = staged_convert(rt, (float *)dev, (unsigned char *)host, count, to_device != 0); break;
+    case THCL_RT_I8: rc = staged_convert(rt, (float *)dev, (char *)host, count, to_device != 0); break;
+    case THCL_RT_I16: rc = staged_convert(rt, (float *)dev, (short *)host, count, to_device != 0); break;
+    case THCL_RT_I32: rc = staged_convert(rt, (float *)dev, (int *)host, count, to_device != 0); break;
+    case THCL_RT_I64: rc = staged_convert(rt, (float *)dev, (long *)host, count, to_device != 0); break;
+    case THCL_RT_F64: rc = staged_convert(rt, (float *)dev, (double *)host, count, to_device != 0); break;
+    default: g_err = "thcl_rt_copy_converted: unknown element kind"; return -1;
+  }
+  if (rc != 0) return rc;
+  if (to_device) return 0;
+  RT_CHECK(hipStreamSynchronize(rt->stream));
+  return check_fault(rt);
+}
 
 int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
   if (!bytes) return 0;

@@ -56,6 +56,10 @@ void thcl_rt_memory_stats(thcl_rt *rt, size_t *live_bytes, size_t *cached_bytes,
                           unsigned long long *cache_hits);
 int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
 int thcl_rt_memcpy_d2h(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
+/* `count` dense host elements of another type to or from device floats, converted by C casts on the way
+ * (to_device != 0: host -> device).  Returns when done. */
+enum { THCL_RT_U8 = 0, THCL_RT_I8 = 1, THCL_RT_I16 = 2, THCL_RT_I32 = 3, THCL_RT_I64 = 4, THCL_RT_F64 = 5 };
+int thcl_rt_copy_converted(thcl_rt *rt, void *dev, void *host, size_t count, int kind, int to_device);
 int thcl_rt_memcpy_d2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* queued            */
 
 /* queue */

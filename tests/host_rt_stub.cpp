@@ -83,6 +83,7 @@ void thcl_rt_memory_stats(thcl_rt *rt, size_t *live_bytes, size_t *cached_bytes,
 }
 int thcl_rt_memcpy_h2d(thcl_rt *, void *dst, const void *src, size_t bytes) { memcpy(dst, src, bytes); return 0; }
 int thcl_rt_memcpy_d2h(thcl_rt *, void *dst, const void *src, size_t bytes) { memcpy(dst, src, bytes); return 0; }
+int thcl_rt_copy_converted(thcl_rt *, void *, void *, size_t, int, int) { return -1; }
 int thcl_rt_memcpy_d2d(thcl_rt *, void *dst, const void *src, size_t bytes) { memmove(dst, src, bytes); return 0; }
 void *thcl_rt_stream(thcl_rt *) { return nullptr; }
 int thcl_rt_sync(thcl_rt *) { return 0; }

@@ -314,6 +314,37 @@ def test_ordinary_host_memory_in_pieces(cl, n):
         assert np.array_equal(s.to_host(np.float64), d.astype(F).astype(np.float64))
 
 
+@pytest.mark.parametrize("n", [(1 << 16) - 1, 1 << 16, (1 << 19) + 5, (3 << 20) + 1, (17 << 20) - 3])
+def test_host_arrays_of_other_element_types(cl, n):
+    """Dense host arrays of the six other element types: from 65536 elements up they are converted by host threads on
+    their way through the page-locked buffers; the values are those of a C cast to float and back, whichever way
+    they went.  Storages and LongTensors, lengths on both sides of the switch and of the piece boundaries."""
+    rng = np.random.RandomState(n % 997)
+    base = rng.standard_normal(n) * 90.0
+    for dt in (np.float64, np.int64, np.int32, np.int16, np.int8, np.uint8):
+        a = (np.abs(base) if dt == np.uint8 else base).astype(dt)
+        s = cl.ClStorage(n)
+        s.copy(a)
+        want = a.astype(F)
+        assert_bit_equal(s.to_host(), want)
+        assert np.array_equal(s.to_host(dt), want.astype(dt))
+    # LongTensor <-> ClTensor (the host form of index vectors)
+    from cltorch_amd.tensor import _call, _long_vector, _LongTensorStruct
+    import ctypes as C
+    lib = cl.state().lib
+    vals = (rng.randint(-10 ** 6, 10 ** 6, size=n)).astype(np.int64)
+    lt = _long_vector(vals)
+    t = cl.ClTensor(n)
+    _call("THClTensor_copyLong", t._h, lt)
+    assert_bit_equal(t.float(), vals.astype(F))
+    t.add(1.0)
+    _call("THLongTensor_copyCl", lt, t._h)
+    st = C.cast(lt, C.POINTER(_LongTensorStruct)).contents
+    got = np.ctypeslib.as_array(st.storage.contents.data, shape=(n,)).copy()
+    lib.THLongTensor_free(lt)
+    assert np.array_equal(got, (vals.astype(F) + F(1.0)).astype(np.int64))
+
+
 def test_pinned_host_arrays(cl):
     """Page-locked host arrays: a round trip through a tensor is exact and views keep the allocation
     alive.  (Transfer rates are a measurement, not a parity property: bench.py reports them.)"""
