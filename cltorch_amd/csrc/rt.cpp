@@ -294,6 +294,7 @@ class HostCopiers {
       f(0, n);
       return;
     }
+    std::lock_guard<std::mutex> one_caller(callers_);   // copies of two host threads take turns
     std::unique_lock<std::mutex> lock(mu_);
     n_ = n;
     f_ = &f;
@@ -338,7 +339,7 @@ class HostCopiers {
       }
     }
   }
-  std::mutex mu_;
+  std::mutex mu_, callers_;
   std::condition_variable wake_, done_;
   std::vector<std::thread> threads_;
   size_t n_ = 0;
