@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
+#include <pthread.h>
 #include <unistd.h>
 
 #include <cstdio>
@@ -285,8 +286,11 @@ constexpr size_t kStagedFrom = 128u << 10;   // below this the driver's own path
 class HostCopiers {
  public:
   static HostCopiers &get() {
-    static HostCopiers *pool = new HostCopiers();   // never destroyed: its threads sleep until the process ends
-    return *pool;
+    // never destroyed: its threads sleep until the process ends.  A forked child has none of them, so it starts over.
+    static std::once_flag at_fork;
+    std::call_once(at_fork, [] { pthread_atfork(nullptr, nullptr, [] { pool_ = nullptr; }); });
+    if (!pool_) pool_ = new HostCopiers();
+    return *pool_;
   }
   // f(first, last) over [0, n) cut into one range per thread (multiples of 1024)
   void run(size_t n, const std::function<void(size_t, size_t)> &f) {
@@ -339,6 +343,7 @@ class HostCopiers {
       }
     }
   }
+  static HostCopiers *pool_;
   std::mutex mu_, callers_;
   std::condition_variable wake_, done_;
   std::vector<std::thread> threads_;
@@ -347,6 +352,8 @@ class HostCopiers {
   unsigned generation_ = 0;
   int pending_ = 0;
 };
+
+HostCopiers *HostCopiers::pool_ = nullptr;
 
 // page-locked memory (this library's or anybody's) goes the direct way
 bool host_memory_is_pagelocked(const void *p) {
