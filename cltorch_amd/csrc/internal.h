@@ -131,6 +131,8 @@ enum ThclReduce : int {
 void thcl_dot_dense(THClState *state, thcl_rt *rt, const float *a, const float *b, long n, float *out, unsigned host_tag = 0);
 // queues a launch that hands the device scalar at `src` to the host through the tagged word pair
 void thcl_scalar_to_host(THClState *state, thcl_rt *rt, const float *src, unsigned host_tag);
+// n dense floats (at most the runtime's mailbox) to the mailbox, then the tagged pair
+void thcl_small_to_host(THClState *state, thcl_rt *rt, const float *src, long n, unsigned host_tag);
 void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *src, long dim);
 // host_tag != 0: `out` is the pinned word pair of thcl_rt_tagged_word_device, which receives {result, tag} in one store
 void thcl_reduce_all(THClState *state, ThclReduce kind, THClTensor *src, float *out, float exponent = 0.f, unsigned host_tag = 0);

@@ -462,7 +462,19 @@ void THFloatTensor_copyCl(THClState *state, THFloatTensor *self, THClTensor *src
   float *hdst = self->storage->data + self->storageOffset;
   std::vector<float> stage;
   if (!hdense) stage.resize((size_t)n);
-  int rc = thcl_rt_memcpy_d2h(rt, hdense ? hdst : stage.data(), thcl_dptr(srcc), (size_t)n * sizeof(float));
+  int rc;
+  size_t box_floats = 0;
+  const float *box = thcl_rt_mailbox_host(rt, &box_floats);
+  if ((size_t)n <= box_floats) {
+    // small: a kernel leaves it in page-locked memory and the host waits for its tag, not for the stream
+    const unsigned tag = thcl_rt_next_tag(rt);
+    thcl_small_to_host(state, rt, thcl_dptr(srcc), n, tag);
+    float unused;
+    rc = thcl_rt_await_tagged(rt, tag, &unused);
+    if (rc == 0) memcpy(hdense ? hdst : stage.data(), box, (size_t)n * sizeof(float));
+  } else {
+    rc = thcl_rt_memcpy_d2h(rt, hdense ? hdst : stage.data(), thcl_dptr(srcc), (size_t)n * sizeof(float));
+  }
   THClTensor_free(state, srcc);
   THCL_CHECK(rc == 0, "%s", thcl_rt_error());
   if (!hdense) {

@@ -60,6 +60,7 @@ struct thcl_rt_timer {
 namespace {
 constexpr int kMaxDevices = 64;
 constexpr size_t kScratchBytes = 8u << 20;
+constexpr size_t kMailboxFloats = 16384;   // behind the 64 pinned words: room for a small tensor on its way to the host
 thcl_rt *g_ctx[kMaxDevices] = {nullptr};
 std::mutex g_mu;
 thread_local std::string g_err;
@@ -135,7 +136,7 @@ thcl_rt *thcl_rt_get(int device) {
   }
   e = hipMalloc(&rt->scratch, kScratchBytes);
   if (e == hipSuccess) e = hipMemset(rt->scratch, 0, kScratchBytes);
-  if (e == hipSuccess) e = hipHostMalloc((void **)&rt->host_word, 64 * sizeof(float), hipHostMallocMapped);
+  if (e == hipSuccess) e = hipHostMalloc((void **)&rt->host_word, (64 + kMailboxFloats) * sizeof(float), hipHostMallocMapped);
   if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&rt->host_word_dev, rt->host_word, 0);
   if (e == hipSuccess) e = hipDeviceSynchronize();
   if (e != hipSuccess) {
@@ -280,7 +281,7 @@ static int check_fault(thcl_rt *rt);
 namespace {
 constexpr size_t kStageBytes = 16u << 20;
 constexpr int kStages = 3;
-constexpr size_t kStagedFrom = 128u << 10;   // below this the driver's own path is as quick (64 KiB: 35 us)
+constexpr size_t kStagedFrom = 2u << 10;   // (64 KiB up: 39 -> 18 us, 4 KiB: 18 -> 14 us; a few bytes stay with the driver)
 
 // a handful of threads that copy slices of one buffer side by side; made at the first large copy, then asleep
 class HostCopiers {
@@ -536,6 +537,11 @@ unsigned *thcl_rt_fault_word_device(thcl_rt *rt) { return (unsigned *)(rt->host_
 // scalar up as soon as it lands instead of waiting for the stream's completion signal.
 constexpr int kTaggedWord = 40;  // 8-byte aligned
 float *thcl_rt_tagged_word_device(thcl_rt *rt) { return rt->host_word_dev + kTaggedWord; }
+float *thcl_rt_mailbox_device(thcl_rt *rt) { return rt->host_word_dev + 64; }
+const float *thcl_rt_mailbox_host(thcl_rt *rt, size_t *floats) {
+  if (floats) *floats = kMailboxFloats;
+  return rt->host_word + 64;
+}
 unsigned thcl_rt_next_tag(thcl_rt *rt) {
   if (++rt->tag == 0u) ++rt->tag;
   return rt->tag;

@@ -89,6 +89,11 @@ unsigned *thcl_rt_fault_word_device(thcl_rt *rt);
  * kernel is unaffected: the stream stays in order.  The reference reads such scalars back with a blocking copy
  * (src/lib/THClTensorMath.cpp:346-368). */
 float *thcl_rt_tagged_word_device(thcl_rt *rt);
+/* Page-locked room behind those words for a small tensor on its way to the host: a kernel copies it there
+ * (thcl_rt_mailbox_device), then stores the tagged pair; the host awaits the tag and reads thcl_rt_mailbox_host
+ * (`floats` receives its size).  One copy at a time: the caller reads the mailbox before anything else uses it. */
+float *thcl_rt_mailbox_device(thcl_rt *rt);
+const float *thcl_rt_mailbox_host(thcl_rt *rt, size_t *floats);
 unsigned thcl_rt_next_tag(thcl_rt *rt);
 int thcl_rt_await_tagged(thcl_rt *rt, unsigned tag, float *value);
 

@@ -97,6 +97,8 @@ float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
 float *thcl_rt_host_word_device(thcl_rt *rt) { return rt->host_word; }
 unsigned *thcl_rt_fault_word_device(thcl_rt *rt) { return (unsigned *)rt->host_word + 32; }
 float *thcl_rt_tagged_word_device(thcl_rt *rt) { return rt->host_word + 40; }
+float *thcl_rt_mailbox_device(thcl_rt *rt) { return rt->host_word; }
+const float *thcl_rt_mailbox_host(thcl_rt *rt, size_t *floats) { if (floats) *floats = 0; return rt->host_word; }
 unsigned thcl_rt_next_tag(thcl_rt *) { return 1u; }
 int thcl_rt_await_tagged(thcl_rt *, unsigned, float *value) { *value = 0.f; return 0; }
 thcl_rt_timer *thcl_rt_timer_new(thcl_rt *) { return new thcl_rt_timer(); }

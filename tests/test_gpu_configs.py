@@ -281,9 +281,9 @@ def test_released_blocks_are_reused_without_stalling_or_mixing_owners(cl):
     assert x.sum() == 2.0 * n
 
 
-@pytest.mark.parametrize("n", [(128 << 8) - 1, 128 << 8, (1 << 18) + 3, (2 << 18) + 1, (9 << 18) - 5, (33 << 18) + 12, (64 << 18), (70 << 18) + 7])
+@pytest.mark.parametrize("n", [511, 512, 513, 16383, 16384, 16385, (128 << 8) - 1, 128 << 8, (1 << 18) + 3, (2 << 18) + 1, (9 << 18) - 5, (33 << 18) + 12, (64 << 18), (70 << 18) + 7])
 def test_ordinary_host_memory_in_pieces(cl, n):
-    """From 128 KiB up, copies from and to ordinary host memory travel in pieces through page-locked buffers with host
+    """From 2 KiB up, copies from and to ordinary host memory travel in pieces through page-locked buffers with host
     threads copying beside the DMA: lengths on both sides of every piece boundary, both directions, into a fresh array
     and into one that already holds something, float and double hosts, with kernels queued before and after."""
     rng = np.random.RandomState(n % 1000)
