@@ -98,8 +98,8 @@ unsigned thcl_rt_next_tag(thcl_rt *rt);
 int thcl_rt_await_tagged(thcl_rt *rt, unsigned tag, float *value);
 
 /* Page-locked host memory for callers that stage their own transfers: copies between a
- * tensor and such a buffer run at the link's rate (57 GB/s measured on MI355X, against
- * 30 GB/s in and 17 GB/s out for pageable memory).  The reference keeps its host mirrors
+ * tensor and such a buffer run at the link's rate (57 GB/s measured on MI355X; ordinary memory,
+ * which the runtime moves through page-locked buffers of its own, gets 41-52).  The reference keeps its host mirrors
  * in ordinary memory (src/lib/THClStorage.cpp:112-140); this has no counterpart there. */
 void *thcl_rt_host_alloc(size_t bytes);
 int thcl_rt_host_free(void *ptr);
