@@ -50,6 +50,11 @@ struct thcl_rt {
   // page-locked staging buffers of the large copies from and to ordinary host memory (made at the first such copy)
   void *stage[3] = {nullptr, nullptr, nullptr};
   hipEvent_t stage_done[3] = {nullptr, nullptr, nullptr};
+  // small uploads leave through a ring of page-locked slots and do not wait for their DMA
+  char *ring = nullptr;
+  hipEvent_t ring_done[16] = {};
+  unsigned ring_next = 0;
+  bool ring_used[16] = {};
 };
 
 struct thcl_rt_timer {
@@ -172,6 +177,9 @@ void thcl_rt_release_all(void) {
       if (rt->stage[i]) (void)hipHostFree(rt->stage[i]);
       if (rt->stage_done[i]) (void)hipEventDestroy(rt->stage_done[i]);
     }
+    if (rt->ring) (void)hipHostFree(rt->ring);
+    for (auto &e : rt->ring_done)
+      if (e) (void)hipEventDestroy(e);
     (void)hipStreamDestroy(rt->stream);
     delete rt;
     g_ctx[d] = nullptr;
@@ -482,9 +490,32 @@ int thcl_rt_copy_converted(thcl_rt *rt, void *dev, void *host, size_t count, int
   return check_fault(rt);
 }
 
+// Uploads of up to 64 KiB: the bytes are copied into the next of 16 page-locked slots and their DMA is queued on the
+// stream; the call returns without waiting for it (the caller's memory is free again, and whatever uses the
+// destination is queued behind the DMA).  A slot is waited for only when the ring comes round to it while its DMA is
+// still pending.  4 KiB: 14 us with the wait, 5 us without.
+constexpr size_t kRingSlot = 64u << 10;
+constexpr unsigned kRingSlots = 16;
+static int ring_upload(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
+  if (!rt->ring) {
+    RT_CHECK(hipHostMalloc((void **)&rt->ring, kRingSlot * kRingSlots, hipHostMallocDefault));
+    for (unsigned i = 0; i < kRingSlots; i++) RT_CHECK(hipEventCreateWithFlags(&rt->ring_done[i], hipEventDisableTiming));
+  }
+  const unsigned slot = rt->ring_next;
+  rt->ring_next = (slot + 1) % kRingSlots;
+  if (rt->ring_used[slot]) RT_CHECK(hipEventSynchronize(rt->ring_done[slot]));
+  rt->ring_used[slot] = true;
+  char *at = rt->ring + (size_t)slot * kRingSlot;
+  memcpy(at, src, bytes);
+  RT_CHECK(hipMemcpyAsync(dst, at, bytes, hipMemcpyHostToDevice, rt->stream));
+  RT_CHECK(hipEventRecord(rt->ring_done[slot], rt->stream));
+  return 0;
+}
+
 int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
   if (!bytes) return 0;
   DeviceGuard g(rt->device);
+  if (bytes <= kRingSlot) return ring_upload(rt, dst, src, bytes);
   if (bytes >= kStagedFrom && !host_memory_is_pagelocked(src)) return staged_copy(rt, (char *)dst, (char *)src, bytes, true);
   RT_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, rt->stream));
   RT_CHECK(hipStreamSynchronize(rt->stream));

@@ -54,7 +54,8 @@ int thcl_rt_free(thcl_rt *rt, void *dptr);
 int thcl_rt_empty_cache(thcl_rt *rt);
 void thcl_rt_memory_stats(thcl_rt *rt, size_t *live_bytes, size_t *cached_bytes, unsigned long long *device_mallocs,
                           unsigned long long *cache_hits);
-int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
+int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when `src` may be reused;
+                                                                                 * the stream sees the bytes in order */
 int thcl_rt_memcpy_d2h(thcl_rt *rt, void *dst, const void *src, size_t bytes); /* returns when done */
 /* `count` dense host elements of another type to or from device floats, converted by C casts on the way
  * (to_device != 0: host -> device).  Returns when done. */
