@@ -447,6 +447,264 @@ __global__ __launch_bounds__(256) void scale_result(GemmParams P) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Products with one short side (n <= 64 here, i.e. a row-major result of at most 64 rows) and a long operand that
+// is contiguous along m.  The tiled kernel above spends a third of such a product between its multiply phases (LDS
+// store, barrier, fragment reads of both operands every 16 k) and needs a second kernel to add its K slices.  Here
+// the long operand never touches LDS: a lane loads four adjacent m-values of one k row straight into registers,
+// lanes 0-31 from row k and lanes 32-63 from row k + 1, which is the layout the MFMA wants for its second operand
+// when value c of the load is fed to the MFMA that computes result columns 4 j + c.  The MFMA computes the result
+// transposed (rows = the short side), so a lane ends up with four adjacent m-values of one n: 16-byte stores.
+//   A block of four waves (one per SIMD: the accumulators alone take 128 registers) owns 128 values of m; the
+//   waves split the block's K range between them, each streaming its own rows, and meet once at the end, where
+//   their accumulators are added through LDS in wave order.  The grid slices K as well (blockIdx.y) until about
+//   every CU has a block.  Two slices are folded in the same launch: a block writes its sums through to device
+//   scope, waits for the stores' acknowledgement and takes a ticket of its column block; the second arrival adds
+//   the first one's sums to its own (the sum of two numbers does not depend on their order, so a product gives
+//   the same bits every time) and writes the result.  More slices go to `work` and are added in slice order by
+//   splitk_reduce.
+//   The short operand passes through LDS in chunks of 32 k, each wave staging the rows of its own K range in a
+//   buffer of its own: there is no barrier inside the K loop.  Rows n..63 of a chunk hold whatever the clamped
+//   loads delivered: they only reach accumulator rows that are never stored.
+//   A wave requests the long operand 16 k-pairs (one chunk) ahead through a ring of registers whose slots are
+//   fixed at compile time: the refills of a chunk all belong to the next chunk, so they share one scalar base and
+//   each slot keeps its own constant 32-bit offset (no address arithmetic in the loop: every vector instruction
+//   beside an MFMA costs the matrix pipe about six cycles).
+// Needs: k even (a multiple of 4 when the short operand is contiguous along k), m a multiple of 4, the long
+// operand, the result and the workspace 16-byte aligned with leading dimensions that are multiples of 4; the short
+// operand in whole aligned 16-byte groups along its contiguous dim; lda < 2^24 and the short operand below 4 GiB.
+constexpr int ST_CW = 128;      // values of m per block
+constexpr int ST_WAVES = 4;
+constexpr int ST_CK = 32;       // k per staged chunk of the short operand
+constexpr int ST_PAIRS = ST_CK / 2;   // k-pairs per chunk = pairs of the long operand in flight per wave
+
+struct StreamFold {
+  unsigned *ticket;   // one arrival counter per column block, zero between launches; null: no fold in the launch
+};
+
+__device__ __forceinline__ void st_store_shared(float *p, f4 v) {   // through to device scope, 8 bytes at a time
+  unsigned long long lo = (unsigned long long)__float_as_uint(v[0]) | ((unsigned long long)__float_as_uint(v[1]) << 32);
+  unsigned long long hi = (unsigned long long)__float_as_uint(v[2]) | ((unsigned long long)__float_as_uint(v[3]) << 32);
+  __hip_atomic_store((unsigned long long *)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((unsigned long long *)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f4 st_load_fresh(const float *p) {       // past the caches
+  const unsigned long long lo = __atomic_load_n((const unsigned long long *)p, __ATOMIC_RELAXED);
+  const unsigned long long hi = __atomic_load_n((const unsigned long long *)p + 1, __ATOMIC_RELAXED);
+  return f4{__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)), __uint_as_float((unsigned)hi),
+            __uint_as_float((unsigned)(hi >> 32))};
+}
+
+template <int NT, bool SKC>
+__global__ __launch_bounds__(64 * ST_WAVES) void sgemm_stream(GemmParams P, StreamFold F) {
+  constexpr int VW = ST_CW / 32;          // m-values per lane and load
+  constexpr int SP = 32 * NT;             // n-values held per k row in LDS
+  constexpr int PAIRS = ST_PAIRS;
+  constexpr int SV = ST_CK * SP / 4 / 64; // 16-byte groups of a chunk per lane
+  constexpr int STAGE = ST_WAVES * ST_CK * SP, RED = ST_WAVES * SP * ST_CW;
+  typedef float VT __attribute__((ext_vector_type(VW)));
+  __shared__ __attribute__((aligned(16))) float lds[STAGE > RED ? STAGE : RED];
+  __shared__ unsigned s_last;
+
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same for the whole wave: what follows from it stays in scalar registers
+  const int kb = blockIdx.y * P.kchunk;
+  const int ke = (kb + P.kchunk < P.k) ? (kb + P.kchunk) : P.k;
+  // the wave's own K range: a multiple of the chunk, the last one takes what is left
+  const int kw = ((ke - kb + ST_WAVES - 1) / ST_WAVES + ST_CK - 1) / ST_CK * ST_CK;
+  const int k_begin = (kb + wave * kw < ke) ? kb + wave * kw : ke;
+  const int k_end = (k_begin + kw < ke) ? k_begin + kw : ke;
+  const int np = (k_end - k_begin) >> 1;           // k-pairs of this wave
+  const int nchunks = (np + PAIRS - 1) / PAIRS;
+  const int k_first = np > 0 ? k_begin : ke - 2;   // a wave without work still issues its first loads, from the last rows
+
+  const int col = blockIdx.x * ST_CW + VW * l32;
+  const int col_c = col + VW <= P.m ? col : P.m - VW;     // m is a multiple of VW: a lane's group is inside or outside
+  // long operand: a uniform row base per chunk + the slot's constant byte offset (row parity, column, pair)
+  const unsigned pair_bytes = 8u * (unsigned)P.lda;
+  unsigned a_off[PAIRS];
+#pragma unroll
+  for (int i = 0; i < PAIRS; i++) a_off[i] = ((unsigned)h * (unsigned)P.lda + (unsigned)col_c) * 4u + (unsigned)i * pair_bytes;
+  const unsigned lastp = np > 0 ? (unsigned)(np - 1) : 0u;
+  // pair p of the wave's range, or the last one beyond it
+  auto a_fetch_any = [&](unsigned p) {
+    const char *rows = (const char *)(P.a + (size_t)k_first * P.lda) + (unsigned long long)(p < lastp ? p : lastp) * pair_bytes;
+    return __builtin_nontemporal_load((const VT *)(rows + a_off[0]));
+  };
+
+  f16v acc[NT][VW];
+#pragma unroll
+  for (int t = 0; t < NT; t++)
+#pragma unroll
+    for (int c = 0; c < VW; c++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[t][c][r] = 0.f;
+
+  // The short operand's chunk `ch` of this wave's range into registers.  Group i of lane l: rows of n (SKC false):
+  // k row l / (SP/4) + (256/SP) i, group l % (SP/4); rows of k (SKC true): n = l % SP, k group l / SP + (64/SP) i.
+  // Either way the lane's part of the address never changes and the rest is the same for the whole wave.
+  // whole: the chunk lies inside the wave's range; else rows past its end are clamped to the last one.
+  float *stage = lds + wave * (ST_CK * SP);
+  f4 sreg[SV];
+  const int s_row = SKC ? lane / SP : lane / (SP / 4), s_col = SKC ? lane % SP : lane % (SP / 4);
+  const unsigned s_lane = SKC ? ((unsigned)(s_col < P.n ? s_col : P.n - 1) * (unsigned)P.ldb + 4u * s_row) * 4u
+                              : ((unsigned)s_row * (unsigned)P.ldb + (4 * s_col < P.n ? 4u * s_col : 0u)) * 4u;
+  const int s_last_row = np > 0 ? k_end : ke;   // rows below this exist
+  auto s_fetch = [&](auto whole, int ch) {
+    const int k0 = k_first + ch * ST_CK;
+#pragma unroll
+    for (int i = 0; i < SV; i++) {
+      const int kofs = SKC ? 4 * (64 / SP) * i : (256 / SP) * i;   // uniform part of the group's k
+      const char *base = (const char *)(SKC ? P.b + (k0 + kofs) : P.b + (size_t)(k0 + kofs) * P.ldb);
+      if constexpr (decltype(whole)::value) {
+        sreg[i] = *(const f4 *)(base + s_lane);
+      } else {
+        const int kk = k0 + kofs + (SKC ? 4 * s_row : s_row);
+        const int kc = SKC ? (kk + 4 <= s_last_row ? kk : s_last_row - 4) : (kk < s_last_row ? kk : s_last_row - 1);
+        const int back = kk - kc;      // rows (or k) the lane's own part overshoots by
+        sreg[i] = *(const f4 *)(base + s_lane - (size_t)back * (SKC ? 4u : 4u * (unsigned)P.ldb));
+      }
+    }
+  };
+  auto s_store = [&](float *buf) {
+#pragma unroll
+    for (int i = 0; i < SV; i++) {
+      if (SKC) {
+        const int kq = s_row + (64 / SP) * i;
+#pragma unroll
+        for (int c = 0; c < 4; c++) buf[(4 * kq + c) * SP + s_col] = sreg[i][c];
+      } else {
+        const int row = s_row + (256 / SP) * i;
+        *(f4 *)(buf + row * SP + 4 * s_col) = sreg[i];
+      }
+    }
+  };
+
+  VT ring[PAIRS];
+  s_fetch(std::false_type{}, 0);
+  // the ring fills in slot order: the wait counts the compiler derives for the loop below follow the later of the
+  // positions a slot's load has here and in the loop, so a reordered fill would make the loop wait for loads it
+  // does not need yet
+#pragma unroll
+  for (int i = 0; i < PAIRS; i++) {
+    __builtin_amdgcn_sched_barrier(0);
+    ring[i] = a_fetch_any((unsigned)i);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  s_store(stage);
+
+  // One step: the short operand's fragments of the next two pairs are requested from LDS, each pair's MFMAs run and
+  // the ring slot they emptied is refilled with the same pair of the next chunk.  The scheduling barrier keeps
+  // that order: left alone the compiler gathers the refills into batches at the end of the chunk, where they no
+  // longer run a chunk ahead.  The staging buffer is the wave's own and LDS serves a wave's accesses in order, so
+  // one buffer is enough: in front of a chunk's last pair, whose fragments are already in registers, the next
+  // chunk replaces it and its first fragments are requested, all behind that pair's MFMAs.
+  // MFMA tile t takes the rows n = NT * i + t of the short side (i = the MFMA's own row index), so that a lane's
+  // NT fragments of one k are neighbours in LDS and arrive with one read; two pairs are requested per step.
+  typedef float FT __attribute__((ext_vector_type(NT)));
+  const float *S = stage + h * SP + NT * l32;
+  FT fa[2], fn[2];
+  fa[0] = *(const FT *)S;
+  fa[1] = *(const FT *)(S + 2 * SP);
+  auto chunk = [&](auto full, auto next_whole, int ch) {
+    const int p0 = ch * PAIRS;
+    s_fetch(next_whole, ch + 1 < nchunks ? ch + 1 : ch);
+    const char *next_rows = (const char *)(P.a + (size_t)(k_first + 2 * (p0 + PAIRS)) * P.lda);   // used when the next chunk is whole
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int pp = 0; pp < PAIRS; pp += 2) {
+      if (pp + 2 == PAIRS) s_store(stage);
+      fn[0] = *(const FT *)(S + (pp + 2 < PAIRS ? 2 * (pp + 2) * SP : 0));
+      fn[1] = *(const FT *)(S + (pp + 2 < PAIRS ? 2 * (pp + 3) * SP : 2 * SP));
+#pragma unroll
+      for (int q = 0; q < 2; q++) {
+        // a range's last chunk may be short (the test is the same for the whole wave); the loads go on regardless
+        if (decltype(full)::value || p0 + pp + q < np) {
+          const VT v = ring[pp + q];
+#pragma unroll
+          for (int c = 0; c < VW; c++)
+#pragma unroll
+            for (int t = 0; t < NT; t++) acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[q][t], v[c], acc[t][c], 0, 0, 0);
+        }
+        if constexpr (decltype(next_whole)::value) ring[pp + q] = __builtin_nontemporal_load((const VT *)(next_rows + a_off[pp + q]));
+        else ring[pp + q] = a_fetch_any((unsigned)(p0 + pp + q + PAIRS));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      fa[0] = fn[0];
+      fa[1] = fn[1];
+    }
+  };
+  // chunks whose successor is whole as well run the plain loads; the range's last two the clamped ones
+  const int nfull = np / PAIRS;
+  int ch = 0;
+  for (; ch + 2 < nchunks; ch++) chunk(std::true_type{}, std::true_type{}, ch);
+  for (; ch < nfull; ch++) chunk(std::true_type{}, std::false_type{}, ch);
+  if (ch < nchunks) chunk(std::false_type{}, std::false_type{}, ch);
+
+  // acc[t][c][r] = C[m = col + c][n = NT (8 (r / 4) + 4 h + r % 4) + t]: the waves' parts meet in LDS as
+  // [wave][n][m] and are added in wave order
+  __syncthreads();
+  float *red = lds + wave * (SP * ST_CW);
+#pragma unroll
+  for (int t = 0; t < NT; t++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int nn = NT * (8 * (r / 4) + 4 * h + r % 4) + t;
+      VT v;
+#pragma unroll
+      for (int c = 0; c < VW; c++) v[c] = acc[t][c][r];
+      *(VT *)(red + nn * ST_CW + VW * l32) = v;
+    }
+  __syncthreads();
+  constexpr int GROUPS = SP * ST_CW / 4 / (64 * ST_WAVES);   // 16-byte groups of the block's result per thread
+  f4 sum[GROUPS];
+#pragma unroll
+  for (int i = 0; i < GROUPS; i++) {
+    const int g = tid + 64 * ST_WAVES * i;
+    const int nn = g / (ST_CW / 4), c4 = g % (ST_CW / 4);
+    sum[i] = *(const f4 *)(lds + nn * ST_CW + 4 * c4);
+#pragma unroll
+    for (int w = 1; w < ST_WAVES; w++) sum[i] += *(const f4 *)(lds + w * (SP * ST_CW) + nn * ST_CW + 4 * c4);
+  }
+  auto finish = [&](auto op) {   // op(i, nn, mcol) for the thread's groups inside the result
+#pragma unroll
+    for (int i = 0; i < GROUPS; i++) {
+      const int g = tid + 64 * ST_WAVES * i;
+      const int nn = g / (ST_CW / 4), mcol = blockIdx.x * ST_CW + 4 * (g % (ST_CW / 4));
+      if (nn < P.n && mcol < P.m) op(i, nn, mcol);
+    }
+  };
+  auto write_result = [&](int i, int nn, int mcol) {
+    f4 *cp = (f4 *)(P.c + (size_t)nn * P.ldc + mcol);
+    f4 v = P.alpha * sum[i];
+    if (P.beta != 0.f) v += P.beta * *cp;
+    *cp = v;
+  };
+  if (P.ksplit == 1) {
+    finish(write_result);
+    return;
+  }
+  if (F.ticket == nullptr) {   // more than two slices: splitk_reduce adds them in slice order
+    finish([&](int i, int nn, int mcol) { *(f4 *)(P.work + ((size_t)blockIdx.y * P.n + nn) * P.m + mcol) = sum[i]; });
+    return;
+  }
+  // Two slices.  The sums go through to where all XCDs meet (device-scope stores leave nothing dirty in this
+  // XCD's L2); every wave waits for its stores' acknowledgement, the block meets, and one lane takes the column
+  // block's ticket.  Whoever draws the second ticket knows that the other block's stores were acknowledged before
+  // its ticket, reads them with loads that bypass the caches, and finishes the result.
+  finish([&](int i, int nn, int mcol) { st_store_shared(P.work + ((size_t)blockIdx.y * P.n + nn) * P.m + mcol, sum[i]); });
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (tid == 0) s_last = atomicAdd(F.ticket + blockIdx.x, 1u) == 1u ? 1u : 0u;
+  __syncthreads();
+  if (!s_last) return;
+  finish([&](int i, int nn, int mcol) {
+    sum[i] += st_load_fresh(P.work + ((size_t)(1 - blockIdx.y) * P.n + nn) * P.m + mcol);
+    write_result(i, nn, mcol);
+  });
+  if (tid == 0) F.ticket[blockIdx.x] = 0u;
+}
+
 template <int BM, int BN, int EDGE>
 void launch_tt(bool ta, bool tb, dim3 grid, hipStream_t s, const GemmParams &P) {
   dim3 block(256);
@@ -522,6 +780,27 @@ static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, 
     }
   }
 }
+// The streaming kernel's launch for a product with n <= 64: a block per 128 values of m, and K sliced over the grid
+// as well while that leaves CUs without a block; a slice is a multiple of 128 k (32 k for each of a block's waves).
+static void plan_stream(long m, long k, int cus, int &ksplit, int &kchunk) {
+  const long bx = (m + ST_CW - 1) / ST_CW;
+  long want = cus / bx;
+  if (want > k / 256) want = k / 256;
+  if (want < 1) want = 1;
+  const long per = ST_WAVES * ST_CK;
+  const long chunk = ((k + want - 1) / want + per - 1) / per * per;
+  kchunk = (int)chunk;
+  ksplit = (int)((k + chunk - 1) / chunk);
+}
+
+static void launch_stream(bool skc, int nt, dim3 grid, hipStream_t s, const GemmParams &P, const StreamFold &F) {
+  dim3 block(64 * ST_WAVES);
+  if (nt == 1 && skc) hipLaunchKernelGGL((sgemm_stream<1, true>), grid, block, 0, s, P, F);
+  else if (nt == 1) hipLaunchKernelGGL((sgemm_stream<1, false>), grid, block, 0, s, P, F);
+  else if (skc) hipLaunchKernelGGL((sgemm_stream<2, true>), grid, block, 0, s, P, F);
+  else hipLaunchKernelGGL((sgemm_stream<2, false>), grid, block, 0, s, P, F);
+}
+
 // the block tile and the K slicing a product of this shape gets on a chip with `cus` compute units
 void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk) {
   choose_tile(m, n, k, cus, k % BK == 0, *bm, *bn);
@@ -556,6 +835,32 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
     hipLaunchKernelGGL(scale_result, dim3((unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256)), dim3(256), 0, stream, P);
     hipError_t e0 = hipGetLastError();
     THCL_CHECK(e0 == hipSuccess, "gemm launch failed: %s", hipGetErrorString(e0));
+    thcl_after_launch(state, rt);
+    return;
+  }
+  const int cus = thcl_rt_get_props(rt)->compute_units;
+  // one short side and a long operand contiguous along m: the long operand streams from memory into the matrix cores
+  const bool b_groups = tb ? (n % 4 == 0) : (k % 4 == 0);
+  if (!ta && n <= 64 && m >= 2048 && k >= 512 && k % 2 == 0 && m % 4 == 0 && lda % 4 == 0 && ldc % 4 == 0 && al16(a) && al16(c) &&
+      ldb % 4 == 0 && al16(b) && b_groups && lda < (1L << 24) && (tb ? k : n) * ldb < (1L << 30)) {
+    plan_stream(m, k, cus, P.ksplit, P.kchunk);
+    if (P.ksplit > 1) {
+      P.work = (float *)thcl_rt_workspace(rt, (size_t)P.ksplit * m * n * sizeof(float));
+      THCL_CHECK(P.work != nullptr, "gemm workspace: %s", thcl_rt_error());
+    }
+    dim3 grid((unsigned)((m + ST_CW - 1) / ST_CW), (unsigned)P.ksplit);
+    // two slices are folded inside the launch; the tickets are the column-tile counters of the context's scratch
+    // block (uint32 [64, 4096), zero between launches; launches of one context run in order)
+    StreamFold F{nullptr};
+    if (P.ksplit == 2 && grid.x <= 4096 - 64) F.ticket = (unsigned *)thcl_rt_scratch(rt, nullptr) + 64;
+    launch_stream(!tb, n <= 32 ? 1 : 2, grid, stream, P, F);
+    if (P.ksplit > 1 && !F.ticket) {
+      const size_t total = (size_t)m * n / 4;
+      unsigned rg = (unsigned)((total + 255) / 256 > 65536 ? 65536 : (total + 255) / 256);
+      hipLaunchKernelGGL(splitk_reduce<true>, dim3(rg), dim3(256), 0, stream, P);
+    }
+    hipError_t e1 = hipGetLastError();
+    THCL_CHECK(e1 == hipSuccess, "gemm launch failed: %s", hipGetErrorString(e1));
     thcl_after_launch(state, rt);
     return;
   }

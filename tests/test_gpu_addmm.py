@@ -276,3 +276,31 @@ def test_sliced_products_repeat_bit_exactly(cl):
         view.addmm(0.25, 2.0, A, B)
         w = wide.float()
         assert np.array_equal(w[:, :N].view(np.uint32), first.view(np.uint32)) and not w[:, N:].any()
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 2048, 512), (64, 4096, 1024), (48, 2052, 640), (33, 8192, 514), (32, 4100, 1000), (20, 2048, 4098),
+                                   (8, 16384, 768), (4, 3000, 512), (64, 66048, 512), (12, 70000, 520), (64, 16384, 4096)])
+def test_short_side_with_a_long_streamed_operand(cl, M, N, K):
+    """At most 64 rows (or columns) against a long operand that is contiguous along the long side: the long operand is
+    streamed from memory into the matrix cores and only the short one passes through LDS.  Short sides that are no
+    multiple of 32 (padded in LDS), long sides that are no multiple of a block's 256 or 512, K that is no multiple of
+    a 128-k chunk (the last chunk is short), slices of K and none, both layouts of the short operand, a row-major
+    result and the mirrored product into a column-major one, beta = 0 over NaNs, and the same bits on a repeat."""
+    rng = np.random.RandomState(M * 13 + N * 3 + K)
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
+    b = rng.standard_normal((K, N)).astype(F)
+    c = rng.standard_normal((M, N)).astype(F)
+    want = 0.5 * c.astype(np.float64) + 1.5 * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = float(np.sqrt(np.mean(want ** 2)))
+    B = cl.ClTensor(b)
+    for A in (cl.ClTensor(a), cl.ClTensor(np.ascontiguousarray(a.T)).t()):
+        first = cl.ClTensor(c).addmm(0.5, 1.5, A, B).float()
+        assert np.max(np.abs(first - want)) / scale < RTOL, A.stride()
+        again = cl.ClTensor(c).addmm(0.5, 1.5, A, B).float()
+        assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+        nan = cl.ClTensor(np.full((M, N), np.nan, dtype=F)).addmm(0.0, 1.0, A, B).float()
+        assert np.max(np.abs(nan - a.astype(np.float64) @ b.astype(np.float64))) / scale < RTOL
+        # mirrored: (N x K) @ (K x M) into a column-major result, the long operand given as the transpose of a dense array
+        Ct = cl.ClTensor(np.ascontiguousarray(c)).t()                 # N x M with strides (1, N)
+        Ct.addmm(0.5, 1.5, B.t(), A.t())
+        assert np.max(np.abs(Ct.float().T - want)) / scale < RTOL, ("mirrored", A.stride())
