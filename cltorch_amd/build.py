@@ -20,7 +20,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libthcl_hip.so")
 
 ARCH = "gfx950"
-SOURCES = ["rt.cpp", "state.cpp", "tensor.cpp", "layout.cpp", "expr.cpp", "math.cpp", "host_copy.cpp", "catalogue.cpp", "user_kernel.cpp", "blas.cpp",
+SOURCES = ["rt.cpp", "state.cpp", "tensor.cpp", "layout.cpp", "expr.cpp", "math.cpp", "host_copy.cpp", "catalogue.cpp", "user_kernel.cpp", "blas.cpp", "unavailable.cpp",
            "apply.hip", "apply_catalogue.hip", "reduce.hip", "scan.hip", "index.hip", "blas12.hip", "gemm.hip"]
 
 COMMON = ["-O3", "-fPIC", "-fvisibility=hidden", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function", "-Wno-unused-const-variable",

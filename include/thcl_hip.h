@@ -592,6 +592,32 @@ void THClKernel_run(THClState *state, THClKernel *kernel, const int *ints, const
                     THClTensor *const *tensors, long numWorkgroups, long workgroupSize);
 int THClKernel_compileCheck(THClKernel *kernel, const char *arch, size_t *code_bytes);
 
+/* ------------------------------------------------------------------------- */
+/* Defined by the reference only to raise an error; kept so that a binding     */
+/* built from the reference's own sources resolves every name it mentions      */
+/* (src/Storage.cpp:75 calls THClStorage_copyCl, src/TensorMath.lua:849 wraps  */
+/* THClTensor_baddbmm).  Each reports the reference's message:                 */
+/* "not available yet for THClStorage" (src/lib/THClStorage.cpp:142-200,       */
+/* THClStorageCopy.cpp:27-32) or "Not implemented" (src/lib/THClBlas.cpp:      */
+/* 67-147,451-470, THClTensorMathBlas.cpp:279-380).                            */
+/* ------------------------------------------------------------------------- */
+THClStorage *THClStorage_newWithSize1(THClState *state, int device, float data0);
+THClStorage *THClStorage_newWithSize2(THClState *state, int device, float data0, float data1);
+THClStorage *THClStorage_newWithSize3(THClState *state, int device, float data0, float data1, float data2);
+THClStorage *THClStorage_newWithSize4(THClState *state, int device, float data0, float data1, float data2, float data3);
+THClStorage *THClStorage_newWithMapping(THClState *state, int device, const char *filename, long size, int shared);
+THClStorage *THClStorage_newWithData(THClState *state, int device, float *data, long size);
+void THClStorage_copyCl(THClState *state, THClStorage *self, THClStorage *src);
+void THClBlas_swap(THClState *state, long n, float *x, long incx, float *y, long incy);
+void THClBlas_scal(THClState *state, long n, float a, float *x, long incx);
+void THClBlas_copy(THClState *state, long n, float *x, long incx, float *y, long incy);
+void THClBlas_axpy(THClState *state, long n, float a, float *x, long incx, float *y, long incy);
+void THClBlas_gemmBatched(THClState *state, char transa, char transb, long m, long n, long k, float alpha,
+                          const float **a, long lda, const float **b, long ldb, float beta, float **c, long ldc,
+                          long batchCount);
+void THClTensor_baddbmm(THClState *state, THClTensor *result, float beta, THClTensor *t, float alpha,
+                        THClTensor *batch1, THClTensor *batch2);
+
 #pragma GCC visibility pop
 #ifdef __cplusplus
 }

@@ -56,6 +56,48 @@ def test_library_exports_only_what_the_headers_declare():
     assert not any("dbg" in n for n in exported)
 
 
+def test_library_defines_every_function_the_reference_library_defines():
+    """tests/golden/reference_defined_exports.json lists the functions the reference declares THCL_API in a header and
+    defines in a .cpp file of its tensor library (written by tests/golden/make_reference_exports.py from the
+    reference's text): a binding linked from the reference's unchanged sources may name any of them, so the library
+    that takes its place has to resolve them all -- also the ones the reference defines only to raise an error."""
+    import json
+    import subprocess
+    names = json.load(open(os.path.join(ROOT, "tests", "golden", "reference_defined_exports.json")))["names"]
+    assert len(names) > 150
+    out = subprocess.check_output(["nm", "-D", "--defined-only", _lib.LIB_PATH], text=True)
+    exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    missing = [n for n in names if n not in exported]
+    assert not missing, missing
+
+
+def test_reference_stubs_report_the_reference_messages(lib):
+    """The entry points the reference defines only to raise (src/lib/THClStorage.cpp:142-200, THClStorageCopy.cpp:27-32,
+    THClBlas.cpp:67-147,451-470, THClTensorMathBlas.cpp:279-380) raise here with the same text, before any device
+    is touched."""
+    lib.THClLastError.restype = C.c_char_p
+    f = C.c_float
+    calls = {
+        "THClStorage_newWithSize1": (None, 0, f(1)), "THClStorage_newWithSize2": (None, 0, f(1), f(2)),
+        "THClStorage_newWithSize3": (None, 0, f(1), f(2), f(3)), "THClStorage_newWithSize4": (None, 0, f(1), f(2), f(3), f(4)),
+        "THClStorage_newWithMapping": (None, 0, b"file", 4, 0), "THClStorage_newWithData": (None, 0, None, 4),
+        "THClStorage_copyCl": (None, None, None),
+    }
+    for name, args in calls.items():
+        r = getattr(lib, name)(*args)
+        assert not r
+        assert lib.THClLastError() == b"not available yet for THClStorage", name
+    blas = {
+        "THClBlas_swap": (None, 4, None, 1, None, 1), "THClBlas_scal": (None, 4, f(2), None, 1),
+        "THClBlas_copy": (None, 4, None, 1, None, 1), "THClBlas_axpy": (None, 4, f(2), None, 1, None, 1),
+        "THClBlas_gemmBatched": (None, b"n", b"n", 2, 2, 2, f(1), None, 2, None, 2, f(0), None, 2, 1),
+        "THClTensor_baddbmm": (None, None, f(1), None, f(1), None, None),
+    }
+    for name, args in blas.items():
+        getattr(lib, name)(*args)
+        assert lib.THClLastError() == b"Not implemented", name
+
+
 def test_product_never_touches_the_oracle():
     pat = re.compile(r"\boracle\b")
     for base, _, files in os.walk(os.path.join(ROOT, "cltorch_amd")):
