@@ -2,6 +2,8 @@
 // in-order stream, the hipRTC kernel cache and event timers.
 #include "thcl_rt.h"
 
+#include "host_copiers.h"
+
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 #include <pthread.h>
@@ -53,8 +55,7 @@ struct thcl_rt {
   // small uploads leave through a ring of page-locked slots and do not wait for their DMA
   char *ring = nullptr;
   hipEvent_t ring_done[16] = {};
-  unsigned ring_next = 0;
-  bool ring_used[16] = {};
+  thcl_host::UploadRing ring_state;
 };
 
 struct thcl_rt_timer {
@@ -68,6 +69,9 @@ constexpr size_t kScratchBytes = 8u << 20;
 constexpr size_t kMailboxFloats = 16384;   // behind the 64 pinned words: room for a small tensor on its way to the host
 thcl_rt *g_ctx[kMaxDevices] = {nullptr};
 std::mutex g_mu;
+// What the embedding process allows the host side to do; both are read when the first context is opened.
+int g_copy_threads = 1;          // THCL_HOST_COPY_THREADS (0: the library starts no thread)
+long g_scalar_spin_us = 2000;    // THCL_SCALAR_SPIN_US: how long a scalar-returning call polls before it waits for the stream (0: never polls)
 thread_local std::string g_err;
 
 int fail(const char *what, hipError_t e) {
@@ -127,6 +131,13 @@ thcl_rt *thcl_rt_get(int device) {
   }
   snprintf(rt->props.name, sizeof(rt->props.name), "%s", p.name);
   snprintf(rt->props.arch, sizeof(rt->props.arch), "%s", p.gcnArchName);
+  // The kernels are built for gfx950 only, and their hand-overs between blocks (relaxed device-scope atomics plus
+  // waits for store acknowledgements) rely on that chip's cache rules: another device is refused, not tried.
+  if (strncmp(p.gcnArchName, "gfx950", 6) != 0) {
+    g_err = std::string("device ") + std::to_string(device) + " is a " + p.gcnArchName + ": this library is built for gfx950 (MI355X) only";
+    delete rt;
+    return nullptr;
+  }
   rt->props.compute_units = p.multiProcessorCount;
   rt->props.wavefront = p.warpSize;
   rt->props.max_threads_per_block = p.maxThreadsPerBlock;
@@ -152,6 +163,12 @@ thcl_rt *thcl_rt_get(int device) {
   rt->scratch_bytes = kScratchBytes;
   rt->cache_limit = rt->props.total_mem / 2;
   if (const char *mb = getenv("THCL_ALLOC_CACHE_MB")) rt->cache_limit = (size_t)strtoull(mb, nullptr, 10) << 20;
+  g_copy_threads = thcl_host::copy_threads_setting();
+  if (const char *us = getenv("THCL_SCALAR_SPIN_US")) {
+    char *end = nullptr;
+    const long v = strtol(us, &end, 10);
+    if (end != us && v >= 0) g_scalar_spin_us = v;
+  }
   g_ctx[device] = rt;
   return rt;
 }
@@ -184,6 +201,7 @@ void thcl_rt_release_all(void) {
     delete rt;
     g_ctx[d] = nullptr;
   }
+  thcl_host::HostCopiers::shutdown();   // joined: nothing of this library keeps running once the contexts are gone
 }
 
 const thcl_rt_props *thcl_rt_get_props(thcl_rt *rt) { return &rt->props; }
@@ -285,84 +303,14 @@ static int check_fault(thcl_rt *rt);
 // jumps about (256 KiB: 115 us, 512 KiB: 35 us; 1 MiB up: 47 or 221 us from run to run).  From kStagedFrom bytes up
 // the copy is cut into pieces that travel through three page-locked buffers of this library: the DMA of one piece
 // runs while a few host threads move the piece before it between its buffer and the caller's memory (256 MiB:
-// 50 GB/s back into touched memory, 41-46 into a new array, 48-52 out; 256 KiB: 27 us).
+// 50 GB/s back into touched memory, 41-46 into a new array, 48-52 out; 256 KiB: 27 us).  The threads and the piece
+// loops live in host_copiers.h; THCL_HOST_COPY_THREADS=0 keeps the library from starting any thread, and float
+// copies then go the driver's way.
 namespace {
-constexpr size_t kStageBytes = 16u << 20;
-constexpr int kStages = 3;
+using thcl_host::HostCopiers;
+using thcl_host::kStageBytes;
+using thcl_host::kStages;
 constexpr size_t kStagedFrom = 2u << 10;   // (64 KiB up: 39 -> 18 us, 4 KiB: 18 -> 14 us; a few bytes stay with the driver)
-
-// a handful of threads that copy slices of one buffer side by side; made at the first large copy, then asleep
-class HostCopiers {
- public:
-  static HostCopiers &get() {
-    // never destroyed: its threads sleep until the process ends.  A forked child has none of them, so it starts over.
-    static std::once_flag at_fork;
-    std::call_once(at_fork, [] { pthread_atfork(nullptr, nullptr, [] { pool_ = nullptr; }); });
-    if (!pool_) pool_ = new HostCopiers();
-    return *pool_;
-  }
-  // f(first, last) over [0, n) cut into one range per thread (multiples of 1024)
-  void run(size_t n, const std::function<void(size_t, size_t)> &f) {
-    if (n < (1u << 18)) {   // not worth waking anybody
-      f(0, n);
-      return;
-    }
-    std::lock_guard<std::mutex> one_caller(callers_);   // copies of two host threads take turns
-    std::unique_lock<std::mutex> lock(mu_);
-    n_ = n;
-    f_ = &f;
-    pending_ = (int)threads_.size();
-    generation_++;
-    wake_.notify_all();
-    done_.wait(lock, [this] { return pending_ == 0; });
-  }
-  void copy(void *dst, const void *src, size_t bytes) {
-    if (bytes < (1u << 20)) {
-      memcpy(dst, src, bytes);
-      return;
-    }
-    run(bytes, [&](size_t a, size_t b) { memcpy((char *)dst + a, (const char *)src + a, b - a); });
-  }
-
- private:
-  HostCopiers() {
-    unsigned n = std::thread::hardware_concurrency();
-    n = n >= 16 ? 8 : (n >= 4 ? n / 2 : 1);
-    for (unsigned i = 0; i < n; i++) threads_.emplace_back([this, i, n] { work(i, n); });
-    for (auto &t : threads_) t.detach();
-  }
-  void work(unsigned me, unsigned n) {
-    unsigned seen = 0;
-    for (;;) {
-      size_t count;
-      const std::function<void(size_t, size_t)> *f;
-      {
-        std::unique_lock<std::mutex> lock(mu_);
-        wake_.wait(lock, [&] { return generation_ != seen; });
-        seen = generation_;
-        count = n_;
-        f = f_;
-      }
-      const size_t per = ((count + n - 1) / n + 4095) / 4096 * 4096;   // whole pages (of bytes) per thread
-      const size_t from = (size_t)me * per;
-      if (from < count) (*f)(from, count - from < per ? count : from + per);
-      {
-        std::lock_guard<std::mutex> lock(mu_);
-        if (--pending_ == 0) done_.notify_one();
-      }
-    }
-  }
-  static HostCopiers *pool_;
-  std::mutex mu_, callers_;
-  std::condition_variable wake_, done_;
-  std::vector<std::thread> threads_;
-  size_t n_ = 0;
-  const std::function<void(size_t, size_t)> *f_ = nullptr;
-  unsigned generation_ = 0;
-  int pending_ = 0;
-};
-
-HostCopiers *HostCopiers::pool_ = nullptr;
 
 // page-locked memory (this library's or anybody's) goes the direct way
 bool host_memory_is_pagelocked(const void *p) {
@@ -383,44 +331,40 @@ int stage_ready(thcl_rt *rt) {
   return 0;
 }
 
+// the DMA side of the piece loops: the context's stream, its three staging buffers and their events
+struct StreamDma {
+  thcl_rt *rt;
+  char *dev;
+  void *stage(int b) { return rt->stage[b]; }
+  int wait(int b) {
+    RT_CHECK(hipEventSynchronize(rt->stage_done[b]));
+    return 0;
+  }
+  int to_device(size_t off, int b, size_t bytes) {
+    RT_CHECK(hipMemcpyAsync(dev + off, rt->stage[b], bytes, hipMemcpyHostToDevice, rt->stream));
+    RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
+    return 0;
+  }
+  int to_host(int b, size_t off, size_t bytes) {
+    RT_CHECK(hipMemcpyAsync(rt->stage[b], dev + off, bytes, hipMemcpyDeviceToHost, rt->stream));
+    RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
+    return 0;
+  }
+  int drain() {
+    RT_CHECK(hipStreamSynchronize(rt->stream));
+    return 0;
+  }
+};
+
 // to_device: host -> staging (threads) -> device (DMA); otherwise device -> staging (DMA) -> host (threads)
 int staged_copy(thcl_rt *rt, char *dev, char *host, size_t bytes, bool to_device) {
   if (stage_ready(rt) != 0) return -1;
   HostCopiers &copiers = HostCopiers::get();
-  // a quarter of the copy per piece, between 2 and 16 MiB: small copies still overlap their halves, large ones
-  // keep the per-piece costs (an event wait, a wake-up of the copiers) small (256 MiB back into a new array:
-  // 25 GB/s in pieces of 4 MiB, 41-46 in pieces of 16)
-  size_t piece = (bytes / 4 + (1u << 20) - 1) >> 20 << 20;
-  if (piece < (2u << 20)) piece = 2u << 20;
-  if (piece > kStageBytes) piece = kStageBytes;
-  const size_t pieces = (bytes + piece - 1) / piece;
-  auto len = [&](size_t c) { return c + 1 < pieces ? piece : bytes - c * piece; };
-  if (to_device) {
-    for (size_t c = 0; c < pieces; c++) {
-      const int b = (int)(c % kStages);
-      if (c >= (size_t)kStages) RT_CHECK(hipEventSynchronize(rt->stage_done[b]));   // the buffer's last piece has left
-      copiers.copy(rt->stage[b], host + c * piece, len(c));
-      RT_CHECK(hipMemcpyAsync(dev + c * piece, rt->stage[b], len(c), hipMemcpyHostToDevice, rt->stream));
-      RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
-    }
-    RT_CHECK(hipStreamSynchronize(rt->stream));
-    return 0;
-  }
-  for (size_t c = 0; c < pieces && c < (size_t)kStages; c++) {
-    RT_CHECK(hipMemcpyAsync(rt->stage[c], dev + c * piece, len(c), hipMemcpyDeviceToHost, rt->stream));
-    RT_CHECK(hipEventRecord(rt->stage_done[c], rt->stream));
-  }
-  for (size_t c = 0; c < pieces; c++) {
-    const int b = (int)(c % kStages);
-    RT_CHECK(hipEventSynchronize(rt->stage_done[b]));
-    copiers.copy(host + c * piece, rt->stage[b], len(c));
-    const size_t next = c + kStages;
-    if (next < pieces) {
-      RT_CHECK(hipMemcpyAsync(rt->stage[b], dev + next * piece, len(next), hipMemcpyDeviceToHost, rt->stream));
-      RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
-    }
-  }
-  return 0;
+  StreamDma dma{rt, dev};
+  const size_t piece = thcl_host::staged_piece_bytes(bytes);
+  if (to_device)
+    return thcl_host::staged_upload(dma, bytes, 1, piece, [&](void *st, size_t first, size_t n) { copiers.copy(st, host + first, n); });
+  return thcl_host::staged_download(dma, bytes, 1, piece, [&](size_t first, void *st, size_t n) { copiers.copy(host + first, st, n); });
 }
 // host elements of another type <-> device floats, converted by the host threads on the way through the buffers
 extern "C++" {
@@ -428,45 +372,23 @@ template <class T>
 int staged_convert(thcl_rt *rt, float *dev, T *host, size_t count, bool to_device) {
   if (stage_ready(rt) != 0) return -1;
   HostCopiers &copiers = HostCopiers::get();
-  size_t piece = (count / 4 + (1u << 18) - 1) >> 18 << 18;   // in elements: a quarter of the copy, 512 Ki to 4 Mi
-  if (piece < (1u << 19)) piece = 1u << 19;
-  if (piece > kStageBytes / sizeof(float)) piece = kStageBytes / sizeof(float);
-  const size_t pieces = (count + piece - 1) / piece;
-  auto len = [&](size_t c) { return c + 1 < pieces ? piece : count - c * piece; };
-  if (to_device) {
-    for (size_t c = 0; c < pieces; c++) {
-      const int b = (int)(c % kStages);
-      if (c >= (size_t)kStages) RT_CHECK(hipEventSynchronize(rt->stage_done[b]));
-      float *st = (float *)rt->stage[b];
-      const T *from = host + c * piece;
-      copiers.run(len(c), [&](size_t i0, size_t i1) {
+  StreamDma dma{rt, (char *)dev};
+  const size_t piece = thcl_host::converted_piece_elems(count);
+  if (to_device)
+    return thcl_host::staged_upload(dma, count, sizeof(float), piece, [&](void *stage, size_t first, size_t n) {
+      float *st = (float *)stage;
+      const T *from = host + first;
+      copiers.run(n, [&](size_t i0, size_t i1) {
         for (size_t i = i0; i < i1; i++) st[i] = (float)from[i];
       });
-      RT_CHECK(hipMemcpyAsync(dev + c * piece, st, len(c) * sizeof(float), hipMemcpyHostToDevice, rt->stream));
-      RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
-    }
-    RT_CHECK(hipStreamSynchronize(rt->stream));
-    return 0;
-  }
-  for (size_t c = 0; c < pieces && c < (size_t)kStages; c++) {
-    RT_CHECK(hipMemcpyAsync(rt->stage[c], dev + c * piece, len(c) * sizeof(float), hipMemcpyDeviceToHost, rt->stream));
-    RT_CHECK(hipEventRecord(rt->stage_done[c], rt->stream));
-  }
-  for (size_t c = 0; c < pieces; c++) {
-    const int b = (int)(c % kStages);
-    RT_CHECK(hipEventSynchronize(rt->stage_done[b]));
-    const float *st = (const float *)rt->stage[b];
-    T *to = host + c * piece;
-    copiers.run(len(c), [&](size_t i0, size_t i1) {
+    });
+  return thcl_host::staged_download(dma, count, sizeof(float), piece, [&](size_t first, void *stage, size_t n) {
+    const float *st = (const float *)stage;
+    T *to = host + first;
+    copiers.run(n, [&](size_t i0, size_t i1) {
       for (size_t i = i0; i < i1; i++) to[i] = (T)st[i];
     });
-    const size_t next = c + kStages;
-    if (next < pieces) {
-      RT_CHECK(hipMemcpyAsync(rt->stage[b], dev + next * piece, len(next) * sizeof(float), hipMemcpyDeviceToHost, rt->stream));
-      RT_CHECK(hipEventRecord(rt->stage_done[b], rt->stream));
-    }
-  }
-  return 0;
+  });
 }
 }  // extern "C++"
 }  // namespace
@@ -495,16 +417,16 @@ int thcl_rt_copy_converted(thcl_rt *rt, void *dev, void *host, size_t count, int
 // destination is queued behind the DMA).  A slot is waited for only when the ring comes round to it while its DMA is
 // still pending.  4 KiB: 14 us with the wait, 5 us without.
 constexpr size_t kRingSlot = 64u << 10;
-constexpr unsigned kRingSlots = 16;
+constexpr unsigned kRingSlots = thcl_host::UploadRing::kSlots;
 static int ring_upload(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
-  if (!rt->ring) {
+  if (!rt->ring) {   // the events first, the buffer last: a ring that exists is complete
+    for (unsigned i = 0; i < kRingSlots; i++)
+      if (!rt->ring_done[i]) RT_CHECK(hipEventCreateWithFlags(&rt->ring_done[i], hipEventDisableTiming));
     RT_CHECK(hipHostMalloc((void **)&rt->ring, kRingSlot * kRingSlots, hipHostMallocDefault));
-    for (unsigned i = 0; i < kRingSlots; i++) RT_CHECK(hipEventCreateWithFlags(&rt->ring_done[i], hipEventDisableTiming));
   }
-  const unsigned slot = rt->ring_next;
-  rt->ring_next = (slot + 1) % kRingSlots;
-  if (rt->ring_used[slot]) RT_CHECK(hipEventSynchronize(rt->ring_done[slot]));
-  rt->ring_used[slot] = true;
+  bool must_wait;
+  const unsigned slot = rt->ring_state.take(&must_wait);
+  if (must_wait) RT_CHECK(hipEventSynchronize(rt->ring_done[slot]));
   char *at = rt->ring + (size_t)slot * kRingSlot;
   memcpy(at, src, bytes);
   RT_CHECK(hipMemcpyAsync(dst, at, bytes, hipMemcpyHostToDevice, rt->stream));
@@ -516,7 +438,7 @@ int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
   if (!bytes) return 0;
   DeviceGuard g(rt->device);
   if (bytes <= kRingSlot) return ring_upload(rt, dst, src, bytes);
-  if (bytes >= kStagedFrom && !host_memory_is_pagelocked(src)) return staged_copy(rt, (char *)dst, (char *)src, bytes, true);
+  if (bytes >= kStagedFrom && g_copy_threads > 0 && !host_memory_is_pagelocked(src)) return staged_copy(rt, (char *)dst, (char *)src, bytes, true);
   RT_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, rt->stream));
   RT_CHECK(hipStreamSynchronize(rt->stream));
   return 0;
@@ -537,7 +459,7 @@ static int check_fault(thcl_rt *rt) {
 int thcl_rt_memcpy_d2h(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
   if (!bytes) return 0;
   DeviceGuard g(rt->device);
-  if (bytes >= kStagedFrom && !host_memory_is_pagelocked(dst)) {
+  if (bytes >= kStagedFrom && g_copy_threads > 0 && !host_memory_is_pagelocked(dst)) {
     if (staged_copy(rt, (char *)src, (char *)dst, bytes, false) != 0) return -1;
     RT_CHECK(hipStreamSynchronize(rt->stream));
     return check_fault(rt);
@@ -579,9 +501,10 @@ unsigned thcl_rt_next_tag(thcl_rt *rt) {
 }
 int thcl_rt_await_tagged(thcl_rt *rt, unsigned tag, float *value) {
   volatile unsigned long long *w = (volatile unsigned long long *)(rt->host_word + kTaggedWord);
-  // poll for up to 2 ms (a reduction of 2^28 elements takes 0.15 ms), then wait for the stream the ordinary way
+  // poll for up to 2 ms (a reduction of 2^28 elements takes 0.15 ms; THCL_SCALAR_SPIN_US sets another limit, 0 none at
+  // all), then wait for the stream the ordinary way
   const auto t0 = std::chrono::steady_clock::now();
-  for (;;) {
+  while (g_scalar_spin_us > 0) {
     for (int i = 0; i < 64; i++) {
       const unsigned long long pair = *w;
       if ((unsigned)(pair >> 32) == tag) {
@@ -590,7 +513,7 @@ int thcl_rt_await_tagged(thcl_rt *rt, unsigned tag, float *value) {
         return check_fault(rt);
       }
     }
-    if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(2000)) break;
+    if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(g_scalar_spin_us)) break;
   }
   const int rc = thcl_rt_sync(rt);
   const unsigned long long pair = *w;

@@ -29,11 +29,14 @@ def _string(text: str) -> bytes:
 
 def encode_tensor(sizes: Sequence[int], strides: Sequence[int], offset0: int, storage: Optional[np.ndarray],
                   tensor_class: str = "torch.ClTensor", storage_class: str = "torch.ClStorage") -> bytes:
-    """The bytes ``torch.save`` writes for one tensor over one storage (``offset0`` counts from 0)."""
+    """The bytes ``torch.save`` writes for one tensor over one storage (``offset0`` counts from 0).  The dimension
+    count is the header's own field, written as it stands (src/torch/generic/Tensor.cpp:1296): an empty tensor,
+    which has no storage, holds -1 there (src/lib/THClTensor.cpp:635); 0 means a point tensor, with its storage."""
     nd = len(sizes)
     assert len(strides) == nd
+    nd_field = -1 if (nd == 0 and storage is None) else nd
     out = [struct.pack("=ii", TYPE_TORCH, 1), _string("V 1"), _string(tensor_class),
-           struct.pack("=i", nd), struct.pack("=%dq" % nd, *sizes), struct.pack("=%dq" % nd, *strides),
+           struct.pack("=i", nd_field), struct.pack("=%dq" % nd, *sizes), struct.pack("=%dq" % nd, *strides),
            struct.pack("=q", offset0 + 1)]
     if storage is None:
         out.append(struct.pack("=i", TYPE_NIL))

@@ -47,5 +47,5 @@ def hooks_lib():
         flags = [f for f in b.COMMON if f != "-fvisibility=hidden"]
         subprocess.check_call([b.hipcc()] + b.HOST_ONLY + flags + ["-DTHCL_HOOKS_PLANNERS", "-c", src, "-o", obj])
         # -Bsymbolic: calls between the entry points stay inside this library even when the shipped one is loaded too
-        subprocess.check_call([b.hipcc(), "-shared", "-fPIC", "-Wl,-Bsymbolic", f"--offload-arch={b.ARCH}", "-o", so, obj] + objs + ["-lhiprtc"])
+        subprocess.check_call([b.hipcc(), "-shared", "-fPIC", "-Wl,-Bsymbolic", f"--offload-arch={b.ARCH}", "-o", so, obj] + objs + ["-lhiprtc", "-pthread"])
     return C.CDLL(so)

@@ -401,8 +401,23 @@ def test_torch7_file_framing_known_bytes():
     sizes, strides, off, storage, tclass, sclass = S.decode_tensor(got)
     assert (sizes, strides, off, tclass, sclass) == ([2, 3], [3, 1], 1, "torch.ClTensor", "torch.ClStorage")
     assert np.array_equal(storage, data)
+    # an empty tensor: the header's dimension field is -1 and the storage is nil, as the reference writes it
+    # (src/lib/THClTensor.cpp:635, src/torch/generic/Tensor.cpp:1296-1310)
     empty = S.encode_tensor([], [], 0, None)
-    assert empty.endswith(struct.pack("<q", 1) + struct.pack("<i", 0)) and S.decode_tensor(empty)[3] is None
+    assert empty == b"".join([struct.pack("<ii", 4, 1), struct.pack("<i", 3), b"V 1", struct.pack("<i", 14), b"torch.ClTensor",
+                              struct.pack("<i", -1), struct.pack("<q", 1), struct.pack("<i", 0)])
+    assert S.decode_tensor(empty)[:4] == ([], [], 0, None)
+    # a point tensor: no dimensions, but a storage of one value
+    point = S.encode_tensor([], [], 0, np.array([2.5], dtype=np.float32))
+    assert point == b"".join([struct.pack("<ii", 4, 1), struct.pack("<i", 3), b"V 1", struct.pack("<i", 14), b"torch.ClTensor",
+                              struct.pack("<i", 0), struct.pack("<q", 1),
+                              struct.pack("<ii", 4, 2), struct.pack("<i", 3), b"V 1", struct.pack("<i", 15), b"torch.ClStorage",
+                              struct.pack("<q", 1), struct.pack("<f", 2.5)])
+    sizes, strides, off, storage, _, _ = S.decode_tensor(point)
+    assert (sizes, strides, off) == ([], [], 0) and storage.tolist() == [2.5]
+    # and a 1-d tensor over the whole of its storage
+    one = S.encode_tensor([3], [1], 0, np.array([1, 2, 3], dtype=np.float32))
+    assert S.decode_tensor(one)[:3] == ([3], [1], 0) and S.decode_tensor(one)[3].tolist() == [1, 2, 3]
     for bad in (got[:-2], got[:40], got.replace(b"torch.ClTensor", b"torch.XxTensor"), struct.pack("<ii", 3, 1) + got[8:]):
         with pytest.raises(ValueError):
             S.decode_tensor(bad)

@@ -139,6 +139,42 @@ def _c4_chain(cl, A, ref):
     return ref
 
 
+def test_config1_sequence_2p28(cl):
+    """The same sequence at the size the bandwidth figures are quoted on: add, cmul and the map2 expression over 2^28
+    elements compared bit for bit with the dense OpenMP loops of the CPU restatement (a few seconds of host time), then
+    sum and max of a copy with the NaNs set to zero against the serial CPU reductions."""
+    import ctypes as C
+    n = 1 << 28
+    L = oracle.lib()
+    x, y, z = (oracle.uniform(s, n) for s in (1, 2, 3))
+    X, Y, Z = cl.ClTensor(x), cl.ClTensor(y), cl.ClTensor(z)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+
+    def host(op, val, a, b):          # x = op(a, b), in place in x
+        L.th_pointwise_contig_omp(C.c_int(oracle.OPS[op]), C.c_float(val), p(x), p(a), p(b), C.c_long(n))
+
+    X.add(Y)
+    host("cadd", 1.0, x, y)
+    assert_bit_equal(X.float(), x, "add at 2^28")
+    X.cmul(Y)
+    host("cmul", 0.0, x, y)
+    assert_bit_equal(X.float(), x, "cmul at 2^28")
+    X.map2_on_gpu(Y, Z, EXPR1)
+    host("map2_c1", 0.0, y, z)
+    got = X.float()
+    assert_bit_equal(got, x, "map2 at 2^28")
+    del got, Y, Z, y, z
+    nan = np.isnan(x)
+    assert nan.any() and not nan.all()
+    assert np.isnan(X.sum()) and np.isnan(X.max())          # Torch7's CPU rule: a NaN decides both
+    X.apply_on_gpu("x = (x != x) ? 0.0 : x")
+    np.copyto(x, F(0), where=nan)
+    v = View.contiguous(x)
+    want = oracle.sumall(v)
+    assert abs(X.sum() - want) <= 1e-5 * abs(want)
+    assert X.max() == oracle.maxall(v) and X.min() == oracle.minall(v)
+
+
 def test_config4_point_tensor_chain_2p28(cl):
     n = 1 << 28
     a = oracle.uniform(7, n, 0.0, 1.0)
@@ -312,6 +348,21 @@ def test_ordinary_host_memory_in_pieces(cl, n):
         s.copy(d)
         assert_bit_equal(s.to_host(), d.astype(F))
         assert np.array_equal(s.to_host(np.float64), d.astype(F).astype(np.float64))
+
+
+def test_host_threads_and_polling_switched_off(cl):
+    """THCL_HOST_COPY_THREADS=0 and THCL_SCALAR_SPIN_US=0 hand the host side back to the embedding process: the
+    library starts no thread (float copies go the driver's way, conversions run on the caller) and scalar-returning
+    calls wait for the stream instead of polling.  Both are read when the first context is opened, so the
+    piece-boundary copies run again in a process of their own (tests/host_side_off_child.py)."""
+    import os
+    import subprocess
+    import sys
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "host_side_off_child.py")
+    env = dict(os.environ, THCL_HOST_COPY_THREADS="0", THCL_SCALAR_SPIN_US="0")
+    r = subprocess.run([sys.executable, child], capture_output=True, text=True, env=env, timeout=280)
+    assert r.returncode == 0, (r.stdout + r.stderr)[-3000:]
+    assert "host side off ok" in r.stdout
 
 
 @pytest.mark.parametrize("n", [(1 << 16) - 1, 1 << 16, (1 << 19) + 5, (3 << 20) + 1, (17 << 20) - 3])

@@ -370,7 +370,13 @@ def test_save_and_load(cl, tmp_path):
     import struct
     from cltorch_amd import serialize
     raw = serialize.encode_tensor([], [], 0, None)
-    at = raw.index(struct.pack("=i", 0), raw.index(b"torch.ClTensor") + len(b"torch.ClTensor"))
+    at = raw.index(b"torch.ClTensor") + len(b"torch.ClTensor")
+    assert raw[at:at + 4] == struct.pack("=i", -1)
     with open(path, "wb") as f:
-        f.write(raw[:at] + struct.pack("=i", -1) + raw[at + 4:])
+        f.write(raw)
     assert cl.load(path).nElement() == 0
+    with open(path, "wb") as f:          # a writer that puts 0 there reads back as empty as well
+        f.write(raw[:at] + struct.pack("=i", 0) + raw[at + 4:])
+    assert cl.load(path).nElement() == 0
+    cl.save(path, cl.ClTensor())
+    assert open(path, "rb").read() == raw

@@ -301,6 +301,32 @@ def test_catalogue_special_values_and_identities():
     assert cat.atan2([1.0, -1.0, 0.0], [0.0, 0.0, -1.0]).tolist() == [np.float32(np.pi / 2), np.float32(-np.pi / 2), np.float32(np.pi)]
 
 
+def test_catalogue_remaining_unary_names_by_special_values():
+    """exp, log, tanh, floor, ceil, sqrt and abs: each name pinned by values that a swapped table entry (floor for
+    ceil, exp for log, abs for sqrt ...) gets wrong."""
+    from oracle import catalogue as cat
+    bits = lambda a: np.asarray(a, dtype=np.float32).view(np.uint32).tolist()
+    assert bits(cat.unary("floor", [-0.5, 0.5, -2.0, 2.75, -2.75])) == bits([-1.0, 0.0, -2.0, 2.0, -3.0])
+    assert bits(cat.unary("ceil", [-0.5, 0.5, -2.0, 2.75, -2.75])) == bits([-0.0, 1.0, -2.0, 3.0, -2.0])    # ceil(-0.5) keeps the sign
+    assert cat.unary("sqrt", [2.25, 0.0, 16.0, 1e-38]).tolist()[:3] == [1.5, 0.0, 4.0]
+    assert np.isnan(cat.unary("sqrt", [-1.0])[0]) and bits(cat.unary("sqrt", [-0.0])) == bits([-0.0])
+    assert bits(cat.unary("abs", [-0.0, -3.5, 3.5, -np.inf])) == bits([0.0, 3.5, 3.5, np.inf])              # sign bit cleared, also on zero
+    assert cat.unary("exp", [0.0])[0] == 1.0 and cat.unary("log", [1.0])[0] == 0.0
+    assert abs(float(cat.unary("exp", [1.0])[0]) - np.e) <= 3e-7 and abs(cat.unary("log", [np.float32(np.e)])[0] - 1.0) <= 1e-7   # one ulp
+    assert cat.unary("exp", [-np.inf])[0] == 0.0 and cat.unary("log", [0.0])[0] == -np.inf and np.isnan(cat.unary("log", [-1.0])[0])
+    x = np.linspace(-6.0, 6.0, 241).astype(np.float32)
+    t = cat.unary("tanh", x)
+    assert np.array_equal(t, -cat.unary("tanh", -x)) and np.all(np.abs(t) < 1.0) and t[120] == 0.0           # odd, bounded
+    assert np.all(np.diff(t.astype(np.float64)) >= 0) and abs(t[-1] - 1.0) < 2e-5
+    assert np.allclose(t, np.sinh(x.astype(np.float64)) / np.cosh(x.astype(np.float64)), atol=1e-6)
+    # exp and log undo one another, sqrt undoes squaring, floor <= x <= ceil with a gap of 0 or 1
+    y = np.linspace(0.05, 20.0, 400).astype(np.float32)
+    assert np.allclose(cat.unary("log", cat.unary("exp", y)), y, rtol=2e-6)
+    assert np.allclose(cat.unary("sqrt", (y * y).astype(np.float32)), y, rtol=1e-6)
+    f, c = cat.unary("floor", x), cat.unary("ceil", x)
+    assert np.all(f <= x) and np.all(x <= c) and set((c - f).tolist()) <= {0.0, 1.0}
+
+
 def test_scan_norm_truth_closed_forms():
     from oracle import catalogue as cat
     n = 3000
