@@ -153,6 +153,8 @@ def main():
                     help="where --pmc-configs writes (and --summarise reads) the list of operations")
     ap.add_argument("--summarise", nargs=3, metavar=("TRACE_DB", "FETCH_DB", "WRITE_DB"),
                     help="print the text summary of three rocprofv3 runs of --pmc-configs (no GPU needed)")
+    ap.add_argument("--write-path", metavar="WPATH_DB", help="with --summarise: a fourth counter run of --pmc-configs (write requests "
+                    "of the L2 to memory, their stall cycles, write latency seen by the vector caches); adds two columns")
     ap.add_argument("--summarise-trace", metavar="TRACE_DB", help="print per-kernel totals of a --kernel-trace --stats run of this script")
     ap.add_argument("--summarise-mfma", metavar="PMC_DB", help="print the matrix-core duty summary of a --pmc-gemm counter run")
     ap.add_argument("--pmc-gemm", action="store_true",
@@ -168,9 +170,10 @@ def main():
         cmds = [f"rocprofv3 --kernel-trace --stats -d $OUT/cfg_trace -o t -- {w}",
                 f"rocprofv3 --pmc FETCH_SIZE --kernel-trace -d $OUT/cfg_fetch -o f -- {w}",
                 f"rocprofv3 --pmc WRITE_SIZE --kernel-trace -d $OUT/cfg_write -o w -- {w}",
+                "rocprofv3 --pmc " + " ".join(WPATH_COUNTERS) + f" --kernel-trace -d $OUT/cfg_wpath -o p -- {w}",
                 "python3 bench.py --manifest $OUT/pmc_configs_manifest.json --summarise $OUT/cfg_trace/t_results.db "
-                "$OUT/cfg_fetch/f_results.db $OUT/cfg_write/w_results.db > " + PROFILE_SUMMARY]
-        sys.stdout.write(summarise(*args.summarise, args.manifest, cmds))
+                "$OUT/cfg_fetch/f_results.db $OUT/cfg_write/w_results.db --write-path $OUT/cfg_wpath/p_results.db > " + PROFILE_SUMMARY]
+        sys.stdout.write(summarise(*args.summarise, args.manifest, cmds, args.write_path))
         return
     if args.summarise_trace:
         sys.stdout.write(summarise_trace(args.summarise_trace))
@@ -248,7 +251,14 @@ def main():
     }
 
     if not args.no_detail:
-        out["detail"] = detail(cl, oracle, T, X, Y, Z, n)
+        d = detail(cl, oracle, T, X, Y, Z, n)
+        # the rows of the five benchmark configurations go last, so that they sit in the tail of the line
+        out["detail"] = dict([(k, v) for k, v in d.items() if not k.startswith("c")] + [(k, v) for k, v in d.items() if k.startswith("c")])
+        out["roofline"]["configs"] = config_summary(kernels, d, prof if prof.get("elements") == n else {})
+        out["roofline"]["configs_note"] = ("per operation of the five configurations: frac = algorithmic bytes (or flops) / time / peak with "
+                                           "calls in a row timed live (ms); kernel_us and traffic (HBM bytes moved / algorithmic bytes) from "
+                                           "the committed rocprofv3 summary " + PROFILE_SUMMARY + ", whose own frac is work / kernel_us / peak")
+        out["roofline"] = out.pop("roofline")          # after `detail` in the line
     if not args.no_cpu:
         del X, Y, Z
         base = cpu_baseline(1 << args.cpu_log2n)
@@ -267,10 +277,35 @@ def main():
     print(json.dumps(out))
 
 
+def config_summary(kernels, d, prof):
+    """{operation: {frac, ms, kernel_us, traffic}} for every row of the five configurations, a few hundred bytes."""
+    ops = prof.get("ops", {})
+    out = {}
+
+    def row(name, frac, ms):
+        p = ops.get(name)
+        r = {"frac": round(frac, 3), "ms": round(ms, 4)}
+        if p:
+            r["kernel_us"] = round(p["kernel_us"], 1)
+            if p["unit"] == "GB/s":
+                r["traffic"] = round((p["read_bytes"] + p["written_bytes"]) / p["work"], 3)
+        out[name] = r
+
+    for k, v in kernels.items():          # config 1 at the headline size, from the timed steps
+        row("c1_" + k, v["frac_of_peak"], v["avg_ms"])
+    for name, v in d.items():
+        if name.startswith("c") and isinstance(v, dict) and "frac_of_peak" in v:
+            row(name, v["frac_of_peak"], v["avg_ms"])
+    ch = d.get("c4_chain_10_launches")
+    if ch:
+        out["c4_chain_10_launches"] = {"frac": round(ch["achieved"] / HBM_PEAK_GBS, 3), "ms": ch["gpu_ms"]}
+    return out
+
+
 def pmc_gemm(cl, oracle):
     """Launches for a matrix-core counter run: config 5's square product five times (the clock
-    settles over the first launches) and its skinny product 600 times (its time keeps changing over the first
-    tens of ms of such work)."""
+    settles over the first launches), its skinny product 600 times (its time keeps changing over the first
+    tens of ms of such work) and two ragged products 12 times each."""
     k = 8192
     sd = 1.0 / np.sqrt(k)
     Am, Bm, Cm = (cl.ClTensor(oracle.normal(s, k * k, 0.0, sd)).resize(k, k) for s in (8, 9, 10))
@@ -286,6 +321,16 @@ def pmc_gemm(cl, oracle):
     for _ in range(600):
         Cs.addmm(0.5, 1.0, At.t(), Bs)
     cl.synchronize()
+    del At, Bs, Cs
+    # two ragged products: nothing aligned (4095^3, the kernel with moved-back 16-byte windows) and whole 16-byte
+    # groups with edge tiles (3000 x 5000 x 7000); 12 launches each, the summary lists the last
+    rs = np.random.RandomState(0)
+    for (m_, n_, k_) in ((4095, 4095, 4095), (3000, 5000, 7000)):
+        a, b, c = (cl.ClTensor((rs.standard_normal(sh) / np.sqrt(k_)).astype(np.float32)) for sh in ((m_, k_), (k_, n_), (m_, n_)))
+        for _ in range(12):
+            c.addmm(0.0, 1.0, a, b)
+        cl.synchronize()
+        del a, b, c
     print(json.dumps({"pmc_gemm": "done"}))
 
 
@@ -457,7 +502,7 @@ def detail(cl, oracle, T, X, Y, Z, n):
             s["kernel_only_ms"] = round(p["kernel_us"] * 1e-3, 4)
             s["frac_of_peak_kernel_only"] = round(work / (p["kernel_us"] * 1e-6) * scale / peak, 4)
             if unit == "TFLOP/s":
-                s["kernel_only_note"] = "trace of 3 launches after a wait: clocks not settled, so it can exceed avg_ms"
+                s["kernel_only_note"] = "mean of the last %d of 12 traced launches" % p.get("kept_calls", 5)
         d[name] = s
     if profiled:
         d["kernel_only_source"] = PROFILE_SUMMARY + " (rocprofv3 --kernel-trace of `bench.py --pmc-configs`, committed)"
@@ -546,8 +591,8 @@ def committed_profile():
 
 def pmc_configs(cl, oracle, n, manifest_path):
     """Launches for hardware-counter and kernel-trace runs over every configuration: a marker (a fill of
-    7 elements) opens and closes each operation, which runs 1 + 3 times in between; the first call (it may
-    compile) is dropped by the summariser.  The first operation is a dense copy of known size, the calibration point
+    7 elements) opens and closes each operation, which runs 1 + 3 times in between (matrix products 12 times); the
+    first calls (the first may compile, matrix products start on cool clocks) are dropped by the summariser.  The first operation is a dense copy of known size, the calibration point
     of FETCH_SIZE / WRITE_SIZE.  Writes the list of operations with their algorithmic work to
     ``manifest_path``."""
     X, Y, Z = (cl.ClTensor(oracle.uniform(s, n)) for s in (1, 2, 3))
@@ -566,12 +611,15 @@ def pmc_configs(cl, oracle, n, manifest_path):
 
     def run(op):
         name, fn, work, unit, _, peak = op
+        # bandwidth kernels: 1 + 3 calls, the mean of the last 3 is kept.  Matrix products: 12 calls, the mean of the
+        # last 5 (the clocks settle over the first launches of such work after a wait)
+        calls, keep = (4, 3) if unit == "GB/s" else (12, 5)
         mk.fill(0.0)
-        for _ in range(4):
+        for _ in range(calls):
             fn()
         mk.fill(0.0)              # closes the operation: what follows (the next one's set-up) is not part of it
         cl.synchronize()
-        manifest.append({"name": name, "work": work, "unit": unit, "peak": peak})
+        manifest.append({"name": name, "work": work, "unit": unit, "peak": peak, "calls": calls, "keep": keep})
 
     for op in ops:
         run(op)
@@ -579,7 +627,7 @@ def pmc_configs(cl, oracle, n, manifest_path):
     for op in config_ops(cl, oracle, X, Y, Z, n):
         run(op)
     with open(manifest_path, "w") as f:
-        json.dump({"elements": n, "calls_per_op": 4, "ops": manifest}, f)
+        json.dump({"elements": n, "ops": manifest}, f)
     print(json.dumps({"pmc_configs": "done", "ops": len(manifest), "manifest": manifest_path}))
 
 
@@ -613,25 +661,34 @@ def _short(name):
     return name[:i] if i > 0 else name
 
 
-def summarise(trace_db, fetch_db, write_db, manifest_path, commands):
-    """Text summary of three rocprofv3 runs of ``--pmc-configs`` (kernel trace; FETCH_SIZE; WRITE_SIZE)."""
+WPATH_COUNTERS = ["TCC_EA0_WRREQ_sum", "TCC_EA0_WRREQ_64B_sum", "TCC_EA0_WRREQ_STALL_sum", "TCC_TOO_MANY_EA_WRREQS_STALL_sum",
+                  "TCP_TCC_WRITE_REQ_sum", "TCP_TCC_WRITE_REQ_LATENCY_sum"]
+
+
+def summarise(trace_db, fetch_db, write_db, manifest_path, commands, wpath_db=None):
+    """Text summary of three rocprofv3 runs of ``--pmc-configs`` (kernel trace; FETCH_SIZE; WRITE_SIZE), and of a
+    fourth with the write-path counters when given."""
     man = json.load(open(manifest_path))
-    ops, calls = man["ops"], man["calls_per_op"]
+    ops = man["ops"]
     tr, fe, wr = _segments(trace_db, False), _segments(fetch_db, True), _segments(write_db, True)
     assert len(tr) == len(fe) == len(wr) == len(ops), (len(tr), len(fe), len(wr), len(ops))
+    wp = _segments(wpath_db, True) if wpath_db else None
+    assert wp is None or len(wp) == len(ops)
     out = ["commands (each run from /tmp with TMPDIR=/tmp; $R is the repository root, $OUT a scratch directory):"]
     out += ["  " + c for c in commands]
     out += ["workload: every operation runs 1 + 3 times behind a marker launch; the first call is dropped, the figures are means",
-            "  of the other three.  Durations come from the --kernel-trace run (no counters), KiB from the two counter runs.", ""]
+            "  of the other three.  Matrix products (TFLOP/s rows) run 12 times and the figures are means of the last five.",
+            "  Durations come from the --kernel-trace run (no counters), KiB from the two counter runs.", ""]
 
-    def per_call(seg):
+    def per_call(seg, op=None):
+        calls, keep = (op or {}).get("calls", 4), (op or {}).get("keep", 3)
         assert len(seg) % calls == 0, (len(seg), calls)
         k = len(seg) // calls
-        return k, seg[k:]          # drop the first call
+        return k, seg[k * (calls - keep):]          # the kept calls
 
     # calibration on the dense copy: reads and writes 4 bytes per element
-    k, cal_f = per_call(fe[0])
-    _, cal_w = per_call(wr[0])
+    k, cal_f = per_call(fe[0], ops[0])
+    _, cal_w = per_call(wr[0], ops[0])
     n = man["elements"]
     want_kib = 4.0 * n / 1024
     f_read = sum(r["c"].get("FETCH_SIZE", 0.0) for r in cal_f) / (len(cal_f) / k)
@@ -641,12 +698,15 @@ def summarise(trace_db, fetch_db, write_db, manifest_path, commands):
             f"  FETCH_SIZE reports {f_read:.1f} KiB -> scale {fs:.4f}; WRITE_SIZE reports {w_read:.1f} KiB -> scale {ws:.4f}", ""]
     hdr = "%-34s %-44s %3s %9s %11s %11s %9s %9s %7s %7s" % ("operation", "kernel", "x", "dur_us", "FETCH_KiB", "WRITE_KiB", "read_MiB",
                                                                "wrote_MiB", "traf/alg", "frac")
+    if wp:
+        hdr += " %10s %9s %9s" % ("wr_req", "stall/req", "lat/req")
     out += [hdr, "-" * len(hdr)]
     js = {"elements": n, "fetch_scale": round(fs, 4), "write_scale": round(ws, 4), "ops": {}}
-    for op, st, sf, sw in zip(ops, tr, fe, wr):
-        k, t = per_call(st)
-        _, f = per_call(sf)
-        _, w = per_call(sw)
+    for idx, (op, st, sf, sw) in enumerate(zip(ops, tr, fe, wr)):
+        k, t = per_call(st, op)
+        _, f = per_call(sf, op)
+        _, w = per_call(sw, op)
+        wpc = per_call(wp[idx], op)[1] if wp else None
         ncalls = len(t) // k if k else 0
         if not k:
             out.append("%-34s (no device kernel)" % op["name"])
@@ -666,14 +726,23 @@ def summarise(trace_db, fetch_db, write_db, manifest_path, commands):
         frac = op["work"] / (tot_us * 1e-6) * (1e-9 if is_bw else 1e-12) / op["peak"]
         for j, (kn, us, fk, wk) in enumerate(lines):
             first = j == 0
-            out.append("%-34s %-44s %3s %9.1f %11.1f %11.1f %9s %9s %7s %7s" % (
+            line = "%-34s %-44s %3s %9.1f %11.1f %11.1f %9s %9s %7s %7s" % (
                 op["name"][:34] if first else "", kn, "", us, fk, wk,
                 "%.1f" % (tot_rd / 2 ** 20) if first else "", "%.1f" % (tot_wr / 2 ** 20) if first else "",
-                ("%.3f" % ratio if ratio is not None else "-") if first else "", "%.3f" % frac if first else ""))
+                ("%.3f" % ratio if ratio is not None else "-") if first else "", "%.3f" % frac if first else "")
+            if wpc and len(wpc) == len(t):
+                cnt = lambda name: float(np.mean([wpc[i * k + j]["c"].get(name, 0.0) for i in range(ncalls)]))
+                req, tcp = cnt("TCC_EA0_WRREQ_sum"), cnt("TCP_TCC_WRITE_REQ_sum")
+                line += " %10.4g %9s %9s" % (req, "%.2f" % (cnt("TCC_EA0_WRREQ_STALL_sum") / req) if req > 1e4 else "-",
+                                             "%.0f" % (cnt("TCP_TCC_WRITE_REQ_LATENCY_sum") / tcp) if tcp > 1e4 else "-")
+            out.append(line)
         js["ops"][op["name"]] = {"kernel_us": round(tot_us, 2), "read_bytes": int(tot_rd), "written_bytes": int(tot_wr),
-                                 "work": op["work"], "unit": op["unit"], "frac": round(frac, 4)}
+                                 "work": op["work"], "unit": op["unit"], "frac": round(frac, 4), "kept_calls": ncalls}
     out += ["", "columns: dur_us = mean kernel duration; FETCH/WRITE_KiB = counter values per dispatch; read/wrote_MiB = scaled HBM bytes of one call;",
             "  traf/alg = (read + written) / algorithmic bytes of the call; frac = algorithmic work / kernel time / peak (8000 GB/s or 157.3 TFLOP/s).",
+            "  wr_req = write requests of the L2s to memory per dispatch (TCC_EA0_WRREQ_sum; all of 64 bytes in every row here);",
+            "  stall/req = TCC_EA0_WRREQ_STALL_sum / wr_req (cycles a request waited for credits on its way out of the L2);",
+            "  lat/req = TCP_TCC_WRITE_REQ_LATENCY_sum / TCP_TCC_WRITE_REQ_sum (cycles from a vector cache's write request to its acknowledgement).",
             "json: " + json.dumps(js)]
     return "\n".join(out) + "\n"
 
@@ -709,21 +778,27 @@ def summarise_mfma(db_path):
     out = ["command (run from /tmp with TMPDIR=/tmp; $R is the repository root, $OUT a scratch directory):",
            "  rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES GRBM_GUI_ACTIVE --kernel-trace -d $OUT/pmc_gemm -o g -- python3 $R/bench.py --pmc-gemm",
            "  python3 bench.py --summarise-mfma $OUT/pmc_gemm/g_results.db > profiles/addmm_8192_and_skinny_pmc_mfma_duty.txt",
-           "workload: addmm 8192^3 five times, then addmm 64x16384x4096 (A given transposed) 600 times; fp32, random normal operands", "",
+           "workload: addmm 8192^3 five times, addmm 64x16384x4096 (A given transposed) 600 times, then 4095^3 and 3000x5000x7000",
+           "  12 times each (their last three launches are listed); fp32, random normal operands", "",
            "how to read it: every v_mfma_f32_32x32x2_f32 books 64 busy cycles on its SIMD, so flops = busy / 64 * 4096;",
            "  duty = SQ_VALU_MFMA_BUSY_CYCLES / (1024 SIMDs * GRBM_GUI_ACTIVE / 8 XCDs); clock = GRBM_GUI_ACTIVE / 8 / duration.",
            "  For kernels shorter than ~0.2 ms GRBM_GUI_ACTIVE also covers some time around the launch, so their clock reads a little",
            "  high and their duty a little low.  Of the 600 skinny launches every hundredth is listed.", "",
            "%-52s %10s %8s %14s %14s %8s %10s %8s" % ("kernel", "grid", "dur_us", "MFMA_BUSY", "GRBM_ACTIVE", "duty", "clock_GHz", "TFLOP/s")]
-    seen = {}
+    total, seen = {}, {}
+    for r in rows.values():
+        if "gemm" in r["name"]:
+            total[_short(r["name"])] = total.get(_short(r["name"]), 0) + 1
     for did in sorted(rows):
         r = rows[did]
         if "gemm" not in r["name"]:
             continue
         key = _short(r["name"])
         seen[key] = seen.get(key, 0) + 1
-        big = r["dur"] > 2e6
-        if not big and seen[key] % 100:
+        # kernels launched a few times: all of the square product's five, else the last three; the 600: every hundredth
+        if total[key] > 20 and seen[key] % 100:
+            continue
+        if 5 < total[key] <= 20 and seen[key] <= total[key] - 3:
             continue
         busy, act = r["c"].get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0), max(r["c"].get("GRBM_GUI_ACTIVE", 1.0), 1.0)
         flops = busy / 64.0 * 4096.0
