@@ -463,20 +463,24 @@ __global__ __launch_bounds__(256) void scale_result(GemmParams P) {
 //   the first one's sums to its own (the sum of two numbers does not depend on their order, so a product gives
 //   the same bits every time) and writes the result.  More slices go to `work` and are added in slice order by
 //   splitk_reduce.
-//   The short operand passes through LDS in chunks of 32 k, each wave staging the rows of its own K range in a
-//   buffer of its own: there is no barrier inside the K loop.  Rows n..63 of a chunk hold whatever the clamped
-//   loads delivered: they only reach accumulator rows that are never stored.
-//   A wave requests the long operand 16 k-pairs (one chunk) ahead through a ring of registers whose slots are
-//   fixed at compile time: the refills of a chunk all belong to the next chunk, so they share one scalar base and
-//   each slot keeps its own constant 32-bit offset (no address arithmetic in the loop: every vector instruction
-//   beside an MFMA costs the matrix pipe about six cycles).
+//   The short operand is small and stays in L2.  Stored in rows of n, a lane's fragments of a k-pair are 4 or 8
+//   adjacent bytes of memory and are loaded as such, through a second ring of registers beside the long
+//   operand's: nothing passes through LDS and the K loop holds, per pair, eight MFMAs, two loads and scalar
+//   address arithmetic.  Stored in rows of k, chunks of 32 k pass through LDS to be transposed, each wave staging
+//   the rows of its own K range in a buffer of its own: there is no barrier inside the K loop either way.
+//   A wave requests 16 k-pairs (one chunk) ahead through rings of registers whose slots are fixed at compile time.
+//   All loads are buffer loads: descriptor base + the lane's constant 32-bit offset + a scalar offset per pair
+//   (no vector instruction for addresses: beside an MFMA every vector instruction costs the matrix pipe several
+//   cycles, scalar ones none), and what lies beyond a wave's rows reads as zero, so the rings run past the end
+//   of a range without clamping.
 // Needs: k even (a multiple of 4 when the short operand is contiguous along k), m a multiple of 4, the long
 // operand, the result and the workspace 16-byte aligned with leading dimensions that are multiples of 4; the short
-// operand in whole aligned 16-byte groups along its contiguous dim; lda < 2^24 and the short operand below 4 GiB.
+// operand in whole aligned 16-byte groups along its contiguous dim; a wave's rows of the long operand and the
+// short operand within 4 GiB of their first byte.
 constexpr int ST_CW = 128;      // values of m per block
 constexpr int ST_WAVES = 4;
-constexpr int ST_CK = 32;       // k per staged chunk of the short operand
-constexpr int ST_PAIRS = ST_CK / 2;   // k-pairs per chunk = pairs of the long operand in flight per wave
+constexpr int ST_CK = 32;       // k per chunk
+constexpr int ST_PAIRS = ST_CK / 2;   // k-pairs per chunk = pairs in flight per wave
 
 struct StreamFold {
   unsigned *ticket;   // one arrival counter per column block, zero between launches; null: no fold in the launch
@@ -495,14 +499,32 @@ __device__ __forceinline__ f4 st_load_fresh(const float *p) {       // past the 
             __uint_as_float((unsigned)(hi >> 32))};
 }
 
+// Buffer loads: the address is a descriptor's base + a per-lane 32-bit offset + a scalar 32-bit offset, so a loop
+// that walks rows needs no vector arithmetic for its addresses, and what lies at or beyond the descriptor's extent
+// reads as zero instead of being fetched (no clamping of addresses past the end of a range).
+typedef unsigned st_u4 __attribute__((ext_vector_type(4)));
+typedef unsigned st_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t st_buffer(const void *base, unsigned long long bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes > 0xffffffffull ? 0xffffffffu : (unsigned)bytes), 0x00020000);
+}
+template <int N, bool STREAM>
+__device__ __forceinline__ auto st_buffer_load(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned uniform_off) {
+  typedef float T __attribute__((ext_vector_type(N)));
+  constexpr int aux = STREAM ? 2 : 0;   // nontemporal: the long operand is read once
+  if constexpr (N == 4) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, aux));
+  else if constexpr (N == 2) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, uniform_off, aux));
+  else return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, uniform_off, aux));
+}
+
 template <int NT, bool SKC>
 __global__ __launch_bounds__(64 * ST_WAVES) void sgemm_stream(GemmParams P, StreamFold F) {
   constexpr int VW = ST_CW / 32;          // m-values per lane and load
-  constexpr int SP = 32 * NT;             // n-values held per k row in LDS
+  constexpr int SP = 32 * NT;             // n-values per k row
   constexpr int PAIRS = ST_PAIRS;
-  constexpr int SV = ST_CK * SP / 4 / 64; // 16-byte groups of a chunk per lane
-  constexpr int STAGE = ST_WAVES * ST_CK * SP, RED = ST_WAVES * SP * ST_CW;
+  constexpr int SV = ST_CK * SP / 4 / 64; // rows of k: 16-byte groups of a chunk per lane
+  constexpr int STAGE = SKC ? ST_WAVES * ST_CK * SP : 0, RED = ST_WAVES * SP * ST_CW;
   typedef float VT __attribute__((ext_vector_type(VW)));
+  typedef float FT __attribute__((ext_vector_type(NT)));
   __shared__ __attribute__((aligned(16))) float lds[STAGE > RED ? STAGE : RED];
   __shared__ unsigned s_last;
 
@@ -516,21 +538,15 @@ __global__ __launch_bounds__(64 * ST_WAVES) void sgemm_stream(GemmParams P, Stre
   const int k_end = (k_begin + kw < ke) ? k_begin + kw : ke;
   const int np = (k_end - k_begin) >> 1;           // k-pairs of this wave
   const int nchunks = (np + PAIRS - 1) / PAIRS;
-  const int k_first = np > 0 ? k_begin : ke - 2;   // a wave without work still issues its first loads, from the last rows
 
   const int col = blockIdx.x * ST_CW + VW * l32;
   const int col_c = col + VW <= P.m ? col : P.m - VW;     // m is a multiple of VW: a lane's group is inside or outside
-  // long operand: a uniform row base per chunk + the slot's constant byte offset (row parity, column, pair)
-  const unsigned pair_bytes = 8u * (unsigned)P.lda;
-  unsigned a_off[PAIRS];
-#pragma unroll
-  for (int i = 0; i < PAIRS; i++) a_off[i] = ((unsigned)h * (unsigned)P.lda + (unsigned)col_c) * 4u + (unsigned)i * pair_bytes;
-  const unsigned lastp = np > 0 ? (unsigned)(np - 1) : 0u;
-  // pair p of the wave's range, or the last one beyond it
-  auto a_fetch_any = [&](unsigned p) {
-    const char *rows = (const char *)(P.a + (size_t)k_first * P.lda) + (unsigned long long)(p < lastp ? p : lastp) * pair_bytes;
-    return __builtin_nontemporal_load((const VT *)(rows + a_off[0]));
-  };
+  // long operand: the wave's rows behind one descriptor; a lane's offset is its row parity and column, a pair's
+  // the same for the whole wave
+  const __amdgpu_buffer_rsrc_t a_rows = st_buffer(P.a + (size_t)k_begin * P.lda, (unsigned long long)(k_end - k_begin) * P.lda * 4ull);
+  const unsigned a_lane = ((unsigned)h * (unsigned)P.lda + (unsigned)col_c) * 4u;
+  const unsigned a_pair = 8u * (unsigned)P.lda;
+  auto a_fetch = [&](int p) { return st_buffer_load<VW, true>(a_rows, a_lane, (unsigned)p * a_pair); };
 
   f16v acc[NT][VW];
 #pragma unroll
@@ -540,106 +556,103 @@ __global__ __launch_bounds__(64 * ST_WAVES) void sgemm_stream(GemmParams P, Stre
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[t][c][r] = 0.f;
 
-  // The short operand's chunk `ch` of this wave's range into registers.  Group i of lane l: rows of n (SKC false):
-  // k row l / (SP/4) + (256/SP) i, group l % (SP/4); rows of k (SKC true): n = l % SP, k group l / SP + (64/SP) i.
-  // Either way the lane's part of the address never changes and the rest is the same for the whole wave.
-  // whole: the chunk lies inside the wave's range; else rows past its end are clamped to the last one.
+  // MFMA tile t takes the rows n = NT * i + t of the short side (i = the MFMA's own row index), so a lane's NT
+  // fragments of one k are neighbours in memory and in LDS and arrive with one access.
+  //
+  // Short operand in rows of n (SKC false): a lane's fragments of a pair come straight from memory (the operand is
+  // small and stays in L2), through a second ring that runs beside the long operand's.  Values of n at or beyond
+  // P.n read the row's pitch or the next row: they only reach accumulator rows that are never stored.
+  const __amdgpu_buffer_rsrc_t s_rows = st_buffer(SKC ? P.b : P.b + (size_t)k_begin * P.ldb,
+                                                  SKC ? (unsigned long long)P.n * P.ldb * 4ull : (unsigned long long)(k_end - k_begin) * P.ldb * 4ull);
+  const unsigned s_pair = 8u * (unsigned)P.ldb;
+  const unsigned s_frag_lane = ((unsigned)h * (unsigned)P.ldb + (unsigned)(NT * l32)) * 4u;
+  auto s_frag = [&](int p) { return st_buffer_load<NT, false>(s_rows, s_frag_lane, (unsigned)p * s_pair); };
+  // Short operand in rows of k (SKC true): chunks of 32 k pass through LDS to be transposed, each wave staging the
+  // rows of its own range in a buffer of its own (LDS serves a wave's accesses in order: no barrier, one buffer).
+  // Group i of lane l: n = l % SP, k group l / SP + (64/SP) i.
   float *stage = lds + wave * (ST_CK * SP);
-  f4 sreg[SV];
-  const int s_row = SKC ? lane / SP : lane / (SP / 4), s_col = SKC ? lane % SP : lane % (SP / 4);
-  const unsigned s_lane = SKC ? ((unsigned)(s_col < P.n ? s_col : P.n - 1) * (unsigned)P.ldb + 4u * s_row) * 4u
-                              : ((unsigned)s_row * (unsigned)P.ldb + (4 * s_col < P.n ? 4u * s_col : 0u)) * 4u;
-  const int s_last_row = np > 0 ? k_end : ke;   // rows below this exist
-  auto s_fetch = [&](auto whole, int ch) {
-    const int k0 = k_first + ch * ST_CK;
+  f4 sreg[SKC ? SV : 1];
+  const int s_row = lane / SP, s_col = lane % SP;
+  const unsigned s_stage_lane = ((unsigned)s_col * (unsigned)P.ldb + 4u * s_row + (unsigned)k_begin) * 4u;
+  auto s_fetch = [&](int ch) {
 #pragma unroll
-    for (int i = 0; i < SV; i++) {
-      const int kofs = SKC ? 4 * (64 / SP) * i : (256 / SP) * i;   // uniform part of the group's k
-      const char *base = (const char *)(SKC ? P.b + (k0 + kofs) : P.b + (size_t)(k0 + kofs) * P.ldb);
-      if constexpr (decltype(whole)::value) {
-        sreg[i] = *(const f4 *)(base + s_lane);
-      } else {
-        const int kk = k0 + kofs + (SKC ? 4 * s_row : s_row);
-        const int kc = SKC ? (kk + 4 <= s_last_row ? kk : s_last_row - 4) : (kk < s_last_row ? kk : s_last_row - 1);
-        const int back = kk - kc;      // rows (or k) the lane's own part overshoots by
-        sreg[i] = *(const f4 *)(base + s_lane - (size_t)back * (SKC ? 4u : 4u * (unsigned)P.ldb));
-      }
+    for (int i = 0; i < (SKC ? SV : 0); i++)
+      sreg[i] = st_buffer_load<4, false>(s_rows, s_stage_lane, (unsigned)(ch * ST_CK + 4 * (64 / SP) * i) * 4u);
+  };
+  auto s_store = [&]() {
+#pragma unroll
+    for (int i = 0; i < (SKC ? SV : 0); i++) {
+      const int kq = s_row + (64 / SP) * i;
+#pragma unroll
+      for (int c = 0; c < 4; c++) stage[(4 * kq + c) * SP + s_col] = sreg[i][c];
     }
   };
-  auto s_store = [&](float *buf) {
-#pragma unroll
-    for (int i = 0; i < SV; i++) {
-      if (SKC) {
-        const int kq = s_row + (64 / SP) * i;
-#pragma unroll
-        for (int c = 0; c < 4; c++) buf[(4 * kq + c) * SP + s_col] = sreg[i][c];
-      } else {
-        const int row = s_row + (256 / SP) * i;
-        *(f4 *)(buf + row * SP + 4 * s_col) = sreg[i];
-      }
-    }
-  };
+  const float *S = stage + h * SP + NT * l32;
 
-  VT ring[PAIRS];
-  s_fetch(std::false_type{}, 0);
-  // the ring fills in slot order: the wait counts the compiler derives for the loop below follow the later of the
+  // The rings fill in slot order: the wait counts the compiler derives for the loop below follow the later of the
   // positions a slot's load has here and in the loop, so a reordered fill would make the loop wait for loads it
-  // does not need yet
+  // does not need yet.
+  VT ring[PAIRS];
+  FT sring[SKC ? 1 : PAIRS];
+  if constexpr (SKC) s_fetch(0);
 #pragma unroll
   for (int i = 0; i < PAIRS; i++) {
     __builtin_amdgcn_sched_barrier(0);
-    ring[i] = a_fetch_any((unsigned)i);
+    if constexpr (!SKC) sring[i] = s_frag(i);
+    ring[i] = a_fetch(i);
   }
   __builtin_amdgcn_sched_barrier(0);
-  s_store(stage);
-
-  // One step: the short operand's fragments of the next two pairs are requested from LDS, each pair's MFMAs run and
-  // the ring slot they emptied is refilled with the same pair of the next chunk.  The scheduling barrier keeps
-  // that order: left alone the compiler gathers the refills into batches at the end of the chunk, where they no
-  // longer run a chunk ahead.  The staging buffer is the wave's own and LDS serves a wave's accesses in order, so
-  // one buffer is enough: in front of a chunk's last pair, whose fragments are already in registers, the next
-  // chunk replaces it and its first fragments are requested, all behind that pair's MFMAs.
-  // MFMA tile t takes the rows n = NT * i + t of the short side (i = the MFMA's own row index), so that a lane's
-  // NT fragments of one k are neighbours in LDS and arrive with one read; two pairs are requested per step.
-  typedef float FT __attribute__((ext_vector_type(NT)));
-  const float *S = stage + h * SP + NT * l32;
   FT fa[2], fn[2];
-  fa[0] = *(const FT *)S;
-  fa[1] = *(const FT *)(S + 2 * SP);
-  auto chunk = [&](auto full, auto next_whole, int ch) {
+  if constexpr (SKC) {
+    s_store();
+    fa[0] = *(const FT *)S;
+    fa[1] = *(const FT *)(S + 2 * SP);
+  }
+
+  // One chunk of 16 k-pairs.  Per pair: its MFMAs run, then the slots they emptied are refilled with the same pair
+  // of the next chunk (beyond the wave's range the descriptors deliver zeros).  The scheduling barriers keep that
+  // order: left alone the compiler gathers the refills into batches at the end of the chunk, where they no longer
+  // run a chunk ahead.  Rows of k: the next chunk is requested at the top, and in front of the chunk's last two
+  // pairs, whose fragments are already in registers, it replaces the staged chunk and its first fragments are
+  // requested, all behind those pairs' MFMAs.
+  auto chunk = [&](auto full, int ch) {
     const int p0 = ch * PAIRS;
-    s_fetch(next_whole, ch + 1 < nchunks ? ch + 1 : ch);
-    const char *next_rows = (const char *)(P.a + (size_t)(k_first + 2 * (p0 + PAIRS)) * P.lda);   // used when the next chunk is whole
+    if constexpr (SKC) s_fetch(ch + 1);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int pp = 0; pp < PAIRS; pp += 2) {
-      if (pp + 2 == PAIRS) s_store(stage);
-      fn[0] = *(const FT *)(S + (pp + 2 < PAIRS ? 2 * (pp + 2) * SP : 0));
-      fn[1] = *(const FT *)(S + (pp + 2 < PAIRS ? 2 * (pp + 3) * SP : 2 * SP));
+      if constexpr (SKC) {
+        if (pp + 2 == PAIRS) s_store();
+        fn[0] = *(const FT *)(S + (pp + 2 < PAIRS ? 2 * (pp + 2) * SP : 0));
+        fn[1] = *(const FT *)(S + (pp + 2 < PAIRS ? 2 * (pp + 3) * SP : 2 * SP));
+      }
 #pragma unroll
       for (int q = 0; q < 2; q++) {
         // a range's last chunk may be short (the test is the same for the whole wave); the loads go on regardless
         if (decltype(full)::value || p0 + pp + q < np) {
           const VT v = ring[pp + q];
+          FT f;
+          if constexpr (SKC) f = fa[q];
+          else f = sring[pp + q];
 #pragma unroll
           for (int c = 0; c < VW; c++)
 #pragma unroll
-            for (int t = 0; t < NT; t++) acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[q][t], v[c], acc[t][c], 0, 0, 0);
+            for (int t = 0; t < NT; t++) acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[t], v[c], acc[t][c], 0, 0, 0);
         }
-        if constexpr (decltype(next_whole)::value) ring[pp + q] = __builtin_nontemporal_load((const VT *)(next_rows + a_off[pp + q]));
-        else ring[pp + q] = a_fetch_any((unsigned)(p0 + pp + q + PAIRS));
+        if constexpr (!SKC) sring[pp + q] = s_frag(p0 + pp + q + PAIRS);
+        ring[pp + q] = a_fetch(p0 + pp + q + PAIRS);
         __builtin_amdgcn_sched_barrier(0);
       }
-      fa[0] = fn[0];
-      fa[1] = fn[1];
+      if constexpr (SKC) {
+        fa[0] = fn[0];
+        fa[1] = fn[1];
+      }
     }
   };
-  // chunks whose successor is whole as well run the plain loads; the range's last two the clamped ones
   const int nfull = np / PAIRS;
   int ch = 0;
-  for (; ch + 2 < nchunks; ch++) chunk(std::true_type{}, std::true_type{}, ch);
-  for (; ch < nfull; ch++) chunk(std::true_type{}, std::false_type{}, ch);
-  if (ch < nchunks) chunk(std::false_type{}, std::false_type{}, ch);
+  for (; ch < nfull; ch++) chunk(std::true_type{}, ch);
+  if (ch < nchunks) chunk(std::false_type{}, ch);
 
   // acc[t][c][r] = C[m = col + c][n = NT (8 (r / 4) + 4 h + r % 4) + t]: the waves' parts meet in LDS as
   // [wave][n][m] and are added in wave order
@@ -841,9 +854,15 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   const int cus = thcl_rt_get_props(rt)->compute_units;
   // one short side and a long operand contiguous along m: the long operand streams from memory into the matrix cores
   const bool b_groups = tb ? (n % 4 == 0) : (k % 4 == 0);
+  bool stream_fits = false;
   if (!ta && n <= 64 && m >= 2048 && k >= 512 && k % 2 == 0 && m % 4 == 0 && lda % 4 == 0 && ldc % 4 == 0 && al16(a) && al16(c) &&
-      ldb % 4 == 0 && al16(b) && b_groups && lda < (1L << 24) && (tb ? k : n) * ldb < (1L << 30)) {
+      ldb % 4 == 0 && al16(b) && b_groups) {
     plan_stream(m, k, cus, P.ksplit, P.kchunk);
+    // the kernel's buffer descriptors address a wave's rows of the long operand, and the short operand, with 32-bit
+    // byte offsets (a wave's range is at most a slice long, and reads a chunk past it)
+    stream_fits = ((long)P.kchunk + 2 * ST_CK) * lda < (1L << 30) && (tb ? (long)P.kchunk + 2 * ST_CK : n) * ldb < (1L << 30);
+  }
+  if (stream_fits) {
     if (P.ksplit > 1) {
       P.work = (float *)thcl_rt_workspace(rt, (size_t)P.ksplit * m * n * sizeof(float));
       THCL_CHECK(P.work != nullptr, "gemm workspace: %s", thcl_rt_error());
