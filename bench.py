@@ -502,7 +502,7 @@ def detail(cl, oracle, T, X, Y, Z, n):
             s["kernel_only_ms"] = round(p["kernel_us"] * 1e-3, 4)
             s["frac_of_peak_kernel_only"] = round(work / (p["kernel_us"] * 1e-6) * scale / peak, 4)
             if unit == "TFLOP/s":
-                s["kernel_only_note"] = "mean of the last %d of 12 traced launches" % p.get("kept_calls", 5)
+                s["kernel_only_note"] = "mean of the last %d traced launches after about 40 ms of them" % p.get("kept_calls", 5)
         d[name] = s
     if profiled:
         d["kernel_only_source"] = PROFILE_SUMMARY + " (rocprofv3 --kernel-trace of `bench.py --pmc-configs`, committed)"
@@ -591,8 +591,9 @@ def committed_profile():
 
 def pmc_configs(cl, oracle, n, manifest_path):
     """Launches for hardware-counter and kernel-trace runs over every configuration: a marker (a fill of
-    7 elements) opens and closes each operation, which runs 1 + 3 times in between (matrix products 12 times); the
-    first calls (the first may compile, matrix products start on cool clocks) are dropped by the summariser.  The first operation is a dense copy of known size, the calibration point
+    7 elements) opens and closes each operation, which runs 1 + 3 times in between (matrix products 12 to 600 times:
+    about 40 ms of launches); the first calls (the first may compile, matrix products start on cool clocks) are dropped
+    by the summariser.  The first operation is a dense copy of known size, the calibration point
     of FETCH_SIZE / WRITE_SIZE.  Writes the list of operations with their algorithmic work to
     ``manifest_path``."""
     X, Y, Z = (cl.ClTensor(oracle.uniform(s, n)) for s in (1, 2, 3))
@@ -611,9 +612,9 @@ def pmc_configs(cl, oracle, n, manifest_path):
 
     def run(op):
         name, fn, work, unit, _, peak = op
-        # bandwidth kernels: 1 + 3 calls, the mean of the last 3 is kept.  Matrix products: 12 calls, the mean of the
-        # last 5 (the clocks settle over the first launches of such work after a wait)
-        calls, keep = (4, 3) if unit == "GB/s" else (12, 5)
+        # bandwidth kernels: 1 + 3 calls, the mean of the last 3 is kept.  Matrix products: at least 12 calls and about
+        # 40 ms of them (the clocks settle over the first tens of ms of such work after a wait), the mean of the last 5
+        calls, keep = (4, 3) if unit == "GB/s" else (max(12, min(600, int(40e-3 / (work / (100e12))))), 5)
         mk.fill(0.0)
         for _ in range(calls):
             fn()
@@ -677,7 +678,8 @@ def summarise(trace_db, fetch_db, write_db, manifest_path, commands, wpath_db=No
     out = ["commands (each run from /tmp with TMPDIR=/tmp; $R is the repository root, $OUT a scratch directory):"]
     out += ["  " + c for c in commands]
     out += ["workload: every operation runs 1 + 3 times behind a marker launch; the first call is dropped, the figures are means",
-            "  of the other three.  Matrix products (TFLOP/s rows) run 12 times and the figures are means of the last five.",
+            "  of the other three.  Matrix products (TFLOP/s rows) run 12 times or more (about 40 ms of launches, at most 600) and the",
+            "  figures are means of the last five.",
             "  Durations come from the --kernel-trace run (no counters), KiB from the two counter runs.", ""]
 
     def per_call(seg, op=None):
