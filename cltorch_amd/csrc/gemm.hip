@@ -46,6 +46,23 @@ struct GemmParams {
   int vec_a, vec_b;
 };
 
+// Buffer loads: the address is a descriptor's base + a per-lane 32-bit offset + a scalar 32-bit offset, so a loop
+// that walks rows needs no vector arithmetic for its addresses, and what lies at or beyond the descriptor's extent
+// reads as zero instead of being fetched (no clamping of addresses past the end of a range).
+typedef unsigned st_u4 __attribute__((ext_vector_type(4)));
+typedef unsigned st_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t st_buffer(const void *base, unsigned long long bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes > 0xffffffffull ? 0xffffffffu : (unsigned)bytes), 0x00020000);
+}
+template <int N, bool STREAM>
+__device__ __forceinline__ auto st_buffer_load(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned uniform_off) {
+  typedef float T __attribute__((ext_vector_type(N)));
+  constexpr int aux = STREAM ? 2 : 0;   // nontemporal: the long operand is read once
+  if constexpr (N == 4) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, aux));
+  else if constexpr (N == 2) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, uniform_off, aux));
+  else return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, uniform_off, aux));
+}
+
 // One operand tile in LDS.  KC: contiguous along k in global memory.
 template <int BMN, bool KC>
 struct TileLds {
@@ -154,6 +171,24 @@ struct TileLoader {
       }
     }
   }
+  // Whole aligned tiles through a buffer descriptor whose base is the slab's first element (the same for the whole
+  // block, moved from slab to slab with scalar arithmetic): a thread's groups keep constant 32-bit byte offsets, so
+  // the loop spends no vector instruction on addresses.
+  __device__ __forceinline__ void set_offsets(int ld, unsigned (&off)[NV]) const {
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
+      if (KC) off[p] = ((unsigned)(f / (BK / 4)) * (unsigned)ld + (unsigned)(f % (BK / 4)) * 4u) * 4u;
+      else off[p] = ((unsigned)(f / (BMN / 4)) * (unsigned)ld + (unsigned)(f % (BMN / 4)) * 4u) * 4u;
+    }
+  }
+  __device__ __forceinline__ void load_buf(__amdgpu_buffer_rsrc_t slab, const unsigned (&off)[NV]) {
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      r[p] = st_buffer_load<4, false>(slab, off[p], 0u);
+      keep[p] = 15u;
+    }
+  }
   // plain loads, for tiles and slabs that the caller knows to lie inside the operand (EDGE 0 and 1: aligned as well)
   __device__ __forceinline__ void load_whole(const float *g, int ld, int mn0, int k0) {
 #pragma unroll
@@ -197,22 +232,36 @@ struct TileLoader {
   }
 };
 
-// fragments of one 8-k group for the wave's sub-tiles: frag[t][s], t = 32-wide sub-tile, s = MFMA step
+// fragments of one 8-k group for the wave's sub-tiles: frag[t][s], t = 32-wide sub-tile, s = MFMA step.
+// An operand stored as [k][mn] interleaves its sub-tiles: sub-tile t holds the lines mn_wave0 + NT * i + t (i = the
+// MFMA's own row or column index), so a lane's NT fragments of one k are neighbours and arrive with one 8-byte read,
+// two steps with one instruction (every LDS read beside the MFMAs costs the matrix pipe some cycles).  An operand
+// stored as [mn][k] keeps sub-tile t at mn_wave0 + 32 t + i: its four steps are one 16-byte read already.
 template <int BMN, bool KC, int NT>
 __device__ __forceinline__ void read_frags(const float *lds, int mn_wave0, int kgroup, float (&frag)[NT][4]) {
   const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
+  if (KC) {
 #pragma unroll
-  for (int t = 0; t < NT; t++) {
-    const int mn = mn_wave0 + t * 32 + l32;
-    if (KC) {
+    for (int t = 0; t < NT; t++) {
+      const int mn = mn_wave0 + t * 32 + l32;
       const f4 v = *(const f4 *)(lds + mn * KPITCH + kgroup * 8 + 4 * h);
 #pragma unroll
       for (int s = 0; s < 4; s++) frag[t][s] = v[s];
-    } else {
+    }
+  } else {
+    typedef float FT __attribute__((ext_vector_type(NT)));
 #pragma unroll
-      for (int s = 0; s < 4; s++) frag[t][s] = lds[(kgroup * 8 + 4 * h + s) * BMN + mn];
+    for (int s = 0; s < 4; s++) {
+      const FT v = *(const FT *)(lds + (kgroup * 8 + 4 * h + s) * BMN + mn_wave0 + NT * l32);
+#pragma unroll
+      for (int t = 0; t < NT; t++) frag[t][s] = v[t];
     }
   }
+}
+// where a lane's accumulators lie in the block tile, by the same rule: line of sub-tile t, index i
+template <bool KC, int NT>
+__device__ __forceinline__ int frag_line(int t, int i) {
+  return KC ? 32 * t + i : NT * i + t;
 }
 
 // TA: op(A) = A^T (A stored k-contiguous); TB: op(B) = B^T (B stored n-contiguous)
@@ -278,13 +327,18 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
     ea.set(P.a, P.lda, m0, P.m);
     eb.set(P.b, P.ldb, n0, P.n);
   }
+  unsigned off_a[TileLoader<BM, AKC, EDGE>::NV], off_b[TileLoader<BN, BKC, EDGE>::NV];
+  if (EDGE == 0) {
+    la.set_offsets(P.lda, off_a);
+    lb.set_offsets(P.ldb, off_b);
+  }
   auto fetch = [&](auto &to_a, auto &to_b, int k0) {
     if constexpr (EDGE != 0) {
       to_a.load_edge(ea, P.lda, k0, k_end);
       to_b.load_edge(eb, P.ldb, k0, k_end);
     } else {
-      to_a.load_whole(P.a, P.lda, m0, k0);
-      to_b.load_whole(P.b, P.ldb, n0, k0);
+      to_a.load_buf(st_buffer(AKC ? P.a + (size_t)m0 * P.lda + k0 : P.a + (size_t)k0 * P.lda + m0, 0xffffffffull), off_a);
+      to_b.load_buf(st_buffer(BKC ? P.b + (size_t)n0 * P.ldb + k0 : P.b + (size_t)k0 * P.ldb + n0, 0xffffffffull), off_b);
     }
   };
   fetch(la, lb, slab_k(0));
@@ -342,70 +396,67 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   }
   if (kt < KT) step(any_slab, kt, 0, la, lb, la1, lb1);
 
-  // epilogue: lane holds rows 8*(r/4) + 4*(lane/32) + (r%4) of column lane%32.  The edge kernels use 16-byte accesses
-  // that need no alignment wherever the four rows lie inside the result, and single elements for the group that
-  // straddles its last row.
+  // epilogue: of sub-tile (i, j) a lane holds the tile's rows 8 (r / 4) + 4 (lane / 32) + r % 4, r = 0..15, of the tile's
+  // column lane % 32; frag_line() tells where those lie in the wave's tile.  Per column sub-tile j and quarter rq the
+  // lane's MT * 4 values form MT groups of four consecutive rows of the result: with interleaved row sub-tiles one run
+  // of MT * 4 rows, else one group per sub-tile.  The edge kernels use 16-byte accesses that need no alignment wherever
+  // a group's four rows lie inside the result, and single elements for the group that straddles its last row.
   using CT = typename std::conditional<EDGE == 0, f4, f4u>::type;
   const int lane = threadIdx.x & 63, l32 = lane & 31, h = lane >> 5;
-  if (P.ksplit > 1) {
-    // raw partial product of this K slice, dense [n][m]; scaled and summed by splitk_reduce
-    float *w = P.work + (size_t)blockIdx.y * P.m * P.n;
+  auto group = [&](int j, int rq, int g, int &row, f4 &v) {   // group g of (j, rq): its first row and its raw sums
+    if (AKC) {
+      row = m0 + wm0 + 32 * g + rq * 8 + h * 4;
 #pragma unroll
-    for (int i = 0; i < MT; i++)
+      for (int e = 0; e < 4; e++) v[e] = acc[g][j][rq * 4 + e];
+    } else {
+      row = m0 + wm0 + MT * (rq * 8 + h * 4) + 4 * g;
 #pragma unroll
-      for (int j = 0; j < NT; j++) {
-        const int col = n0 + wn0 + j * 32 + l32;
+      for (int e = 0; e < 4; e++) v[e] = acc[(4 * g + e) % MT][j][rq * 4 + (4 * g + e) / MT];
+    }
+  };
+  float *w = P.ksplit > 1 ? P.work + (size_t)blockIdx.y * P.m * P.n : nullptr;   // raw partial product of this K slice, dense [n][m]
 #pragma unroll
-        for (int rq = 0; rq < 4; rq++) {
-          const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
+  for (int j = 0; j < NT; j++) {
+    const int col = n0 + wn0 + frag_line<BKC, NT>(j, l32);
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++)
+#pragma unroll
+      for (int g = 0; g < MT; g++) {
+        int row;
+        f4 v;
+        group(j, rq, g, row, v);
+        if (P.ksplit > 1) {   // scaled and summed by splitk_reduce
           float *wp = w + (size_t)col * P.m + row;
-          if (!EDGE || (col < P.n && row + 3 < P.m)) {  // edge kernels: a 16-byte store that needs no alignment
-            f4 v;
-#pragma unroll
-            for (int c = 0; c < 4; c++) v[c] = acc[i][j][rq * 4 + c];
+          if (!EDGE || (col < P.n && row + 3 < P.m)) {
             *(CT *)wp = v;
           } else if (col < P.n) {
 #pragma unroll
             for (int c = 0; c < 4; c++)
-              if (row + c < P.m) wp[c] = acc[i][j][rq * 4 + c];
+              if (row + c < P.m) wp[c] = v[c];
           }
+          continue;
         }
-      }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < MT; i++) {
-#pragma unroll
-    for (int j = 0; j < NT; j++) {
-      const int col = n0 + wn0 + j * 32 + l32;
-#pragma unroll
-      for (int rq = 0; rq < 4; rq++) {
-        const int row = m0 + wm0 + i * 32 + rq * 8 + h * 4;
         float *cp = P.c + (size_t)col * P.ldc + row;
         if (!EDGE || (col < P.n && row + 3 < P.m)) {
-          f4 v;
 #pragma unroll
-          for (int c = 0; c < 4; c++) v[c] = P.alpha * acc[i][j][rq * 4 + c];
+          for (int c = 0; c < 4; c++) v[c] = P.alpha * v[c];
           if (P.beta != 0.f) {
             const f4 old = *(const CT *)cp;
 #pragma unroll
             for (int c = 0; c < 4; c++) v[c] += P.beta * old[c];
           }
           *(CT *)cp = v;
-        } else {
-          if (col < P.n) {
+        } else if (col < P.n) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-              if (row + c < P.m) {
-                float v = P.alpha * acc[i][j][rq * 4 + c];
-                if (P.beta != 0.f) v += P.beta * cp[c];
-                cp[c] = v;
-              }
+          for (int c = 0; c < 4; c++) {
+            if (row + c < P.m) {
+              float x = P.alpha * v[c];
+              if (P.beta != 0.f) x += P.beta * cp[c];
+              cp[c] = x;
             }
           }
         }
       }
-    }
   }
 }
 
@@ -497,23 +548,6 @@ __device__ __forceinline__ f4 st_load_fresh(const float *p) {       // past the 
   const unsigned long long hi = __atomic_load_n((const unsigned long long *)p + 1, __ATOMIC_RELAXED);
   return f4{__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)), __uint_as_float((unsigned)hi),
             __uint_as_float((unsigned)(hi >> 32))};
-}
-
-// Buffer loads: the address is a descriptor's base + a per-lane 32-bit offset + a scalar 32-bit offset, so a loop
-// that walks rows needs no vector arithmetic for its addresses, and what lies at or beyond the descriptor's extent
-// reads as zero instead of being fetched (no clamping of addresses past the end of a range).
-typedef unsigned st_u4 __attribute__((ext_vector_type(4)));
-typedef unsigned st_u2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t st_buffer(const void *base, unsigned long long bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes > 0xffffffffull ? 0xffffffffu : (unsigned)bytes), 0x00020000);
-}
-template <int N, bool STREAM>
-__device__ __forceinline__ auto st_buffer_load(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned uniform_off) {
-  typedef float T __attribute__((ext_vector_type(N)));
-  constexpr int aux = STREAM ? 2 : 0;   // nontemporal: the long operand is read once
-  if constexpr (N == 4) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, uniform_off, aux));
-  else if constexpr (N == 2) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(r, lane_off, uniform_off, aux));
-  else return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, uniform_off, aux));
 }
 
 template <int NT, bool SKC>
@@ -891,7 +925,8 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   // fewer than 4 elements along an operand's contiguous dim and no alignment to rely on: one element at a time, one tile shape
   const bool by_element = !(lda % 4 == 0 && a_run % 4 == 0 && al16(a) && ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) && (a_run < 4 || b_run < 4);
   if (by_element) bm = bn = 64;
-  const bool fast = aligned && (m % bm == 0) && (n % bn == 0);
+  // (the whole-tile kernel addresses a slab of a tile with 32-bit byte offsets: 128 rows of either operand)
+  const bool fast = aligned && (m % bm == 0) && (n % bn == 0) && lda < (1L << 22) && ldb < (1L << 22);
   P.vec_a = (lda % 4 == 0 && a_run % 4 == 0 && al16(a)) ? 1 : 0;
   P.vec_b = (ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) ? 1 : 0;
   P.tiles_m = (int)((m + bm - 1) / bm);
