@@ -42,8 +42,6 @@ struct GemmParams {
   int ksplit;   // blockIdx.y slices of K; > 1: raw partial products go to `work`
   int kchunk;   // K per slice (multiple of BK)
   float *work;  // [ksplit][n][m] dense partials
-  // the operand's 16-byte groups along its contiguous dim are whole and aligned (a and b: picks the edge kernel)
-  int vec_a, vec_b;
 };
 
 // Buffer loads: the address is a descriptor's base + a per-lane 32-bit offset + a scalar 32-bit offset, so a loop
@@ -69,14 +67,15 @@ struct TileLds {
   static constexpr int FLOATS = KC ? BMN * KPITCH : BK * BMN;
 };
 
-// Edge kernels: what a lane's loads of one operand keep from slab to slab, worked out once per tile (with the extent
-// tests and the 64-bit products redone at every slab a tile on the rim took 1.6 times as long as a whole one).
-// EDGE 1: at[p] is the lane's 16-byte group in k row 0 (operands contiguous along m/n) or the start of its row
+// Edge kernels 2 and 3 (pitches too long for a buffer descriptor's 32-bit offsets): what a lane's loads of one operand
+// keep from slab to slab, worked out once per tile (with the extent tests and the 64-bit products redone at every slab
+// a tile on the rim took 1.6 times as long as a whole one).
+// EDGE 2: at[p] is the lane's 16-byte group in k row 0 (operands contiguous along m/n) or the start of its row
 // (operands contiguous along k), moved to the operand's last group or row when it lies beyond the m/n extent; in[p]
-// is 15 when it lies inside.  EDGE 2: the same with groups that may straddle the extent: the 16-byte window is then
-// moved back to end at the extent and sh[p] tells by how many elements.  EDGE 3: per element: for operands
-// contiguous along m/n at[p] is the operand's base, mo[p][c] the element's offset along m/n (the last one when it
-// lies beyond), in[p] one bit per element.
+// is 15 when it lies inside; a group that straddles the extent is read through a 16-byte window moved back to end at
+// the extent and sh[p] tells by how many elements.  EDGE 3: per element: for operands contiguous along m/n at[p] is
+// the operand's base, mo[p][c] the element's offset along m/n (the last one when it lies beyond), in[p] one bit per
+// element.
 template <int BMN, bool KC, int EDGE>
 struct EdgeLanes {
   static constexpr int GROUPS = BMN * BK / 4;
@@ -95,9 +94,9 @@ struct EdgeLanes {
         const int mn = mn0 + f / (BK / 4);
         in[p] = mn < lim_mn ? 15u : 0u;
         at[p] = g + (size_t)(mn < lim_mn ? mn : lim_mn - 1) * ld;
-      } else if (EDGE == 1 || EDGE == 2) {
+      } else if (EDGE == 2) {
         const int mq = mn0 + (f % (BMN / 4)) * 4;
-        const int mw = mq + 4 <= lim_mn ? mq : lim_mn - 4;   // EDGE 1: extents are multiples of 4, so mw is mq or outside
+        const int mw = mq + 4 <= lim_mn ? mq : lim_mn - 4;
         in[p] = mq < lim_mn ? 15u : 0u;
         sh[p] = mq < lim_mn ? (unsigned)(mq - mw) : 0u;
         at[p] = g + mw;
@@ -116,16 +115,21 @@ struct EdgeLanes {
 };
 
 // global -> registers: each thread carries BMN*BK/256/4 float4 (a 32-wide tile has 128 of them: the upper half of the
-// block loads the same groups again and does not store them).  EDGE 0: the tile is whole and aligned.  EDGE 1: a
-// 16-byte group of the operand is either inside it or outside, and aligned; every load is issued (from the operand's
-// last row or group when the lane's own lies outside) and groups outside become zeros, so there is no branch around
-// a load.
-// EDGE 2: any pitch and alignment, with 16-byte loads that need no alignment; a group that straddles the operand's
-// extent is read through a window moved back to end there and shifted into place on the way to LDS.  Needs at least
-// 4 elements along each operand's contiguous dimension.  EDGE 3: one element at a time, for what is left.
+// block loads the same groups again and does not store them).  EDGE 0: the tile is whole and aligned.
+// EDGE 1: any extents and alignment, through the same buffer loads as EDGE 0 with the descriptor ending at the
+// operand's last element.  Line i of op(A) only reaches row i of the result and line j of op(B) only column j, so
+// what a tile on the rim reads for lines beyond m or n (the neighbouring row's elements, or zeros past the
+// descriptor's end) lands in results that are never stored and needs no masking; only k beyond the extent has to
+// read as zero, in both operands.  For an operand stored as [k][mn] every such row lies past the descriptor's end
+// (the range check is per 4-byte element, so the last row's groups that straddle the end keep their elements
+// inside); for one stored as [mn][k] the slabs that reach past k get a mask per group, applied on the way to LDS.
+// EDGE 2: the same cases for pitches beyond the descriptor's 32-bit offsets, with 16-byte loads that need no
+// alignment; every load is issued (from the operand's last row or group when the lane's own lies outside), a group
+// that straddles the operand's extent is read through a window moved back to end there and shifted into place on the
+// way to LDS.  Needs at least 4 elements along each operand's contiguous dimension.  EDGE 3: one element at a time,
+// for what is left.
 // The choice is made at compile time: a run-time branch between two edge forms made the compiler wait for all loads
-// at every slab (aligned 4096^3 through the edge kernel: 101 TFLOP/s with the branch against 138 through the
-// whole-tile kernel).
+// at every slab (aligned 4096^3 through such an edge kernel: 101 TFLOP/s with the branch against 138 without).
 template <int BMN, bool KC, int EDGE>
 struct TileLoader {
   using LoadT = typename std::conditional<EDGE == 2, f4u, f4>::type;
@@ -144,7 +148,7 @@ struct TileLoader {
       const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
       if (KC) {
         const int kc = k0 + (f % (BK / 4)) * 4;
-        if (EDGE == 1 || EDGE == 2) {
+        if (EDGE == 2) {
           const int kw = kc + 4 <= lim_k ? kc : lim_k - 4;
           r[p] = *(const LoadT *)(e.at[p] + kw);
           keep[p] = kc < lim_k ? (e.in[p] | (unsigned)(kc - kw) << 4) : 0u;
@@ -160,7 +164,7 @@ struct TileLoader {
       } else {
         const int kr = k0 + f / (BMN / 4);
         const float *row = e.at[p] + (size_t)(kr < lim_k ? kr : lim_k - 1) * ld;
-        if (EDGE == 1 || EDGE == 2) {
+        if (EDGE == 2) {
           r[p] = *(const LoadT *)row;
           keep[p] = kr < lim_k ? (e.in[p] | e.sh[p] << 4) : 0u;
         } else {
@@ -171,9 +175,9 @@ struct TileLoader {
       }
     }
   }
-  // Whole aligned tiles through a buffer descriptor whose base is the slab's first element (the same for the whole
-  // block, moved from slab to slab with scalar arithmetic): a thread's groups keep constant 32-bit byte offsets, so
-  // the loop spends no vector instruction on addresses.
+  // EDGE 0 and 1: through a buffer descriptor whose base is the slab's first element (the same for the whole block,
+  // moved from slab to slab with scalar arithmetic): a thread's groups keep constant 32-bit byte offsets, so the loop
+  // spends no vector instruction on addresses.
   __device__ __forceinline__ void set_offsets(int ld, unsigned (&off)[NV]) const {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
@@ -189,7 +193,17 @@ struct TileLoader {
       keep[p] = 15u;
     }
   }
-  // plain loads, for tiles and slabs that the caller knows to lie inside the operand (EDGE 0 and 1: aligned as well)
+  // EDGE 1, operands contiguous along k: which of a group's elements lie below the k extent, for slabs that may reach past it
+  __device__ __forceinline__ void mask_k(int k0, int lim_k) {
+    if (!KC) return;
+#pragma unroll
+    for (int p = 0; p < NV; p++) {
+      const int f = PART ? (int)(threadIdx.x % GROUPS) : (int)(threadIdx.x + 256 * p);
+      const int left = lim_k - (k0 + (f % (BK / 4)) * 4);
+      keep[p] = left >= 4 ? 15u : left <= 0 ? 0u : (1u << left) - 1u;
+    }
+  }
+  // plain loads, for tiles and slabs that the caller knows to lie inside the operand
   __device__ __forceinline__ void load_whole(const float *g, int ld, int mn0, int k0) {
 #pragma unroll
     for (int p = 0; p < NV; p++) {
@@ -204,13 +218,17 @@ struct TileLoader {
       keep[p] = 15u;
     }
   }
+  template <bool MASKED = true>
   __device__ __forceinline__ void store(float *lds) const {
     if (PART && threadIdx.x >= GROUPS) return;
 #pragma unroll
     for (int p = 0; p < NV; p++) {
       const int f = threadIdx.x + 256 * p;
       f4 v = r[p];
-      if (EDGE == 1) v = keep[p] ? v : f4{0.f, 0.f, 0.f, 0.f};
+      if (EDGE == 1 && KC && MASKED) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) v[c] = (keep[p] >> c & 1u) ? v[c] : 0.f;
+      }
       if (EDGE == 2) {   // element c of the group sits at c + (how far the window was moved back)
         const unsigned back = keep[p] >> 4;
         const f4 w = r[p];
@@ -323,26 +341,39 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   auto slab_k = [&](int kt) { return k_begin + (kt < last ? kt : last) * BK; };
   EdgeLanes<BM, AKC, EDGE> ea;
   EdgeLanes<BN, BKC, EDGE> eb;
-  if (EDGE != 0) {
+  constexpr bool DESCRIPTOR = EDGE == 0 || EDGE == 1;
+  if (!DESCRIPTOR) {
     ea.set(P.a, P.lda, m0, P.m);
     eb.set(P.b, P.ldb, n0, P.n);
   }
   unsigned off_a[TileLoader<BM, AKC, EDGE>::NV], off_b[TileLoader<BN, BKC, EDGE>::NV];
-  if (EDGE == 0) {
+  if (DESCRIPTOR) {
     la.set_offsets(P.lda, off_a);
     lb.set_offsets(P.ldb, off_b);
   }
-  auto fetch = [&](auto &to_a, auto &to_b, int k0) {
-    if constexpr (EDGE != 0) {
+  // one past each operand's last element (k > 0 here)
+  const float *a_end = P.a + (AKC ? (size_t)(P.m - 1) * P.lda + P.k : (size_t)(P.k - 1) * P.lda + P.m);
+  const float *b_end = P.b + (BKC ? (size_t)(P.n - 1) * P.ldb + P.k : (size_t)(P.k - 1) * P.ldb + P.n);
+  constexpr std::true_type whole_slab{};
+  constexpr std::false_type any_slab{};
+  // `whole`: the caller knows that the slab ends at or below the k extent
+  auto fetch = [&](auto whole, auto &to_a, auto &to_b, int k0) {
+    if constexpr (DESCRIPTOR) {
+      const float *sa = AKC ? P.a + (size_t)m0 * P.lda + k0 : P.a + (size_t)k0 * P.lda + m0;
+      const float *sb = BKC ? P.b + (size_t)n0 * P.ldb + k0 : P.b + (size_t)k0 * P.ldb + n0;
+      to_a.load_buf(st_buffer(sa, EDGE == 0 ? 0xffffffffull : (unsigned long long)(a_end - sa) * 4ull), off_a);
+      to_b.load_buf(st_buffer(sb, EDGE == 0 ? 0xffffffffull : (unsigned long long)(b_end - sb) * 4ull), off_b);
+      if constexpr (EDGE == 1 && !decltype(whole)::value) {
+        to_a.mask_k(k0, k_end);
+        to_b.mask_k(k0, k_end);
+      }
+    } else {
       to_a.load_edge(ea, P.lda, k0, k_end);
       to_b.load_edge(eb, P.ldb, k0, k_end);
-    } else {
-      to_a.load_buf(st_buffer(AKC ? P.a + (size_t)m0 * P.lda + k0 : P.a + (size_t)k0 * P.lda + m0, 0xffffffffull), off_a);
-      to_b.load_buf(st_buffer(BKC ? P.b + (size_t)n0 * P.ldb + k0 : P.b + (size_t)k0 * P.ldb + n0, 0xffffffffull), off_b);
     }
   };
-  fetch(la, lb, slab_k(0));
-  fetch(la1, lb1, slab_k(1));
+  fetch(any_slab, la, lb, slab_k(0));
+  fetch(any_slab, la1, lb1, slab_k(1));
   la.store(lds);
   lb.store(lds + AF);
   __syncthreads();
@@ -350,11 +381,11 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
   auto step = [&](auto inside, int kt, int cur, auto &issue_a, auto &issue_b, auto &keep_a, auto &keep_b) {
     float *As = lds + cur * (AF + BF);
     float *Bs = As + AF;
-    if constexpr (decltype(inside)::value) {
+    if constexpr (decltype(inside)::value && !DESCRIPTOR) {
       issue_a.load_whole(P.a, P.lda, m0, slab_k(kt + 2));
       issue_b.load_whole(P.b, P.ldb, n0, slab_k(kt + 2));
     } else {
-      fetch(issue_a, issue_b, slab_k(kt + 2));
+      fetch(inside, issue_a, issue_b, slab_k(kt + 2));
     }
     __builtin_amdgcn_sched_barrier(0);   // keep the loads at the top of the step
     {
@@ -373,17 +404,15 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
       }
     }
     float *An = lds + (cur ^ 1) * (AF + BF);
-    keep_a.store(An);
-    keep_b.store(An + AF);
+    keep_a.template store<!decltype(inside)::value>(An);
+    keep_b.template store<!decltype(inside)::value>(An + AF);
     __syncthreads();
   };
   int kt = 0;
-  constexpr std::true_type whole_slab{};
-  constexpr std::false_type any_slab{};
-  if ((EDGE == 1 || EDGE == 2) && m0 + BM <= P.m && n0 + BN <= P.n) {
-    // a tile inside the matrix (the same for the whole block): its slabs are whole except the last ones, so the
-    // steps that request a whole slab (kt + 2 and kt + 3 below KF) use the plain loads, and the edge form is left
-    // to the tiles on the rim and to the end of K
+  if (EDGE == 1 || (EDGE == 2 && m0 + BM <= P.m && n0 + BN <= P.n)) {
+    // slabs are whole except the last ones, so the steps that store and request whole slabs (kt + 1, and kt + 2 and
+    // kt + 3 below KF) go without the k masks (EDGE 1) or, for a tile inside the matrix (the same for the whole
+    // block), with plain loads (EDGE 2); the general form is left to the end of K and to EDGE 2's tiles on the rim
     const int KF = (k_end - k_begin) / BK;
     for (; kt + 3 < KF; kt += 2) {
       step(whole_slab, kt, 0, la, lb, la1, lb1);
@@ -922,13 +951,12 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   choose_tile(m, n, k, thcl_rt_get_props(rt)->compute_units, aligned, bm, bn);
   // an operand's contiguous dim is m for a 'n', k for a 't'; n for b 't', k for b 'n'
   const long a_run = ta ? k : m, b_run = tb ? n : k;
-  // fewer than 4 elements along an operand's contiguous dim and no alignment to rely on: one element at a time, one tile shape
-  const bool by_element = !(lda % 4 == 0 && a_run % 4 == 0 && al16(a) && ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) && (a_run < 4 || b_run < 4);
+  // the descriptor kernels address a slab of a tile with 32-bit byte offsets: 128 rows of either operand
+  const bool short_pitch = lda < (1L << 22) && ldb < (1L << 22);
+  // longer pitches with fewer than 4 elements along an operand's contiguous dim: one element at a time, one tile shape
+  const bool by_element = !short_pitch && (a_run < 4 || b_run < 4);
   if (by_element) bm = bn = 64;
-  // (the whole-tile kernel addresses a slab of a tile with 32-bit byte offsets: 128 rows of either operand)
-  const bool fast = aligned && (m % bm == 0) && (n % bn == 0) && lda < (1L << 22) && ldb < (1L << 22);
-  P.vec_a = (lda % 4 == 0 && a_run % 4 == 0 && al16(a)) ? 1 : 0;
-  P.vec_b = (ldb % 4 == 0 && b_run % 4 == 0 && al16(b)) ? 1 : 0;
+  const bool fast = aligned && (m % bm == 0) && (n % bn == 0) && short_pitch;
   P.tiles_m = (int)((m + bm - 1) / bm);
   P.tiles_n = (int)((n + bn - 1) / bn);
   P.group_m = P.tiles_m < 8 ? P.tiles_m : 8;
@@ -940,7 +968,7 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   dim3 grid((unsigned)(P.tiles_m * P.tiles_n), (unsigned)P.ksplit);
 #define GO(BM_, BN_)                                                   \
   if (fast) launch_tt<BM_, BN_, 0>(ta, tb, grid, stream, P);                        \
-  else if (P.vec_a && P.vec_b) launch_tt<BM_, BN_, 1>(ta, tb, grid, stream, P);     \
+  else if (short_pitch) launch_tt<BM_, BN_, 1>(ta, tb, grid, stream, P);            \
   else launch_tt<BM_, BN_, 2>(ta, tb, grid, stream, P);
   if (by_element) launch_tt<64, 64, 3>(ta, tb, grid, stream, P);
   else if (bm == 128 && bn == 128) { GO(128, 128) }

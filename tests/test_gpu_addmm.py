@@ -227,8 +227,8 @@ def _odd_pitch(cl, arr, transposed):
 @pytest.mark.parametrize("M,N,K", [(50, 3, 37), (3, 50, 37), (50, 40, 3), (2, 2, 2), (70, 3, 3), (1, 300, 2), (301, 299, 5),
                                    (129, 131, 67), (1001, 515, 130)])
 def test_unaligned_operands_of_any_extent(cl, M, N, K):
-    """Operands whose rows start at odd element offsets: 16-byte loads that need no alignment, a window moved back
-    at the end of a row, and, with fewer than four elements along a row, one element at a time.  All eight layouts."""
+    """Operands whose rows start at odd element offsets: 16-byte loads that need no alignment, groups that straddle
+    the end of a row or of the operand, fewer than four elements along a row.  All eight layouts."""
     rng = np.random.RandomState(M * 5 + N * 11 + K)
     a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
     b = rng.standard_normal((K, N)).astype(F)
@@ -239,6 +239,38 @@ def test_unaligned_operands_of_any_extent(cl, M, N, K):
         A, B, Cd = _odd_pitch(cl, a, lay & 1), _odd_pitch(cl, b, lay & 2), _odd_pitch(cl, c, lay & 4)
         Cd.addmm(-0.5, 1.25, A, B)
         assert np.max(np.abs(Cd.float() - want)) / scale < RTOL, lay
+
+
+def _nan_window(cl, arr, transposed, before, after):
+    """device tensor equal to arr (2-D): a window of a larger storage that holds NaN everywhere else (`before` rows
+    and elements in front of it, `after` behind it), optionally stored transposed"""
+    a = np.ascontiguousarray(arr.T if transposed else arr)
+    big = np.full((a.shape[0] + before + after, a.shape[1] + before + after), np.nan, F)
+    big[before:before + a.shape[0], before:before + a.shape[1]] = a
+    t = cl.ClTensor(big).narrow(1, before + 1, a.shape[0]).narrow(2, before + 1, a.shape[1])
+    return t.t() if transposed else t
+
+
+@pytest.mark.parametrize("M,N,K", [(130, 129, 67), (257, 140, 35), (64, 64, 16), (100, 37, 1), (5, 6, 7), (300, 200, 2050),
+                                   (96, 1500, 4099), (1030, 1029, 131)])
+@pytest.mark.parametrize("before,after", [(1, 2), (4, 0), (0, 0)])
+def test_operand_windows_inside_nan_filled_storage(cl, M, N, K, before, after):
+    """What lies beside an operand in its storage never reaches the result: tiles on the rim read beyond m and n
+    (into the pitch's padding and the neighbouring rows) and the last slab reads beyond k, here all NaN; with
+    (0, 0) the operands end exactly where their storage ends.  All eight layouts, K sliced for the longer ones."""
+    rng = np.random.RandomState(M * 3 + N * 5 + K * 7)
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
+    b = rng.standard_normal((K, N)).astype(F)
+    c = rng.standard_normal((M, N)).astype(F)
+    want = 0.75 * c.astype(np.float64) + 1.25 * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = max(1.0, float(np.sqrt(np.mean(want ** 2))))
+    for lay in range(8):
+        A, B = _nan_window(cl, a, lay & 1, before, after), _nan_window(cl, b, lay & 2, before, after)
+        Cd = cl.ClTensor(np.ascontiguousarray(c.T)).t() if lay & 4 else cl.ClTensor(c)
+        Cd.addmm(0.75, 1.25, A, B)
+        got = Cd.float()
+        assert np.isfinite(got).all(), lay
+        assert np.max(np.abs(got - want)) / scale < RTOL, lay
 
 
 def test_sliced_products_repeat_bit_exactly(cl):
