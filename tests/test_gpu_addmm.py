@@ -273,6 +273,34 @@ def test_operand_windows_inside_nan_filled_storage(cl, M, N, K, before, after):
         assert np.max(np.abs(got - want)) / scale < RTOL, lay
 
 
+def _long_pitch(cl, arr, transposed, pitch, first):
+    """device tensor equal to arr (2-D) whose rows lie `pitch` elements apart in a NaN-filled storage, the first
+    one `first` elements into it, optionally stored transposed"""
+    a = np.ascontiguousarray(arr.T if transposed else arr)
+    store = cl.ClTensor((a.shape[0] - 1) * pitch + a.shape[1] + first).fill(float("nan"))
+    t = store.strided(a.shape, (pitch, 1), first + 1)
+    t.copy(cl.ClTensor(a))
+    return t.t() if transposed else t
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 6, 7), (70, 3, 3), (130, 129, 67), (40, 260, 150)])
+def test_pitches_beyond_the_descriptor_kernels_reach(cl, M, N, K):
+    """Rows 2^22 and more elements apart: the tiled kernels with 64-bit addressing, with windows moved back at the
+    end of a row and, below four elements along a row, one element at a time.  All four layouts of A and B."""
+    rng = np.random.RandomState(M + 2 * N + 3 * K)
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
+    b = rng.standard_normal((K, N)).astype(F)
+    c = rng.standard_normal((M, N)).astype(F)
+    want = 0.5 * c.astype(np.float64) + 1.5 * (a.astype(np.float64) @ b.astype(np.float64))
+    scale = max(1.0, float(np.sqrt(np.mean(want ** 2))))
+    for lay in range(4):
+        A, B = _long_pitch(cl, a, lay & 1, (1 << 22) + 3, 1), _long_pitch(cl, b, lay & 2, 1 << 22, 0)
+        got = cl.ClTensor(c).addmm(0.5, 1.5, A, B).float()
+        assert np.max(np.abs(got - want)) / scale < RTOL, lay
+        del A, B
+    cl.emptyCache()
+
+
 def test_sliced_products_repeat_bit_exactly(cl):
     """K-sliced products sum their slices in slice order: every repetition gives the same
     bits, also with other reductions in between, with ragged shapes, with beta = 0 over
