@@ -42,7 +42,22 @@ struct GemmParams {
   int ksplit;   // blockIdx.y slices of K; > 1: raw partial products go to `work`
   int kchunk;   // K per slice (multiple of BK)
   float *work;  // [ksplit][n][m] dense partials
+  // A launch of several tiles per CU whose tile count is no multiple of the CUs: the first `whole_tiles` logical
+  // tiles (a multiple of the CUs) get a block each, and each of the `tail_tiles` after them gets `tail_split` blocks
+  // that share its K (`tail_kchunk` each), numbered behind the others so that they fill the CUs as those run dry.
+  // Their raw partial products go to `work` as [slice][tail tile][BN][BM] and tail_reduce adds them in slice order.
+  int whole_tiles, tail_tiles, tail_split, tail_kchunk;
 };
+
+// logical tile id -> tile coordinates, grouped order: walk group_m tiles down m, then step along n
+__device__ __forceinline__ void tile_of(const GemmParams &P, int bid, int &tm, int &tn) {
+  const int gsz = P.group_m * P.tiles_n;
+  const int g = bid / gsz, r = bid % gsz;
+  const int m_first = g * P.group_m;
+  const int m_count = (P.tiles_m - m_first < P.group_m) ? (P.tiles_m - m_first) : P.group_m;
+  tm = m_first + r % m_count;
+  tn = r / m_count;
+}
 
 // Buffer loads: the address is a descriptor's base + a per-lane 32-bit offset + a scalar 32-bit offset, so a loop
 // that walks rows needs no vector arithmetic for its addresses, and what lies at or beyond the descriptor's extent
@@ -295,22 +310,19 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
 
   // XCD-aware renumbering: consecutive hardware block ids go to different
   // XCDs, so give XCD x the x-th contiguous chunk of logical ids.
-  const int nblocks = P.tiles_m * P.tiles_n;
   int bid = blockIdx.x;
-  {
-    const int per = nblocks / 8;
+  const bool tail = bid >= P.whole_tiles;   // one of several blocks that share a tile's K
+  int tail_tile = 0, tail_slice = 0;
+  if (tail) {
+    tail_tile = (bid - P.whole_tiles) / P.tail_split;
+    tail_slice = (bid - P.whole_tiles) % P.tail_split;
+    bid = P.whole_tiles + tail_tile;
+  } else {
+    const int per = P.whole_tiles / 8;
     if (per > 0 && bid < per * 8) bid = (bid % 8) * per + bid / 8;
   }
-  // grouped order: walk group_m tiles down m, then step along n
   int tm, tn;
-  {
-    const int gsz = P.group_m * P.tiles_n;
-    const int g = bid / gsz, r = bid % gsz;
-    const int m_first = g * P.group_m;
-    const int m_count = (P.tiles_m - m_first < P.group_m) ? (P.tiles_m - m_first) : P.group_m;
-    tm = m_first + r % m_count;
-    tn = r / m_count;
-  }
+  tile_of(P, bid, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int wave = threadIdx.x >> 6;
@@ -326,8 +338,9 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
 
   TileLoader<BM, AKC, EDGE> la;
   TileLoader<BN, BKC, EDGE> lb;
-  const int k_begin = blockIdx.y * P.kchunk;
-  const int k_end = (k_begin + P.kchunk < P.k) ? (k_begin + P.kchunk) : P.k;
+  const int k_begin = tail ? tail_slice * P.tail_kchunk : blockIdx.y * P.kchunk;
+  const int k_len = tail ? P.tail_kchunk : P.kchunk;
+  const int k_end = (k_begin + k_len < P.k) ? (k_begin + k_len) : P.k;
   const int KT = (k_end - k_begin + BK - 1) / BK;
 
   // Two register sets: while slab kt is multiplied out of LDS, slab kt+1 waits in one
@@ -454,6 +467,10 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
         int row;
         f4 v;
         group(j, rq, g, row, v);
+        if (tail) {   // scaled and summed by tail_reduce
+          *(f4 *)(P.work + ((size_t)tail_slice * P.tail_tiles + tail_tile) * (BM * BN) + (col - n0) * BM + (row - m0)) = v;
+          continue;
+        }
         if (P.ksplit > 1) {   // scaled and summed by splitk_reduce
           float *wp = w + (size_t)col * P.m + row;
           if (!EDGE || (col < P.n && row + 3 < P.m)) {
@@ -486,6 +503,33 @@ __global__ __launch_bounds__(256) void sgemm_mfma(GemmParams P) {
           }
         }
       }
+  }
+}
+
+// The tiles whose K was shared by several blocks: C = alpha * (sum over their slices, in slice order) + beta * C.
+// A thread takes four rows of a column of one tile; ALIGNED: the result's 16-byte groups are whole and aligned.
+template <int BM, int BN, bool ALIGNED>
+__global__ __launch_bounds__(256) void tail_reduce(GemmParams P) {
+  constexpr int UNITS = BM * BN / 4;   // per tile
+  const int u = (int)(((size_t)blockIdx.x * 256 + threadIdx.x) % UNITS), t = (int)(((size_t)blockIdx.x * 256 + threadIdx.x) / UNITS);
+  if (t >= P.tail_tiles) return;
+  const f4 *w = (const f4 *)P.work + (size_t)t * UNITS + u;
+  const size_t step = (size_t)P.tail_tiles * UNITS;
+  f4 s = w[0];
+  for (int k = 1; k < P.tail_split; k++) s += w[(size_t)k * step];
+  int tm, tn;
+  tile_of(P, P.whole_tiles + t, tm, tn);
+  const int col = tn * BN + u / (BM / 4), row = tm * BM + (u % (BM / 4)) * 4;
+  if (col >= P.n || row >= P.m) return;
+  float *cp = P.c + (size_t)col * P.ldc + row;
+  if (ALIGNED || row + 3 < P.m) {
+    f4 v = P.alpha * s;
+    if (P.beta != 0.f) v += P.beta * *(const f4u *)cp;
+    if (ALIGNED) *(f4 *)cp = v;
+    else *(f4u *)cp = v;
+  } else {
+    for (int c = 0; c < 4; c++)
+      if (row + c < P.m) cp[c] = P.beta != 0.f ? P.alpha * s[c] + P.beta * cp[c] : P.alpha * s[c];
   }
 }
 
@@ -814,6 +858,24 @@ static void choose_ksplit(long tiles, long k, int cus, int &ksplit, int &kchunk)
     kchunk = (int)chunk;
   }
 }
+// Several tiles per CU, but not a whole number of them: the tiles beyond the last multiple of the CUs would occupy
+// some CUs for a whole tile time while the others idle (3072^3 in 128 x 128 tiles: 576 tiles on 256 CUs, 2.25 tile
+// times of work in a launch that takes close to 3).  When they are at most half the CUs, each of them is shared by
+// `split` blocks along K, so that the tail takes 1 / split of a tile time on all CUs, at the price of a pass over
+// those tiles' partial sums.
+static bool plan_tail(long tiles, long k, int cus, int &whole, int &split, int &chunk) {
+  const long q = tiles / cus, r = tiles % cus;
+  if (q < 1 || r == 0 || 2 * r > cus) return false;
+  long s = cus / r;
+  if (s > k / 256) s = k / 256;   // at least 16 slabs a slice
+  if (s > 16) s = 16;
+  if (s < 2) return false;
+  const long c = ((k + s - 1) / s + BK - 1) / BK * BK;
+  whole = (int)(q * cus);
+  split = (int)((k + c - 1) / c);
+  chunk = (int)c;
+  return split >= 2;
+}
 // Tile choice by a small model of the launch, fitted to measurements on 256 CUs (cubes of 1024 to 6144 and ragged
 // shapes, predicted within a few percent):
 //   rate     what the tile's kernel sustains on a large product, in TFLOP/s: whole tiles / tiles with edges
@@ -843,7 +905,9 @@ static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, 
     int ks, kc;
     choose_ksplit(tiles, k, cus, ks, kc);
     const long blocks = tiles * ks, rounds = (blocks + cus - 1) / cus;
-    const double balance = (double)blocks / (double)(rounds * cus);
+    double balance = (double)blocks / (double)(rounds * cus);
+    int tw, tsp, tch;
+    if (ks == 1 && plan_tail(tiles, k, cus, tw, tsp, tch)) balance = ((double)tiles / cus) / ((double)(tiles / cus) + 1.0 / tsp + 0.05);
     const double useful = ((double)m * (double)n) / ((double)(tm * c.bm) * (double)(tn * c.bn));
     const long held = rounds < c.resident ? rounds : c.resident;
     const double fill = held >= 3 ? 1.0 : held == 2 ? 0.9 : 0.75;
@@ -878,9 +942,15 @@ static void launch_stream(bool skc, int nt, dim3 grid, hipStream_t s, const Gemm
 }
 
 // the block tile and the K slicing a product of this shape gets on a chip with `cus` compute units
-void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk) {
+void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk, int *tail_tiles, int *tail_split) {
   choose_tile(m, n, k, cus, k % BK == 0, *bm, *bn);
-  choose_ksplit(((m + *bm - 1) / *bm) * ((n + *bn - 1) / *bn), k, cus, *ksplit, *kchunk);
+  const long tiles = ((m + *bm - 1) / *bm) * ((n + *bn - 1) / *bn);
+  choose_ksplit(tiles, k, cus, *ksplit, *kchunk);
+  int whole = 0, chunk = 0;
+  *tail_tiles = 0;
+  *tail_split = 1;
+  if (*ksplit == 1 && plan_tail(tiles, k, cus, whole, *tail_split, chunk)) *tail_tiles = (int)(tiles - whole);
+  else *tail_split = 1;
 }
 
 void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m, long n, long k, float alpha,
@@ -965,7 +1035,20 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
     P.work = (float *)thcl_rt_workspace(rt, (size_t)P.ksplit * m * n * sizeof(float));
     THCL_CHECK(P.work != nullptr, "gemm workspace: %s", thcl_rt_error());
   }
-  dim3 grid((unsigned)(P.tiles_m * P.tiles_n), (unsigned)P.ksplit);
+  P.whole_tiles = P.tiles_m * P.tiles_n;
+  P.tail_split = 1;
+  if (P.ksplit == 1) {
+    int whole, split, chunk;
+    if (plan_tail((long)P.tiles_m * P.tiles_n, k, cus, whole, split, chunk)) {
+      P.tail_tiles = P.whole_tiles - whole;
+      P.whole_tiles = whole;
+      P.tail_split = split;
+      P.tail_kchunk = chunk;
+      P.work = (float *)thcl_rt_workspace(rt, (size_t)split * P.tail_tiles * bm * bn * sizeof(float));
+      THCL_CHECK(P.work != nullptr, "gemm workspace: %s", thcl_rt_error());
+    }
+  }
+  dim3 grid((unsigned)(P.whole_tiles + P.tail_tiles * P.tail_split), (unsigned)P.ksplit);
 #define GO(BM_, BN_)                                                   \
   if (fast) launch_tt<BM_, BN_, 0>(ta, tb, grid, stream, P);                        \
   else if (short_pitch) launch_tt<BM_, BN_, 1>(ta, tb, grid, stream, P);            \
@@ -978,6 +1061,17 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
   else if (bm == 32 && bn == 128) { GO(32, 128) }
   else { GO(64, 64) }
 #undef GO
+  if (P.tail_tiles > 0) {
+    const bool vec = m % 4 == 0 && ldc % 4 == 0 && al16(c);
+    const unsigned rg = (unsigned)(((size_t)P.tail_tiles * bm * bn / 4 + 255) / 256);
+#define GO(BM_, BN_)                                                                                        \
+  if (bm == BM_ && bn == BN_) {                                                                             \
+    if (vec) hipLaunchKernelGGL((tail_reduce<BM_, BN_, true>), dim3(rg), dim3(256), 0, stream, P);          \
+    else hipLaunchKernelGGL((tail_reduce<BM_, BN_, false>), dim3(rg), dim3(256), 0, stream, P);             \
+  }
+    GO(128, 128) GO(128, 64) GO(64, 128) GO(64, 64) GO(128, 32) GO(32, 128)
+#undef GO
+  }
   if (P.ksplit > 1) {
     const bool vec = m % 4 == 0 && ldc % 4 == 0 && al16(c);
     const size_t total = (size_t)m * n / (vec ? 4 : 1);

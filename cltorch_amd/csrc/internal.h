@@ -151,7 +151,7 @@ void thcl_sgemm(THClState *state, thcl_rt *rt, char transa, char transb, long m,
                 const float *a, long lda, const float *b, long ldb, float beta, float *c, long ldc);
 
 // the block tile and the K slicing a product of this shape gets on a chip with `cus` compute units
-void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk);
+void thcl_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk, int *tail_tiles, int *tail_split);
 
 // ------------------------------------------------------------------ misc ---
 // contiguous device fill / copy kernels used by storage-level calls

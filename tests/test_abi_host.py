@@ -341,17 +341,22 @@ def test_gemm_tile_choice(lib):
     """The tile comes from a model of the launch: the kernel's rate, whole rounds of tiles per CU, the tiles' area
     outside the matrix, blocks per CU, K slicing.  Known outcomes on 256 CUs, each confirmed by measurement."""
     def tile(m, n, k, cus=256):
-        bm, bn, ks, kc = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
-        lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(k), C.c_int(cus), C.byref(bm), C.byref(bn), C.byref(ks), C.byref(kc))
+        bm, bn, ks, kc, tt, ts = (C.c_int(0) for _ in range(6))
+        lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(k), C.c_int(cus), C.byref(bm), C.byref(bn), C.byref(ks), C.byref(kc),
+                               C.byref(tt), C.byref(ts))
         return bm.value, bn.value
     assert tile(8192, 8192, 8192) == (128, 128) and tile(4096, 4096, 4096) == (128, 128) and tile(6144, 6144, 6144) == (128, 128)
     assert tile(16384, 64, 4096) == (128, 64)    # the skinny configuration after the row-major swap
-    assert tile(4608, 4608, 4608) == (128, 64) and tile(5120, 5120, 5120) == (128, 64)   # 6 and 7 rounds of 128x128 tiles leave CUs idle
-    assert tile(3072, 3072, 3072) == (64, 64) and tile(2560, 2560, 2560) == (64, 64)     # 9 and 7 whole rounds of 64x64 tiles
+    # a few tiles more than a whole number per CU: the surplus tiles share their K, so the large tile keeps its rate
+    # (4608^3: 135 TFLOP/s in 128x64 tiles -> 147; 3072^3: 123 in 64x64 tiles -> 145)
+    assert tile(4608, 4608, 4608) == (128, 128) and tile(5120, 5120, 5120) == (128, 128) and tile(3072, 3072, 3072) == (128, 128)
+    assert tile(2560, 2560, 2560) == (128, 64)     # 400 tiles of 128x128 leave more than half the CUs a second tile; 800 of 128x64 leave 32
     assert tile(2048, 2048, 2048) == (64, 64) and tile(1024, 1024, 1024) == (64, 64)
     assert tile(100, 100, 100) == (64, 64)
     # ragged sizes: every tile shape has edges, the larger tiles' edge kernels keep the higher rate
-    assert tile(3000, 5000, 7000) == (128, 128) and tile(6000, 6000, 2000) == (128, 128)
+    assert tile(6000, 6000, 2000) == (128, 128)
+    # 960 tiles of 128x128 are 3.75 per CU; 1920 of 128x64 are 7.5 with the last 104 sharing their K (125 -> 134 TFLOP/s)
+    assert tile(3000, 5000, 7000) == (128, 64)
     # 63 x 64 rows and columns: whole 64-wide tiles (123 x 0.97 for the last round) lose to 128-wide ones with edges (128 x 0.97 of area)
     assert tile(4032, 4032, 4096) == (128, 128)
     # a side of at most 32: thin tiles halve the padding of a 64-wide tile; they never stand for wider products
@@ -365,9 +370,9 @@ def test_gemm_k_slicing(lib):
     two tiles per CU from K = 2048 up, below half a tile per CU from K = 512 up; slices are multiples of the K slab (16)
     and at least 256 long, or 128 where slices of 256 would leave CUs without a block."""
     def plan(m, n, k, cus=256):
-        bm, bn, ks, kc = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
+        bm, bn, ks, kc, tt, ts = (C.c_int(0) for _ in range(6))
         lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(k), C.c_int(cus), C.byref(bm), C.byref(bn),
-                               C.byref(ks), C.byref(kc))
+                               C.byref(ks), C.byref(kc), C.byref(tt), C.byref(ts))
         return bm.value, bn.value, ks.value, kc.value
     assert plan(8192, 8192, 8192) == (128, 128, 1, 8192)
     assert plan(16384, 64, 4096) == (128, 64, 4, 1024)           # skinny: 128 tiles on 256 CUs
@@ -379,6 +384,17 @@ def test_gemm_k_slicing(lib):
     assert plan(128, 128, 1000)[2:] == (7, 144)                  # very few tiles: slices down to 128 (23 -> 9.6 us)
     assert plan(512, 512, 512)[2:] == (4, 128)                   # 64 tiles: 13.2 -> 10.6 us
     assert plan(256, 1024, 1024)[2:] == (4, 256)                 # 64 tiles, and slices of 256 already give every CU a block
+    # several tiles per CU and a few left over (at most half the CUs): those are each shared by floor(CUs / leftover)
+    # blocks along K, at most 16, slices of at least 256
+    def tail(m, n, k, cus=256):
+        v = [C.c_int(0) for _ in range(6)]
+        lib.thcl_dbg_gemm_plan(C.c_long(m), C.c_long(n), C.c_long(k), C.c_int(cus), *[C.byref(x) for x in v])
+        return v[4].value, v[5].value
+    assert tail(3072, 3072, 3072) == (64, 4) and tail(4608, 4608, 4608) == (16, 16) and tail(4100, 4100, 4100) == (65, 3)
+    assert tail(3072, 3072, 600) == (128, 2) and tail(3072, 3072, 500) == (0, 1)     # 1152 tiles of 128x64; K too short to share
+    assert tail(8192, 8192, 8192) == (0, 1) and tail(4095, 4095, 4095) == (0, 1)     # whole numbers of tiles per CU
+    assert tail(6000, 6000, 2000) == (0, 1)                                          # 2209 tiles: 161 left over, more than half the CUs
+    assert tail(64, 64, 100000) == (0, 1)                                            # sliced over the whole grid instead
     for k in (1024, 1040, 3000, 5555):
         _, _, ks, kc = plan(64, 64, k)
         assert kc % 16 == 0 and (ks - 1) * kc < k <= ks * kc and (ks == 1 or kc >= 128)

@@ -241,6 +241,34 @@ def test_unaligned_operands_of_any_extent(cl, M, N, K):
         assert np.max(np.abs(Cd.float() - want)) / scale < RTOL, lay
 
 
+@pytest.mark.parametrize("M,N,K", [(2176, 2176, 1024), (2100, 2200, 1000), (3072, 3072, 512), (4608, 4608, 300), (2049, 2303, 777),
+                                   (2304, 2176, 4100)])
+def test_tiles_beyond_a_whole_number_per_cu_share_their_k(cl, M, N, K):
+    """A few more 128 x 128 tiles than a multiple of the 256 CUs (289, 306, 576, 1296, 306, 306): the surplus tiles are
+    each computed by several blocks along K and summed in slice order.  Whole result against an fp64 product, all four
+    layouts of A and B, whole and ragged sizes, beta = 0 over NaNs, and the same bits on a repeat."""
+    rng = np.random.RandomState(M + N + K)
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(F)
+    b = rng.standard_normal((K, N)).astype(F)
+    c = rng.standard_normal((M, N)).astype(F)
+    prod = a.astype(np.float64) @ b.astype(np.float64)
+    want = 0.5 * c.astype(np.float64) + 1.5 * prod
+    scale = float(np.sqrt(np.mean(want ** 2)))
+    As = (cl.ClTensor(a), cl.ClTensor(np.ascontiguousarray(a.T)).t())
+    Bs = (cl.ClTensor(b), cl.ClTensor(np.ascontiguousarray(b.T)).t())
+    for A in As:
+        for B in Bs:
+            got = cl.ClTensor(c).addmm(0.5, 1.5, A, B).float()
+            assert np.max(np.abs(got - want)) / scale < RTOL, (A.stride(), B.stride())
+    over_nan = cl.ClTensor(np.full((M, N), np.nan, dtype=F)).addmm(0.0, 1.0, As[0], Bs[0]).float()
+    assert np.max(np.abs(over_nan - prod)) / scale < RTOL
+    again = cl.ClTensor(np.full((M, N), np.nan, dtype=F)).addmm(0.0, 1.0, As[0], Bs[0]).float()
+    assert np.array_equal(over_nan, again)
+    Ct = cl.ClTensor(np.ascontiguousarray(c.T)).t()
+    Ct.addmm(0.5, 1.5, As[1], Bs[0])
+    assert np.max(np.abs(Ct.float() - want)) / scale < RTOL
+
+
 def _nan_window(cl, arr, transposed, before, after):
     """device tensor equal to arr (2-D): a window of a larger storage that holds NaN everywhere else (`before` rows
     and elements in front of it, `after` behind it), optionally stored transposed"""

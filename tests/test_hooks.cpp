@@ -105,8 +105,8 @@ int thcl_dbg_plan_kind(int n, const int *nd, long *sizes, long *strides, const l
 // n / d the way the kernels compute it (multiply, shift)
 unsigned thcl_dbg_divide(unsigned n, long d) { return thcl_host_divide(n, d); }
 
-void thcl_dbg_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk) {
-  thcl_gemm_plan(m, n, k, cus, bm, bn, ksplit, kchunk);
+void thcl_dbg_gemm_plan(long m, long n, long k, int cus, int *bm, int *bn, int *ksplit, int *kchunk, int *tail_tiles, int *tail_split) {
+  thcl_gemm_plan(m, n, k, cus, bm, bn, ksplit, kchunk, tail_tiles, tail_split);
 }
 #endif
 }
