@@ -40,6 +40,13 @@ struct IndexParams {
 
 enum Mode { SELECT = 0, COPY = 1, FILL = 2, GATHER = 3, SCATTER = 4, SCATTER_FILL = 5 };
 
+// Called by the lanes that met a bad index (inside their branch): one of them sets the pinned word, so a wave full
+// of bad entries sends one store over the link to host memory, not 64.
+__device__ __forceinline__ void raise_fault(unsigned *word) {
+  const unsigned long long here = __builtin_amdgcn_ballot_w64(true);
+  if ((int)__lane_id() == __ffsll((long long)here) - 1) *word = 1u;
+}
+
 // For duplicate targets the sequential CPU loop leaves the last source slice;
 // winner[j] = max position i with index[i] == j + 1 reproduces that in parallel.
 __global__ __launch_bounds__(kThreads) void index_winner(IndexParams P) {
@@ -47,7 +54,7 @@ __global__ __launch_bounds__(kThreads) void index_winner(IndexParams P) {
   if (i >= P.M) return;
   const long j = (long)P.index[i] - 1;
   if (j >= 0 && j < (long)P.N) atomicMax(P.winner + j, (int)i);
-  else *P.fault = 1u;
+  else raise_fault(P.fault);
 }
 
 template <int MODE, int VEC>
@@ -68,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void index_move(IndexParams P) {
     for (int c = 0; c < VEC; c++) {
       const long j = (long)P.index[boff + c] - 1;
       if (j < 0 || j >= (long)P.N) {
-        *P.fault = 1u;
+        raise_fault(P.fault);
         continue;
       }
       const thcl_u64 aoff = ((thcl_u64)o * P.N + (thcl_u64)j) * P.I + k + c;
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(kThreads) void index_move(IndexParams P) {
   }
   const long j = (long)P.index[i] - 1;
   if (j < 0 || j >= (long)P.N) {
-    if (ku == 0 && o == 0) *P.fault = 1u;  // once per bad entry, not once per unit of its slice
+    if (ku == 0 && o == 0) raise_fault(P.fault);  // once per bad entry, not once per unit of its slice
     return;
   }
   if (MODE == COPY && P.winner[j] != (int)i) return;
@@ -142,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void index_move_by_element(IndexParams P)
 #pragma unroll
   for (int k = 0; k < U; k++) {
     const bool in = j[k] >= 0 && j[k] < (long)P.N;
-    if (!in && ok[k] && !(slice[k] & 0x80000000u)) *P.fault = 1u;
+    if (!in && ok[k] && !(slice[k] & 0x80000000u)) raise_fault(P.fault);
     ok[k] = ok[k] && in;
     aoff[k] += (thcl_u64)(in ? j[k] : 0) * P.I;
   }

@@ -14,6 +14,15 @@
 
 #define THCL_MAX_DIMS 25
 
+// The kernels hand results from block to block with relaxed device-scope accesses ordered by `s_waitcnt vmcnt(0)`
+// and by tickets, which is enough on this chip because its stores complete in the L2 that the reader's loads come
+// from (reduce.hip, index.hip, gemm.hip say so where they do it); tile shapes, LDS sizes and the matrix instructions
+// are this chip's too.  A device pass for any other target stops here instead of building code whose ordering would
+// silently no longer hold; at run time thcl_rt_get refuses devices of another architecture.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "libthcl_hip's kernels are written for gfx950 only: build with --offload-arch=gfx950"
+#endif
+
 // ---------------------------------------------------------------- errors ---
 // A failed check throws ThclError; every extern "C" entry point is wrapped in
 // THCL_GUARD which converts it into the recorded message + handler call, so no

@@ -485,6 +485,7 @@ int thcl_rt_sync(thcl_rt *rt) {
 }
 
 unsigned *thcl_rt_fault_word_device(thcl_rt *rt) { return (unsigned *)(rt->host_word_dev + kFaultWord); }
+int thcl_rt_check_fault(thcl_rt *rt) { return check_fault(rt); }
 
 // A pinned pair of words {value, tag} that a kernel fills with one 8-byte store, so the host can pick a
 // scalar up as soon as it lands instead of waiting for the stream's completion signal.

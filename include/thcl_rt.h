@@ -82,6 +82,9 @@ float *thcl_rt_host_word_device(thcl_rt *rt);
  * the host must hear about (an index outside its range).  thcl_rt_sync and thcl_rt_memcpy_d2h
  * look at it after they have waited: if it is set they clear it and return -3 with a message. */
 unsigned *thcl_rt_fault_word_device(thcl_rt *rt);
+/* The same look without a wait, for a caller that has just waited for the stream by other means (its own event, a
+ * copy through another library): 0, or -3 with the message after clearing the word. */
+int thcl_rt_check_fault(thcl_rt *rt);
 
 /* A scalar handed to the host without waiting for the stream's completion signal: a kernel that is given
  * thcl_rt_tagged_word_device() and a tag from thcl_rt_next_tag() writes {value, tag} there in one 8-byte store when

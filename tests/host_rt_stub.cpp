@@ -96,6 +96,7 @@ int thcl_rt_host_free(void *ptr) { free(ptr); return 0; }
 float *thcl_rt_host_word(thcl_rt *rt) { return rt->host_word; }
 float *thcl_rt_host_word_device(thcl_rt *rt) { return rt->host_word; }
 unsigned *thcl_rt_fault_word_device(thcl_rt *rt) { return (unsigned *)rt->host_word + 32; }
+int thcl_rt_check_fault(thcl_rt *) { return 0; }
 float *thcl_rt_tagged_word_device(thcl_rt *rt) { return rt->host_word + 40; }
 float *thcl_rt_mailbox_device(thcl_rt *rt) { return rt->host_word; }
 const float *thcl_rt_mailbox_host(thcl_rt *rt, size_t *floats) { if (floats) *floats = 0; return rt->host_word; }
