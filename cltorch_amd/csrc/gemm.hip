@@ -879,10 +879,13 @@ static bool plan_tail(long tiles, long k, int cus, int &whole, int &split, int &
 // Tile choice by a small model of the launch, fitted to measurements on 256 CUs (cubes of 1024 to 6144 and ragged
 // shapes, predicted within a few percent):
 //   rate     what the tile's kernel sustains on a large product, in TFLOP/s: whole tiles / tiles with edges
-//   balance  a CU works through whole tiles, so the launch takes ceil(tiles / CUs) tile times
+//   balance  a CU works through whole tiles, so the launch takes ceil(tiles / CUs) tile times, or, when the last
+//            tiles share their K (plan_tail), the whole rounds plus that share of one
 //   useful   the part of the tiles' area that lies inside the matrix
 //   fill     one or two blocks on a CU do not keep its matrix pipes busy
-//   start    a block's first loads and its epilogue cost about as much as 8 of its K slabs
+//   start    a block's first loads and its epilogue cost about as much as 8 of its K slabs, 12 for the largest tile
+//            (whose CU holds few other blocks to work meanwhile; 4096 x 4096 x 256: 92 TFLOP/s in 128 x 128 tiles,
+//            109 in 128 x 64)
 // Products with few tiles are sliced along K as well (choose_ksplit), which fills the chip at the price of a
 // second pass over the result.
 static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, int &bn) {
@@ -890,10 +893,11 @@ static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, 
     int bm, bn;
     double whole, edge;
     int resident;  // blocks a CU holds
+    double start;  // what a block's first loads and its epilogue cost, in K slabs
   };
   // the two thin tiles only stand for products with a side of at most 32, where they halve the padding
-  static const Cand cands[6] = {{128, 128, 138., 134., 3}, {128, 64, 133., 129., 5}, {64, 128, 126., 116., 5},
-                                {64, 64, 123., 119., 8},   {128, 32, 115., 110., 8}, {32, 128, 115., 110., 8}};
+  static const Cand cands[6] = {{128, 128, 147., 140., 3, 12.}, {128, 64, 131., 133., 5, 8.}, {64, 128, 139., 133., 5, 8.},
+                                {64, 64, 127., 127., 8, 8.},    {128, 32, 115., 110., 8, 8.}, {32, 128, 115., 110., 8, 8.}};
   double best = -1.;
   bm = bn = 64;
   for (const Cand &c : cands) {
@@ -911,7 +915,7 @@ static void choose_tile(long m, long n, long k, int cus, bool aligned, int &bm, 
     const double useful = ((double)m * (double)n) / ((double)(tm * c.bm) * (double)(tn * c.bn));
     const long held = rounds < c.resident ? rounds : c.resident;
     const double fill = held >= 3 ? 1.0 : held == 2 ? 0.9 : 0.75;
-    const double slabs = (double)((kc + BK - 1) / BK), start = slabs / (slabs + 8.);
+    const double slabs = (double)((kc + BK - 1) / BK), start = slabs / (slabs + c.start);
     const double score = (whole ? c.whole : c.edge) * balance * useful * fill * start * (ks > 1 ? 0.93 : 1.0);
     if (score > best) {
       best = score;

@@ -346,15 +346,17 @@ def test_gemm_tile_choice(lib):
                                C.byref(tt), C.byref(ts))
         return bm.value, bn.value
     assert tile(8192, 8192, 8192) == (128, 128) and tile(4096, 4096, 4096) == (128, 128) and tile(6144, 6144, 6144) == (128, 128)
-    assert tile(16384, 64, 4096) == (128, 64)    # the skinny configuration after the row-major swap
+    # the skinny configuration after the row-major swap, when the streaming kernel cannot take it (calls in a row: 64x64
+    # tiles in 2 slices 90 us, 128x64 tiles in 4 slices 94)
+    assert tile(16384, 64, 4096) == (64, 64)
     # a few tiles more than a whole number per CU: the surplus tiles share their K, so the large tile keeps its rate
     # (4608^3: 135 TFLOP/s in 128x64 tiles -> 147; 3072^3: 123 in 64x64 tiles -> 145)
     assert tile(4608, 4608, 4608) == (128, 128) and tile(5120, 5120, 5120) == (128, 128) and tile(3072, 3072, 3072) == (128, 128)
-    assert tile(2560, 2560, 2560) == (128, 64)     # 400 tiles of 128x128 leave more than half the CUs a second tile; 800 of 128x64 leave 32
+    assert tile(2560, 2560, 2560) == (64, 128)     # 400 tiles of 128x128 leave more than half the CUs a second tile; 800 of 64x128 leave 32
     assert tile(2048, 2048, 2048) == (64, 64) and tile(1024, 1024, 1024) == (64, 64)
     assert tile(100, 100, 100) == (64, 64)
     # ragged sizes: every tile shape has edges, the larger tiles' edge kernels keep the higher rate
-    assert tile(6000, 6000, 2000) == (128, 128)
+    assert tile(6000, 6000, 2000) == (128, 64)     # 4418 tiles, the last 66 share their K (135 TFLOP/s in 128x128 tiles, 139)
     # 960 tiles of 128x128 are 3.75 per CU; 1920 of 128x64 are 7.5 with the last 104 sharing their K (125 -> 134 TFLOP/s)
     assert tile(3000, 5000, 7000) == (128, 64)
     # 63 x 64 rows and columns: whole 64-wide tiles (123 x 0.97 for the last round) lose to 128-wide ones with edges (128 x 0.97 of area)
@@ -375,8 +377,8 @@ def test_gemm_k_slicing(lib):
                                C.byref(ks), C.byref(kc), C.byref(tt), C.byref(ts))
         return bm.value, bn.value, ks.value, kc.value
     assert plan(8192, 8192, 8192) == (128, 128, 1, 8192)
-    assert plan(16384, 64, 4096) == (128, 64, 4, 1024)           # skinny: 128 tiles on 256 CUs
-    assert plan(2048, 512, 4096) == (128, 64, 4, 1024)           # 128 tiles, long K: the same 512 blocks as 256 tiles in 2 slices, at the larger tile's rate
+    assert plan(16384, 64, 4096) == (64, 64, 2, 2048)            # skinny: 256 tiles on 256 CUs, a long K
+    assert plan(2048, 512, 4096) == (64, 128, 4, 1024)           # 128 tiles, long K: the same 512 blocks as 256 tiles in 2 slices, at the larger tile's rate
     assert plan(1024, 1024, 1024) == (64, 64, 1, 1024)           # 256 tiles but K too short to pay for a second pass
     assert plan(64, 64, 100000)[2] == 368                        # one tile: as many slices of at least 256 as fit
     assert plan(32, 32, 1 << 20)[2] == 512                       # capped
@@ -393,7 +395,8 @@ def test_gemm_k_slicing(lib):
     assert tail(3072, 3072, 3072) == (64, 4) and tail(4608, 4608, 4608) == (16, 16) and tail(4100, 4100, 4100) == (65, 3)
     assert tail(3072, 3072, 600) == (128, 2) and tail(3072, 3072, 500) == (0, 1)     # 1152 tiles of 128x64; K too short to share
     assert tail(8192, 8192, 8192) == (0, 1) and tail(4095, 4095, 4095) == (0, 1)     # whole numbers of tiles per CU
-    assert tail(6000, 6000, 2000) == (0, 1)                                          # 2209 tiles: 161 left over, more than half the CUs
+    assert tail(4096, 6016, 4096) == (0, 1)                                          # 1504 tiles: 224 left over, more than half the CUs
+    assert tail(4096, 7680, 4096) == (128, 2)                                        # 1920 tiles: exactly half the CUs left over
     assert tail(64, 64, 100000) == (0, 1)                                            # sliced over the whole grid instead
     for k in (1024, 1040, 3000, 5555):
         _, _, ks, kc = plan(64, 64, k)
