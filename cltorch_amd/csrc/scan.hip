@@ -304,7 +304,8 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
 // contiguous bytes), so 256 / TC rows per column are combined side by side: thread totals, a
 // shuffle scan over the row groups of a wave, the 4 waves' totals through LDS, then the rows are
 // finished from the registers.  One barrier a step; the rows of the next two steps are requested before
-// this step's work (two steps ahead instead of one: 108 -> 103 us on 4096 x 16384).  TC = 8 for wide tensors; with 4 to 28 columns TC = 1, 2, 4 or 8 covers the whole
+// this step's work (two steps ahead instead of one: 108 -> 103 us on 4096 x 16384).  TC = 16 for wide tensors that
+// have a strip of 64 columns for every CU, else 8; with 4 to 28 columns TC = 1, 2, 4 or 8 covers the whole
 // width and consecutive rows are adjacent in memory, so a step reads one contiguous run.  PHASE 0 leaves the segment's
 // totals, PHASE 1 scans (from the segment's carry when the lines are cut into segments).
 // ANY: the width need not be a multiple of 4 nor the rows 16-byte aligned (narrow tensors only): a thread's up to 4
@@ -719,6 +720,12 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     // Widths that are no multiple of 4, or rows that are not 16-byte aligned, take the same strips one element
     // at a time (2^20 x 3: 106 us with a thread per column, 30 us this way; 2^18 x 27: 37 us).
     int strip_tc = 8;
+    // strips of 64 columns (runs of 256 bytes) when those still give every CU a block: 4096 x 16384 104 -> 98 us,
+    // 2048 x 32768 118 -> 99 us
+    if (strip && P.O * ((P.I / 4 + 15) / 16) >= (thcl_u64)cus) {
+      strip_tc = 16;
+      strips = P.O * ((P.I / 4 + 15) / 16);
+    }
     bool narrow = false, narrow_any = false;
     // (from 1.5 million elements per tensor slice up: below that the three launches of the strips cost more than the
     // thread-per-column walk, 20000 x 8: 42 us against 10)
@@ -798,7 +805,9 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     case 8: STRIP_CASE(false, 4, PH) break;                                                                    \
     case 9: STRIP_CASE(true, 4, PH) break;                                                                     \
     case 16: STRIP_CASE(false, 8, PH) break;                                                                   \
-    default: STRIP_CASE(true, 8, PH) break;                                                                    \
+    case 17: STRIP_CASE(true, 8, PH) break;                                                                    \
+    case 32: STRIP_CASE(false, 16, PH) break;                                                                  \
+    default: STRIP_CASE(true, 16, PH) break;                                                                   \
   }
       if (P.S > 1) {
         STRIP_PHASE(0)

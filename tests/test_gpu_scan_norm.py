@@ -27,7 +27,10 @@ def _scan_close(got, want, what):
 SHAPES = [(1,), (5,), (1023,), (1024,), (4099,), (300000,), (7, 5), (3, 2000), (2000, 3), (64, 4096), (33, 70, 9),
           (4, 300, 128), (2, 3, 4, 5), (1, 50000), (50000, 1), (6, 1 << 16),
           (5000, 2), (5000, 3), (3000, 16), (3000, 18), (700, 100), (700, 256), (300, 1000), (20000, 2048), (9, 7, 130),
-          (1000, 16384), (777, 8200), (3, 700, 4096), (513, 32768),   # outer scans over strips of 32 columns
+          (1000, 16384), (777, 8200), (3, 700, 4096), (513, 32768),
+          # outer scans of 1024 rows and more over strips of 32 columns, and of 64 where those give every CU a block
+          # (whole and ragged last strips, one and two outer slices)
+          (1030, 8192), (1100, 16384), (1500, 16400), (2, 1100, 8200), (1025, 4100), (2600, 16384),
           # a handful of columns and long lines: strips as wide as the tensor, lines cut into segments
           (1 << 20, 4), (300001, 8), (100003, 12), (70000, 28), (3, 40000, 8), (2, 20000, 20), (16384, 16)]
 
@@ -40,7 +43,8 @@ def test_cumsum_every_dim(cl, shape):
         _scan_close(X.cumsum(d + 1).float(), cat.cumulate(x, d), f"cumsum {shape} dim {d + 1}")
 
 
-@pytest.mark.parametrize("shape", [(37,), (5000,), (40, 300), (300, 40), (9, 33, 17), (600, 8200), (50000, 4), (2, 30000, 12)])
+@pytest.mark.parametrize("shape", [(37,), (5000,), (40, 300), (300, 40), (9, 33, 17), (600, 8200), (50000, 4), (2, 30000, 12),
+                                   (1200, 16384), (1040, 8200)])
 def test_cumprod_every_dim(cl, shape):
     x = oracle.uniform(62, int(np.prod(shape)), 0.9, 1.1)
     x[::7] *= -1
