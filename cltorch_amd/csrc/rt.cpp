@@ -449,8 +449,14 @@ int thcl_rt_memcpy_h2d(thcl_rt *rt, void *dst, const void *src, size_t bytes) {
 constexpr int kFaultWord = 32;
 static int check_fault(thcl_rt *rt) {
   volatile unsigned *w = (volatile unsigned *)(rt->host_word + kFaultWord);
-  if (*w == 0u) return 0;
+  const unsigned what = *w;
+  if (what == 0u) return 0;
   *w = 0u;
+  if (what == 2u) {
+    g_err = "scan: the blocks of a single-pass scan did not run at the same time (a wait inside the kernel ran out); "
+            "the result of that scan is not valid";
+    return -3;
+  }
   g_err = "index out of range: an indexing kernel met an index outside 1..size of the indexed dimension "
           "(that entry moved nothing; reported at the first wait after the launch)";
   return -3;

@@ -24,6 +24,7 @@
 
 #include <type_traits>
 
+#include <cstdlib>
 #include <cstring>
 
 #include "apply_device.h"
@@ -571,6 +572,202 @@ __global__ __launch_bounds__(kThreads) void scan_wave_rows(ScanParams P) {
   }
 }
 
+// One long row in one pass over memory (8 bytes an element where the three passes move 12): a launch whose blocks all
+// run at the same time (a cooperative launch, two blocks per CU) walks the row in rounds; in round r block b owns the
+// chunk r * G + b of 8192 elements, so a round is one contiguous run of G chunks.  A block keeps three chunks in
+// registers: the one it scans, the next one, whose total it has already published, and the one after, on its way
+// from memory.  What lies ahead of a chunk is the row's value at the start of the round (published by the round's
+// last block) combined with the totals of the round's chunks in front of it; both were published a whole round
+// earlier, so the block that needs them hardly ever waits, and no block waits for anything published later than its
+// own position in the row: the waits cannot form a cycle.
+// A total travels as one 8-byte word whose bit pattern is the double itself; all ones means "not there yet".  That
+// pattern cannot be a total: it is a NaN whose low mantissa bits are set, and sums and products of values converted
+// from float keep the 29 low bits of every NaN they meet at zero.  Stores and loads of the words are relaxed atomics
+// at device scope (the value is its own flag, nothing else has to be ordered with it).
+// Waits are bounded: after `spin_limit` polls a thread raises the fault word and goes on with what it has, so every
+// wave leaves the kernel whatever happens, and the host reports the launch as failed at its next wait.
+struct ChainParams {
+  const float *in;
+  float *out;
+  thcl_u64 n;                    // elements of the row, a multiple of 4; both pointers 16-byte aligned
+  unsigned long long *totals;    // [rounds][G]
+  unsigned long long *carries;   // [rounds + 1]
+  thcl_u32 rounds;
+  thcl_u32 spin_limit;
+  thcl_u32 mute;                 // a block that publishes nothing (tests of the give-up path; no block otherwise)
+  unsigned *fault;
+};
+constexpr unsigned long long kChainNotYet = ~0ull;
+constexpr int kChainSteps = 2;                       // steps of 4096 elements per chunk
+constexpr thcl_u64 kChainChunk = kChainSteps * 4096;
+constexpr thcl_u64 kChainFrom = 1ull << 24;          // rows from this length up (2^24: 34.5 us against 36.8 for the three passes, 2^28: 400 against 504)
+
+__global__ __launch_bounds__(kThreads) void scan_chain_init(unsigned long long *words, thcl_u64 count) {
+  const thcl_u64 i = (thcl_u64)blockIdx.x * kThreads + threadIdx.x;
+  if (i < count) words[i] = kChainNotYet;
+}
+
+template <bool PROD>
+__global__ __launch_bounds__(kThreads) void scan_chain(ChainParams P) {
+  constexpr int WAVES = kThreads / kWave, PER = 4, RUN = kThreads * PER, UNR = 4, STEP = RUN * UNR, SPC = kChainSteps;
+  __shared__ double wave_tot[UNR][WAVES];
+  __shared__ double fold[2][WAVES];
+  const thcl_u32 G = gridDim.x, b = blockIdx.x;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const thcl_u64 last_group = P.n - PER;
+  bool gave_up = false;   // this thread has met a wait that did not end: it does not wait again
+  auto await = [&](const unsigned long long *p) {
+    unsigned long long bits = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    thcl_u32 spins = 0;
+    while (bits == kChainNotYet && !gave_up) {
+      if (++spins > P.spin_limit) {
+        gave_up = true;
+        *P.fault = 2u;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+      bits = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return __builtin_bit_cast(double, bits);
+  };
+  auto publish = [&](unsigned long long *p, double v) {
+    if (b == P.mute) return;
+    __hip_atomic_store(p, __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // block-wide combination in a fixed order: lanes by butterfly, then the waves in order
+  // (two values at a time: one pair of barriers serves a chunk's total and what lies ahead of another chunk)
+  auto block_fold = [&](double &p, double &q) {
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+      p = Op<PROD>::comb(p, __shfl_xor(p, d, kWave));
+      q = Op<PROD>::comb(q, __shfl_xor(q, d, kWave));
+    }
+    if (lane == 0) {
+      fold[0][wave] = p;
+      fold[1][wave] = q;
+    }
+    __syncthreads();
+    p = fold[0][0];
+    q = fold[1][0];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) {
+      p = Op<PROD>::comb(p, fold[0][w]);
+      q = Op<PROD>::comb(q, fold[1][w]);
+    }
+    __syncthreads();
+  };
+  typedef float Chunk[SPC][UNR][PER];
+  // every load is issued: groups past the end of the row read its last group again and count as the identity below
+  auto fetch = [&](Chunk &x, thcl_u64 chunk) {
+    const thcl_u64 base = chunk * kChainChunk + (thcl_u64)threadIdx.x * PER;
+#pragma unroll
+    for (int st = 0; st < SPC; st++)
+#pragma unroll
+      for (int u = 0; u < UNR; u++) {
+        const thcl_u64 j = base + (thcl_u64)st * STEP + (thcl_u64)u * RUN;
+        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(P.in + (j < P.n ? j : last_group)));
+#pragma unroll
+        for (int c = 0; c < PER; c++) x[st][u][c] = v[c];
+      }
+  };
+  const float fill = PROD ? 1.0f : 0.0f;
+  auto chunk_partial = [&](const Chunk &x, thcl_u64 chunk) {   // this thread's part of a chunk's total
+    const thcl_u64 base = chunk * kChainChunk + (thcl_u64)threadIdx.x * PER;
+    double t = Op<PROD>::identity();
+#pragma unroll
+    for (int st = 0; st < SPC; st++)
+#pragma unroll
+      for (int u = 0; u < UNR; u++) {
+        const bool in = base + (thcl_u64)st * STEP + (thcl_u64)u * RUN < P.n;
+#pragma unroll
+        for (int c = 0; c < PER; c++) t = Op<PROD>::comb(t, (double)(in ? x[st][u][c] : fill));
+      }
+    return t;
+  };
+  // the scan of one chunk from its registers, `carry` being everything ahead of it (as in scan_row)
+  auto scan_chunk = [&](const Chunk &x, thcl_u64 chunk, double carry) {
+#pragma unroll
+    for (int st = 0; st < SPC; st++) {
+      const thcl_u64 base = chunk * kChainChunk + (thcl_u64)st * STEP;
+      double a[UNR][PER], incl[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; u++) {
+        const bool in = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER < P.n;
+        a[u][0] = (double)(in ? x[st][u][0] : fill);
+#pragma unroll
+        for (int c = 1; c < PER; c++) a[u][c] = Op<PROD>::comb(a[u][c - 1], (double)(in ? x[st][u][c] : fill));
+        incl[u] = wave_inclusive<PROD>(a[u][PER - 1]);
+      }
+      __syncthreads();  // wave_tot of the previous step has been read
+      if (lane == kWave - 1) {
+#pragma unroll
+        for (int u = 0; u < UNR; u++) wave_tot[u][wave] = incl[u];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < UNR; u++) {
+        double before = carry;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) {
+          if (w < wave) before = Op<PROD>::comb(before, wave_tot[u][w]);
+          carry = Op<PROD>::comb(carry, wave_tot[u][w]);
+        }
+        const double prev = __shfl_up(incl[u], 1, kWave);
+        if (lane > 0) before = Op<PROD>::comb(before, prev);
+        const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
+        if (j < P.n) {
+          thcl_f4 v;
+#pragma unroll
+          for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[u][c]);
+          __builtin_nontemporal_store(v, (thcl_f4 *)(P.out + j));
+        }
+      }
+    }
+  };
+  double tot_cur;   // this block's total of the chunk it scans next
+  auto peek = [&](const unsigned long long *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+  auto round = [&](Chunk &cur, Chunk &next, Chunk &far, thcl_u32 r) {
+    // what lies ahead of this round's chunk was published a round ago: its words are requested first, so that their
+    // trip through memory runs beside the work on the next chunk's total, and they are looked at after it
+    const thcl_u32 k0 = threadIdx.x, k1 = threadIdx.x + kThreads;
+    const unsigned long long *row = P.totals + (thcl_u64)r * G;
+    unsigned long long w0 = 0, w1 = 0, wc = 0;
+    if (k0 < b) w0 = peek(row + k0);
+    if (k1 < b) w1 = peek(row + k1);
+    if (threadIdx.x == 0 && r > 0) wc = peek(P.carries + r);
+    fetch(far, (thcl_u64)(r + 2) * G + b);
+    __builtin_amdgcn_sched_barrier(0);
+    double tot_next = chunk_partial(next, (thcl_u64)(r + 1) * G + b);
+    double mine = Op<PROD>::identity();
+    if (threadIdx.x == 0 && r > 0) mine = wc != kChainNotYet ? __builtin_bit_cast(double, wc) : await(P.carries + r);
+    if (k0 < b) mine = Op<PROD>::comb(mine, w0 != kChainNotYet ? __builtin_bit_cast(double, w0) : await(row + k0));
+    if (k1 < b) mine = Op<PROD>::comb(mine, w1 != kChainNotYet ? __builtin_bit_cast(double, w1) : await(row + k1));
+    block_fold(tot_next, mine);
+    const double ahead = mine;
+    if (threadIdx.x == 0 && r + 1 < P.rounds) publish(P.totals + (thcl_u64)(r + 1) * G + b, tot_next);
+    if (b == G - 1 && threadIdx.x == 0) publish(P.carries + r + 1, Op<PROD>::comb(ahead, tot_cur));
+    scan_chunk(cur, (thcl_u64)r * G + b, ahead);
+    tot_cur = tot_next;
+  };
+  Chunk xa, xb, xc;
+  fetch(xa, b);
+  fetch(xb, (thcl_u64)G + b);
+  {
+    double none = Op<PROD>::identity();
+    tot_cur = chunk_partial(xa, b);
+    block_fold(tot_cur, none);
+  }
+  if (threadIdx.x == 0) publish(P.totals + b, tot_cur);
+  for (thcl_u32 r = 0;;) {
+    round(xa, xb, xc, r);
+    if (++r >= P.rounds) break;
+    round(xb, xc, xa, r);
+    if (++r >= P.rounds) break;
+    round(xc, xa, xb, r);
+    if (++r >= P.rounds) break;
+  }
+}
+
 template <bool PROD, int G>
 void launch_short(hipStream_t stream, const ScanParams &P, bool vec) {
   const dim3 grid((unsigned)((P.O + kThreads / G - 1) / (kThreads / G))), block(kThreads);
@@ -607,6 +804,48 @@ void launch_carries(hipStream_t stream, const ScanParams &P) {
   else
     hipLaunchKernelGGL((scan_carries<PROD>), dim3((unsigned)((lines + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, P);
   check("scan carries");
+}
+
+// The single-pass scan of a few long rows, one launch per row.  The grid is what the chip holds at one time (the
+// occupancy the runtime reports for the kernel, at most two blocks per CU); the launches of a context run in order on
+// its one stream, so nothing of the library's competes for the CUs, and should another client of the GPU keep blocks
+// from starting, the kernel's bounded waits end the launch with an error report instead of a result.
+// False: not started (the kernel does not fit a CU), and the caller takes the three passes.
+template <bool PROD>
+bool run_chain(thcl_rt *rt, hipStream_t stream, const ScanParams &S) {
+  static int per_cu = -1;   // blocks of scan_chain a CU holds at a time, at most 2
+  static thcl_u32 spin_limit = 1u << 20, mute = ~0u;
+  if (per_cu < 0) {
+    int nb = 0, nbp = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, scan_chain<false>, kThreads, 0) != hipSuccess) nb = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nbp, scan_chain<true>, kThreads, 0) != hipSuccess) nbp = 0;
+    if (nbp < nb) nb = nbp;
+    (void)hipGetLastError();
+    per_cu = nb > 2 ? 2 : nb;
+    // for tests of the give-up path: how often a wait polls before it gives up, and a block that publishes nothing
+    if (const char *e = getenv("THCL_SCAN_CHAIN_SPINS")) spin_limit = (thcl_u32)strtoul(e, nullptr, 10);
+    if (const char *e = getenv("THCL_SCAN_CHAIN_MUTE")) mute = (thcl_u32)strtoul(e, nullptr, 10);
+  }
+  if (per_cu <= 0) return false;
+  const thcl_u32 G = (thcl_u32)(thcl_rt_get_props(rt)->compute_units * per_cu);
+  ChainParams C;
+  C.n = S.R;
+  C.rounds = (thcl_u32)((S.R + (thcl_u64)G * kChainChunk - 1) / ((thcl_u64)G * kChainChunk));
+  C.spin_limit = spin_limit;
+  C.mute = mute;
+  C.fault = thcl_rt_fault_word_device(rt);
+  const thcl_u64 words = (thcl_u64)C.rounds * G + C.rounds + 1;
+  C.totals = (unsigned long long *)thcl_rt_workspace(rt, (size_t)words * sizeof(unsigned long long));
+  THCL_CHECK(C.totals != nullptr, "%s", thcl_rt_error());
+  C.carries = C.totals + (thcl_u64)C.rounds * G;
+  for (thcl_u64 o = 0; o < S.O; o++) {
+    C.in = S.in + o * S.R;
+    C.out = S.out + o * S.R;
+    hipLaunchKernelGGL(scan_chain_init, dim3((unsigned)((words + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, C.totals, words);
+    hipLaunchKernelGGL(scan_chain<PROD>, dim3(G), dim3(kThreads), 0, stream, C);
+  }
+  check("scan");
+  return true;
 }
 
 template <bool PROD>
@@ -819,6 +1058,8 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
 #undef STRIP_PHASE
 #undef STRIP_CASE
       check("scan");
+    } else if (rows && vec && P.O <= 16 && P.S > 1 && P.R >= kChainFrom && (prod ? run_chain<true>(rt, stream, P) : run_chain<false>(rt, stream, P))) {
+      // a few long rows: a single pass over each
     } else if (prod) {
       run_scan<true>(stream, P, rows, vec);
     } else {

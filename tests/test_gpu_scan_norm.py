@@ -54,6 +54,37 @@ def test_cumprod_every_dim(cl, shape):
         _scan_close(X.cumprod(d + 1).float(), cat.cumulate(x, d, prod=True), f"cumprod {shape} dim {d + 1}")
 
 
+@pytest.mark.parametrize("shape,prod", [(((1 << 24) + 4096,), False), (((1 << 25) + 8200 * 4,), False), ((3, 1 << 24), False),
+                                        (((1 << 24) + 12,), True), ((1 << 27,), False)])
+def test_long_rows_in_one_pass(cl, shape, prod):
+    """Rows of 2^24 elements and more (a multiple of 4, aligned) are scanned in one pass by blocks that hand their
+    totals on while they run: whole and ragged last rounds, several rows, sums and products."""
+    n = int(np.prod(shape))
+    x = (oracle.uniform(71, n, 0.9995, 1.0005) if prod else oracle.uniform(72, n)).reshape(shape)
+    X = cl.ClTensor(x)
+    d = len(shape)
+    got = (X.cumprod(d) if prod else X.cumsum(d)).float()
+    _scan_close(got, cat.cumulate(x, d - 1, prod=prod), f"long rows {shape}")
+    if not prod and len(shape) == 1:
+        ones = cl.ClTensor(n)
+        ones.fill(1.0)
+        assert np.array_equal(ones.cumsum().float(), np.arange(1, n + 1, dtype=np.float64).astype(F))   # exact below 2^24, rounded above
+
+
+def test_single_pass_scan_gives_up_instead_of_hanging(cl):
+    """A block of the single-pass scan that never publishes its totals (forced from the host, with waits that poll
+    once): every kernel still ends, the failure is reported at the next wait and the library keeps working
+    (tests/scan_give_up_child.py, in a process of its own because both switches are read once)."""
+    import os
+    import subprocess
+    import sys
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "scan_give_up_child.py")
+    env = dict(os.environ, THCL_SCAN_CHAIN_SPINS="0", THCL_SCAN_CHAIN_MUTE="0")
+    r = subprocess.run([sys.executable, child], capture_output=True, text=True, env=env, timeout=110)
+    assert r.returncode == 0, (r.stdout + r.stderr)[-3000:]
+    assert "scan give-up ok" in r.stdout
+
+
 def test_scan_closed_forms_views_and_in_place(cl):
     n = 1 << 22                                             # long row: segments + carries
     ones = cl.ClTensor(n)
