@@ -572,12 +572,14 @@ __global__ __launch_bounds__(kThreads) void scan_wave_rows(ScanParams P) {
   }
 }
 
-// One long row in one pass over memory (8 bytes an element where the three passes move 12): a launch whose blocks all
-// run at the same time (a cooperative launch, two blocks per CU) walks the row in rounds; in round r block b owns the
-// chunk r * G + b of 8192 elements, so a round is one contiguous run of G chunks.  A block keeps three chunks in
+// Long rows, too few to fill the chip with a block each, in one pass over memory (8 bytes an element where the three
+// passes move 12): a launch whose blocks all run at the same time (two per CU) walks the rows in rounds.  Every row is
+// cut into chunks of 8192 elements (its last one may be short), the chunks of all rows are numbered in memory order,
+// and in round r block b owns chunk r * G + b, so a round is one run of G chunks.  A block keeps three chunks in
 // registers: the one it scans, the next one, whose total it has already published, and the one after, on its way
-// from memory.  What lies ahead of a chunk is the row's value at the start of the round (published by the round's
-// last block) combined with the totals of the round's chunks in front of it; both were published a whole round
+// from memory.  What lies ahead of a chunk is its row's value at the start of the round (published by the last block
+// of the round before, and used when the row began before this round) combined with the totals of the round's chunks
+// in front of it in the same row; both were published a whole round
 // earlier, so the block that needs them hardly ever waits, and no block waits for anything published later than its
 // own position in the row: the waits cannot form a cycle.
 // A total travels as one 8-byte word whose bit pattern is the double itself; all ones means "not there yet".  That
@@ -589,7 +591,9 @@ __global__ __launch_bounds__(kThreads) void scan_wave_rows(ScanParams P) {
 struct ChainParams {
   const float *in;
   float *out;
-  thcl_u64 n;                    // elements of the row, a multiple of 4; both pointers 16-byte aligned
+  thcl_u64 R;                    // elements of a row, a multiple of 4; both pointers 16-byte aligned
+  thcl_u64 total;                // elements of all rows
+  thcl_u32 cpr, nchunks;         // chunks per row (the last one may be short), chunks of all rows
   unsigned long long *totals;    // [rounds][G]
   unsigned long long *carries;   // [rounds + 1]
   thcl_u32 rounds;
@@ -614,7 +618,19 @@ __global__ __launch_bounds__(kThreads) void scan_chain(ChainParams P) {
   __shared__ double fold[2][WAVES];
   const thcl_u32 G = gridDim.x, b = blockIdx.x;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const thcl_u64 last_group = P.n - PER;
+  const thcl_u64 last_group = P.total - PER;
+  // chunk q of the whole tensor: where it starts, where its row ends, and which chunk is its row's first
+  // (a chunk past the last one holds nothing and stands for a row of its own)
+  auto place = [&](thcl_u64 q, thcl_u64 &base, thcl_u64 &lim) {
+    if (q >= P.nchunks) {
+      base = lim = P.total;
+      return (thcl_u32)q;
+    }
+    const thcl_u32 row = (thcl_u32)q / P.cpr, cin = (thcl_u32)q - row * P.cpr;
+    base = (thcl_u64)row * P.R + (thcl_u64)cin * kChainChunk;
+    lim = (thcl_u64)row * P.R + P.R;
+    return row * P.cpr;
+  };
   bool gave_up = false;   // this thread has met a wait that did not end: it does not wait again
   auto await = [&](const unsigned long long *p) {
     unsigned long long bits = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -659,26 +675,30 @@ __global__ __launch_bounds__(kThreads) void scan_chain(ChainParams P) {
   typedef float Chunk[SPC][UNR][PER];
   // every load is issued: groups past the end of the row read its last group again and count as the identity below
   auto fetch = [&](Chunk &x, thcl_u64 chunk) {
-    const thcl_u64 base = chunk * kChainChunk + (thcl_u64)threadIdx.x * PER;
+    thcl_u64 base, lim;
+    place(chunk, base, lim);
+    base += (thcl_u64)threadIdx.x * PER;
 #pragma unroll
     for (int st = 0; st < SPC; st++)
 #pragma unroll
       for (int u = 0; u < UNR; u++) {
         const thcl_u64 j = base + (thcl_u64)st * STEP + (thcl_u64)u * RUN;
-        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(P.in + (j < P.n ? j : last_group)));
+        const thcl_f4 v = __builtin_nontemporal_load((const thcl_f4 *)(P.in + (j < lim ? j : last_group)));
 #pragma unroll
         for (int c = 0; c < PER; c++) x[st][u][c] = v[c];
       }
   };
   const float fill = PROD ? 1.0f : 0.0f;
   auto chunk_partial = [&](const Chunk &x, thcl_u64 chunk) {   // this thread's part of a chunk's total
-    const thcl_u64 base = chunk * kChainChunk + (thcl_u64)threadIdx.x * PER;
+    thcl_u64 base, lim;
+    place(chunk, base, lim);
+    base += (thcl_u64)threadIdx.x * PER;
     double t = Op<PROD>::identity();
 #pragma unroll
     for (int st = 0; st < SPC; st++)
 #pragma unroll
       for (int u = 0; u < UNR; u++) {
-        const bool in = base + (thcl_u64)st * STEP + (thcl_u64)u * RUN < P.n;
+        const bool in = base + (thcl_u64)st * STEP + (thcl_u64)u * RUN < lim;
 #pragma unroll
         for (int c = 0; c < PER; c++) t = Op<PROD>::comb(t, (double)(in ? x[st][u][c] : fill));
       }
@@ -686,13 +706,15 @@ __global__ __launch_bounds__(kThreads) void scan_chain(ChainParams P) {
   };
   // the scan of one chunk from its registers, `carry` being everything ahead of it (as in scan_row)
   auto scan_chunk = [&](const Chunk &x, thcl_u64 chunk, double carry) {
+    thcl_u64 first, lim;
+    place(chunk, first, lim);
 #pragma unroll
     for (int st = 0; st < SPC; st++) {
-      const thcl_u64 base = chunk * kChainChunk + (thcl_u64)st * STEP;
+      const thcl_u64 base = first + (thcl_u64)st * STEP;
       double a[UNR][PER], incl[UNR];
 #pragma unroll
       for (int u = 0; u < UNR; u++) {
-        const bool in = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER < P.n;
+        const bool in = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER < lim;
         a[u][0] = (double)(in ? x[st][u][0] : fill);
 #pragma unroll
         for (int c = 1; c < PER; c++) a[u][c] = Op<PROD>::comb(a[u][c - 1], (double)(in ? x[st][u][c] : fill));
@@ -715,7 +737,7 @@ __global__ __launch_bounds__(kThreads) void scan_chain(ChainParams P) {
         const double prev = __shfl_up(incl[u], 1, kWave);
         if (lane > 0) before = Op<PROD>::comb(before, prev);
         const thcl_u64 j = base + (thcl_u64)u * RUN + (thcl_u64)threadIdx.x * PER;
-        if (j < P.n) {
+        if (j < lim) {
           thcl_f4 v;
 #pragma unroll
           for (int c = 0; c < PER; c++) v[c] = (float)Op<PROD>::comb(before, a[u][c]);
@@ -729,19 +751,27 @@ __global__ __launch_bounds__(kThreads) void scan_chain(ChainParams P) {
   auto round = [&](Chunk &cur, Chunk &next, Chunk &far, thcl_u32 r) {
     // what lies ahead of this round's chunk was published a round ago: its words are requested first, so that their
     // trip through memory runs beside the work on the next chunk's total, and they are looked at after it
+    // (of this chunk's own row only: the round's chunks from the row's first one on, and the value at the start of
+    // the round when the row began before it)
+    thcl_u64 unused0, unused1;
+    const thcl_u64 round_first = (thcl_u64)r * G;
+    const thcl_u32 row_first = place(round_first + b, unused0, unused1);
+    const thcl_u32 k_lo = row_first > round_first ? (thcl_u32)(row_first - round_first) : 0u;
+    const bool began_before = r > 0 && row_first < round_first;
     const thcl_u32 k0 = threadIdx.x, k1 = threadIdx.x + kThreads;
-    const unsigned long long *row = P.totals + (thcl_u64)r * G;
+    const bool take0 = k0 >= k_lo && k0 < b, take1 = k1 >= k_lo && k1 < b, takec = threadIdx.x == 0 && began_before;
+    const unsigned long long *row = P.totals + round_first;
     unsigned long long w0 = 0, w1 = 0, wc = 0;
-    if (k0 < b) w0 = peek(row + k0);
-    if (k1 < b) w1 = peek(row + k1);
-    if (threadIdx.x == 0 && r > 0) wc = peek(P.carries + r);
+    if (take0) w0 = peek(row + k0);
+    if (take1) w1 = peek(row + k1);
+    if (takec) wc = peek(P.carries + r);
     fetch(far, (thcl_u64)(r + 2) * G + b);
     __builtin_amdgcn_sched_barrier(0);
     double tot_next = chunk_partial(next, (thcl_u64)(r + 1) * G + b);
     double mine = Op<PROD>::identity();
-    if (threadIdx.x == 0 && r > 0) mine = wc != kChainNotYet ? __builtin_bit_cast(double, wc) : await(P.carries + r);
-    if (k0 < b) mine = Op<PROD>::comb(mine, w0 != kChainNotYet ? __builtin_bit_cast(double, w0) : await(row + k0));
-    if (k1 < b) mine = Op<PROD>::comb(mine, w1 != kChainNotYet ? __builtin_bit_cast(double, w1) : await(row + k1));
+    if (takec) mine = wc != kChainNotYet ? __builtin_bit_cast(double, wc) : await(P.carries + r);
+    if (take0) mine = Op<PROD>::comb(mine, w0 != kChainNotYet ? __builtin_bit_cast(double, w0) : await(row + k0));
+    if (take1) mine = Op<PROD>::comb(mine, w1 != kChainNotYet ? __builtin_bit_cast(double, w1) : await(row + k1));
     block_fold(tot_next, mine);
     const double ahead = mine;
     if (threadIdx.x == 0 && r + 1 < P.rounds) publish(P.totals + (thcl_u64)(r + 1) * G + b, tot_next);
@@ -806,7 +836,7 @@ void launch_carries(hipStream_t stream, const ScanParams &P) {
   check("scan carries");
 }
 
-// The single-pass scan of a few long rows, one launch per row.  The grid is what the chip holds at one time (the
+// The single-pass scan of rows that are too few to fill the chip with a block each.  The grid is what the chip holds at one time (the
 // occupancy the runtime reports for the kernel, at most two blocks per CU); the launches of a context run in order on
 // its one stream, so nothing of the library's competes for the CUs, and should another client of the GPU keep blocks
 // from starting, the kernel's bounded waits end the launch with an error report instead of a result.
@@ -828,9 +858,16 @@ bool run_chain(thcl_rt *rt, hipStream_t stream, const ScanParams &S) {
   }
   if (per_cu <= 0) return false;
   const thcl_u32 G = (thcl_u32)(thcl_rt_get_props(rt)->compute_units * per_cu);
+  const thcl_u64 cpr = (S.R + kChainChunk - 1) / kChainChunk;
+  if (cpr * S.O >= (1ull << 31)) return false;
   ChainParams C;
-  C.n = S.R;
-  C.rounds = (thcl_u32)((S.R + (thcl_u64)G * kChainChunk - 1) / ((thcl_u64)G * kChainChunk));
+  C.in = S.in;
+  C.out = S.out;
+  C.R = S.R;
+  C.total = S.O * S.R;
+  C.cpr = (thcl_u32)cpr;
+  C.nchunks = (thcl_u32)(cpr * S.O);
+  C.rounds = (C.nchunks + G - 1) / G;
   C.spin_limit = spin_limit;
   C.mute = mute;
   C.fault = thcl_rt_fault_word_device(rt);
@@ -838,12 +875,8 @@ bool run_chain(thcl_rt *rt, hipStream_t stream, const ScanParams &S) {
   C.totals = (unsigned long long *)thcl_rt_workspace(rt, (size_t)words * sizeof(unsigned long long));
   THCL_CHECK(C.totals != nullptr, "%s", thcl_rt_error());
   C.carries = C.totals + (thcl_u64)C.rounds * G;
-  for (thcl_u64 o = 0; o < S.O; o++) {
-    C.in = S.in + o * S.R;
-    C.out = S.out + o * S.R;
-    hipLaunchKernelGGL(scan_chain_init, dim3((unsigned)((words + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, C.totals, words);
-    hipLaunchKernelGGL(scan_chain<PROD>, dim3(G), dim3(kThreads), 0, stream, C);
-  }
+  hipLaunchKernelGGL(scan_chain_init, dim3((unsigned)((words + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, C.totals, words);
+  hipLaunchKernelGGL(scan_chain<PROD>, dim3(G), dim3(kThreads), 0, stream, C);
   check("scan");
   return true;
 }
@@ -1058,8 +1091,8 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
 #undef STRIP_PHASE
 #undef STRIP_CASE
       check("scan");
-    } else if (rows && vec && P.O <= 16 && P.S > 1 && P.R >= kChainFrom && (prod ? run_chain<true>(rt, stream, P) : run_chain<false>(rt, stream, P))) {
-      // a few long rows: a single pass over each
+    } else if (rows && vec && P.S > 1 && total >= kChainFrom && (prod ? run_chain<true>(rt, stream, P) : run_chain<false>(rt, stream, P))) {
+      // rows too few to fill the chip, 2^24 elements and more: a single pass
     } else if (prod) {
       run_scan<true>(stream, P, rows, vec);
     } else {

@@ -55,10 +55,14 @@ def test_cumprod_every_dim(cl, shape):
 
 
 @pytest.mark.parametrize("shape,prod", [(((1 << 24) + 4096,), False), (((1 << 25) + 8200 * 4,), False), ((3, 1 << 24), False),
-                                        (((1 << 24) + 12,), True), ((1 << 27,), False)])
+                                        (((1 << 24) + 12,), True), ((1 << 27,), False),
+                                        ((64, 1 << 20), False), ((5, (1 << 22) + 4000), False), ((256, 1 << 16), False),
+                                        ((700, 30000), False), ((2, 3, (1 << 22) - 8), True), ((767, 21880), False)])
 def test_long_rows_in_one_pass(cl, shape, prod):
-    """Rows of 2^24 elements and more (a multiple of 4, aligned) are scanned in one pass by blocks that hand their
-    totals on while they run: whole and ragged last rounds, several rows, sums and products."""
+    """2^24 elements and more in rows (a multiple of 4 long, aligned) that are too few for a block each are scanned in
+    one pass by blocks that hand their totals on while they run: whole and ragged last chunks and rounds, one row and
+    several hundred (a row's chunks in one round, across rounds, rows that begin in the middle of a round), sums and
+    products."""
     n = int(np.prod(shape))
     x = (oracle.uniform(71, n, 0.9995, 1.0005) if prod else oracle.uniform(72, n)).reshape(shape)
     X = cl.ClTensor(x)
