@@ -8,13 +8,18 @@
 // BM x BN block tile (4x1 or 1x4 over the 128x32 and 32x128 tiles that serve
 // products with one side of at most 32); K advances in slabs of 16 staged through double-buffered
 // LDS (one barrier per slab), the next slab's global loads are issued before
-// the current slab's MFMAs.  Operands that are contiguous along m/n in memory
-// sit in LDS as [k][mn] and are read one dword per MFMA; operands contiguous
-// along k sit as [mn][k+4] and are read 128 bits per four MFMAs.  Within a
-// group of 8 k-values, MFMA step s consumes k = s (lanes 0-31) and k = 4+s
-// (lanes 32-63) for both operands, which is what makes the 128-bit read usable.
-// Blocks are renumbered so the blocks an XCD receives form a compact patch of
-// the tile grid and share its L2.
+// the current slab's MFMAs (two slabs ahead, through buffer descriptors whose
+// base moves with scalar arithmetic, so the loop computes no address with vector
+// instructions).  Operands that are contiguous along m/n in memory sit in LDS as
+// [k][mn] with the wave's sub-tiles interleaved, and are read 64 bits per two
+// MFMAs; operands contiguous along k sit as [mn][k+4] and are read 128 bits per
+// four MFMAs.  Within a group of 8 k-values, MFMA step s consumes k = s (lanes
+// 0-31) and k = 4+s (lanes 32-63) for both operands, which is what makes the
+// 128-bit read usable.  Blocks are renumbered so the blocks an XCD receives form
+// a compact patch of the tile grid and share its L2; tiles beyond a whole number
+// per CU share their K among several blocks of the same launch (plan_tail).
+// A product with a short side streams its long operand from memory straight into
+// the matrix cores (sgemm_stream, further down).
 #include <hip/hip_runtime.h>
 
 #include <cstring>
