@@ -508,6 +508,10 @@ def detail(cl, oracle, T, X, Y, Z, n):
         d["kernel_only_source"] = PROFILE_SUMMARY + " (rocprofv3 --kernel-trace of `bench.py --pmc-configs`, committed)"
     sk = d["c5_addmm_skinny_64x16384x4096"]
     sk["hbm_GBs"] = round(4.0 * (64 * 4096 + 4096 * 16384 + 2 * 64 * 16384) / (sk["avg_ms"] * 1e-3) * 1e-9, 1)
+    if "w_addmm_32x16384x4096" in d:   # bound by its long operand's bytes rather than by the matrix cores
+        sk = d["w_addmm_32x16384x4096"]
+        sk["hbm_GBs"] = round(4.0 * (32 * 4096 + 4096 * 16384 + 2 * 32 * 16384) / (sk["avg_ms"] * 1e-3) * 1e-9, 1)
+        sk["frac_of_hbm_peak"] = round(sk["hbm_GBs"] / 8000.0, 4)
 
     # config 4 as one chain: sumall_gpu + div_gpu + 8 in-place ops, one sync at the end
     pt = cl.ClTensor()
