@@ -788,23 +788,34 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
   }
   __syncthreads();
   if (!s_last) return;
+  // J = UB * VEC slices (a power of two, at most 256) share the block's threads: kThreads / J threads walk a slice's
+  // partials side by side (split index `parts` apart, up to 8 loads requested together), meet in LDS and are folded in
+  // order of their first split index
   const T *partials = (const T *)P.partials;
-  for (thcl_u32 j = threadIdx.x; j < UB * VEC; j += kThreads) {
-    const thcl_u32 s = blockIdx.x * (UB * VEC) + j;
-    if (s < P.nslices) {
-      T t = S::init();
-      thcl_u32 k = 0;
-      constexpr int B = 16;  // partials fetched together
-      for (; k + B <= P.split; k += B) {
-        T v[B];
+  const thcl_u32 J = UB * VEC, parts = (thcl_u32)kThreads / J;
+  const thcl_u32 j = threadIdx.x % J, part = threadIdx.x / J;
+  const thcl_u32 sj = blockIdx.x * J + j;
+  const bool live = sj < P.nslices;
+  T t = S::init();
+  if (live) {
+    constexpr int B = 8;
+    thcl_u32 k = part;
+    for (; k + (B - 1) * parts < P.split; k += B * parts) {
+      T v[B];
 #pragma unroll
-        for (int b = 0; b < B; b++) v[b] = load_fresh(partials + (thcl_u64)(k + b) * P.nslices + s);
+      for (int b = 0; b < B; b++) v[b] = load_fresh(partials + (thcl_u64)(k + b * parts) * P.nslices + sj);
 #pragma unroll
-        for (int b = 0; b < B; b++) t = S::comb(t, v[b]);
-      }
-      for (; k < P.split; k++) t = S::comb(t, load_fresh(partials + (thcl_u64)k * P.nslices + s));
-      S::store(P, s, t);
+      for (int b = 0; b < B; b++) t = S::comb(t, v[b]);
     }
+    for (; k < P.split; k += parts) t = S::comb(t, load_fresh(partials + (thcl_u64)k * P.nslices + sj));
+  }
+  T *meet = &lds[0][0];   // kThreads entries
+  meet[part * J + j] = t;
+  __syncthreads();
+  if (part == 0 && live) {
+    T r = meet[j];
+    for (thcl_u32 g = 1; g < parts; g++) r = S::comb(r, meet[g * J + j]);
+    S::store(P, sj, r);
   }
   if (threadIdx.x == 0) P.ticket[blockIdx.x] = 0u;
 }
@@ -879,8 +890,18 @@ __global__ __launch_bounds__(kThreads) void reduce_cols_finish(ReduceDimParams P
   const int sl = threadIdx.x % kFinSlices, part = threadIdx.x / kFinSlices;
   const thcl_u32 s = blockIdx.x * kFinSlices + sl;
   T r = S::init();
-  if (s < P.nslices)
-    for (thcl_u32 k = part; k < P.split; k += kFinParts) r = S::comb(r, partials[(thcl_u64)k * P.nslices + s]);
+  if (s < P.nslices) {
+    constexpr int B = 8;   // partials requested together (one after the other a long split of one slice took 24 us)
+    thcl_u32 k = part;
+    for (; k + (B - 1) * kFinParts < P.split; k += B * kFinParts) {
+      T v[B];
+#pragma unroll
+      for (int b = 0; b < B; b++) v[b] = partials[(thcl_u64)(k + b * kFinParts) * P.nslices + s];
+#pragma unroll
+      for (int b = 0; b < B; b++) r = S::comb(r, v[b]);
+    }
+    for (; k < P.split; k += kFinParts) r = S::comb(r, partials[(thcl_u64)k * P.nslices + s]);
+  }
   lds[part][sl] = r;
   __syncthreads();
   if (part == 0 && s < P.nslices) {
@@ -1316,6 +1337,9 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
           P.split = (thcl_u32)split;
           P.rows_per_split = (thcl_u32)rps;
           grid.y = (unsigned)split;
+          // (folding the pieces in the same launch, the last arrival at a ticket per slice, measured slower: these
+          // blocks live for a microsecond or two, and a write-through, its acknowledgement and an atomic at the end
+          // of each keep its CU slot twice as long: 64 x 2^20 41.4 -> 46.6 us, 16 x 2^22 44.2 -> 52.0)
         }
       }
     }
@@ -1370,9 +1394,9 @@ void thcl_reduce_dim(THClState *state, ThclReduce kind, THClTensor *values, THCl
     split = (R + rps - 1) / rps;
     P.split = (thcl_u32)split;
     P.rows_per_split = (thcl_u32)rps;
-    // One block folding a tile's partials is quick while they are few; a long
-    // split (few, tall slices) is folded by a second, chip-wide kernel.
-    P.fused = (split > 1 && split <= 32 && tiles <= (long)kColTickets) ? 1u : 0u;
+    // One block folding a tile's partials is quick while each of its threads has few of them to fetch (the tile's
+    // slices share the block's 256 threads); beyond 64 a thread the fold is left to a second, chip-wide kernel.
+    P.fused = (split > 1 && split * ub * vec <= 64 * (long)kThreads && tiles <= (long)kColTickets) ? 1u : 0u;
     grid.x = (unsigned)(tiles > (1l << 20) ? (1l << 20) : tiles);
     grid.y = (unsigned)split;
     }
