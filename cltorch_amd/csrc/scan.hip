@@ -311,11 +311,13 @@ __global__ __launch_bounds__(kThreads) void scan_row(ScanParams P) {
 // totals, PHASE 1 scans (from the segment's carry when the lines are cut into segments).
 // ANY: the width need not be a multiple of 4 nor the rows 16-byte aligned (narrow tensors only): a thread's up to 4
 // columns are read and written one element each, columns past the width are dead.
-template <bool PROD, int TC, int PHASE, bool ANY = false>
+template <bool PROD, int TC, int PHASE, bool ANY = false, bool HALF = false>
 __global__ __launch_bounds__(kThreads) void scan_strip(ScanParams P) {
   // rows per thread: 8; 2 on the narrowest strips, where a thread's 8 rows would be 128 or 256 contiguous
-  // bytes read 16 at a time (measured 0.6 TB/s on 4 columns against 2.0 with 2 rows)
-  constexpr int K = (TC >= 4 && !ANY) ? 8 : 2;  // element-wise strips: lanes that share an instruction stay 2 rows apart
+  // bytes read 16 at a time (measured 0.6 TB/s on 4 columns against 2.0 with 2 rows); HALF: 4, for launches of
+  // one block per CU (8192 x 8192: 104 -> 90 us, 4096 x 16384: 98 -> 88; with two blocks per CU or half a
+  // block 8 rows stay ahead: 2048 x 32768 99 against 102 us, 16384 x 4096 126 against 138)
+  constexpr int K = HALF ? 4 : (TC >= 4 && !ANY) ? 8 : 2;  // element-wise strips: lanes that share an instruction stay 2 rows apart
   constexpr int WAVES = kThreads / kWave, ROWS = kThreads / TC * K, CW = TC * 4;
   __shared__ double wave_tot[2][WAVES][CW];
   const thcl_u64 strips = ((P.I + 3) / 4 + TC - 1) / TC;
@@ -994,9 +996,15 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
     int strip_tc = 8;
     // strips of 64 columns (runs of 256 bytes) when those still give every CU a block: 4096 x 16384 104 -> 98 us,
     // 2048 x 32768 118 -> 99 us
+    // (unless they leave the CUs unevenly loaded where the narrower strips do not: 4096 x 20480 is 320 strips of 64
+    // columns, two rounds of blocks on 256 CUs for 1.25 rounds of work, 157 us against 146 in 640 strips of 32)
     if (strip && P.O * ((P.I / 4 + 15) / 16) >= (thcl_u64)cus) {
-      strip_tc = 16;
-      strips = P.O * ((P.I / 4 + 15) / 16);
+      const thcl_u64 wide = P.O * ((P.I / 4 + 15) / 16);
+      auto balance = [&](thcl_u64 blocks) { return (double)blocks / (double)((blocks + cus - 1) / cus * cus); };
+      if (balance(wide) * 1.08 >= balance(strips)) {
+        strip_tc = 16;
+        strips = wide;
+      }
     }
     bool narrow = false, narrow_any = false;
     // (from 1.5 million elements per tensor slice up: below that the three launches of the strips cost more than the
@@ -1065,8 +1073,12 @@ void thcl_scan_dim(THClState *state, bool prod, THClTensor *self, THClTensor *sr
       check("scan");
     } else if (strip) {
       const dim3 grid((unsigned)(strips * P.S)), block(kThreads);
+      // one block on (nearly) every CU and two on none: four rows a thread instead of eight (with 1.125 to 1.375
+      // blocks per CU the CUs that hold two set the time and prefer eight rows: 4096 x 10240 84 us against 89)
+      const bool strip_half = !narrow && strip_tc >= 8 && strips * P.S * 5 >= (thcl_u64)cus * 4 && strips * P.S <= (thcl_u64)cus;
 #define STRIP_CASE(PR, TC_, PH)                                                                               \
   if (narrow_any) hipLaunchKernelGGL((scan_strip<PR, TC_, PH, true>), grid, block, 0, stream, P);              \
+  else if (strip_half && TC_ >= 8) hipLaunchKernelGGL((scan_strip<PR, (TC_ >= 8 ? TC_ : 8), PH, false, true>), grid, block, 0, stream, P); \
   else hipLaunchKernelGGL((scan_strip<PR, TC_, PH, false>), grid, block, 0, stream, P);
 #define STRIP_PHASE(PH)                                                                                        \
   switch (strip_tc * 2 + (prod ? 1 : 0)) {                                                                     \
