@@ -78,9 +78,11 @@ float *thcl_rt_host_word(thcl_rt *rt);
  * directly, and the host reads it after thcl_rt_sync (no copy in between) */
 float *thcl_rt_host_word_device(thcl_rt *rt);
 
-/* A pinned word, at the address kernels use, that a kernel sets to non-zero when it meets input
- * the host must hear about (an index outside its range).  thcl_rt_sync and thcl_rt_memcpy_d2h
- * look at it after they have waited: if it is set they clear it and return -3 with a message. */
+/* A pinned word, at the address kernels use, that a kernel sets to non-zero when the host must hear
+ * about something: 1 = an index outside its range (that entry moved nothing), 2 = a wait inside a
+ * single-pass scan ran out because its blocks did not run at the same time (that scan's result is
+ * not valid).  thcl_rt_sync and thcl_rt_memcpy_d2h look at it after they have waited: if it is set
+ * they clear it and return -3 with a message. */
 unsigned *thcl_rt_fault_word_device(thcl_rt *rt);
 /* The same look without a wait, for a caller that has just waited for the stream by other means (its own event, a
  * copy through another library): 0, or -3 with the message after clearing the word. */
