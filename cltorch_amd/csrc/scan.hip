@@ -846,7 +846,7 @@ void launch_carries(hipStream_t stream, const ScanParams &P) {
 template <bool PROD>
 bool run_chain(thcl_rt *rt, hipStream_t stream, const ScanParams &S) {
   static int per_cu = -1;   // blocks of scan_chain a CU holds at a time, at most 2
-  static thcl_u32 spin_limit = 1u << 20, mute = ~0u;
+  static thcl_u32 spin_limit = 1u << 23, mute = ~0u;   // some seconds of polling before a wait gives up
   if (per_cu < 0) {
     int nb = 0, nbp = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, scan_chain<false>, kThreads, 0) != hipSuccess) nb = 0;
