@@ -1,7 +1,8 @@
 """Many launches in a row of every kernel whose blocks hand partial results to one another
 (reduce-all dense and strided, dot, the column reduction that folds its splits in the same
 launch, the column and row reductions with a finishing kernel, the matrix-vector kernels with
-partials, the K-sliced matrix product), on inputs with closed-form answers: all ones, 1..n,
+partials, the K-sliced matrix product and the one whose surplus tiles share their K, the single-pass scan
+whose blocks hand their totals on while they run), on inputs with closed-form answers: all ones, 1..n,
 and a matrix whose column maxima sit at known rows.  Every result of every launch is compared
 exactly and the test stops at the first mismatch.  The launches of a round are queued without
 waiting in between, so kernels that share tickets and partial slots follow one another the
@@ -47,6 +48,12 @@ def test_two_thousand_launches_with_closed_form_results(cl):
     vlong, v4 = cl.ClTensor(1 << 22).fill(1.0), cl.ClTensor(4).fill(1.0)
     M, N, K = 64, 4096, 4096
     A, B = cl.ClTensor(M * K).fill(1.0).resize(M, K), cl.ClTensor(K * N).fill(0.5).resize(K, N)
+    # 17 x 17 tiles of 128: the 33 tiles beyond the CUs' whole share are computed by several blocks each along K
+    T2, K2 = 2176, 512
+    A2, B2 = cl.ClTensor(T2 * K2).fill(1.0).resize(T2, K2), cl.ClTensor(K2 * T2).fill(0.5).resize(K2, T2)
+    # two rows of 2^23 ones: scanned in one pass by blocks that run together and pass their chunk totals along
+    scan_rows = cl.ClTensor(2 << 23).fill(1.0).resize(2, 1 << 23)
+    scan_want = np.tile(np.arange(1, (1 << 23) + 1, dtype=F), 2)
 
     launches = 0
     for rnd in range(ROUNDS):
@@ -77,6 +84,10 @@ def test_two_thousand_launches_with_closed_form_results(cl):
         checks.append(("ones(2^22 x 4) . ones", ylong.addmv(0.0, 1.0, mv.t(), v4), np.full(1 << 22, 4.0, dtype=F)))
         Cm = cl.ClTensor(M, N).fill(1.0)
         checks.append(("K-sliced product of constants", Cm.addmm(0.5, 1.0, A, B), np.full((M, N), 0.5 + K * 0.5, dtype=F)))
+        C2 = cl.ClTensor(T2, T2).fill(1.0)
+        checks.append(("product whose last tiles share their K", C2.addmm(0.5, 1.0, A2, B2), np.full((T2, T2), 0.5 + K2 * 0.5, dtype=F)))
+        if rnd % 4 == 0:
+            checks.append(("running sums of two rows of 2^23 ones", scan_rows.cumsum(2), scan_want))
         assert ones[1 << 20].dot(ones[1 << 20]) == float(1 << 20), f"round {rnd}: dot of ones"   # waits for its result
         launches += len(checks) + 5                                 # + the fills above
         cl.synchronize()
