@@ -6,7 +6,7 @@
 //
 // The tensor is taken as dense [O][R][I] (outer, scanned, inner).  Numerics
 // follow Torch7's CPU path: the running value is fp64 and every output is its
-// rounding to fp32.  Four kernels:
+// rounding to fp32.  The kernels:
 //   * scan_seq: one thread per (o, i) walks r; adjacent threads are adjacent in
 //     i, so accesses coalesce whenever I is not tiny.
 //   * scan_row: I == 1 and long rows; a block walks the row 1024 elements at a
@@ -16,9 +16,11 @@
 //   * scan_wave_rows: I == 1 and many aligned rows of 1024 to 8191 elements; a
 //     wave per row with the next 1024 elements requested ahead.
 //   * scan_strip: I > 1 with fewer columns than the chip has threads; a block
-//     walks 32 columns, 256 rows a step.
-// When O * I alone cannot fill the chip, R is cut into S segments and the scan
-// becomes three passes: segment totals, an exclusive scan of the totals, then
+//     walks 32 or 64 columns, 64 to 256 rows a step.
+//   * scan_chain: I == 1 and rows too few for a block each, 2^24 elements and more:
+//     one pass by blocks that run together and hand their chunk totals on.
+// When O * I alone cannot fill the chip otherwise, R is cut into S segments and the
+// scan becomes three passes: segment totals, an exclusive scan of the totals, then
 // the scan proper with each segment's carry-in.
 #include <hip/hip_runtime.h>
 
