@@ -677,7 +677,7 @@ __global__ __launch_bounds__(kThreads) void reduce_cols(ReduceDimParams P) {
       }
       // this wave takes rows r_begin + wave, + WAVES, ...; FLY of them are loaded
       // before any is consumed, the address advances by a constant step
-      constexpr int FLY = 8;
+      constexpr int FLY = 4;   // (batches of 8 rows: the arg-max of 4096 x 16384 along dim 1 took 41.5 us against 40.0, sums the same)
       thcl_u32 r = r_begin + wave * RL + rl;
       const float *ptr = P.in + off + (thcl_u64)r * P.rstride;
       const thcl_u64 step = (thcl_u64)RSTEP * P.rstride;
